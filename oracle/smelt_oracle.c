@@ -1,0 +1,689 @@
+/*
+ * smelt_oracle.c — CPU restatement of Smelt's quantized-weight numerics.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker that the HIP kernels are
+ * compared against; nothing that ships (the C-ABI runtime, the kernels, the
+ * record emitters) links, loads or calls it.  Only tests/, the smoke check and
+ * the benchmark's cpu_baseline leg may use it.
+ *
+ * Every function cites the reference file:line it restates (paths relative to
+ * the Smelt repository root).  Scalar C, no dependencies, one translation unit.
+ *
+ * Pin status (what fixes each function independently of this file):
+ *   - f16/bf16 conversions ........ exhaustive vs numpy float16 / closed form
+ *   - affine_u4 pack + dequant .... SmeltAffineU4Tests.swift:67-80,120-128
+ *   - binary1/ternary2 codec ...... SmeltSignedQuantCodecTests.swift:16-107
+ *   - MLX scale normalisation ..... SmeltSignedQuantCodecTests.swift:109-204
+ *   - ternary affine QMV .......... MLX golden bits, SignedQuantKernelTests.swift:87-199
+ *   - affine / signed matvec ...... exact-rational recomputation on dyadic fixtures,
+ *                                   brute-force dequant-then-dot cross-check
+ *   - argmax key .................. special cases (ties, signed zero) + brute force
+ *   - trit5 codec ................. PARITY UNPINNED BY THE REFERENCE: the format does
+ *                                   not exist there; pinned by closed form, exhaustive
+ *                                   243-entry check and agreement with ternary2
+ *   - signed SwiGLU epilogue ...... PARITY UNPINNED: Metal's half-precision exp() is not
+ *                                   specified bit-exactly; restated with fp32 expf rounded
+ *                                   to fp16 at each materialisation point
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#define SO_EXPORT __attribute__((visibility("default")))
+
+/* error codes mirror SmeltSignedQuantError (SmeltSignedQuantCodec.swift:38-68) */
+enum {
+    SO_OK = 0,
+    SO_ERR_GEOMETRY = -1,
+    SO_ERR_BUFFER_TOO_SMALL = -2,
+    SO_ERR_INVALID_CODE = -3,
+    SO_ERR_MLX_SCALE = -4,
+    SO_ERR_MLX_BIAS = -5,
+};
+
+/* element types for activations / scales */
+enum { SO_F16 = 0, SO_BF16 = 1, SO_F32 = 2 };
+/* signed formats: binary1 / ternary2 follow SmeltSignedQuantFormat; trit5 is new */
+enum { SO_BINARY1 = 0, SO_TERNARY2 = 1, SO_TRIT5 = 2 };
+
+/* ------------------------------------------------------------------------- */
+/* IEEE conversions. Swift Float16(x) is round-to-nearest-even narrowing and   */
+/* Float(Float16) is exact widening.                                           */
+/* ------------------------------------------------------------------------- */
+
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+SO_EXPORT float so_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    if (exp == 0) {
+        if (man == 0) return bits_f32(sign);
+        /* subnormal: value = man * 2^-24 */
+        float v = (float)man * 5.9604644775390625e-08f;
+        return (sign ? -v : v);
+    }
+    if (exp == 31) return bits_f32(sign | 0x7F800000u | (man << 13));
+    return bits_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+SO_EXPORT uint16_t so_f32_to_f16(float f) {
+    uint32_t x = f32_bits(f);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t absx = x & 0x7FFFFFFFu;
+    if (absx >= 0x7F800000u) { /* inf / nan */
+        if (absx > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((absx >> 13) & 0x3FFu));
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (absx >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u); /* rounds to inf: >= 65520 */
+    if (absx < 0x33000001u) return sign;                          /* <= 2^-25 rounds to zero */
+    int32_t e = (int32_t)(absx >> 23) - 127;
+    uint32_t m = (absx & 0x7FFFFFu) | 0x800000u; /* 24-bit significand */
+    uint32_t shift;
+    uint32_t base;
+    if (e < -14) { /* subnormal result: units of 2^-24 */
+        shift = (uint32_t)(13 + (-14 - e));
+        base = 0;
+    } else {
+        shift = 13;
+        base = ((uint32_t)(e + 15) << 10) - 0x400u; /* hidden bit adds 0x400 back */
+    }
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q += 1;
+    return (uint16_t)(sign | (base + q));
+}
+
+/* SmeltBF16.swift:6-15 */
+SO_EXPORT uint16_t so_f32_to_bf16(float f) {
+    uint32_t bits = f32_bits(f);
+    uint32_t rounded = bits + 0x7FFFu + ((bits >> 16) & 1u);
+    return (uint16_t)(rounded >> 16);
+}
+SO_EXPORT float so_bf16_to_f32(uint16_t v) { return bits_f32((uint32_t)v << 16); }
+
+static inline float widen(uint16_t bits, int dtype) {
+    return dtype == SO_BF16 ? so_bf16_to_f32(bits) : so_f16_to_f32(bits);
+}
+static inline uint16_t narrow(float v, int dtype) {
+    return dtype == SO_BF16 ? so_f32_to_bf16(v) : so_f32_to_f16(v);
+}
+SO_EXPORT float so_round_through(float v, int dtype) {
+    if (dtype == SO_F32) return v;
+    return widen(narrow(v, dtype), dtype);
+}
+
+/* ------------------------------------------------------------------------- */
+/* affine_u4 — SmeltAffineU4.swift                                             */
+/* ------------------------------------------------------------------------- */
+
+/* SmeltAffineU4.swift:17-19 */
+SO_EXPORT int so_affine_num_groups(int cols, int group) { return (cols + group - 1) / group; }
+/* SmeltAffineU4.swift:22-23 */
+SO_EXPORT int so_affine_packed_row_stride(int cols) { return (cols + 1) / 2; }
+
+/* SmeltAffineU4.swift:30-34 — scale = (hi-lo)/15, bias = lo, degenerate range -> scale 1 */
+SO_EXPORT void so_affine_params(float lo, float hi, int dtype, float *scale, float *bias,
+                                uint16_t *scale_bits, uint16_t *bias_bits) {
+    float range = hi - lo;
+    float s = range < 1e-12f ? 1.0f : range / 15.0f;
+    *scale = s;
+    *bias = lo;
+    *scale_bits = narrow(s, dtype);
+    *bias_bits = narrow(lo, dtype);
+}
+
+/* SmeltAffineU4.swift:59-91 — endpoint choice; clip 0 = minMax, 1 = mseOptimal */
+static void clip_endpoints(const float *values, int c0, int c1, float minv, float maxv, int clip,
+                           const float *importance, int dtype, float *lo_out, float *hi_out) {
+    if (clip == 0) { *lo_out = minv; *hi_out = maxv; return; }
+    float half = (maxv - minv) / 2;
+    if (half < 1e-12f) { *lo_out = minv; *hi_out = maxv; return; }
+    float best_lo = minv, best_hi = maxv, best_err = INFINITY;
+    for (int step = 0; step <= 8; ++step) {
+        float c = 1.0f - (float)step * 0.075f;
+        float lo = minv + (1 - c) * half, hi = maxv - (1 - c) * half;
+        float scale = (hi - lo) / 15.0f;
+        float scale_f = so_round_through(scale, dtype), lo_f = so_round_through(lo, dtype);
+        float inv = 1.0f / scale;
+        float err = 0;
+        for (int k = c0; k < c1; ++k) {
+            float v = values[k];
+            float nib = fminf(fmaxf(roundf((v - lo) * inv), 0.0f), 15.0f);
+            float d = v - (nib * scale_f + lo_f);
+            err += (importance ? importance[k] : 1.0f) * d * d;
+        }
+        if (err < best_err) { best_err = err; best_lo = lo; best_hi = hi; }
+    }
+    *lo_out = best_lo; *hi_out = best_hi;
+}
+
+/* SmeltAffineU4.swift:94-136. Swift's .rounded() is round-half-away-from-zero = roundf. */
+SO_EXPORT void so_affine_quantize_row(const float *values, int cols, int group, int clip,
+                                      const float *importance, int dtype, uint8_t *packed,
+                                      uint16_t *scales, uint16_t *biases) {
+    int groups = so_affine_num_groups(cols, group);
+    for (int g = 0; g < groups; ++g) {
+        int c0 = g * group;
+        int c1 = c0 + group < cols ? c0 + group : cols;
+        float minv = INFINITY, maxv = -INFINITY;
+        for (int c = c0; c < c1; ++c) {
+            float v = values[c];
+            if (v < minv) minv = v;
+            if (v > maxv) maxv = v;
+        }
+        float lo, hi, scale, bias;
+        clip_endpoints(values, c0, c1, minv, maxv, clip, importance, dtype, &lo, &hi);
+        so_affine_params(lo, hi, dtype, &scale, &bias, &scales[g], &biases[g]);
+        float inv = 1.0f / scale;
+        for (int c = c0; c < c1; ++c) {
+            float normalized = (values[c] - bias) * inv;
+            float clamped = fminf(fmaxf(normalized, 0.0f), 15.0f);
+            uint8_t nib = (uint8_t)roundf(clamped);
+            int bi = c >> 1;
+            if ((c & 1) == 0) packed[bi] = nib;
+            else packed[bi] |= (uint8_t)(nib << 4);
+        }
+    }
+}
+
+/* SmeltAffineU4.swift:141-161: out[c] = Float(nibble) * scale + bias (one mul, one add). */
+SO_EXPORT void so_affine_dequantize_row(const uint8_t *packed, const uint16_t *scales,
+                                        const uint16_t *biases, int cols, int group, int dtype,
+                                        float *out) {
+    int groups = so_affine_num_groups(cols, group);
+    for (int g = 0; g < groups; ++g) {
+        int c0 = g * group;
+        int c1 = c0 + group < cols ? c0 + group : cols;
+        float scale = widen(scales[g], dtype);
+        float bias = widen(biases[g], dtype);
+        for (int c = c0; c < c1; ++c) {
+            uint8_t byte = packed[c >> 1];
+            uint8_t nib = (c & 1) == 0 ? (byte & 0x0F) : (byte >> 4);
+            volatile float prod = (float)nib * scale; /* forbid fma contraction */
+            out[c] = prod + bias;
+        }
+    }
+}
+
+/* SmeltRuntime.swift:2522-2595 — embedding-row form: Float16(Float(nib)*scale+bias) */
+SO_EXPORT void so_affine_dequantize_row_narrow(const uint8_t *packed, const uint16_t *scales,
+                                               const uint16_t *biases, int cols, int group,
+                                               int dtype, int out_dtype, uint16_t *out) {
+    int groups = so_affine_num_groups(cols, group);
+    int stride = so_affine_packed_row_stride(cols);
+    int bytes_per_group = group / 2;
+    for (int g = 0; g < groups; ++g) {
+        float scale = widen(scales[g], dtype);
+        float bias = widen(biases[g], dtype);
+        int c1 = (g + 1) * group < cols ? (g + 1) * group : cols;
+        int b0 = g * bytes_per_group;
+        int b1 = b0 + bytes_per_group < stride ? b0 + bytes_per_group : stride;
+        for (int b = b0; b < b1; ++b) {
+            uint8_t byte = packed[b];
+            int col0 = b * 2;
+            if (col0 < c1) {
+                volatile float p = (float)(byte & 0x0F) * scale;
+                out[col0] = narrow(p + bias, out_dtype);
+            }
+            if (col0 + 1 < c1) {
+                volatile float p = (float)(byte >> 4) * scale;
+                out[col0 + 1] = narrow(p + bias, out_dtype);
+            }
+        }
+    }
+}
+
+/* MetalKernelTestSupport.swift:396-428 / PrefillKernelTests.swift:266-300.
+ * Group-wise  acc += scale*dot + bias*xsum  in fp32, sequential order; result unrounded. */
+SO_EXPORT void so_affine_matvec(const uint8_t *packed, const uint16_t *scales,
+                                const uint16_t *biases, const float *x, int rows, int cols,
+                                int group, int dtype, float *out) {
+    int gpr = cols / group;
+    int stride = cols / 2;
+    for (int r = 0; r < rows; ++r) {
+        const uint8_t *w = packed + (size_t)r * stride;
+        float acc = 0;
+        for (int g = 0; g < gpr; ++g) {
+            float scale = widen(scales[(size_t)r * gpr + g], dtype);
+            float bias = widen(biases[(size_t)r * gpr + g], dtype);
+            int cb = g * group;
+            float dot = 0, xsum = 0;
+            for (int i = 0; i < group; ++i) {
+                int col = cb + i;
+                uint8_t byte = w[col / 2];
+                uint8_t nib = (col & 1) == 0 ? (byte & 0x0F) : (byte >> 4);
+                dot += (float)nib * x[col];
+                xsum += x[col];
+            }
+            acc += scale * dot + bias * xsum;
+        }
+        out[r] = acc;
+    }
+}
+
+/* Independent formulation used to cross-check so_affine_matvec: dequantise each
+ * element (SmeltAffineU4.swift:141-161) and accumulate the dot product in double. */
+SO_EXPORT void so_affine_matvec_dequant_f64(const uint8_t *packed, const uint16_t *scales,
+                                            const uint16_t *biases, const float *x, int rows,
+                                            int cols, int group, int dtype, double *out) {
+    int gpr = so_affine_num_groups(cols, group);
+    int stride = so_affine_packed_row_stride(cols);
+    for (int r = 0; r < rows; ++r) {
+        double acc = 0;
+        for (int c = 0; c < cols; ++c) {
+            uint8_t byte = packed[(size_t)r * stride + (c >> 1)];
+            uint8_t nib = (c & 1) == 0 ? (byte & 0x0F) : (byte >> 4);
+            float s = widen(scales[(size_t)r * gpr + c / group], dtype);
+            float b = widen(biases[(size_t)r * gpr + c / group], dtype);
+            volatile float p = (float)nib * s;
+            float w = p + b;
+            acc += (double)w * (double)x[c];
+        }
+        out[r] = acc;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* signed codec — SmeltSignedQuantCodec.swift                                  */
+/* ------------------------------------------------------------------------- */
+
+static inline int bits_per_code(int format) { return format == SO_BINARY1 ? 1 : 2; }
+
+/* SmeltSignedQuantCodec.swift:72-84 (trit5: ceil(n/5) bytes) */
+SO_EXPORT int64_t so_signed_packed_byte_count(int64_t logical_count, int format) {
+    if (logical_count < 0) return SO_ERR_GEOMETRY;
+    if (format == SO_TRIT5) return (logical_count + 4) / 5;
+    return (logical_count * bits_per_code(format) + 7) / 8;
+}
+
+/* SmeltSignedQuantCodec.swift:88-98 */
+SO_EXPORT int so_signed_groups_per_row(int padded_cols, int group) {
+    if (padded_cols <= 0) return SO_ERR_GEOMETRY;
+    if (group <= 0 || padded_cols % group != 0) return SO_ERR_GEOMETRY;
+    return padded_cols / group;
+}
+
+/* SmeltSignedQuantCodec.swift:102-124 — LSB-first code extraction */
+SO_EXPORT int so_signed_code_at(int64_t index, const uint8_t *bytes, int64_t byte_count,
+                                int format) {
+    if (index < 0) return SO_ERR_GEOMETRY;
+    if (format == SO_TRIT5) {
+        int64_t bi = index / 5;
+        if (bi >= byte_count) return SO_ERR_BUFFER_TOO_SMALL;
+        unsigned v = bytes[bi];
+        if (v >= 243) return SO_ERR_INVALID_CODE;
+        for (int i = (int)(index % 5); i > 0; --i) v /= 3;
+        return (int)(v % 3);
+    }
+    int bpc = bits_per_code(format);
+    int64_t bit = index * bpc;
+    int64_t bi = bit >> 3;
+    if (bi >= byte_count) return SO_ERR_BUFFER_TOO_SMALL;
+    int shift = (int)(bit & 7);
+    int mask = (1 << bpc) - 1;
+    return (bytes[bi] >> shift) & mask;
+}
+
+/* SmeltSignedQuantCodec.swift:22-35 */
+SO_EXPORT int so_signed_semantic(int format, int packed_code, int *out) {
+    if (format == SO_BINARY1) {
+        if (packed_code >= 2 || packed_code < 0) return SO_ERR_INVALID_CODE;
+        *out = packed_code == 0 ? -1 : 1;
+        return SO_OK;
+    }
+    if (packed_code >= 3 || packed_code < 0) return SO_ERR_INVALID_CODE;
+    *out = packed_code - 1;
+    return SO_OK;
+}
+
+/* SmeltSignedQuantCodec.swift:128-145; on failure *bad_index = first offending index */
+SO_EXPORT int so_signed_validate_codes(const uint8_t *bytes, int64_t byte_count,
+                                       int64_t logical_count, int format, int64_t *bad_index) {
+    int64_t need = so_signed_packed_byte_count(logical_count, format);
+    if (need < 0) return (int)need;
+    if (byte_count < need) return SO_ERR_BUFFER_TOO_SMALL;
+    if (format == SO_BINARY1) return SO_OK;
+    for (int64_t i = 0; i < logical_count; ++i) {
+        int v = so_signed_code_at(i, bytes, byte_count, format);
+        if (v == 3 || v == SO_ERR_INVALID_CODE) {
+            if (bad_index) *bad_index = i;
+            return SO_ERR_INVALID_CODE;
+        }
+    }
+    return SO_OK;
+}
+
+static int f16_is_finite(uint16_t h) { return ((h >> 10) & 0x1F) != 31; }
+static float f16_ulp(uint16_t h) {
+    /* Swift Float16.ulp: spacing at |h|; for zero/subnormal it is the least nonzero value */
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    if (exp == 0) return 5.9604644775390625e-08f;
+    return ldexpf(1.0f, (int)exp - 15 - 10);
+}
+
+/* SmeltSignedQuantCodec.swift:180-215 */
+SO_EXPORT int so_signed_canonical_mlx_scale_bits(int format, uint16_t source_scale_bits,
+                                                 uint16_t bias_bits, uint16_t *out) {
+    float source = so_f16_to_f32(source_scale_bits);
+    if (!f16_is_finite(source_scale_bits) || !(source >= 0)) return SO_ERR_MLX_SCALE;
+    uint16_t canonical = format == SO_BINARY1 ? so_f32_to_f16(source * 0.5f) : source_scale_bits;
+    float canonical_f = so_f16_to_f32(canonical);
+    uint16_t expected_bias = so_f32_to_f16(-canonical_f);
+    float actual = so_f16_to_f32(bias_bits);
+    int equivalent = f16_is_finite(bias_bits) && actual <= 0 &&
+                     fabsf(actual - so_f16_to_f32(expected_bias)) <= f16_ulp(canonical);
+    if (!(bias_bits == expected_bias || equivalent)) return SO_ERR_MLX_BIAS;
+    *out = canonical;
+    return SO_OK;
+}
+
+/* SmeltSignedQuantCodec.swift:154-176; on failure *bad_group is the failing group */
+SO_EXPORT int so_signed_normalize_mlx_scales(int format, const uint16_t *scales,
+                                             const uint16_t *biases, int group_count,
+                                             uint16_t *out, int *bad_group) {
+    if (group_count < 0) return SO_ERR_GEOMETRY;
+    for (int g = 0; g < group_count; ++g) {
+        int rc = so_signed_canonical_mlx_scale_bits(format, scales[g], biases[g], &out[g]);
+        if (rc != SO_OK) { if (bad_group) *bad_group = g; return rc; }
+    }
+    return SO_OK;
+}
+
+/* SmeltSignedQuantCodec.swift:219-257 (fp32 row) */
+SO_EXPORT int so_signed_dequantize_row(int format, const uint8_t *codes, int64_t code_bytes,
+                                       const uint16_t *scales, int64_t scale_bytes, int cols,
+                                       int padded_cols, int group, float *out) {
+    if (cols <= 0 || cols > padded_cols) return SO_ERR_GEOMETRY;
+    int groups = so_signed_groups_per_row(padded_cols, group);
+    if (groups < 0) return groups;
+    int64_t need = so_signed_packed_byte_count(padded_cols, format);
+    if (code_bytes < need) return SO_ERR_BUFFER_TOO_SMALL;
+    if (scale_bytes < (int64_t)groups * 2) return SO_ERR_BUFFER_TOO_SMALL;
+    int rc = so_signed_validate_codes(codes, code_bytes, padded_cols, format, NULL);
+    if (rc != SO_OK) return rc;
+    for (int col = 0; col < cols; ++col) {
+        int packed = so_signed_code_at(col, codes, code_bytes, format);
+        int sem;
+        rc = so_signed_semantic(format, packed, &sem);
+        if (rc != SO_OK) return rc;
+        out[col] = (float)sem * so_f16_to_f32(scales[col / group]);
+    }
+    return SO_OK;
+}
+
+/* SmeltSignedQuantCodec.swift:262-324 (fp16 row) */
+SO_EXPORT int so_signed_dequantize_row_f16(int format, const uint8_t *codes, int64_t code_bytes,
+                                           const uint16_t *scales, int64_t scale_bytes, int cols,
+                                           int padded_cols, int group, uint16_t *out) {
+    if (cols <= 0 || cols > padded_cols) return SO_ERR_GEOMETRY;
+    int groups = so_signed_groups_per_row(padded_cols, group);
+    if (groups < 0) return groups;
+    int64_t need = so_signed_packed_byte_count(padded_cols, format);
+    if (code_bytes < need) return SO_ERR_BUFFER_TOO_SMALL;
+    if (scale_bytes < (int64_t)groups * 2) return SO_ERR_BUFFER_TOO_SMALL;
+    int rc = so_signed_validate_codes(codes, code_bytes, padded_cols, format, NULL);
+    if (rc != SO_OK) return rc;
+    for (int col = 0; col < cols; ++col) {
+        int packed = so_signed_code_at(col, codes, code_bytes, format);
+        int sem;
+        rc = so_signed_semantic(format, packed, &sem);
+        if (rc != SO_OK) return rc;
+        out[col] = so_f32_to_f16((float)sem * so_f16_to_f32(scales[col / group]));
+    }
+    return SO_OK;
+}
+
+/* Test-fixture packer, SignedQuantKernelTests.swift:7-22 (LSB-first, row stride
+ * cols*bits/8) and the trit5 closed form byte = sum d_i * 3^i (digit 0 = lowest
+ * column; tail digits beyond cols encode 1, i.e. semantic zero). */
+SO_EXPORT void so_signed_pack_row(int format, const uint8_t *codes, int cols, uint8_t *out,
+                                  int64_t out_bytes) {
+    memset(out, 0, (size_t)out_bytes);
+    if (format == SO_TRIT5) {
+        for (int64_t b = 0; b < out_bytes; ++b) {
+            unsigned v = 0, p = 1;
+            for (int i = 0; i < 5; ++i) {
+                int64_t c = b * 5 + i;
+                unsigned d = c < cols ? codes[c] : 1u;
+                v += d * p;
+                p *= 3;
+            }
+            out[b] = (uint8_t)v;
+        }
+        return;
+    }
+    int bpc = bits_per_code(format);
+    for (int c = 0; c < cols; ++c) {
+        int bit = c * bpc;
+        out[bit / 8] |= (uint8_t)(codes[c] << (bit & 7));
+    }
+}
+
+/* trit5 decode table: entry[byte] packs five 2-bit ternary2-style codes (digit i at
+ * bits 2i..2i+1); bytes 243..255 are invalid and map to 0xFFFF. */
+SO_EXPORT void so_trit5_build_lut(uint16_t *lut256) {
+    for (unsigned b = 0; b < 256; ++b) {
+        if (b >= 243) { lut256[b] = 0xFFFFu; continue; }
+        unsigned v = b, e = 0;
+        for (int i = 0; i < 5; ++i) { e |= (v % 3) << (2 * i); v /= 3; }
+        lut256[b] = (uint16_t)e;
+    }
+}
+
+/* SignedQuantKernelTests.swift:1030-1045: expected += x * semantic * scale, fp32, in
+ * column order; result unrounded. x is [batch, cols] already widened to fp32. */
+SO_EXPORT int so_signed_matvec(int format, const uint8_t *codes, int64_t row_stride,
+                               const uint16_t *scales, const float *x, int rows, int cols,
+                               int padded_cols, int group, int batch, float *out) {
+    int groups = so_signed_groups_per_row(padded_cols, group);
+    if (groups < 0) return groups;
+    for (int b = 0; b < batch; ++b) {
+        for (int r = 0; r < rows; ++r) {
+            const uint8_t *row = codes + (size_t)r * row_stride;
+            float expected = 0;
+            for (int c = 0; c < cols; ++c) {
+                int packed = so_signed_code_at(c, row, row_stride, format);
+                int sem;
+                int rc = so_signed_semantic(format, packed, &sem);
+                if (rc != SO_OK) return rc;
+                expected += x[(size_t)b * cols + c] * (float)sem *
+                            so_f16_to_f32(scales[(size_t)r * groups + c / group]);
+            }
+            out[(size_t)b * rows + r] = expected;
+        }
+    }
+    return SO_OK;
+}
+
+/* Cross-check formulation: per-group exact integer-weighted sums in double. */
+SO_EXPORT int so_signed_matvec_f64(int format, const uint8_t *codes, int64_t row_stride,
+                                   const uint16_t *scales, const float *x, int rows, int cols,
+                                   int padded_cols, int group, int batch, double *out) {
+    int groups = so_signed_groups_per_row(padded_cols, group);
+    if (groups < 0) return groups;
+    for (int b = 0; b < batch; ++b)
+        for (int r = 0; r < rows; ++r) {
+            const uint8_t *row = codes + (size_t)r * row_stride;
+            double acc = 0;
+            for (int g = 0; g < groups; ++g) {
+                double part = 0;
+                int c1 = (g + 1) * group < cols ? (g + 1) * group : cols;
+                for (int c = g * group; c < c1; ++c) {
+                    int packed = so_signed_code_at(c, row, row_stride, format);
+                    int sem;
+                    int rc = so_signed_semantic(format, packed, &sem);
+                    if (rc != SO_OK) return rc;
+                    part += (double)sem * (double)x[(size_t)b * cols + c];
+                }
+                acc += part * (double)so_f16_to_f32(scales[(size_t)r * groups + g]);
+            }
+            out[(size_t)b * rows + r] = acc;
+        }
+    return SO_OK;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Ternary "affine" QMV, the arithmetic of MLX affine_qmv_fast<half,128,2>     */
+/* signed_quant_precise.metal:8-25 (qdot16) and :41-108 (kernel).              */
+/* x is fp16 bits [batch, cols]; out fp16 bits [batch, rows].                  */
+/* Lane l of a 32-wide simdgroup owns 16 columns of each 512-column block.     */
+/* ------------------------------------------------------------------------- */
+
+static inline float h2f(uint16_t h) { return so_f16_to_f32(h); }
+static inline float hround(float v) { return so_f16_to_f32(so_f32_to_f16(v)); }
+
+SO_EXPORT void so_ternary_affine_qmv(const uint8_t *codes, const uint16_t *scales,
+                                     const uint16_t *bias_scales, const uint16_t *x, int rows,
+                                     int cols, int batch, uint16_t *out) {
+    const int G = 128, VPL = 16, BLOCK = VPL * 32;
+    int groups = cols / G;
+    int row_bytes = cols / 4;
+    for (int b = 0; b < batch; ++b) {
+        const uint16_t *xb = x + (size_t)b * cols;
+        for (int r = 0; r < rows; ++r) {
+            float lane_result[32];
+            for (int lane = 0; lane < 32; ++lane) {
+                float result = 0;
+                for (int block = 0; block < cols; block += BLOCK) {
+                    int col = block + lane * VPL;
+                    if (col >= cols) continue;
+                    float xt[16];
+                    float sum = 0;
+                    for (int i = 0; i < VPL; i += 4) {
+                        /* half-typed a+b+c+d, then widened into the float accumulator */
+                        float h = hround(h2f(xb[col + i]) + h2f(xb[col + i + 1]));
+                        h = hround(h + h2f(xb[col + i + 2]));
+                        h = hround(h + h2f(xb[col + i + 3]));
+                        sum += h;
+                        xt[i + 0] = h2f(xb[col + i + 0]);
+                        xt[i + 1] = h2f(xb[col + i + 1]) / 4.0f;
+                        xt[i + 2] = h2f(xb[col + i + 2]) / 16.0f;
+                        xt[i + 3] = h2f(xb[col + i + 3]) / 64.0f;
+                    }
+                    uint32_t packed_codes;
+                    memcpy(&packed_codes, codes + (size_t)r * row_bytes + col / 4, 4);
+                    float scale = h2f(scales[(size_t)r * groups + col / G]);
+                    float bias = -h2f(bias_scales[(size_t)r * groups + col / G]);
+                    float accum = 0;
+                    for (int i = 0; i < 4; ++i) {
+                        uint32_t p = (packed_codes >> (i * 8)) & 0xFFu;
+                        volatile float t0 = xt[4 * i + 0] * (float)(p & 0x03u);
+                        volatile float t1 = xt[4 * i + 1] * (float)(p & 0x0Cu);
+                        volatile float t2 = xt[4 * i + 2] * (float)(p & 0x30u);
+                        volatile float t3 = xt[4 * i + 3] * (float)(p & 0xC0u);
+                        volatile float s01 = t0 + t1;
+                        volatile float s012 = s01 + t2;
+                        volatile float s = s012 + t3;
+                        accum += s;
+                    }
+                    volatile float sa = scale * accum;
+                    volatile float sb = sum * bias;
+                    result += sa + sb;
+                }
+                lane_result[lane] = result;
+            }
+            /* simd_sum: butterfly reduction (xor 16, 8, 4, 2, 1) */
+            for (int off = 16; off > 0; off >>= 1)
+                for (int lane = 0; lane < off; ++lane) lane_result[lane] += lane_result[lane + off];
+            out[(size_t)b * rows + r] = so_f32_to_f16(lane_result[0]);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Epilogues                                                                   */
+/* ------------------------------------------------------------------------- */
+
+/* lut_matvec.metal:4574-4577, signed_quant.metal:277-284:
+ * project, round to the activation type, then add the residual in that type. */
+SO_EXPORT uint16_t so_epilogue_residual_add(float acc, uint16_t residual, int dtype) {
+    float projected = so_round_through(acc, dtype);
+    return narrow(projected + widen(residual, dtype), dtype);
+}
+
+/* lut_matvec.metal:5075, agent_affine_qmm.h:329: half(gate/(1+exp(-gate))*up), fp32 g,u */
+SO_EXPORT uint16_t so_epilogue_affine_swiglu(float gate, float up, int dtype) {
+    return narrow(gate / (1.0f + expf(-gate)) * up, dtype);
+}
+
+/* signed_quant.metal:15-20 / signed_quant_precise.metal:31-36: every intermediate is
+ * materialised in the activation type. gate/up arrive already rounded to that type. */
+SO_EXPORT uint16_t so_epilogue_signed_swiglu(uint16_t gate_bits, uint16_t up_bits, int dtype) {
+    float gate = widen(gate_bits, dtype), up = widen(up_bits, dtype);
+    float e = so_round_through(expf(fabsf(gate)), dtype);
+    float denom = so_round_through(1.0f + e, dtype);
+    float tail = so_round_through(1.0f / denom, dtype);
+    float sigmoid = gate < 0.0f ? tail : so_round_through(1.0f - tail, dtype);
+    float activated = so_round_through(gate * sigmoid, dtype);
+    return narrow(activated * up, dtype);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Argmax key — lut_matvec.metal:4045-4074                                     */
+/* ------------------------------------------------------------------------- */
+
+#define SO_ARGMAX_INDEX_BITS 18
+#define SO_ARGMAX_MAX_INDEX ((1u << SO_ARGMAX_INDEX_BITS) - 1u)
+
+SO_EXPORT uint32_t so_argmax_ordered_key16(uint16_t bits16) {
+    uint32_t bits = bits16;
+    if ((bits & 0x7FFFu) == 0u) bits = 0u;
+    return (bits & 0x8000u) != 0u ? (0xFFFFu - bits) : (bits ^ 0x8000u);
+}
+
+SO_EXPORT uint64_t so_argmax_pack_key(uint16_t value_bits, uint32_t index) {
+    uint32_t ordered = so_argmax_ordered_key16(value_bits);
+    uint32_t inverse = (SO_ARGMAX_MAX_INDEX - index) & SO_ARGMAX_MAX_INDEX;
+    return ((uint64_t)ordered << 32) | inverse;
+}
+
+/* argmax over 16-bit float patterns (fp16, or bf16 — same sign/magnitude ordering):
+ * largest value wins, ties to the lowest index, -0 == +0. */
+SO_EXPORT int so_argmax16(const uint16_t *values, int count) {
+    uint64_t best = 0;
+    for (int i = 0; i < count; ++i) {
+        uint64_t k = so_argmax_pack_key(values[i], (uint32_t)i);
+        if (k > best) best = k;
+    }
+    return (int)(SO_ARGMAX_MAX_INDEX - (uint32_t)(best & 0xFFFFFFFFu));
+}
+
+/* ------------------------------------------------------------------------- */
+/* Threaded driver for the benchmark's cpu_baseline leg: rows split over       */
+/* threads with OpenMP if built with -fopenmp; the arithmetic is the scalar    */
+/* restatement above.                                                          */
+/* ------------------------------------------------------------------------- */
+
+SO_EXPORT void so_affine_matvec_mt(const uint8_t *packed, const uint16_t *scales,
+                                   const uint16_t *biases, const float *x, int rows, int cols,
+                                   int group, int dtype, float *out) {
+    int gpr = cols / group;
+    size_t stride = (size_t)cols / 2;
+#pragma omp parallel for schedule(static)
+    for (int r0 = 0; r0 < rows; r0 += 64) {
+        int n = rows - r0 < 64 ? rows - r0 : 64;
+        so_affine_matvec(packed + (size_t)r0 * stride, scales + (size_t)r0 * gpr,
+                         biases + (size_t)r0 * gpr, x, n, cols, group, dtype, out + r0);
+    }
+}
+
+SO_EXPORT int so_signed_matvec_mt(int format, const uint8_t *codes, int64_t row_stride,
+                                  const uint16_t *scales, const float *x, int rows, int cols,
+                                  int padded_cols, int group, float *out) {
+    int groups = so_signed_groups_per_row(padded_cols, group);
+    if (groups < 0) return groups;
+    int rc_all = SO_OK;
+#pragma omp parallel for schedule(static)
+    for (int r0 = 0; r0 < rows; r0 += 64) {
+        int n = rows - r0 < 64 ? rows - r0 : 64;
+        int rc = so_signed_matvec(format, codes + (size_t)r0 * row_stride, row_stride,
+                                  scales + (size_t)r0 * groups, x, n, cols, padded_cols, group, 1,
+                                  out + r0);
+        if (rc != SO_OK) rc_all = rc;
+    }
+    return rc_all;
+}
