@@ -1,0 +1,60 @@
+"""Builds the gfx950 code object and the C-ABI host library in-tree.
+
+    python -m smelt_amd.build          # compile everything
+
+Outputs (git-ignored, shipped to the GPU box as built files):
+    smelt_amd/lib/smelt_kernels.hsaco   hipcc --genco, gfx950 only
+    smelt_amd/lib/libsmelt_hip.so       host runtime + record emitters (links libamdhip64)
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "lib")
+HSACO = os.path.join(LIB, "smelt_kernels.hsaco")
+HOST_LIB = os.path.join(LIB, "libsmelt_hip.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# packed fp32 instructions are switched off for all device code
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+HOST_SOURCES = ["runtime.cpp", "pipeline_table.cpp", "compiler.cpp"]
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout + proc.stderr)
+        raise RuntimeError("build step failed: " + " ".join(cmd))
+
+
+def build_kernels() -> str:
+    os.makedirs(LIB, exist_ok=True)
+    src = os.path.join(CSRC, "kernels", "smelt_kernels.hip")
+    _run([HIPCC, *DEVICE_FLAGS, "--genco", "-o", HSACO, src])
+    return HSACO
+
+
+def build_host() -> str:
+    os.makedirs(LIB, exist_ok=True)
+    srcs = [os.path.join(CSRC, s) for s in HOST_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+          "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", "-o", HOST_LIB, *srcs,
+          f"-L{rocm}/lib", f"-Wl,-rpath,{rocm}/lib", "-lamdhip64", "-lpthread"])
+    return HOST_LIB
+
+
+def build_all() -> None:
+    build_kernels()
+    build_host()
+
+
+if __name__ == "__main__":
+    build_all()
+    print(HSACO)
+    print(HOST_LIB)

@@ -1,0 +1,114 @@
+// Shared device helpers for the gfx950 quantized matvec / qmm kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace smelt {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// Element types of activations / scales as stored in memory (raw 16-bit patterns).
+struct F16 {
+    static __device__ __forceinline__ float widen(uint16_t b) {
+        return (float)__builtin_bit_cast(_Float16, b);
+    }
+    // round-to-nearest-even narrowing
+    static __device__ __forceinline__ uint16_t narrow(float v) {
+        return __builtin_bit_cast(uint16_t, (_Float16)v);
+    }
+    // bits of the same value as fp16 (identity)
+    static __device__ __forceinline__ uint16_t to_f16_bits(uint16_t b) { return b; }
+};
+
+struct BF16 {
+    static __device__ __forceinline__ float widen(uint16_t b) {
+        return __builtin_bit_cast(float, (uint32_t)b << 16);
+    }
+    static __device__ __forceinline__ uint16_t narrow(float v) {
+        uint32_t bits = __builtin_bit_cast(uint32_t, v);
+        uint32_t rounded = bits + 0x7FFFu + ((bits >> 16) & 1u);
+        return (uint16_t)(rounded >> 16);
+    }
+    // bf16 -> fp16: exact for |v| in [2^-14, 65504]; smaller values round to the fp16
+    // subnormal grid (absolute error <= 2^-25), larger ones saturate to +-65504.
+    static __device__ __forceinline__ uint16_t to_f16_bits(uint16_t b) {
+        float v = widen(b);
+        v = __builtin_fminf(__builtin_fmaxf(v, -65504.0f), 65504.0f);
+        return __builtin_bit_cast(uint16_t, (_Float16)v);
+    }
+};
+
+__device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
+
+// D = a.x*b.x + a.y*b.y + acc with fp32 accumulation (v_dot2c_f32_f16).
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), acc, false);
+}
+
+// ---- wave64 reductions with DPP (no LDS) ---------------------------------------------
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_add(float v) {
+    int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, true);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over aligned groups of LANES consecutive lanes; the total is valid in the LAST lane
+// of each group (lane % LANES == LANES-1).
+template <int LANES>
+__device__ __forceinline__ float group_sum_last(float v) {
+    static_assert(LANES == 64 || LANES == 32 || LANES == 16 || LANES == 8 || LANES == 4 ||
+                  LANES == 2 || LANES == 1, "power of two");
+    if (LANES >= 2) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    if (LANES >= 4) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    if (LANES >= 8) v = dpp_add<0x141>(v);  // row_half_mirror
+    if (LANES >= 16) v = dpp_add<0x140>(v); // row_mirror
+    if (LANES >= 32) v = dpp_add<0x142, 0xA>(v);  // row_bcast:15 into rows 1,3
+    if (LANES >= 64) v = dpp_add<0x143, 0xC>(v);  // row_bcast:31 into rows 2,3
+    return v;
+}
+
+// ---- argmax key (value in the high word, inverted index in the low word) ---------------
+constexpr uint32_t kArgmaxIndexBits = 18;
+constexpr uint32_t kArgmaxMaxIndex = (1u << kArgmaxIndexBits) - 1u;
+
+__device__ __forceinline__ uint32_t ordered_key16(uint32_t bits) {
+    if ((bits & 0x7FFFu) == 0u) bits = 0u;  // -0 == +0
+    return (bits & 0x8000u) ? (0xFFFFu - bits) : (bits ^ 0x8000u);
+}
+
+__device__ __forceinline__ uint2_t argmax_pack_key(uint16_t value_bits, uint32_t index) {
+    uint2_t k;
+    k.x = ordered_key16(value_bits);
+    k.y = (kArgmaxMaxIndex - index) & kArgmaxMaxIndex;
+    return k;
+}
+
+__device__ __forceinline__ bool argmax_key_gt(uint2_t a, uint2_t b) {
+    return a.x > b.x || (a.x == b.x && a.y > b.y);
+}
+__device__ __forceinline__ uint2_t argmax_key_max(uint2_t a, uint2_t b) {
+    return argmax_key_gt(a, b) ? a : b;
+}
+
+__device__ __forceinline__ uint2_t wave_argmax_key(uint2_t k) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        uint2_t o;
+        o.x = __shfl_xor(k.x, off);
+        o.y = __shfl_xor(k.y, off);
+        k = argmax_key_max(k, o);
+    }
+    return k;
+}
+
+__device__ __forceinline__ int ilog2(uint32_t v) { return 31 - __builtin_clz(v); }
+
+}  // namespace smelt

@@ -1,0 +1,259 @@
+// Batch-1 / small-batch quantized matvec for gfx950 (wave64).
+//
+// y[b, r] = sum_c w(r, c) * x[b, c]   with w dequantised from packed codes and per-group scales.
+//
+// Shape of the computation
+//   * A "unit" is 16 bytes of one row's packed codes (one 128-bit load per lane): 32 affine-u4
+//     columns, 64 ternary2 columns or 128 binary1 columns.
+//   * A wave owns R rows (x S rows side by side when a row is shorter than 64 units); lane l
+//     walks units l, l+L, ... of each of its rows, so every load instruction of the wave reads
+//     one contiguous run of a row.
+//   * The activation vector is staged once per workgroup into LDS as fp16 *pairs* laid out to
+//     match the bit positions the codes occupy, so codes are turned into fp16 operands with one
+//     AND-OR each and multiplied two at a time by v_dot2c_f32_f16 (fp32 accumulate):
+//         ((dword >> s) & mask) | magic  ==  half2(base + code_a, base + code_b)
+//     The row-independent term  sum base * x  is computed at staging time and subtracted from
+//     each unit's dot product before the group scale is applied.
+//   * Per-row partial sums are reduced across the L lanes of a row with DPP adds.
+#pragma once
+#include "common.hpp"
+
+namespace smelt {
+
+// ---------------------------------------------------------------------------------------
+// Format traits. dot() consumes one dword of codes and kPairsPerDword fp16 pairs of x
+// (pair i = columns (i, i + kPairsPerDword) of that dword's column run).
+// pair_offset(i) = base_i + kSemShift, the constant folded out of pair i.
+// The semantic weight is kSemMul * (code + pair terms - offset) * scale.
+// ---------------------------------------------------------------------------------------
+struct FmtU4 {
+    static constexpr int kBitsPerCode = 4;
+    static constexpr int kPairsPerDword = 4;
+    static constexpr bool kHasBias = true;
+    static constexpr float kSemMul = 1.0f;
+    static __device__ __forceinline__ float pair_offset(int i) { return (i & 1) ? 64.0f : 1024.0f; }
+    static __device__ __forceinline__ float dot(uint32_t c, const uint32_t* xp, float acc) {
+        const uint32_t c8 = c >> 8;
+        acc = dot2((c & 0x000F000Fu) | 0x64006400u, xp[0], acc);   // nibbles 0,4 -> 1024+n
+        acc = dot2((c & 0x00F000F0u) | 0x54005400u, xp[1], acc);   // nibbles 1,5 -> 64+n
+        acc = dot2((c8 & 0x000F000Fu) | 0x64006400u, xp[2], acc);  // nibbles 2,6
+        acc = dot2((c8 & 0x00F000F0u) | 0x54005400u, xp[3], acc);  // nibbles 3,7
+        return acc;
+    }
+};
+
+struct FmtTer2 {
+    static constexpr int kBitsPerCode = 2;
+    static constexpr int kPairsPerDword = 8;
+    static constexpr bool kHasBias = false;
+    static constexpr float kSemMul = 1.0f;
+    // semantic = code - 1; codes sit at mantissa bits 4, 6 or 8 -> bases 64, 16, 4
+    static __device__ __forceinline__ float pair_offset(int i) {
+        const int k = i % 3;
+        return (k == 0 ? 64.0f : (k == 1 ? 16.0f : 4.0f)) + 1.0f;
+    }
+    static __device__ __forceinline__ float dot(uint32_t c, const uint32_t* xp, float acc) {
+        const uint32_t a = c << 4, b = c >> 2, d = c >> 8;
+        acc = dot2((a & 0x00300030u) | 0x54005400u, xp[0], acc);
+        acc = dot2((a & 0x00C000C0u) | 0x4C004C00u, xp[1], acc);
+        acc = dot2((a & 0x03000300u) | 0x44004400u, xp[2], acc);
+        acc = dot2((b & 0x00300030u) | 0x54005400u, xp[3], acc);
+        acc = dot2((b & 0x00C000C0u) | 0x4C004C00u, xp[4], acc);
+        acc = dot2((b & 0x03000300u) | 0x44004400u, xp[5], acc);
+        acc = dot2((d & 0x00300030u) | 0x54005400u, xp[6], acc);
+        acc = dot2((d & 0x00C000C0u) | 0x4C004C00u, xp[7], acc);
+        return acc;
+    }
+};
+
+struct FmtBin {
+    static constexpr int kBitsPerCode = 1;
+    static constexpr int kPairsPerDword = 16;
+    static constexpr bool kHasBias = false;
+    static constexpr float kSemMul = 2.0f;
+    // semantic = 2*bit - 1 = 2*(bit - 0.5); bits sit at mantissa bits 4..9 -> bases 64..2
+    static __device__ __forceinline__ float pair_offset(int i) {
+        const int k = i % 6;
+        return (float)(64 >> k) + 0.5f;
+    }
+    static __device__ __forceinline__ float dot(uint32_t c, const uint32_t* xp, float acc) {
+        const uint32_t a = c << 4, b = c >> 2, d = c >> 8;
+        acc = dot2((a & 0x00100010u) | 0x54005400u, xp[0], acc);
+        acc = dot2((a & 0x00200020u) | 0x50005000u, xp[1], acc);
+        acc = dot2((a & 0x00400040u) | 0x4C004C00u, xp[2], acc);
+        acc = dot2((a & 0x00800080u) | 0x48004800u, xp[3], acc);
+        acc = dot2((a & 0x01000100u) | 0x44004400u, xp[4], acc);
+        acc = dot2((a & 0x02000200u) | 0x40004000u, xp[5], acc);
+        acc = dot2((b & 0x00100010u) | 0x54005400u, xp[6], acc);
+        acc = dot2((b & 0x00200020u) | 0x50005000u, xp[7], acc);
+        acc = dot2((b & 0x00400040u) | 0x4C004C00u, xp[8], acc);
+        acc = dot2((b & 0x00800080u) | 0x48004800u, xp[9], acc);
+        acc = dot2((b & 0x01000100u) | 0x44004400u, xp[10], acc);
+        acc = dot2((b & 0x02000200u) | 0x40004000u, xp[11], acc);
+        acc = dot2((d & 0x00100010u) | 0x54005400u, xp[12], acc);
+        acc = dot2((d & 0x00200020u) | 0x50005000u, xp[13], acc);
+        acc = dot2((d & 0x00400040u) | 0x4C004C00u, xp[14], acc);
+        acc = dot2((d & 0x00800080u) | 0x48004800u, xp[15], acc);
+        return acc;
+    }
+};
+
+template <class F>
+struct FmtGeom {
+    static constexpr int kPPD = F::kPairsPerDword;
+    static constexpr int kColsPerDword = 2 * kPPD;
+    static constexpr int kColsPerUnit = 4 * kColsPerDword;
+    static constexpr int kChunksPerDword = kPPD / 4;       // 16-byte LDS chunks (4 pairs each)
+    static constexpr int kChunksPerUnit = 4 * kChunksPerDword;
+};
+
+// LDS layout for one batch tile of MB activations over U units per row:
+//   pairs : [MB][kChunksPerUnit][U] x 16 B   (chunk-major so consecutive lanes hit consecutive 16 B)
+//   corr  : [MB][U] float4 (one float per dword of the unit)
+//   xsum  : [MB][U] float4 (affine only)
+template <class F>
+__device__ __forceinline__ size_t lds_pairs_bytes(int U, int MB) {
+    return (size_t)MB * FmtGeom<F>::kChunksPerUnit * U * 16;
+}
+
+// Stage x[b0 .. b0+nb) (nb <= MB, rows of `cols` elements of ActT) into LDS.
+template <class F, class ActT, int MB>
+__device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x, int cols, int U,
+                                                  int b0, int nb, uint4_t* lds_pairs,
+                                                  float* lds_corr, float* lds_xsum) {
+    using G = FmtGeom<F>;
+    constexpr int PPD = G::kPPD;
+    constexpr int CPD = G::kColsPerDword;
+    const int dwords = U * 4;
+    for (int item = threadIdx.x; item < MB * dwords; item += blockDim.x) {
+        const int b = item / dwords;
+        const int D = item - b * dwords;
+        const int u = D >> 2, d = D & 3;
+        const int col0 = D * CPD;
+        uint16_t v[CPD];
+        if (b < nb && col0 + CPD <= cols) {
+            const uint4_t* src = reinterpret_cast<const uint4_t*>(x + (size_t)(b0 + b) * cols + col0);
+#pragma unroll
+            for (int q = 0; q < CPD / 8; ++q) {
+                uint4_t t = src[q];
+                v[8 * q + 0] = (uint16_t)(t.x & 0xFFFF); v[8 * q + 1] = (uint16_t)(t.x >> 16);
+                v[8 * q + 2] = (uint16_t)(t.y & 0xFFFF); v[8 * q + 3] = (uint16_t)(t.y >> 16);
+                v[8 * q + 4] = (uint16_t)(t.z & 0xFFFF); v[8 * q + 5] = (uint16_t)(t.z >> 16);
+                v[8 * q + 6] = (uint16_t)(t.w & 0xFFFF); v[8 * q + 7] = (uint16_t)(t.w >> 16);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < CPD; ++i) {
+                const int c = col0 + i;
+                v[i] = (b < nb && c < cols) ? x[(size_t)(b0 + b) * cols + c] : (uint16_t)0;
+            }
+        }
+        float corr = 0.0f, xsum = 0.0f;
+        uint32_t pairs[PPD];
+#pragma unroll
+        for (int i = 0; i < PPD; ++i) {
+            const uint16_t lo = ActT::to_f16_bits(v[i]);
+            const uint16_t hi = ActT::to_f16_bits(v[i + PPD]);
+            pairs[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+            const float s = F16::widen(lo) + F16::widen(hi);
+            corr += F::pair_offset(i) * s;
+            xsum += s;
+        }
+#pragma unroll
+        for (int j = 0; j < G::kChunksPerDword; ++j) {
+            uint4_t ch;
+            ch.x = pairs[4 * j + 0]; ch.y = pairs[4 * j + 1];
+            ch.z = pairs[4 * j + 2]; ch.w = pairs[4 * j + 3];
+            lds_pairs[((size_t)b * G::kChunksPerUnit + d * G::kChunksPerDword + j) * U + u] = ch;
+        }
+        lds_corr[((size_t)b * U + u) * 4 + d] = corr;
+        if (F::kHasBias) lds_xsum[((size_t)b * U + u) * 4 + d] = xsum;
+    }
+}
+
+// One weight matrix as seen by the core.
+struct MatPtrs {
+    const uint8_t* codes;
+    const uint16_t* scales;
+    const uint16_t* biases;  // affine only
+};
+
+// Accumulate acc[m][r][b] for the wave's row tile.
+//   row_base  : first row of this wave's tile; rows row_base + side*R + r
+//   L         : lanes per row (power of two), S = 64 / L rows side by side
+template <class F, class ScaleT, int R, int MB, int NMAT, int L>
+__device__ __forceinline__ void matvec_tile(const MatPtrs (&mats)[NMAT], int rows, int U,
+                                            int row_stride, int groups_per_row, int gshift,
+                                            int row_base, const uint4_t* lds_pairs,
+                                            const float4_t* lds_corr, const float4_t* lds_xsum,
+                                            float (&acc)[NMAT][R][MB]) {
+    using G = FmtGeom<F>;
+    constexpr int NCH = G::kChunksPerUnit;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sub = lane & (L - 1);
+    const int side = lane / L;
+    int row[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int rr = row_base + side * R + r;
+        row[r] = rr < rows ? rr : rows - 1;  // clamped rows are computed but never stored
+    }
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) acc[m][r][b] = 0.0f;
+
+    for (int u = sub; u < U; u += L) {
+        uint4_t c[NMAT][R];
+        float sc[NMAT][R], bi[NMAT][R];
+        const int g = (u * G::kColsPerUnit) >> gshift;
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                c[m][r] = *reinterpret_cast<const uint4_t*>(mats[m].codes + (size_t)row[r] * row_stride + (size_t)u * 16);
+                const size_t si = (size_t)row[r] * groups_per_row + g;
+                sc[m][r] = F::kSemMul * ScaleT::widen(mats[m].scales[si]);
+                bi[m][r] = F::kHasBias ? ScaleT::widen(mats[m].biases[si]) : 0.0f;
+            }
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            uint32_t xp[NCH * 4];
+#pragma unroll
+            for (int q = 0; q < NCH; ++q) {
+                const uint4_t t = lds_pairs[((size_t)b * NCH + q) * U + u];
+                xp[4 * q + 0] = t.x; xp[4 * q + 1] = t.y; xp[4 * q + 2] = t.z; xp[4 * q + 3] = t.w;
+            }
+            const float4_t cr = lds_corr[(size_t)b * U + u];
+            const float corr = (cr.x + cr.y) + (cr.z + cr.w);
+            float xsum = 0.0f;
+            if (F::kHasBias) {
+                const float4_t xs = lds_xsum[(size_t)b * U + u];
+                xsum = (xs.x + xs.y) + (xs.z + xs.w);
+            }
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    float d = -corr;
+                    d = F::dot(c[m][r].x, xp + 0 * G::kPPD, d);
+                    d = F::dot(c[m][r].y, xp + 1 * G::kPPD, d);
+                    d = F::dot(c[m][r].z, xp + 2 * G::kPPD, d);
+                    d = F::dot(c[m][r].w, xp + 3 * G::kPPD, d);
+                    float a = acc[m][r][b];
+                    if (F::kHasBias) a = __builtin_fmaf(bi[m][r], xsum, a);
+                    acc[m][r][b] = __builtin_fmaf(sc[m][r], d, a);
+                }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) acc[m][r][b] = group_sum_last<L>(acc[m][r][b]);
+}
+
+}  // namespace smelt

@@ -1,0 +1,293 @@
+// __global__ entry points for the quantized matvec family.  Argument order of every kernel is
+// the binding order of the Smelt dispatch record that drives it (buffers and 4-byte constants
+// by ascending binding index), followed by the shape arguments the pipeline table appends.
+#pragma once
+#include "matvec.hpp"
+
+namespace smelt {
+
+// ---- epilogues ---------------------------------------------------------------------------
+// Each epilogue receives the reduced fp32 sums of one (batch, row) for NMAT matrices.
+
+template <class ActT>
+struct EpiStore {
+    uint16_t* y;
+    int rows;
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        y[(size_t)b * rows + row] = ActT::narrow(v[0]);
+    }
+};
+
+// project, round to the activation type, add the residual in that type
+template <class ActT>
+struct EpiAdd {
+    uint16_t* y;
+    const uint16_t* residual;
+    int rows;
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        const size_t i = (size_t)b * rows + row;
+        const float projected = ActT::widen(ActT::narrow(v[0]));
+        y[i] = ActT::narrow(projected + ActT::widen(residual[i]));
+    }
+};
+
+// affine SwiGLU: narrow(gate / (1 + exp(-gate)) * up) on the fp32 sums
+template <class ActT>
+struct EpiAffineSwiglu {
+    uint16_t* y;
+    int rows;
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        const float g = v[0], u = v[1];
+        y[(size_t)b * rows + row] = ActT::narrow(g / (1.0f + expf(-g)) * u);
+    }
+};
+
+// signed SwiGLU: gate and up are first rounded to the activation type and every intermediate
+// (exp, 1+e, reciprocal, 1-tail, gate*sigmoid, *up) is materialised in that type
+template <class ActT>
+struct EpiSignedSwiglu {
+    uint16_t* y;
+    int rows;
+    static __device__ __forceinline__ float rt(float v) { return ActT::widen(ActT::narrow(v)); }
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        const float g = rt(v[0]), u = rt(v[1]);
+        const float e = rt(expf(fabsf(g)));
+        const float denom = rt(1.0f + e);
+        const float tail = rt(1.0f / denom);
+        const float sig = g < 0.0f ? tail : rt(1.0f - tail);
+        const float act = rt(g * sig);
+        y[(size_t)b * rows + row] = ActT::narrow(act * u);
+    }
+};
+
+template <class ActT>
+struct EpiDual {
+    uint16_t* y1;
+    uint16_t* y2;
+    int rows;
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        y1[(size_t)b * rows + row] = ActT::narrow(v[0]);
+        y2[(size_t)b * rows + row] = ActT::narrow(v[1]);
+    }
+};
+
+// ---- workgroup body ------------------------------------------------------------------------
+
+template <class F, class ScaleT, int R, int MB, int NMAT, int L, class Epi>
+__device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], int rows, int U,
+                                          int row_stride, int gpr, int gshift, int b0, int nb,
+                                          const uint4_t* lds_pairs, const float4_t* lds_corr,
+                                          const float4_t* lds_xsum, const Epi& epi) {
+    constexpr int S = kWave / L;
+    constexpr int TILE = S * R;
+    const int waves = blockDim.x / kWave;
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sub = lane & (L - 1);
+    const int side = lane / L;
+    const int tiles = (rows + TILE - 1) / TILE;
+    for (int tile = blockIdx.x * waves + wave; tile < tiles; tile += gridDim.x * waves) {
+        float acc[NMAT][R][MB];
+        matvec_tile<F, ScaleT, R, MB, NMAT, L>(mats, rows, U, row_stride, gpr, gshift, tile * TILE,
+                                               lds_pairs, lds_corr, lds_xsum, acc);
+        if (sub == L - 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int row = tile * TILE + side * R + r;
+                if (row < rows) {
+#pragma unroll
+                    for (int b = 0; b < MB; ++b) {
+                        if (b < nb) {
+                            float v[NMAT];
+#pragma unroll
+                            for (int m = 0; m < NMAT; ++m) v[m] = acc[m][r][b];
+                            epi(b0 + b, row, v);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Covers batch rows [batch_lo, batch_hi) in chunks of MB with the activations of one chunk
+// resident in LDS.  x is [batch, cols]; row_stride is the byte stride of one packed row.
+template <class F, class ActT, class ScaleT, int R, int MB, int NMAT, class Epi>
+__device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const uint16_t* x,
+                                            int rows, int cols, int row_stride, int group,
+                                            int batch_lo, int batch_hi, const Epi& epi) {
+    using G = FmtGeom<F>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int U = row_stride / 16;
+    const int gshift = ilog2((uint32_t)group);
+    const int gpr = (cols + group - 1) / group;
+    uint4_t* lds_pairs = reinterpret_cast<uint4_t*>(smem);
+    float* lds_corr = reinterpret_cast<float*>(smem + lds_pairs_bytes<F>(U, MB));
+    float* lds_xsum = lds_corr + (size_t)MB * U * 4;
+    for (int b0 = batch_lo; b0 < batch_hi; b0 += MB) {
+        const int nb = batch_hi - b0 < MB ? batch_hi - b0 : MB;
+        if (b0 != batch_lo) __syncthreads();
+        stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum);
+        __syncthreads();
+        const float4_t* corr4 = reinterpret_cast<const float4_t*>(lds_corr);
+        const float4_t* xsum4 = reinterpret_cast<const float4_t*>(lds_xsum);
+        if (U > 32)
+            run_tiles<F, ScaleT, R, MB, NMAT, 64>(mats, rows, U, row_stride, gpr, gshift, b0, nb, lds_pairs, corr4, xsum4, epi);
+        else if (U > 16)
+            run_tiles<F, ScaleT, R, MB, NMAT, 32>(mats, rows, U, row_stride, gpr, gshift, b0, nb, lds_pairs, corr4, xsum4, epi);
+        else
+            run_tiles<F, ScaleT, R, MB, NMAT, 16>(mats, rows, U, row_stride, gpr, gshift, b0, nb, lds_pairs, corr4, xsum4, epi);
+    }
+}
+
+template <class F>
+__device__ __forceinline__ int packed_row_stride(int cols, int group) {
+    const int padded = F::kHasBias ? cols : (cols + group - 1) / group * group;
+    return (padded * F::kBitsPerCode + 7) / 8;
+}
+
+}  // namespace smelt
+
+// ---- entry points ---------------------------------------------------------------------------
+#define SMELT_KERNEL extern "C" __global__ __launch_bounds__(256)
+using u16 = uint16_t;
+using u8 = uint8_t;
+using u32 = uint32_t;
+
+#define SMELT_AFFINE_KERNELS(T, ACT, SC)                                                          \
+    SMELT_KERNEL void smelt_affine_matvec_##T(const u8* W, const u16* S, const u16* B,            \
+                                              const u16* x, u16* y, u32 rows, u32 cols,           \
+                                              u32 group) {                                        \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{y, (int)rows};                                                          \
+        matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi);                    \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_matvec_add_##T(const u8* W, const u16* S, const u16* B,        \
+                                                  const u16* x, u16* y, const u16* res, u32 rows, \
+                                                  u32 cols, u32 group) {                          \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiAdd<ACT> epi{y, res, (int)rows};                                                       \
+        matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi);                    \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_gate_up_swiglu_##T(                                            \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* x, u16* y, u32 rows, u32 cols, u32 group) {                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiAffineSwiglu<ACT> epi{y, (int)rows};                                                   \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi);                    \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_dual_matvec_##T(                                               \
+        const u8* W1, const u16* S1, const u16* B1, const u8* W2, const u16* S2, const u16* B2,   \
+        const u16* x, u16* y1, u16* y2, u32 rows, u32 cols, u32 group) {                          \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
+        EpiDual<ACT> epi{y1, y2, (int)rows};                                                      \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi);                    \
+    }
+
+#define SMELT_AFFINE_BATCHED(T, ACT, SC, MBV)                                                     \
+    SMELT_KERNEL void smelt_affine_matvec_batched_mb##MBV##_##T(                                  \
+        const u8* W, const u16* S, const u16* B, const u16* X, u16* Y, u32 batch, u32 rows,       \
+        u32 cols, u32 group, u32 batch_tile) {                                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{Y, (int)rows};                                                          \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        matvec_body<FmtU4, ACT, SC, 4, MBV, 1>(mats, X, rows, cols,                               \
+                                               packed_row_stride<FmtU4>(cols, group), group, lo,  \
+                                               hi, epi);                                          \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_matvec_add_batched_mb##MBV##_##T(                              \
+        const u8* W, const u16* S, const u16* B, const u16* X, u16* Y, const u16* res, u32 batch, \
+        u32 rows, u32 cols, u32 group, u32 batch_tile) {                                          \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiAdd<ACT> epi{Y, res, (int)rows};                                                       \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        matvec_body<FmtU4, ACT, SC, 4, MBV, 1>(mats, X, rows, cols,                               \
+                                               packed_row_stride<FmtU4>(cols, group), group, lo,  \
+                                               hi, epi);                                          \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_gate_up_swiglu_batched_mb##MBV##_##T(                          \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* X, u16* Y, u32 batch, u32 rows, u32 cols, u32 group, u32 batch_tile) {         \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiAffineSwiglu<ACT> epi{Y, (int)rows};                                                   \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        matvec_body<FmtU4, ACT, SC, 2, MBV, 2>(mats, X, rows, cols,                               \
+                                               packed_row_stride<FmtU4>(cols, group), group, lo,  \
+                                               hi, epi);                                          \
+    }
+
+// Signed kernels: batch row = blockIdx.y (M = 1 family) or a tile of 4 rows (_b4 family).
+#define SMELT_SIGNED_KERNELS(FN, FMT, T, ACT)                                                     \
+    SMELT_KERNEL void smelt_signed_##FN##_matvec_##T(const u8* C, const u16* S, const u16* X,     \
+                                                     u16* Y, u32 rows, u32 cols) {                \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{Y, (int)rows};                                                          \
+        matvec_body<FMT, ACT, F16, 4, 1, 1>(mats, X, rows, cols,                                  \
+                                            packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
+                                            blockIdx.y + 1, epi);                                 \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_matvec_add_##T(const u8* C, const u16* S, const u16* X, \
+                                                         u16* Y, const u16* res, u32 rows,        \
+                                                         u32 cols) {                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{Y, res, (int)rows};                                                       \
+        matvec_body<FMT, ACT, F16, 4, 1, 1>(mats, X, rows, cols,                                  \
+                                            packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
+                                            blockIdx.y + 1, epi);                                 \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_gate_up_swiglu_##T(                                     \
+        const u8* gC, const u16* gS, const u8* uC, const u16* uS, const u16* X, u16* Y, u32 rows, \
+        u32 cols) {                                                                               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{Y, (int)rows};                                                   \
+        matvec_body<FMT, ACT, F16, 2, 1, 2>(mats, X, rows, cols,                                  \
+                                            packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
+                                            blockIdx.y + 1, epi);                                 \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_matvec_b4_##T(const u8* C, const u16* S, const u16* X,  \
+                                                        u16* Y, u32 rows, u32 cols, u32 batch) {  \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{Y, (int)rows};                                                          \
+        const u32 lo = blockIdx.y * 4;                                                            \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + 4 < batch ? lo + 4 : batch;                                           \
+        matvec_body<FMT, ACT, F16, 4, 2, 1>(mats, X, rows, cols,                                  \
+                                            packed_row_stride<FMT>(cols, 128), 128, lo, hi, epi); \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_gate_up_swiglu_b4_##T(                                  \
+        const u8* gC, const u16* gS, const u8* uC, const u16* uS, const u16* X, u16* Y, u32 rows, \
+        u32 cols, u32 batch) {                                                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{Y, (int)rows};                                                   \
+        const u32 lo = blockIdx.y * 4;                                                            \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + 4 < batch ? lo + 4 : batch;                                           \
+        matvec_body<FMT, ACT, F16, 2, 2, 2>(mats, X, rows, cols,                                  \
+                                            packed_row_stride<FMT>(cols, 128), 128, lo, hi, epi); \
+    }

@@ -1,0 +1,169 @@
+// Element-exact dequant (embedding gathers) and argmax kernels.
+#pragma once
+#include "common.hpp"
+
+namespace smelt {
+
+// w = float(code) * scale + bias with one rounded multiply and one rounded add (never fused),
+// then narrowed to the output type: the per-element contract of the packed formats.
+template <class ScaleT, class OutT>
+__device__ __forceinline__ uint16_t dequant_affine(uint32_t nib, uint16_t s, uint16_t b) {
+    const float p = __fmul_rn((float)nib, ScaleT::widen(s));
+    return OutT::narrow(__fadd_rn(p, ScaleT::widen(b)));
+}
+
+template <class ScaleT, class OutT>
+__device__ __forceinline__ void affine_gather_body(const uint8_t* W, const uint16_t* S,
+                                                   const uint16_t* B, const int* token_ids,
+                                                   uint16_t* out, uint32_t cols, uint32_t group,
+                                                   uint32_t batch, uint32_t batch_count) {
+    const uint32_t half_cols = cols / 2;
+    const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= half_cols || batch >= batch_count) return;
+    const size_t row = (size_t)(uint32_t)token_ids[batch];
+    const uint32_t gpr = cols / group;
+    const uint8_t packed = W[row * half_cols + t];
+    const uint32_t c0 = t * 2, c1 = c0 + 1;
+    const size_t sb = row * gpr;
+    out[(size_t)batch * cols + c0] = dequant_affine<ScaleT, OutT>(packed & 0xFu, S[sb + c0 / group], B[sb + c0 / group]);
+    out[(size_t)batch * cols + c1] = dequant_affine<ScaleT, OutT>(packed >> 4, S[sb + c1 / group], B[sb + c1 / group]);
+}
+
+// FORMAT: 0 binary1, 1 ternary2, 2 trit5 (5 base-3 digits per byte, LUT-decoded).
+// trit5 rows are padded to a 16-byte multiple.
+__device__ __forceinline__ uint32_t trit5_row_stride(uint32_t cols) {
+    return (((cols + 4) / 5) + 15u) & ~15u;
+}
+
+template <int FORMAT, class OutT>
+__device__ __forceinline__ void signed_gather_body(const uint8_t* codes, const uint16_t* scales,
+                                                   const int* token_ids, uint16_t* out,
+                                                   uint32_t hidden, const uint16_t* trit_lut) {
+    const uint32_t col = blockIdx.x * blockDim.x + threadIdx.x;
+    if (col >= hidden) return;
+    const uint32_t b = blockIdx.y;
+    const size_t row = (size_t)(uint32_t)token_ids[b];
+    const uint32_t groups = hidden / 128;
+    float value;
+    if (FORMAT == 1) {
+        const uint32_t packed = (codes[row * (hidden / 4) + col / 4] >> (2u * (col & 3u))) & 3u;
+        value = (float)((int)packed - 1);
+    } else if (FORMAT == 0) {
+        const uint32_t packed = (codes[row * (hidden / 8) + col / 8] >> (col & 7u)) & 1u;
+        value = packed == 0u ? -1.0f : 1.0f;
+    } else {
+        const uint32_t byte = codes[row * trit5_row_stride(hidden) + col / 5];
+        const uint32_t packed = (trit_lut[byte] >> (2u * (col % 5u))) & 3u;
+        value = (float)((int)packed - 1);
+    }
+    out[(size_t)b * hidden + col] = OutT::narrow(__fmul_rn(value, F16::widen(scales[row * groups + col / 128])));
+}
+
+// 243-entry decode table: five 2-bit codes (digit i at bits 2i..2i+1) per byte value.
+__device__ __forceinline__ uint16_t trit5_lut_entry(uint32_t b) {
+    if (b >= 243u) return 0x0155u;  // invalid bytes decode to five semantic zeros
+    uint32_t e = 0;
+#pragma unroll
+    for (int i = 0; i < 5; ++i) { e |= (b % 3u) << (2 * i); b /= 3u; }
+    return (uint16_t)e;
+}
+
+}  // namespace smelt
+
+#define SMELT_MISC_KERNEL extern "C" __global__ __launch_bounds__(256)
+
+#define SMELT_GATHER_KERNELS(T, ACT)                                                              \
+    SMELT_MISC_KERNEL void smelt_affine_embedding_gather_##T(                                     \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const int* token_id,              \
+        uint16_t* out, uint32_t cols, uint32_t group) {                                           \
+        smelt::affine_gather_body<ACT, ACT>(W, S, B, token_id, out, cols, group, 0, 1);           \
+    }                                                                                             \
+    SMELT_MISC_KERNEL void smelt_affine_embedding_gather_batched_##T(                             \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const int* token_ids,             \
+        uint16_t* out, uint32_t cols, uint32_t batch, uint32_t group) {                           \
+        smelt::affine_gather_body<ACT, ACT>(W, S, B, token_ids, out, cols, group, blockIdx.y,     \
+                                            batch);                                               \
+    }                                                                                             \
+    SMELT_MISC_KERNEL void smelt_signed_binary_embedding_gather_##T(                              \
+        const uint8_t* C, const uint16_t* S, const int* ids, uint16_t* out, uint32_t hidden) {    \
+        smelt::signed_gather_body<0, ACT>(C, S, ids, out, hidden, nullptr);                       \
+    }                                                                                             \
+    SMELT_MISC_KERNEL void smelt_signed_ternary_embedding_gather_##T(                             \
+        const uint8_t* C, const uint16_t* S, const int* ids, uint16_t* out, uint32_t hidden) {    \
+        smelt::signed_gather_body<1, ACT>(C, S, ids, out, hidden, nullptr);                       \
+    }                                                                                             \
+    SMELT_MISC_KERNEL void smelt_signed_trit5_embedding_gather_##T(                               \
+        const uint8_t* C, const uint16_t* S, const int* ids, uint16_t* out, uint32_t hidden) {    \
+        __shared__ uint16_t lut[256];                                                             \
+        lut[threadIdx.x & 255] = smelt::trit5_lut_entry(threadIdx.x & 255);                       \
+        if (blockDim.x < 256)                                                                     \
+            for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x)                              \
+                lut[i] = smelt::trit5_lut_entry(i);                                               \
+        __syncthreads();                                                                          \
+        smelt::signed_gather_body<2, ACT>(C, S, ids, out, hidden, lut);                           \
+    }
+
+SMELT_GATHER_KERNELS(f16, smelt::F16)
+SMELT_GATHER_KERNELS(bf16, smelt::BF16)
+
+// ---- argmax over materialised 16-bit logits ---------------------------------------------------
+// Largest value wins, ties go to the lowest index, -0 equals +0.  The ordering of the 16-bit
+// pattern is the same for fp16 and bf16 (sign + magnitude), so one kernel serves both.
+SMELT_MISC_KERNEL void smelt_argmax16_partials(const uint16_t* logits, smelt::uint2_t* partials,
+                                               uint32_t vocab, uint32_t chunk) {
+    using namespace smelt;
+    const uint32_t start = blockIdx.x * chunk;
+    const uint32_t end = start + chunk < vocab ? start + chunk : vocab;
+    uint2_t best = {0u, 0u};
+    for (uint32_t i = start + threadIdx.x; i < end; i += blockDim.x)
+        best = argmax_key_max(best, argmax_pack_key(logits[i], i));
+    best = wave_argmax_key(best);
+    __shared__ uint2_t wave_best[16];
+    const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) wave_best[wave] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t waves = (blockDim.x + kWave - 1) / kWave;
+        for (uint32_t w = 1; w < waves; ++w) best = argmax_key_max(best, wave_best[w]);
+        partials[blockIdx.x] = best;
+    }
+}
+
+// one block per batch row (blockIdx.x); partials are [batch, num_partials]
+SMELT_MISC_KERNEL void smelt_argmax_key_reduce(const smelt::uint2_t* partials, int* output,
+                                               uint32_t num_partials) {
+    using namespace smelt;
+    const uint2_t* row = partials + (size_t)blockIdx.x * num_partials;
+    uint2_t best = {0u, 0u};
+    for (uint32_t i = threadIdx.x; i < num_partials; i += blockDim.x) best = argmax_key_max(best, row[i]);
+    best = wave_argmax_key(best);
+    __shared__ uint2_t wave_best[16];
+    const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) wave_best[wave] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t waves = (blockDim.x + kWave - 1) / kWave;
+        for (uint32_t w = 1; w < waves; ++w) best = argmax_key_max(best, wave_best[w]);
+        output[blockIdx.x] = (int)(kArgmaxMaxIndex - best.y);
+    }
+}
+
+// lm_head reduce: same as above with the batch guard of the fused lm_head path
+SMELT_MISC_KERNEL void smelt_lm_head_argmax_reduce(const smelt::uint2_t* partials, int* output,
+                                                   uint32_t batch, uint32_t num_partials) {
+    using namespace smelt;
+    if (blockIdx.x >= batch) return;
+    const uint2_t* row = partials + (size_t)blockIdx.x * num_partials;
+    uint2_t best = {0u, 0u};
+    for (uint32_t i = threadIdx.x; i < num_partials; i += blockDim.x) best = argmax_key_max(best, row[i]);
+    best = wave_argmax_key(best);
+    __shared__ uint2_t wave_best[16];
+    const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) wave_best[wave] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t waves = (blockDim.x + kWave - 1) / kWave;
+        for (uint32_t w = 1; w < waves; ++w) best = argmax_key_max(best, wave_best[w]);
+        output[blockIdx.x] = (int)(kArgmaxMaxIndex - best.y);
+    }
+}

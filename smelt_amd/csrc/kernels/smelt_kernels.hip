@@ -1,0 +1,18 @@
+// Single translation unit for the gfx950 code object (smelt_kernels.hsaco).
+// Built with:  hipcc --offload-arch=gfx950 --genco -O3 -Xclang -target-feature -Xclang -packed-fp32-ops
+#include "matvec_kernels.hpp"
+#include "misc_kernels.hpp"
+
+SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
+SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
+SMELT_AFFINE_BATCHED(f16, smelt::F16, smelt::F16, 1)
+SMELT_AFFINE_BATCHED(f16, smelt::F16, smelt::F16, 2)
+SMELT_AFFINE_BATCHED(f16, smelt::F16, smelt::F16, 4)
+SMELT_AFFINE_BATCHED(bf16, smelt::BF16, smelt::BF16, 1)
+SMELT_AFFINE_BATCHED(bf16, smelt::BF16, smelt::BF16, 2)
+SMELT_AFFINE_BATCHED(bf16, smelt::BF16, smelt::BF16, 4)
+
+SMELT_SIGNED_KERNELS(binary, smelt::FmtBin, f16, smelt::F16)
+SMELT_SIGNED_KERNELS(binary, smelt::FmtBin, bf16, smelt::BF16)
+SMELT_SIGNED_KERNELS(ternary, smelt::FmtTer2, f16, smelt::F16)
+SMELT_SIGNED_KERNELS(ternary, smelt::FmtTer2, bf16, smelt::BF16)

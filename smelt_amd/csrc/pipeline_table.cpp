@@ -1,0 +1,220 @@
+// Pipeline-name resolution.  The reference resolves a manifest pipeline string to a Metal
+// function by exact name, or by "name:cols:groupSize" function constants
+// (SmeltRuntime.swift:6229-6263); its catalog carries one Metal function per tuned shape
+// (SmeltKernelCatalog.swift).  The HIP kernels take the shape as arguments, so every name of
+// an in-scope family maps onto a handful of symbols plus appended shape values.
+#include "pipeline_table.hpp"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace smelt_host {
+
+namespace {
+
+bool starts_with(const std::string& s, const char* p) { return s.compare(0, strlen(p), p) == 0; }
+
+bool parse_uint(const std::string& s, uint32_t* out) {
+    if (s.empty() || s.size() > 9) return false;
+    uint32_t v = 0;
+    for (char c : s) {
+        if (c < '0' || c > '9') return false;
+        v = v * 10 + (uint32_t)(c - '0');
+    }
+    *out = v;
+    return true;
+}
+
+// "_c1024_r2048_g64<suffix>" -> cols, rows, group, suffix
+bool parse_fixed_shape(const std::string& rest, uint32_t* cols, uint32_t* rows, uint32_t* group,
+                       std::string* suffix) {
+    if (!starts_with(rest, "_c")) return false;
+    size_t p = 2, q = rest.find("_r", p);
+    if (q == std::string::npos || !parse_uint(rest.substr(p, q - p), cols)) return false;
+    p = q + 2;
+    q = rest.find("_g", p);
+    if (q == std::string::npos || !parse_uint(rest.substr(p, q - p), rows)) return false;
+    p = q + 2;
+    q = p;
+    while (q < rest.size() && rest[q] >= '0' && rest[q] <= '9') ++q;
+    if (!parse_uint(rest.substr(p, q - p), group)) return false;
+    *suffix = rest.substr(q);
+    return true;
+}
+
+bool is_pow2(uint32_t v) { return v && !(v & (v - 1)); }
+
+const char* act_suffix(ActDType a) { return a == kActBF16 ? "bf16" : "f16"; }
+
+// resident activation rows per pass for the batched matvec kernels, bounded by LDS
+uint32_t pick_mb(int bits, uint32_t row_stride, uint32_t want, size_t lds_limit) {
+    for (uint32_t mb = want; mb > 1; mb >>= 1)
+        if (matvec_lds_bytes(bits, true, row_stride, mb) <= lds_limit) return mb;
+    return 1;
+}
+
+struct AffineName {
+    const char* prefix;
+    FamilyId m1;
+};
+
+}  // namespace
+
+size_t matvec_lds_bytes(int bits_per_code, bool, uint32_t row_stride_bytes, uint32_t mb) {
+    const size_t U = row_stride_bytes / 16;
+    const size_t chunks = 16 / (size_t)bits_per_code;  // 16-byte LDS chunks of fp16 pairs per unit
+    return (size_t)mb * U * 16 * (chunks + 2);         // + per-dword corrections and sums
+}
+
+uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
+    const uint32_t padded = (cols + 127u) / 128u * 128u;
+    switch (f) {
+        case kFmtBinary1: return padded / 8;
+        case kFmtTernary2: return padded / 4;
+        case kFmtTrit5: return (((cols + 4u) / 5u) + 15u) & ~15u;
+        default: return 0;
+    }
+}
+
+ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act,
+                               size_t lds_limit, ResolvedPipeline* out, std::string* why) {
+    std::string entry = entry_in;
+    ActDType act = default_act;
+    size_t at = entry.find('@');
+    if (at != std::string::npos) {
+        const std::string tag = entry.substr(at + 1);
+        if (tag == "bf16") act = kActBF16;
+        else if (tag == "f16") act = kActF16;
+        else { *why = "unknown dtype tag '" + tag + "'"; return kResolveMalformed; }
+        entry = entry.substr(0, at);
+    }
+    out->act = act;
+    out->appended.clear();
+    out->format = kFmtNone;
+    out->lds_variant = 0;
+    const std::string t = act_suffix(act);
+
+    // ---- function-constant entries: "name:cols:groupSize" --------------------------------
+    size_t colon = entry.find(':');
+    if (colon != std::string::npos) {
+        const std::string name = entry.substr(0, colon);
+        size_t colon2 = entry.find(':', colon + 1);
+        uint32_t cols = 0, group = 0;
+        if (colon2 == std::string::npos || entry.find(':', colon2 + 1) != std::string::npos ||
+            !parse_uint(entry.substr(colon + 1, colon2 - colon - 1), &cols) ||
+            !parse_uint(entry.substr(colon2 + 1), &group)) {
+            *why = "Malformed specialized pipeline entry: '" + entry_in + "'";
+            return kResolveMalformed;
+        }
+        if (name == "affine_matvec") { out->family = kFamAffineMatvec; out->symbol = "smelt_affine_matvec_" + t; out->kinds = "PPPPPUUU"; }
+        else if (name == "fused_affine_matvec_add") { out->family = kFamAffineAdd; out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; }
+        else if (name == "fused_affine_gate_up_swiglu") { out->family = kFamAffineGateUp; out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; }
+        else if (name == "fused_dual_affine_matvec") { out->family = kFamAffineDual; out->symbol = "smelt_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; }
+        else { *why = "no HIP kernel for function-constant pipeline '" + name + "'"; return kResolveUnknown; }
+        if (!is_pow2(group) || group < 32 || cols % 32 != 0 || cols == 0) {
+            *why = "affine kernels need cols % 32 == 0 and a power-of-two group >= 32 (got cols " +
+                   std::to_string(cols) + ", group " + std::to_string(group) + ")";
+            return kResolveMalformed;
+        }
+        out->appended = {cols, group};
+        return kResolveOk;
+    }
+
+    // ---- fixed-shape affine names -----------------------------------------------------------
+    static const AffineName kAffine[] = {
+        {"affine_matvec_argmax", kFamAffineArgmax},
+        {"affine_matvec", kFamAffineMatvec},
+        {"fused_affine_matvec_add", kFamAffineAdd},
+        {"fused_affine_gate_up_swiglu", kFamAffineGateUp},
+        {"fused_dual_affine_matvec", kFamAffineDual},
+    };
+    for (const AffineName& a : kAffine) {
+        const size_t n = strlen(a.prefix);
+        if (entry.compare(0, n, a.prefix) != 0 || entry.size() <= n || entry[n] != '_' || entry[n + 1] != 'c') continue;
+        uint32_t cols, rows, group;
+        std::string suffix;
+        if (!parse_fixed_shape(entry.substr(n), &cols, &rows, &group, &suffix)) continue;
+        if (!is_pow2(group) || group < 32 || cols % 32 != 0 || cols == 0 || rows == 0) {
+            *why = "unsupported affine geometry in '" + entry + "'";
+            return kResolveMalformed;
+        }
+        const uint32_t row_stride = cols / 2;
+        const bool m1 = suffix.empty() || suffix == "_rows4" || suffix == "_rows8" || suffix == "_rows4_sg1";
+        uint32_t bt = 0;
+        bool full = false;
+        if (suffix == "_batched") bt = 8;
+        else if (suffix == "_batched_tile3") bt = 3;
+        else if (suffix == "_batched_tile4" || suffix == "_batched_ext_b4") bt = 4;
+        else if (suffix == "_batched_ext_b5" || suffix == "_batched_sg4_bt5") bt = 5;
+        else if (suffix == "_batched_full") { bt = 16; full = true; }
+        else if (suffix == "_batched_full_b8") { bt = 8; full = true; }
+        else if (!m1) { *why = "unknown kernel variant '" + suffix + "' in '" + entry + "'"; return kResolveUnknown; }
+
+        if (a.m1 == kFamAffineArgmax) {
+            *why = "affine_matvec_argmax is not built yet";
+            return kResolveUnknown;
+        }
+        if (m1) {
+            out->family = a.m1;
+            switch (a.m1) {
+                case kFamAffineMatvec: out->symbol = "smelt_affine_matvec_" + t; out->kinds = "PPPPPUUU"; break;
+                case kFamAffineAdd: out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; break;
+                case kFamAffineGateUp: out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; break;
+                case kFamAffineDual: out->symbol = "smelt_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; break;
+                default: break;
+            }
+            out->appended = {rows, cols, group};
+            return kResolveOk;
+        }
+        if (full) {
+            *why = "affine qmm (batched_full) is not built yet";
+            return kResolveUnknown;
+        }
+        const uint32_t mb = pick_mb(4, row_stride, 4, lds_limit);
+        out->lds_variant = mb;
+        const std::string mbs = "mb" + std::to_string(mb) + "_" + t;
+        if (a.m1 == kFamAffineMatvec) { out->family = kFamAffineBatched; out->symbol = "smelt_affine_matvec_batched_" + mbs; out->kinds = "PPPPPUUUUU"; }
+        else if (a.m1 == kFamAffineGateUp) { out->family = kFamAffineGateUpBatched; out->symbol = "smelt_affine_gate_up_swiglu_batched_" + mbs; out->kinds = "PPPPPPPPUUUUU"; }
+        else { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
+        out->appended = {rows, cols, group, bt};
+        return kResolveOk;
+    }
+
+    // ---- signed g128 names ------------------------------------------------------------------
+    struct SignedName { const char* name; FamilyId fam; SignedFormat fmt; const char* sym; const char* kinds; };
+    static const SignedName kSigned[] = {
+        {"signed_binary_matvec_g128_rows8", kFamSignedMatvec, kFmtBinary1, "smelt_signed_binary_matvec_", "PPPPUU"},
+        {"signed_binary_matvec_add_g128_rows8", kFamSignedAdd, kFmtBinary1, "smelt_signed_binary_matvec_add_", "PPPPPUU"},
+        {"signed_binary_gate_up_swiglu_g128_rows8", kFamSignedGateUp, kFmtBinary1, "smelt_signed_binary_gate_up_swiglu_", "PPPPPPUU"},
+        {"signed_binary_matvec_g128_rows8_batched_b4", kFamSignedB4, kFmtBinary1, "smelt_signed_binary_matvec_b4_", "PPPPUUU"},
+        {"signed_binary_gate_up_swiglu_g128_rows8_batched_b4", kFamSignedGateUpB4, kFmtBinary1, "smelt_signed_binary_gate_up_swiglu_b4_", "PPPPPPUUU"},
+        {"signed_ternary_matvec_g128_rows8", kFamSignedMatvec, kFmtTernary2, "smelt_signed_ternary_matvec_", "PPPPUU"},
+        {"signed_ternary_matvec_add_g128_rows8", kFamSignedAdd, kFmtTernary2, "smelt_signed_ternary_matvec_add_", "PPPPPUU"},
+        {"signed_ternary_gate_up_swiglu_g128_rows8", kFamSignedGateUp, kFmtTernary2, "smelt_signed_ternary_gate_up_swiglu_", "PPPPPPUU"},
+        {"signed_ternary_matvec_g128_rows8_batched_b4", kFamSignedB4, kFmtTernary2, "smelt_signed_ternary_matvec_b4_", "PPPPUUU"},
+        {"signed_ternary_gate_up_swiglu_g128_rows8_batched_b4", kFamSignedGateUpB4, kFmtTernary2, "smelt_signed_ternary_gate_up_swiglu_b4_", "PPPPPPUUU"},
+    };
+    for (const SignedName& s : kSigned) {
+        if (entry == s.name) {
+            out->family = s.fam;
+            out->format = s.fmt;
+            out->symbol = std::string(s.sym) + t;
+            out->kinds = s.kinds;
+            return kResolveOk;
+        }
+    }
+
+    // ---- gathers and argmax -----------------------------------------------------------------
+    if (entry == "affine_embedding_gather") { out->family = kFamAffineGather; out->symbol = "smelt_affine_embedding_gather_" + t; out->kinds = "PPPPPUU"; return kResolveOk; }
+    if (entry == "affine_embedding_gather_batched") { out->family = kFamAffineGatherBatched; out->symbol = "smelt_affine_embedding_gather_batched_" + t; out->kinds = "PPPPPUUU"; return kResolveOk; }
+    if (entry == "signed_binary_embedding_gather_g128") { out->family = kFamSignedGather; out->format = kFmtBinary1; out->symbol = "smelt_signed_binary_embedding_gather_" + t; out->kinds = "PPPPU"; return kResolveOk; }
+    if (entry == "signed_ternary_embedding_gather_g128") { out->family = kFamSignedGather; out->format = kFmtTernary2; out->symbol = "smelt_signed_ternary_embedding_gather_" + t; out->kinds = "PPPPU"; return kResolveOk; }
+    if (entry == "signed_trit5_embedding_gather_g128") { out->family = kFamSignedGather; out->format = kFmtTrit5; out->symbol = "smelt_signed_trit5_embedding_gather_" + t; out->kinds = "PPPPU"; return kResolveOk; }
+    if (entry == "argmax_fp16_partials") { out->family = kFamArgmaxPartials; out->symbol = "smelt_argmax16_partials"; out->kinds = "PPUU"; return kResolveOk; }
+    if (entry == "argmax_key_reduce") { out->family = kFamArgmaxReduce; out->symbol = "smelt_argmax_key_reduce"; out->kinds = "PPU"; return kResolveOk; }
+
+    *why = "no HIP kernel named '" + entry + "'";
+    return kResolveUnknown;
+}
+
+}  // namespace smelt_host

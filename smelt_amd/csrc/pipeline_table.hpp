@@ -1,0 +1,67 @@
+// Pipeline-name resolution: manifest pipeline strings -> (code-object symbol, argument
+// signature, appended shape arguments, validator).  Host-only; shared by the runtime (to
+// launch) and the record emitters (to know what a family binds).
+#pragma once
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+namespace smelt_host {
+
+enum ActDType { kActF16 = 0, kActBF16 = 1 };
+
+enum FamilyId {
+    kFamAffineMatvec = 0,     // W S B x y | rows cols group
+    kFamAffineAdd,            // W S B x y res | rows cols group
+    kFamAffineGateUp,         // gW gS gB uW uS uB x y | rows cols group
+    kFamAffineDual,           // W1 S1 B1 W2 S2 B2 x y1 y2 | rows cols group
+    kFamAffineBatched,        // W S B X Y batch | rows cols group batch_tile
+    kFamAffineGateUpBatched,  // gW gS gB uW uS uB X Y batch | rows cols group batch_tile
+    kFamAffineQmm,            // W S B X Y batch | rows cols group batch_tile
+    kFamAffineQmmAdd,         // W S B X mv res out batch | rows cols group batch_tile
+    kFamAffineQmmGateUp,      // gW gS gB uW uS uB X Y batch | rows cols group batch_tile
+    kFamAffineArgmax,         // W S B X keys batch logit_cap | rows cols group batch_tile rows_per_block
+    kFamLmHeadReduce,         // keys out batch | num_partials(const from record or appended)
+    kFamSignedMatvec,         // C S X Y rows cols                      (batch = grid.y)
+    kFamSignedAdd,            // C S X Y res rows cols
+    kFamSignedGateUp,         // gC gS uC uS X Y rows cols
+    kFamSignedB4,             // C S X Y rows cols batch                (4 batch rows per grid.y)
+    kFamSignedGateUpB4,       // gC gS uC uS X Y rows cols batch
+    kFamTerAffMatvec,         // C S S2 X Y rows cols                   (batch = grid.y)
+    kFamTerAffAdd,            // C S S2 X Y res rows cols
+    kFamTerAffGateUp,         // gC gS gS2 uC uS uS2 X Y rows cols
+    kFamTerAffBank4,          // C S S2 x y0 y1 y2 y3 rows0 rows1 rows2 rows3 cols
+    kFamTerAffQmm,            // C S S2 X Y rows cols batch
+    kFamAffineGather,         // W S B id out cols group
+    kFamAffineGatherBatched,  // W S B ids out cols batch group
+    kFamSignedGather,         // C S ids out hidden
+    kFamArgmaxPartials,       // logits partials vocab chunk
+    kFamArgmaxReduce,         // partials out num_partials
+    kFamCount
+};
+
+enum SignedFormat { kFmtNone = -1, kFmtBinary1 = 0, kFmtTernary2 = 1, kFmtTrit5 = 2 };
+
+struct ResolvedPipeline {
+    FamilyId family;
+    std::string symbol;              // kernel symbol in the code object
+    std::string kinds;               // final argument kinds: 'P' pointer, 'U' u32, 'F' f32
+    std::vector<uint32_t> appended;  // values appended after the record's own bindings
+    ActDType act;
+    SignedFormat format = kFmtNone;
+    uint32_t lds_variant = 0;        // batched families: activations resident per pass (1, 2, 4)
+};
+
+enum ResolveStatus { kResolveOk = 0, kResolveUnknown = 1, kResolveMalformed = 2 };
+
+// entry: "fn", "fn:cols:group", optionally followed by "@f16" / "@bf16".
+ResolveStatus resolve_pipeline(const std::string& entry, ActDType default_act, size_t lds_limit,
+                               ResolvedPipeline* out, std::string* why);
+
+// LDS bytes the matvec kernels need for `cols` columns of a format with `mb` resident rows.
+size_t matvec_lds_bytes(int bits_per_code, bool has_bias, uint32_t row_stride_bytes, uint32_t mb);
+
+uint32_t signed_row_stride(SignedFormat f, uint32_t cols);
+
+}  // namespace smelt_host

@@ -1,0 +1,844 @@
+// libsmelt_hip runtime: the HIP side of Smelt's dispatch-record interpreter.
+// Mirrors what SmeltRuntime does with MTLDevice / MTLLibrary / MTLComputePipelineState /
+// MTLBuffer / MTLComputeCommandEncoder (SmeltRuntime.swift:668-998, 3150-3275, 5990-6207).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/smelt_hip.h"
+#include "pipeline_table.hpp"
+
+using namespace smelt_host;
+
+static_assert(sizeof(SmeltBufferRecord) == 16, "SmeltBufferRecord stride");
+static_assert(sizeof(SmeltConstantRecord) == 8, "SmeltConstantRecord stride");
+static_assert(sizeof(SmeltDispatchRecord) == 360, "SmeltDispatchRecord stride");
+static_assert(offsetof(SmeltDispatchRecord, pipeline) == 2, "pipeline offset");
+static_assert(offsetof(SmeltDispatchRecord, min_seq_len) == 8, "minSeqLen offset");
+static_assert(offsetof(SmeltDispatchRecord, grid_w) == 12, "gridW offset");
+static_assert(offsetof(SmeltDispatchRecord, buffers) == 40, "buffers offset");
+static_assert(offsetof(SmeltDispatchRecord, constants) == 296, "constants offset");
+
+namespace {
+
+constexpr int kMaxSlots = 4096;
+
+struct SlotBuffer {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    bool read_only = false;
+};
+
+struct Pipeline {
+    std::string entry;
+    bool ready = false;
+    hipFunction_t fn = nullptr;
+    ResolvedPipeline res;
+};
+
+thread_local std::string g_global_error;
+
+}  // namespace
+
+struct smelt_hip_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int launches = 0;
+};
+
+struct smelt_hip_context {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_end = nullptr;
+    bool batch_open = false;
+    bool timing_valid = false;
+    hipModule_t module = nullptr;
+    std::vector<Pipeline> pipelines;
+    std::mutex pipeline_mutex;
+    std::vector<SlotBuffer> slots;
+    int weights_slot = -1;
+    ActDType default_act = kActF16;
+    uint32_t cache_seq_capacity = 0;
+    size_t lds_limit = 65536;
+    hipDeviceProp_t props;
+    mutable std::string error;
+};
+
+namespace {
+
+int fail(const smelt_hip_context* ctx, int code, const std::string& msg) {
+    if (ctx) ctx->error = msg;
+    else g_global_error = msg;
+    return code;
+}
+
+int hip_fail(const smelt_hip_context* ctx, hipError_t e, const char* what) {
+    return fail(ctx, SMELT_HIP_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIP_TRY(ctx, call)                                      \
+    do {                                                        \
+        hipError_t _e = (call);                                 \
+        if (_e != hipSuccess) return hip_fail(ctx, _e, #call);  \
+    } while (0)
+
+struct Arg {
+    char kind = 0;  // 'P', 'U', 'F' or 0 (unset)
+    uint32_t value = 0;
+    char* ptr = nullptr;
+    size_t avail = 0;  // bytes from ptr to the end of its slot
+    bool writable = false;
+};
+
+struct Launch {
+    std::vector<Arg> args;
+    uint32_t grid[3];
+    uint32_t block[3];
+    size_t lds = 0;
+};
+
+size_t cdiv(size_t a, size_t b) { return (a + b - 1) / b; }
+
+// Checks operand extents against what the kernel will touch, and computes its LDS need.
+// Every hand-written kernel is only launched after this passes.
+int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
+    const ResolvedPipeline& r = p.res;
+    auto U = [&](size_t i) -> size_t { return L.args[i].value; };
+    std::vector<size_t> need(L.args.size(), 0);
+    std::vector<bool> written(L.args.size(), false);
+    std::vector<size_t> align(L.args.size(), 2);
+    const size_t gy = L.grid[1];
+    auto bad_geom = [&](const std::string& m) {
+        return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
+    };
+    const bool matvec_like = r.family <= kFamTerAffQmm;
+    if (matvec_like) {
+        if (L.block[0] % 64 != 0 || L.block[0] == 0 || L.block[0] > 256 || L.block[1] != 1 || L.block[2] != 1)
+            return bad_geom("threadgroup must be 64..256 threads in whole wavefronts, got " +
+                            std::to_string(L.block[0]) + "x" + std::to_string(L.block[1]) + "x" + std::to_string(L.block[2]));
+        if (L.grid[2] != 1) return bad_geom("grid depth must be 1");
+    }
+    auto affine = [&](size_t w, size_t s, size_t b, size_t rows, size_t cols, size_t group) {
+        need[w] = rows * (cols / 2);
+        align[w] = 16;
+        const size_t gpr = cdiv(cols, group);
+        need[s] = need[b] = rows * gpr * 2;
+    };
+    auto signed_w = [&](size_t c, size_t s, size_t rows, size_t cols) {
+        need[c] = rows * (size_t)signed_row_stride(r.format, (uint32_t)cols);
+        align[c] = 16;
+        need[s] = rows * cdiv(cols, 128) * 2;
+    };
+    auto check_affine_shape = [&](size_t rows, size_t cols, size_t group) -> int {
+        if (rows == 0 || cols == 0 || cols % 32 != 0 || group < 32 || (group & (group - 1)))
+            return bad_geom("affine kernels need rows > 0, cols % 32 == 0 and a power-of-two group >= 32");
+        return 0;
+    };
+    auto check_signed_shape = [&](size_t rows, size_t cols) -> int {
+        if (rows == 0 || cols == 0 || cols % 128 != 0)
+            return bad_geom("signed g128 kernels need rows > 0 and cols % 128 == 0");
+        return 0;
+    };
+    int bits = 4;
+    if (r.format == kFmtBinary1) bits = 1;
+    if (r.format == kFmtTernary2) bits = 2;
+    switch (r.family) {
+        case kFamAffineMatvec:
+        case kFamAffineAdd: {
+            const size_t o = r.family == kFamAffineAdd ? 6 : 5;
+            const size_t rows = U(o), cols = U(o + 1), group = U(o + 2);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            affine(0, 1, 2, rows, cols, group);
+            need[3] = gy * cols * 2; align[3] = 16;
+            need[4] = gy * rows * 2; written[4] = true;
+            if (r.family == kFamAffineAdd) need[5] = gy * rows * 2;
+            L.lds = matvec_lds_bytes(4, true, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamAffineGateUp:
+        case kFamAffineDual: {
+            const size_t o = r.family == kFamAffineDual ? 9 : 8;
+            const size_t rows = U(o), cols = U(o + 1), group = U(o + 2);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            affine(0, 1, 2, rows, cols, group);
+            affine(3, 4, 5, rows, cols, group);
+            need[6] = gy * cols * 2; align[6] = 16;
+            need[7] = gy * rows * 2; written[7] = true;
+            if (r.family == kFamAffineDual) { need[8] = gy * rows * 2; written[8] = true; }
+            L.lds = matvec_lds_bytes(4, true, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamAffineBatched:
+        case kFamAffineGateUpBatched: {
+            const size_t o = r.family == kFamAffineGateUpBatched ? 8 : 5;
+            const size_t batch = U(o), rows = U(o + 1), cols = U(o + 2), group = U(o + 3), bt = U(o + 4);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (bt == 0 || gy * bt < batch) return bad_geom("grid height * batch tile does not cover the batch");
+            affine(0, 1, 2, rows, cols, group);
+            size_t xi = 3, yi = 4;
+            if (r.family == kFamAffineGateUpBatched) { affine(3, 4, 5, rows, cols, group); xi = 6; yi = 7; }
+            need[xi] = batch * cols * 2; align[xi] = 16;
+            need[yi] = batch * rows * 2; written[yi] = true;
+            L.lds = matvec_lds_bytes(4, true, (uint32_t)(cols / 2), r.lds_variant);
+            break;
+        }
+        case kFamSignedMatvec:
+        case kFamSignedAdd: {
+            const size_t o = r.family == kFamSignedAdd ? 5 : 4;
+            const size_t rows = U(o), cols = U(o + 1);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            signed_w(0, 1, rows, cols);
+            need[2] = gy * cols * 2; align[2] = 16;
+            need[3] = gy * rows * 2; written[3] = true;
+            if (r.family == kFamSignedAdd) need[4] = gy * rows * 2;
+            L.lds = matvec_lds_bytes(bits, false, signed_row_stride(r.format, (uint32_t)cols), 1);
+            break;
+        }
+        case kFamSignedGateUp: {
+            const size_t rows = U(6), cols = U(7);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            signed_w(0, 1, rows, cols);
+            signed_w(2, 3, rows, cols);
+            need[4] = gy * cols * 2; align[4] = 16;
+            need[5] = gy * rows * 2; written[5] = true;
+            L.lds = matvec_lds_bytes(bits, false, signed_row_stride(r.format, (uint32_t)cols), 1);
+            break;
+        }
+        case kFamSignedB4:
+        case kFamSignedGateUpB4: {
+            const size_t o = r.family == kFamSignedGateUpB4 ? 6 : 4;
+            const size_t rows = U(o), cols = U(o + 1), batch = U(o + 2);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            if (gy * 4 < batch) return bad_geom("grid height * 4 does not cover the batch");
+            signed_w(0, 1, rows, cols);
+            size_t xi = 2, yi = 3;
+            if (r.family == kFamSignedGateUpB4) { signed_w(2, 3, rows, cols); xi = 4; yi = 5; }
+            need[xi] = batch * cols * 2; align[xi] = 16;
+            need[yi] = batch * rows * 2; written[yi] = true;
+            L.lds = matvec_lds_bytes(bits, false, signed_row_stride(r.format, (uint32_t)cols), 2);
+            break;
+        }
+        case kFamAffineGather:
+        case kFamAffineGatherBatched: {
+            const bool batched = r.family == kFamAffineGatherBatched;
+            const size_t cols = U(5), batch = batched ? U(6) : 1, group = batched ? U(7) : U(6);
+            if (cols == 0 || cols % 2 != 0 || group == 0 || cols % group != 0)
+                return bad_geom("gather needs even cols divisible by the group size");
+            need[3] = batch * 4; align[3] = 4;
+            need[4] = batch * cols * 2; written[4] = true;
+            if (L.grid[0] * (size_t)L.block[0] < cols / 2 || (batched && gy < batch))
+                return bad_geom("grid does not cover the gather");
+            break;
+        }
+        case kFamSignedGather: {
+            const size_t hidden = U(4);
+            if (hidden == 0 || hidden % 128 != 0) return bad_geom("signed gather needs hidden % 128 == 0");
+            need[2] = gy * 4; align[2] = 4;
+            need[3] = gy * hidden * 2; written[3] = true;
+            if (L.grid[0] * (size_t)L.block[0] < hidden) return bad_geom("grid does not cover the gather");
+            break;
+        }
+        case kFamArgmaxPartials: {
+            const size_t vocab = U(2), chunk = U(3);
+            if (chunk == 0 || (size_t)L.grid[0] * chunk < vocab) return bad_geom("chunks do not cover the vocabulary");
+            if (vocab > (1u << 18)) return bad_geom("argmax keys hold 18 index bits");
+            need[0] = vocab * 2;
+            need[1] = (size_t)L.grid[0] * 8; align[1] = 8; written[1] = true;
+            break;
+        }
+        case kFamArgmaxReduce: {
+            need[0] = (size_t)L.grid[0] * U(2) * 8; align[0] = 8;
+            need[1] = (size_t)L.grid[0] * 4; align[1] = 4; written[1] = true;
+            break;
+        }
+        default:
+            return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "pipeline '" + p.entry + "' has no launch validator");
+    }
+    if (L.lds > ctx->lds_limit)
+        return bad_geom("needs " + std::to_string(L.lds) + " bytes of LDS, device allows " + std::to_string(ctx->lds_limit));
+    for (size_t i = 0; i < L.args.size(); ++i) {
+        if (L.args[i].kind != 'P') continue;
+        if (need[i] > L.args[i].avail)
+            return fail(ctx, SMELT_HIP_ERR_OUT_OF_RANGE,
+                        "pipeline '" + p.entry + "': argument " + std::to_string(i) + " needs " +
+                            std::to_string(need[i]) + " bytes, slot has " + std::to_string(L.args[i].avail) + " from its offset");
+        if (((uintptr_t)L.args[i].ptr) % align[i] != 0)
+            return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY,
+                        "pipeline '" + p.entry + "': argument " + std::to_string(i) + " must be " + std::to_string(align[i]) + "-byte aligned");
+        if (written[i] && !L.args[i].writable)
+            return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT,
+                        "pipeline '" + p.entry + "': output argument " + std::to_string(i) + " is bound to the read-only weights slot");
+    }
+    return 0;
+}
+
+struct Dyn {
+    bool prefill;
+    int32_t position;  // decode
+    int32_t seq_len, start_pos;
+};
+
+// resolveDispatchBufferOffset: SmeltRuntime.swift:6158-6184; decode form :3207-3209
+int resolve_offset(smelt_hip_context* ctx, const SmeltBufferRecord& b, const Dyn& d, size_t* out) {
+    if (!d.prefill) {
+        *out = b.offset_kind == 0 ? (size_t)b.offset : (size_t)((int64_t)d.position * (int64_t)b.offset);
+        return 0;
+    }
+    switch (b.offset_kind) {
+        case 0: *out = (size_t)b.offset; return 0;
+        case 1: *out = (size_t)((int64_t)d.start_pos * (int64_t)b.offset); return 0;
+        case 2: *out = (size_t)((int64_t)d.start_pos * (int64_t)(b.offset & 0xFFFFFFFFu) + (int64_t)(b.offset >> 32)); return 0;
+        case 3: *out = (size_t)((int64_t)(d.seq_len - 1) * (int64_t)b.offset); return 0;
+        case 4: {
+            const int64_t stride = (int64_t)(b.offset & 0xFFFFFFFFu);
+            const int64_t divisor = std::max<int64_t>((int64_t)(b.offset >> 32), 1);
+            *out = (size_t)(((int64_t)d.seq_len / divisor) * stride);
+            return 0;
+        }
+        default:
+            return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE,
+                        "unknown dispatch offsetKind " + std::to_string(b.offset_kind) + " - emitter/runtime mismatch");
+    }
+}
+
+// resolveDecodeConstant / resolvePrefillConstant: SmeltRuntime.swift:1189-1252
+uint32_t resolve_constant(const smelt_hip_context* ctx, const SmeltConstantRecord& c, const Dyn& d, bool* skip) {
+    if (!d.prefill) {
+        switch (c.kind) {
+            case SMELT_CONST_POSITION: return (uint32_t)d.position;
+            case SMELT_CONST_POSITION_PLUS1: return (uint32_t)(d.position + 1);
+            case SMELT_CONST_POSITION_PLUS1_LT_LITERAL_SKIP_IF_FALSE: {
+                const uint32_t v = (uint32_t)(d.position + 1) < c.value ? 1 : 0;
+                if (!v) *skip = true;
+                return v;
+            }
+            case SMELT_CONST_POSITION_PLUS1_GE_LITERAL_SKIP_IF_FALSE: {
+                const uint32_t v = (uint32_t)(d.position + 1) >= c.value ? 1 : 0;
+                if (!v) *skip = true;
+                return v;
+            }
+            case SMELT_CONST_CACHE_SEQ_CAPACITY: return ctx->cache_seq_capacity;
+            default: return c.value;
+        }
+    }
+    const uint32_t s = (uint32_t)d.seq_len, p = (uint32_t)d.start_pos;
+    switch (c.kind) {
+        case SMELT_CONST_POSITION: return p;
+        case SMELT_CONST_POSITION_PLUS1: return p + 1;
+        case SMELT_CONST_SEQ_LEN: return s;
+        case SMELT_CONST_SEQ_LEN_MUL_LITERAL: return s * c.value;
+        case SMELT_CONST_SEQ_LEN_MOD_LITERAL: return c.value == 0 ? 0 : s % c.value;
+        case SMELT_CONST_SEQ_LEN_MOD_LITERAL_SKIP_IF_ZERO: {
+            const uint32_t v = c.value == 0 ? 0 : s % c.value;
+            if (!v) *skip = true;
+            return v;
+        }
+        case SMELT_CONST_SEQ_LEN_LT_LITERAL_SKIP_IF_FALSE: {
+            const uint32_t v = s < c.value ? 1 : 0;
+            if (!v) *skip = true;
+            return v;
+        }
+        case SMELT_CONST_START_POS: return p;
+        case SMELT_CONST_START_POS_PLUS_LITERAL: return p + c.value;
+        case SMELT_CONST_CACHE_SEQ_CAPACITY: return ctx->cache_seq_capacity;
+        default: return c.value;
+    }
+}
+
+// resolvePrefillGrid: SmeltRuntime.swift:6186-6207
+uint32_t resolve_grid(uint32_t literal, uint8_t kind, int32_t seq_len) {
+    const int64_t s = std::max<int64_t>(seq_len, 0);
+    switch (kind) {
+        case SMELT_GRID_SEQ_LEN: return (uint32_t)s;
+        case SMELT_GRID_SEQ_LEN_MUL_LITERAL: return (uint32_t)(s * (int64_t)literal);
+        case SMELT_GRID_SEQ_LEN_CEIL_DIV_LITERAL: {
+            const int64_t divisor = std::max<int64_t>(literal & 0x7FFFFFFFu, 1);
+            if (literal & 0x80000000u) return (uint32_t)(s / divisor);
+            return (uint32_t)((s + divisor - 1) / divisor);
+        }
+        default: return literal;
+    }
+}
+
+const Pipeline* pipeline_for(smelt_hip_context* ctx, uint32_t index) {
+    // "fallback to previous": SmeltRuntime.swift:453-456, 6305-6306
+    std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);
+    if (index >= ctx->pipelines.size()) return nullptr;
+    for (int64_t i = index; i >= 0; --i)
+        if (ctx->pipelines[(size_t)i].ready) return &ctx->pipelines[(size_t)i];
+    return nullptr;
+}
+
+// Returns 1 launched, 0 skipped, <0 error.
+int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cur, int alt, const Dyn& d) {
+    if (!ctx || !rec) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or record");
+    if (rec->op_kind != SMELT_OP_DISPATCH) return 0;
+    if (d.prefill && rec->min_seq_len > 0 && (uint32_t)d.seq_len < (uint32_t)rec->min_seq_len) return 0;
+    if (rec->buffer_count > SMELT_MAX_BUFFERS_PER_DISPATCH || rec->constant_count > SMELT_MAX_CONSTANTS_PER_DISPATCH)
+        return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, "record binding counts exceed the table format");
+    const Pipeline* p = pipeline_for(ctx, rec->pipeline);
+    if (!p) return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "record names pipeline index " + std::to_string(rec->pipeline) + " which has no launchable kernel");
+
+    const std::string& kinds = p->res.kinds;
+    Launch L;
+    L.args.resize(kinds.size());
+    const size_t own = kinds.size() - p->res.appended.size();
+    for (int i = 0; i < rec->buffer_count; ++i) {
+        const SmeltBufferRecord& b = rec->buffers[i];
+        int slot = b.slot >= 0 ? b.slot : (b.slot == SMELT_SLOT_CUR ? cur : alt);
+        if (slot < 0 || (size_t)slot >= ctx->slots.size() || !ctx->slots[(size_t)slot].ptr)
+            return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "record binds slot " + std::to_string(slot) + " which has no buffer");
+        size_t off = 0;
+        if (int e = resolve_offset(ctx, b, d, &off)) return e;
+        const SlotBuffer& sb = ctx->slots[(size_t)slot];
+        if (off > sb.bytes)
+            return fail(ctx, SMELT_HIP_ERR_OUT_OF_RANGE, slot == ctx->weights_slot
+                            ? "weight offset " + std::to_string(off) + " is outside the mapped weight segments"
+                            : "offset " + std::to_string(off) + " is outside slot " + std::to_string(slot));
+        if (b.binding_index >= own || kinds[b.binding_index] != 'P')
+            return fail(ctx, SMELT_HIP_ERR_BINDING_MISMATCH, "pipeline '" + p->entry + "' takes no buffer at index " + std::to_string(b.binding_index));
+        Arg& a = L.args[b.binding_index];
+        a.kind = 'P';
+        a.ptr = (char*)sb.ptr + off;
+        a.avail = sb.bytes - off;
+        a.writable = !sb.read_only;
+    }
+    bool skip = false;
+    for (int i = 0; i < rec->constant_count; ++i) {
+        const SmeltConstantRecord& c = rec->constants[i];
+        const uint32_t v = resolve_constant(ctx, c, d, &skip);
+        if (c.binding_index == 0xFF) continue;
+        if (c.binding_index >= own || kinds[c.binding_index] == 'P')
+            return fail(ctx, SMELT_HIP_ERR_BINDING_MISMATCH, "pipeline '" + p->entry + "' takes no constant at index " + std::to_string(c.binding_index));
+        Arg& a = L.args[c.binding_index];
+        a.kind = kinds[c.binding_index];
+        a.value = v;
+    }
+    if (skip) return 0;
+    for (size_t i = 0; i < p->res.appended.size(); ++i) {
+        Arg& a = L.args[own + i];
+        a.kind = 'U';
+        a.value = p->res.appended[i];
+    }
+    for (size_t i = 0; i < L.args.size(); ++i)
+        if (L.args[i].kind == 0)
+            return fail(ctx, SMELT_HIP_ERR_BINDING_MISMATCH, "pipeline '" + p->entry + "': argument " + std::to_string(i) + " is not bound by the record");
+
+    uint32_t gw = rec->grid_w, gh = rec->grid_h, gd = rec->grid_d;
+    if (d.prefill) {
+        gw = resolve_grid(rec->grid_w, (rec->style >> 2) & 3, d.seq_len);
+        gh = resolve_grid(rec->grid_h, (rec->style >> 4) & 3, d.seq_len);
+        gd = resolve_grid(rec->grid_d, (rec->style >> 6) & 3, d.seq_len);
+    }
+    if (gw == 0 || gh == 0 || gd == 0) return 0;
+    if (rec->tg_w == 0 || rec->tg_h == 0 || rec->tg_d == 0)
+        return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, "record has an empty threadgroup");
+    L.block[0] = rec->tg_w; L.block[1] = rec->tg_h; L.block[2] = rec->tg_d;
+    if ((rec->style & 3) == SMELT_STYLE_THREADGROUPS) {
+        L.grid[0] = gw; L.grid[1] = gh; L.grid[2] = gd;
+    } else {  // dispatchThreads: grid counts threads; kernels bounds-check the ragged edge
+        L.grid[0] = (uint32_t)cdiv(gw, rec->tg_w);
+        L.grid[1] = (uint32_t)cdiv(gh, rec->tg_h);
+        L.grid[2] = (uint32_t)cdiv(gd, rec->tg_d);
+    }
+    if ((size_t)L.block[0] * L.block[1] * L.block[2] > 1024)
+        return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "threadgroup exceeds 1024 threads");
+    if (int e = validate_launch(ctx, *p, L)) return e;
+
+    // kernarg block: natural alignment in argument order
+    alignas(16) unsigned char kernarg[512];
+    size_t pos = 0;
+    for (const Arg& a : L.args) {
+        if (a.kind == 'P') {
+            pos = (pos + 7) & ~(size_t)7;
+            void* ptr = a.ptr;
+            memcpy(kernarg + pos, &ptr, 8);
+            pos += 8;
+        } else {
+            memcpy(kernarg + pos, &a.value, 4);
+            pos += 4;
+        }
+    }
+    size_t kernarg_size = pos;
+    void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, kernarg, HIP_LAUNCH_PARAM_BUFFER_SIZE, &kernarg_size, HIP_LAUNCH_PARAM_END};
+    if (!ctx->batch_open) {
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+        ctx->batch_open = true;
+        ctx->timing_valid = false;
+    }
+    HIP_TRY(ctx, hipModuleLaunchKernel(p->fn, L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2],
+                                       (unsigned)L.lds, ctx->stream, nullptr, config));
+    return 1;
+}
+
+int interpret(smelt_hip_context* ctx, const SmeltDispatchRecord* table, size_t count, int cur, int alt, const Dyn& d) {
+    if (!ctx || (!table && count)) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or table");
+    int launched = 0;
+    for (size_t i = 0; i < count; ++i) {
+        if (table[i].op_kind == SMELT_OP_SWAP) { std::swap(cur, alt); continue; }
+        const int rc = encode_record(ctx, &table[i], cur, alt, d);
+        if (rc < 0) {
+            ctx->error = "record " + std::to_string(i) + ": " + ctx->error;
+            return rc;
+        }
+        launched += rc;
+    }
+    return launched;
+}
+
+}  // namespace
+
+extern "C" {
+
+int smelt_hip_context_create(int device_index, smelt_hip_context** out) {
+    if (!out) return fail(nullptr, SMELT_HIP_ERR_INVALID_ARGUMENT, "out is null");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0)
+        return fail(nullptr, SMELT_HIP_ERR_NO_DEVICE, std::string("no HIP device: ") + (e != hipSuccess ? hipGetErrorString(e) : "device count is 0"));
+    if (device_index < 0 || device_index >= count)
+        return fail(nullptr, SMELT_HIP_ERR_INVALID_ARGUMENT, "device index out of range");
+    smelt_hip_context* ctx = new smelt_hip_context();
+    ctx->device = device_index;
+    ctx->slots.resize(64);
+    auto bail = [&](hipError_t err, const char* what) {
+        int rc = hip_fail(nullptr, err, what);
+        delete ctx;
+        return rc;
+    };
+    if ((e = hipSetDevice(device_index)) != hipSuccess) return bail(e, "hipSetDevice");
+    if ((e = hipGetDeviceProperties(&ctx->props, device_index)) != hipSuccess) return bail(e, "hipGetDeviceProperties");
+    if ((e = hipStreamCreate(&ctx->stream)) != hipSuccess) return bail(e, "hipStreamCreate");
+    if ((e = hipEventCreate(&ctx->ev_start)) != hipSuccess) return bail(e, "hipEventCreate");
+    if ((e = hipEventCreate(&ctx->ev_end)) != hipSuccess) return bail(e, "hipEventCreate");
+    ctx->lds_limit = ctx->props.sharedMemPerBlock ? ctx->props.sharedMemPerBlock : 65536;
+    *out = ctx;
+    return SMELT_HIP_OK;
+}
+
+void smelt_hip_context_destroy(smelt_hip_context* ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (SlotBuffer& s : ctx->slots)
+        if (s.ptr) (void)hipFree(s.ptr);
+    if (ctx->module) (void)hipModuleUnload(ctx->module);
+    if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+    if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+const char* smelt_hip_last_error(const smelt_hip_context* ctx) {
+    return ctx ? ctx->error.c_str() : g_global_error.c_str();
+}
+
+int smelt_hip_set_activation_dtype(smelt_hip_context* ctx, int act_dtype) {
+    if (!ctx || (act_dtype != SMELT_HIP_ACT_F16 && act_dtype != SMELT_HIP_ACT_BF16))
+        return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "activation dtype must be SMELT_HIP_ACT_F16 or SMELT_HIP_ACT_BF16");
+    ctx->default_act = act_dtype == SMELT_HIP_ACT_BF16 ? kActBF16 : kActF16;
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_module_load(smelt_hip_context* ctx, const void* code_object, size_t bytes) {
+    if (!ctx || !code_object || bytes == 0) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or empty code object");
+    if (ctx->module) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "a code object is already loaded");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipModuleLoadData(&ctx->module, code_object));
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_module_load_file(smelt_hip_context* ctx, const char* path) {
+    if (!ctx || !path) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or path");
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, std::string("cannot open code object '") + path + "'");
+    std::vector<char> data((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    if (data.empty()) return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, std::string("code object '") + path + "' is empty");
+    return smelt_hip_module_load(ctx, data.data(), data.size());
+}
+
+int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int allow_missing, uint32_t* out_index) {
+    if (!ctx || !entry) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or entry");
+    if (!ctx->module) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "load a code object before creating pipelines");
+    Pipeline p;
+    p.entry = entry;
+    std::string why;
+    const ResolveStatus st = resolve_pipeline(p.entry, ctx->default_act, ctx->lds_limit, &p.res, &why);
+    if (st == kResolveMalformed) return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, why);
+    if (st == kResolveUnknown && !allow_missing) return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, why);
+    if (st == kResolveOk) {
+        hipError_t e = hipModuleGetFunction(&p.fn, ctx->module, p.res.symbol.c_str());
+        if (e != hipSuccess) {
+            if (!allow_missing)
+                return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "code object has no kernel '" + p.res.symbol + "' for pipeline '" + p.entry + "': " + hipGetErrorString(e));
+        } else {
+            p.ready = true;
+        }
+    }
+    std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);
+    if (ctx->pipelines.size() >= 65536) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "pipeline index is 16 bits");
+    ctx->pipelines.push_back(std::move(p));
+    if (out_index) *out_index = (uint32_t)(ctx->pipelines.size() - 1);
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_pipeline_count(const smelt_hip_context* ctx) {
+    return ctx ? (int)ctx->pipelines.size() : SMELT_HIP_ERR_INVALID_ARGUMENT;
+}
+
+int smelt_hip_pipeline_is_ready(const smelt_hip_context* ctx, uint32_t index) {
+    if (!ctx || index >= ctx->pipelines.size()) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    return ctx->pipelines[index].ready ? 1 : 0;
+}
+
+static int alloc_slot(smelt_hip_context* ctx, int slot, size_t bytes, bool read_only) {
+    if (!ctx || slot < 0 || slot >= kMaxSlots) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "slot index out of range");
+    if (bytes == 0) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "zero-length buffer");
+    if ((size_t)slot >= ctx->slots.size()) ctx->slots.resize((size_t)slot + 1);
+    SlotBuffer& s = ctx->slots[(size_t)slot];
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    if (s.ptr) {
+        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        HIP_TRY(ctx, hipFree(s.ptr));
+        s = SlotBuffer();
+    }
+    // 256 bytes of slack keep whole-vector loads of a ragged tail inside the allocation
+    HIP_TRY(ctx, hipMalloc(&s.ptr, bytes + 256));
+    HIP_TRY(ctx, hipMemset(s.ptr, 0, bytes + 256));
+    s.bytes = bytes;
+    s.read_only = read_only;
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_buffer_alloc(smelt_hip_context* ctx, int slot, size_t bytes) {
+    return alloc_slot(ctx, slot, bytes, false);
+}
+
+int smelt_hip_weights_upload(smelt_hip_context* ctx, int weights_slot, const void* bytes, size_t size) {
+    if (!bytes) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null weights");
+    if (int e = alloc_slot(ctx, weights_slot, size, true)) return e;
+    HIP_TRY(ctx, hipMemcpy(ctx->slots[(size_t)weights_slot].ptr, bytes, size, hipMemcpyHostToDevice));
+    ctx->weights_slot = weights_slot;
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_buffer_write(smelt_hip_context* ctx, int slot, size_t offset, const void* src, size_t bytes) {
+    if (!ctx || !src || slot < 0 || (size_t)slot >= ctx->slots.size() || !ctx->slots[(size_t)slot].ptr)
+        return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "bad slot or null source");
+    SlotBuffer& s = ctx->slots[(size_t)slot];
+    if (offset > s.bytes || bytes > s.bytes - offset) return fail(ctx, SMELT_HIP_ERR_OUT_OF_RANGE, "write past the end of the slot");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, hipMemcpy((char*)s.ptr + offset, src, bytes, hipMemcpyHostToDevice));
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_buffer_read(smelt_hip_context* ctx, int slot, size_t offset, void* dst, size_t bytes) {
+    if (!ctx || !dst || slot < 0 || (size_t)slot >= ctx->slots.size() || !ctx->slots[(size_t)slot].ptr)
+        return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "bad slot or null destination");
+    SlotBuffer& s = ctx->slots[(size_t)slot];
+    if (offset > s.bytes || bytes > s.bytes - offset) return fail(ctx, SMELT_HIP_ERR_OUT_OF_RANGE, "read past the end of the slot");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, hipMemcpy(dst, (char*)s.ptr + offset, bytes, hipMemcpyDeviceToHost));
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_buffer_size(const smelt_hip_context* ctx, int slot, size_t* bytes) {
+    if (!ctx || !bytes || slot < 0 || (size_t)slot >= ctx->slots.size() || !ctx->slots[(size_t)slot].ptr)
+        return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "bad slot");
+    *bytes = ctx->slots[(size_t)slot].bytes;
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_set_cache_seq_capacity(smelt_hip_context* ctx, uint32_t capacity) {
+    if (!ctx) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context");
+    ctx->cache_seq_capacity = capacity;
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_dispatch_table_count(size_t table_bytes, size_t* out_count) {
+    if (!out_count) return fail(nullptr, SMELT_HIP_ERR_INVALID_ARGUMENT, "out_count is null");
+    if (table_bytes % sizeof(SmeltDispatchRecord) != 0)
+        return fail(nullptr, SMELT_HIP_ERR_INVALID_PACKAGE,
+                    "dispatch table size " + std::to_string(table_bytes) + " is not a multiple of dispatch stride " + std::to_string(sizeof(SmeltDispatchRecord)));
+    *out_count = table_bytes / sizeof(SmeltDispatchRecord);
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_encode_decode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cur, int alt, int32_t position) {
+    Dyn d{false, position, 0, 0};
+    return encode_record(ctx, rec, cur, alt, d);
+}
+
+int smelt_hip_encode_prefill_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cur, int alt, int32_t seq_len, int32_t start_pos) {
+    Dyn d{true, 0, seq_len, start_pos};
+    return encode_record(ctx, rec, cur, alt, d);
+}
+
+int smelt_hip_interpret_decode_table(smelt_hip_context* ctx, const SmeltDispatchRecord* table, size_t count, int cur0, int alt0, int32_t position) {
+    Dyn d{false, position, 0, 0};
+    return interpret(ctx, table, count, cur0, alt0, d);
+}
+
+int smelt_hip_interpret_prefill_table(smelt_hip_context* ctx, const SmeltDispatchRecord* table, size_t count, int cur0, int alt0, int32_t seq_len, int32_t start_pos) {
+    Dyn d{true, 0, seq_len, start_pos};
+    return interpret(ctx, table, count, cur0, alt0, d);
+}
+
+int smelt_hip_submit(smelt_hip_context* ctx) {
+    if (!ctx) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context");
+    if (ctx->batch_open) {
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_end, ctx->stream));
+        ctx->batch_open = false;
+        ctx->timing_valid = true;
+    }
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_wait(smelt_hip_context* ctx) {
+    if (!ctx) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context");
+    if (ctx->batch_open) {
+        if (int e = smelt_hip_submit(ctx)) return e;
+    }
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_last_gpu_ns(smelt_hip_context* ctx, uint64_t* out_ns) {
+    if (!ctx || !out_ns) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    if (!ctx->timing_valid) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "no submitted batch to time");
+    HIP_TRY(ctx, hipEventSynchronize(ctx->ev_end));
+    float ms = 0;
+    HIP_TRY(ctx, hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_end));
+    *out_ns = (uint64_t)((double)ms * 1e6);
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_benchmark_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cur, int alt, int prefill,
+                               int32_t a, int32_t b, int warmup, int iters, float* out_us) {
+    if (!ctx || !rec || !out_us || iters <= 0 || warmup < 0) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "bad benchmark arguments");
+    Dyn d{prefill != 0, prefill ? 0 : a, prefill ? a : 0, prefill ? b : 0};
+    if (int e = smelt_hip_wait(ctx)) return e;
+    for (int i = 0; i < warmup; ++i) {
+        const int rc = encode_record(ctx, rec, cur, alt, d);
+        if (rc < 0) return rc;
+        if (rc == 0) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "record does not dispatch for these arguments");
+    }
+    if (int e = smelt_hip_wait(ctx)) return e;
+    std::vector<hipEvent_t> ev((size_t)iters * 2);
+    for (hipEvent_t& e : ev) HIP_TRY(ctx, hipEventCreate(&e));
+    int status = SMELT_HIP_OK;
+    ctx->batch_open = true;  // keep encode_record from re-recording the batch start event
+    for (int i = 0; i < iters && status == SMELT_HIP_OK; ++i) {
+        if (hipEventRecord(ev[(size_t)2 * i], ctx->stream) != hipSuccess) { status = fail(ctx, SMELT_HIP_ERR_HIP, "hipEventRecord"); break; }
+        const int rc = encode_record(ctx, rec, cur, alt, d);
+        if (rc < 0) { status = rc; break; }
+        if (hipEventRecord(ev[(size_t)2 * i + 1], ctx->stream) != hipSuccess) { status = fail(ctx, SMELT_HIP_ERR_HIP, "hipEventRecord"); break; }
+    }
+    ctx->batch_open = false;
+    ctx->timing_valid = false;
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess && status == SMELT_HIP_OK) status = fail(ctx, SMELT_HIP_ERR_HIP, "hipStreamSynchronize");
+    if (status == SMELT_HIP_OK) {
+        for (int i = 0; i < iters; ++i) {
+            float ms = 0;
+            if (hipEventElapsedTime(&ms, ev[(size_t)2 * i], ev[(size_t)2 * i + 1]) != hipSuccess) { status = fail(ctx, SMELT_HIP_ERR_HIP, "hipEventElapsedTime"); break; }
+            out_us[i] = ms * 1000.0f;
+        }
+    }
+    for (hipEvent_t& e : ev) (void)hipEventDestroy(e);
+    return status;
+}
+
+static int capture(smelt_hip_context* ctx, const SmeltDispatchRecord* table, size_t count, int cur0, int alt0, const Dyn& d, smelt_hip_graph** out) {
+    if (!ctx || !out) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    *out = nullptr;
+    if (int e = smelt_hip_wait(ctx)) return e;
+    HIP_TRY(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->batch_open = true;  // no event records inside the capture
+    const int launched = interpret(ctx, table, count, cur0, alt0, d);
+    ctx->batch_open = false;
+    ctx->timing_valid = false;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (launched < 0) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return launched;
+    }
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamEndCapture");
+    smelt_hip_graph* g = new smelt_hip_graph();
+    g->graph = graph;
+    g->launches = launched;
+    e = hipGraphInstantiate(&g->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        delete g;
+        return hip_fail(ctx, e, "hipGraphInstantiate");
+    }
+    *out = g;
+    return launched;
+}
+
+int smelt_hip_graph_capture_decode(smelt_hip_context* ctx, const SmeltDispatchRecord* table, size_t count, int cur0, int alt0, int32_t position, smelt_hip_graph** out) {
+    Dyn d{false, position, 0, 0};
+    return capture(ctx, table, count, cur0, alt0, d, out);
+}
+
+int smelt_hip_graph_capture_prefill(smelt_hip_context* ctx, const SmeltDispatchRecord* table, size_t count, int cur0, int alt0, int32_t seq_len, int32_t start_pos, smelt_hip_graph** out) {
+    Dyn d{true, 0, seq_len, start_pos};
+    return capture(ctx, table, count, cur0, alt0, d, out);
+}
+
+int smelt_hip_graph_launch(smelt_hip_context* ctx, smelt_hip_graph* graph) {
+    if (!ctx || !graph) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null argument");
+    if (!ctx->batch_open) {
+        HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+        ctx->batch_open = true;
+        ctx->timing_valid = false;
+    }
+    HIP_TRY(ctx, hipGraphLaunch(graph->exec, ctx->stream));
+    return graph->launches;
+}
+
+void smelt_hip_graph_destroy(smelt_hip_context* ctx, smelt_hip_graph* graph) {
+    if (!graph) return;
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
+}
+
+int smelt_hip_graph_time(smelt_hip_context* ctx, smelt_hip_graph* graph, int iters, float* out_total_us) {
+    if (!ctx || !graph || !out_total_us || iters <= 0) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "bad arguments");
+    if (int e = smelt_hip_wait(ctx)) return e;
+    HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+    for (int i = 0; i < iters; ++i) HIP_TRY(ctx, hipGraphLaunch(graph->exec, ctx->stream));
+    HIP_TRY(ctx, hipEventRecord(ctx->ev_end, ctx->stream));
+    HIP_TRY(ctx, hipEventSynchronize(ctx->ev_end));
+    float ms = 0;
+    HIP_TRY(ctx, hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_end));
+    *out_total_us = ms * 1000.0f;
+    ctx->timing_valid = true;
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_device_info(smelt_hip_context* ctx, char* name, size_t name_cap, int* compute_units, size_t* lds_per_block, size_t* hbm_bytes) {
+    if (!ctx) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context");
+    if (name && name_cap) {
+        std::string n = std::string(ctx->props.name) + " (" + ctx->props.gcnArchName + ")";
+        snprintf(name, name_cap, "%s", n.c_str());
+    }
+    if (compute_units) *compute_units = ctx->props.multiProcessorCount;
+    if (lds_per_block) *lds_per_block = ctx->lds_limit;
+    if (hbm_bytes) *hbm_bytes = ctx->props.totalGlobalMem;
+    return SMELT_HIP_OK;
+}
+
+}  // extern "C"
