@@ -20,6 +20,11 @@
 
 namespace smelt {
 
+// (code & mask) | magic in one full-rate instruction (v_bitop3_b32, truth table 0xEA).
+__device__ __forceinline__ uint32_t and_or(uint32_t c, uint32_t mask, uint32_t magic) {
+    return __builtin_amdgcn_bitop3_b32(c, mask, magic, 0xEA);
+}
+
 // ---------------------------------------------------------------------------------------
 // Format traits. dot() consumes one dword of codes and kPairsPerDword fp16 pairs of x
 // (pair i = columns (i, i + kPairsPerDword) of that dword's column run).
@@ -34,10 +39,10 @@ struct FmtU4 {
     static __device__ __forceinline__ float pair_offset(int i) { return (i & 1) ? 64.0f : 1024.0f; }
     static __device__ __forceinline__ float dot(uint32_t c, const uint32_t* xp, float acc) {
         const uint32_t c8 = c >> 8;
-        acc = dot2((c & 0x000F000Fu) | 0x64006400u, xp[0], acc);   // nibbles 0,4 -> 1024+n
-        acc = dot2((c & 0x00F000F0u) | 0x54005400u, xp[1], acc);   // nibbles 1,5 -> 64+n
-        acc = dot2((c8 & 0x000F000Fu) | 0x64006400u, xp[2], acc);  // nibbles 2,6
-        acc = dot2((c8 & 0x00F000F0u) | 0x54005400u, xp[3], acc);  // nibbles 3,7
+        acc = dot2(and_or(c, 0x000F000Fu, 0x64006400u), xp[0], acc);   // nibbles 0,4 -> 1024+n
+        acc = dot2(and_or(c, 0x00F000F0u, 0x54005400u), xp[1], acc);   // nibbles 1,5 -> 64+n
+        acc = dot2(and_or(c8, 0x000F000Fu, 0x64006400u), xp[2], acc);  // nibbles 2,6
+        acc = dot2(and_or(c8, 0x00F000F0u, 0x54005400u), xp[3], acc);  // nibbles 3,7
         return acc;
     }
 };
@@ -54,14 +59,14 @@ struct FmtTer2 {
     }
     static __device__ __forceinline__ float dot(uint32_t c, const uint32_t* xp, float acc) {
         const uint32_t a = c << 4, b = c >> 2, d = c >> 8;
-        acc = dot2((a & 0x00300030u) | 0x54005400u, xp[0], acc);
-        acc = dot2((a & 0x00C000C0u) | 0x4C004C00u, xp[1], acc);
-        acc = dot2((a & 0x03000300u) | 0x44004400u, xp[2], acc);
-        acc = dot2((b & 0x00300030u) | 0x54005400u, xp[3], acc);
-        acc = dot2((b & 0x00C000C0u) | 0x4C004C00u, xp[4], acc);
-        acc = dot2((b & 0x03000300u) | 0x44004400u, xp[5], acc);
-        acc = dot2((d & 0x00300030u) | 0x54005400u, xp[6], acc);
-        acc = dot2((d & 0x00C000C0u) | 0x4C004C00u, xp[7], acc);
+        acc = dot2(and_or(a, 0x00300030u, 0x54005400u), xp[0], acc);
+        acc = dot2(and_or(a, 0x00C000C0u, 0x4C004C00u), xp[1], acc);
+        acc = dot2(and_or(a, 0x03000300u, 0x44004400u), xp[2], acc);
+        acc = dot2(and_or(b, 0x00300030u, 0x54005400u), xp[3], acc);
+        acc = dot2(and_or(b, 0x00C000C0u, 0x4C004C00u), xp[4], acc);
+        acc = dot2(and_or(b, 0x03000300u, 0x44004400u), xp[5], acc);
+        acc = dot2(and_or(d, 0x00300030u, 0x54005400u), xp[6], acc);
+        acc = dot2(and_or(d, 0x00C000C0u, 0x4C004C00u), xp[7], acc);
         return acc;
     }
 };
@@ -78,22 +83,22 @@ struct FmtBin {
     }
     static __device__ __forceinline__ float dot(uint32_t c, const uint32_t* xp, float acc) {
         const uint32_t a = c << 4, b = c >> 2, d = c >> 8;
-        acc = dot2((a & 0x00100010u) | 0x54005400u, xp[0], acc);
-        acc = dot2((a & 0x00200020u) | 0x50005000u, xp[1], acc);
-        acc = dot2((a & 0x00400040u) | 0x4C004C00u, xp[2], acc);
-        acc = dot2((a & 0x00800080u) | 0x48004800u, xp[3], acc);
-        acc = dot2((a & 0x01000100u) | 0x44004400u, xp[4], acc);
-        acc = dot2((a & 0x02000200u) | 0x40004000u, xp[5], acc);
-        acc = dot2((b & 0x00100010u) | 0x54005400u, xp[6], acc);
-        acc = dot2((b & 0x00200020u) | 0x50005000u, xp[7], acc);
-        acc = dot2((b & 0x00400040u) | 0x4C004C00u, xp[8], acc);
-        acc = dot2((b & 0x00800080u) | 0x48004800u, xp[9], acc);
-        acc = dot2((b & 0x01000100u) | 0x44004400u, xp[10], acc);
-        acc = dot2((b & 0x02000200u) | 0x40004000u, xp[11], acc);
-        acc = dot2((d & 0x00100010u) | 0x54005400u, xp[12], acc);
-        acc = dot2((d & 0x00200020u) | 0x50005000u, xp[13], acc);
-        acc = dot2((d & 0x00400040u) | 0x4C004C00u, xp[14], acc);
-        acc = dot2((d & 0x00800080u) | 0x48004800u, xp[15], acc);
+        acc = dot2(and_or(a, 0x00100010u, 0x54005400u), xp[0], acc);
+        acc = dot2(and_or(a, 0x00200020u, 0x50005000u), xp[1], acc);
+        acc = dot2(and_or(a, 0x00400040u, 0x4C004C00u), xp[2], acc);
+        acc = dot2(and_or(a, 0x00800080u, 0x48004800u), xp[3], acc);
+        acc = dot2(and_or(a, 0x01000100u, 0x44004400u), xp[4], acc);
+        acc = dot2(and_or(a, 0x02000200u, 0x40004000u), xp[5], acc);
+        acc = dot2(and_or(b, 0x00100010u, 0x54005400u), xp[6], acc);
+        acc = dot2(and_or(b, 0x00200020u, 0x50005000u), xp[7], acc);
+        acc = dot2(and_or(b, 0x00400040u, 0x4C004C00u), xp[8], acc);
+        acc = dot2(and_or(b, 0x00800080u, 0x48004800u), xp[9], acc);
+        acc = dot2(and_or(b, 0x01000100u, 0x44004400u), xp[10], acc);
+        acc = dot2(and_or(b, 0x02000200u, 0x40004000u), xp[11], acc);
+        acc = dot2(and_or(d, 0x00100010u, 0x54005400u), xp[12], acc);
+        acc = dot2(and_or(d, 0x00200020u, 0x50005000u), xp[13], acc);
+        acc = dot2(and_or(d, 0x00400040u, 0x4C004C00u), xp[14], acc);
+        acc = dot2(and_or(d, 0x00800080u, 0x48004800u), xp[15], acc);
         return acc;
     }
 };
@@ -178,82 +183,67 @@ struct MatPtrs {
     const uint16_t* biases;  // affine only
 };
 
-// Accumulate acc[m][r][b] for the wave's row tile.
-//   row_base  : first row of this wave's tile; rows row_base + side*R + r
-//   L         : lanes per row (power of two), S = 64 / L rows side by side
-template <class F, class ScaleT, int R, int MB, int NMAT, int L>
-__device__ __forceinline__ void matvec_tile(const MatPtrs (&mats)[NMAT], int rows, int U,
-                                            int row_stride, int groups_per_row, int gshift,
-                                            int row_base, const uint4_t* lds_pairs,
-                                            const float4_t* lds_corr, const float4_t* lds_xsum,
-                                            float (&acc)[NMAT][R][MB]) {
-    using G = FmtGeom<F>;
-    constexpr int NCH = G::kChunksPerUnit;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int sub = lane & (L - 1);
-    const int side = lane / L;
-    int row[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int rr = row_base + side * R + r;
-        row[r] = rr < rows ? rr : rows - 1;  // clamped rows are computed but never stored
-    }
+// Registers of one work item: the 16-byte unit `u` of R rows of NMAT matrices plus the group
+// scale (and bias) each of them needs.
+template <int R, int NMAT>
+struct ItemRegs {
+    uint4_t c[NMAT][R];
+    uint16_t s[NMAT][R];
+    uint16_t b[NMAT][R];
+};
+
+template <class F, int R, int NMAT>
+__device__ __forceinline__ void load_item(const MatPtrs (&mats)[NMAT], const int (&row)[R], int u,
+                                          int row_stride, int groups_per_row, int gshift,
+                                          ItemRegs<R, NMAT>& it) {
+    const int g = (u * FmtGeom<F>::kColsPerUnit) >> gshift;
 #pragma unroll
     for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int b = 0; b < MB; ++b) acc[m][r][b] = 0.0f;
+        for (int r = 0; r < R; ++r) {
+            it.c[m][r] = *reinterpret_cast<const uint4_t*>(mats[m].codes + (size_t)row[r] * row_stride + (size_t)u * 16);
+            const size_t si = (size_t)row[r] * groups_per_row + g;
+            it.s[m][r] = mats[m].scales[si];
+            it.b[m][r] = F::kHasBias ? mats[m].biases[si] : (uint16_t)0;
+        }
+}
 
-    for (int u = sub; u < U; u += L) {
-        uint4_t c[NMAT][R];
-        float sc[NMAT][R], bi[NMAT][R];
-        const int g = (u * G::kColsPerUnit) >> gshift;
+// acc[m][r][b] += scale * (sum (base + code) * x  -  sum base * x) + bias * sum x   for unit u
+template <class F, class ScaleT, int R, int MB, int NMAT>
+__device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u, int U,
+                                             const uint4_t* lds_pairs, const float4_t* lds_corr,
+                                             const float4_t* lds_xsum, float (&acc)[NMAT][R][MB]) {
+    using G = FmtGeom<F>;
+    constexpr int NCH = G::kChunksPerUnit;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        uint32_t xp[NCH * 4];
+#pragma unroll
+        for (int q = 0; q < NCH; ++q) {
+            const uint4_t t = lds_pairs[((size_t)b * NCH + q) * U + u];
+            xp[4 * q + 0] = t.x; xp[4 * q + 1] = t.y; xp[4 * q + 2] = t.z; xp[4 * q + 3] = t.w;
+        }
+        const float4_t cr = lds_corr[(size_t)b * U + u];
+        const float corr = (cr.x + cr.y) + (cr.z + cr.w);
+        float xsum = 0.0f;
+        if (F::kHasBias) {
+            const float4_t xs = lds_xsum[(size_t)b * U + u];
+            xsum = (xs.x + xs.y) + (xs.z + xs.w);
+        }
 #pragma unroll
         for (int m = 0; m < NMAT; ++m)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                c[m][r] = *reinterpret_cast<const uint4_t*>(mats[m].codes + (size_t)row[r] * row_stride + (size_t)u * 16);
-                const size_t si = (size_t)row[r] * groups_per_row + g;
-                sc[m][r] = F::kSemMul * ScaleT::widen(mats[m].scales[si]);
-                bi[m][r] = F::kHasBias ? ScaleT::widen(mats[m].biases[si]) : 0.0f;
+                float d = -corr;
+                d = F::dot(it.c[m][r].x, xp + 0 * G::kPPD, d);
+                d = F::dot(it.c[m][r].y, xp + 1 * G::kPPD, d);
+                d = F::dot(it.c[m][r].z, xp + 2 * G::kPPD, d);
+                d = F::dot(it.c[m][r].w, xp + 3 * G::kPPD, d);
+                float a = acc[m][r][b];
+                if (F::kHasBias) a = __builtin_fmaf(ScaleT::widen(it.b[m][r]), xsum, a);
+                acc[m][r][b] = __builtin_fmaf(F::kSemMul * ScaleT::widen(it.s[m][r]), d, a);
             }
-#pragma unroll
-        for (int b = 0; b < MB; ++b) {
-            uint32_t xp[NCH * 4];
-#pragma unroll
-            for (int q = 0; q < NCH; ++q) {
-                const uint4_t t = lds_pairs[((size_t)b * NCH + q) * U + u];
-                xp[4 * q + 0] = t.x; xp[4 * q + 1] = t.y; xp[4 * q + 2] = t.z; xp[4 * q + 3] = t.w;
-            }
-            const float4_t cr = lds_corr[(size_t)b * U + u];
-            const float corr = (cr.x + cr.y) + (cr.z + cr.w);
-            float xsum = 0.0f;
-            if (F::kHasBias) {
-                const float4_t xs = lds_xsum[(size_t)b * U + u];
-                xsum = (xs.x + xs.y) + (xs.z + xs.w);
-            }
-#pragma unroll
-            for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    float d = -corr;
-                    d = F::dot(c[m][r].x, xp + 0 * G::kPPD, d);
-                    d = F::dot(c[m][r].y, xp + 1 * G::kPPD, d);
-                    d = F::dot(c[m][r].z, xp + 2 * G::kPPD, d);
-                    d = F::dot(c[m][r].w, xp + 3 * G::kPPD, d);
-                    float a = acc[m][r][b];
-                    if (F::kHasBias) a = __builtin_fmaf(bi[m][r], xsum, a);
-                    acc[m][r][b] = __builtin_fmaf(sc[m][r], d, a);
-                }
-        }
     }
-#pragma unroll
-    for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int b = 0; b < MB; ++b) acc[m][r][b] = group_sum_last<L>(acc[m][r][b]);
 }
 
 }  // namespace smelt

@@ -72,12 +72,17 @@ struct EpiDual {
 };
 
 // ---- workgroup body ------------------------------------------------------------------------
+//
+// A wave walks its row tiles (grid-stride, so any grid covers every row) as a flat sequence of
+// work items (tile, unit step).  Items are software-pipelined two deep: the loads of item q+1
+// are issued before item q is computed, and the loads of the very first item are issued before
+// the activations are staged, so a small matrix pays one memory latency, not two.
 
-template <class F, class ScaleT, int R, int MB, int NMAT, int L, class Epi>
-__device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], int rows, int U,
-                                          int row_stride, int gpr, int gshift, int b0, int nb,
-                                          const uint4_t* lds_pairs, const float4_t* lds_corr,
-                                          const float4_t* lds_xsum, const Epi& epi) {
+template <class F, class ActT, class ScaleT, int R, int MB, int NMAT, int L, class Epi>
+__device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uint16_t* x, int rows,
+                                          int cols, int U, int row_stride, int gpr, int gshift,
+                                          int batch_lo, int batch_hi, uint4_t* lds_pairs,
+                                          float* lds_corr, float* lds_xsum, const Epi& epi) {
     constexpr int S = kWave / L;
     constexpr int TILE = S * R;
     const int waves = blockDim.x / kWave;
@@ -86,26 +91,83 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], int rows,
     const int sub = lane & (L - 1);
     const int side = lane / L;
     const int tiles = (rows + TILE - 1) / TILE;
-    for (int tile = blockIdx.x * waves + wave; tile < tiles; tile += gridDim.x * waves) {
+    const int nit = (U + L - 1) / L;
+    const int first = blockIdx.x * waves + wave;
+    const int stride = gridDim.x * waves;
+    const int my_tiles = first < tiles ? (tiles - first + stride - 1) / stride : 0;
+    const int nq = my_tiles * nit;
+    const float4_t* corr4 = reinterpret_cast<const float4_t*>(lds_corr);
+    const float4_t* xsum4 = reinterpret_cast<const float4_t*>(lds_xsum);
+
+    for (int b0 = batch_lo; b0 < batch_hi; b0 += MB) {
+        const int nb = batch_hi - b0 < MB ? batch_hi - b0 : MB;
+        ItemRegs<R, NMAT> regs_a, regs_b;
+        // (tile, step) of the item being computed and of the item being prefetched
+        int tile_c = first, it_c = 0, tile_n = first, it_n = 0;
+        auto load = [&](ItemRegs<R, NMAT>& dst) {
+            const int u = sub + L * it_n;
+            if (u < U) {
+                int row[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int rr = tile_n * TILE + side * R + r;
+                    row[r] = rr < rows ? rr : rows - 1;  // clamped rows are computed, never stored
+                }
+                load_item<F, R, NMAT>(mats, row, u, row_stride, gpr, gshift, dst);
+            }
+            if (++it_n == nit) { it_n = 0; tile_n += stride; }
+        };
+        if (nq > 0) load(regs_a);
+        if (b0 != batch_lo) __syncthreads();
+        stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum);
+        __syncthreads();
+
         float acc[NMAT][R][MB];
-        matvec_tile<F, ScaleT, R, MB, NMAT, L>(mats, rows, U, row_stride, gpr, gshift, tile * TILE,
-                                               lds_pairs, lds_corr, lds_xsum, acc);
-        if (sub == L - 1) {
+        auto step = [&](const ItemRegs<R, NMAT>& cur, ItemRegs<R, NMAT>& nxt, int q) {
+            if (q + 1 < nq) load(nxt);
+            if (it_c == 0) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int row = tile * TILE + side * R + r;
-                if (row < rows) {
+                for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-                    for (int b = 0; b < MB; ++b) {
-                        if (b < nb) {
-                            float v[NMAT];
+                    for (int r = 0; r < R; ++r)
 #pragma unroll
-                            for (int m = 0; m < NMAT; ++m) v[m] = acc[m][r][b];
-                            epi(b0 + b, row, v);
+                        for (int b = 0; b < MB; ++b) acc[m][r][b] = 0.0f;
+            }
+            const int u = sub + L * it_c;
+            if (u < U) compute_item<F, ScaleT, R, MB, NMAT>(cur, u, U, lds_pairs, corr4, xsum4, acc);
+            if (it_c == nit - 1) {
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+#pragma unroll
+                        for (int b = 0; b < MB; ++b) acc[m][r][b] = group_sum_last<L>(acc[m][r][b]);
+                if (sub == L - 1) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const int row = tile_c * TILE + side * R + r;
+                        if (row < rows) {
+#pragma unroll
+                            for (int b = 0; b < MB; ++b) {
+                                if (b < nb) {
+                                    float v[NMAT];
+#pragma unroll
+                                    for (int m = 0; m < NMAT; ++m) v[m] = acc[m][r][b];
+                                    epi(b0 + b, row, v);
+                                }
+                            }
                         }
                     }
                 }
+                it_c = 0;
+                tile_c += stride;
+            } else {
+                ++it_c;
             }
+        };
+        for (int q = 0; q < nq; q += 2) {
+            step(regs_a, regs_b, q);
+            if (q + 1 < nq) step(regs_b, regs_a, q + 1);
         }
     }
 }
@@ -116,7 +178,6 @@ template <class F, class ActT, class ScaleT, int R, int MB, int NMAT, class Epi>
 __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const uint16_t* x,
                                             int rows, int cols, int row_stride, int group,
                                             int batch_lo, int batch_hi, const Epi& epi) {
-    using G = FmtGeom<F>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int U = row_stride / 16;
     const int gshift = ilog2((uint32_t)group);
@@ -124,20 +185,12 @@ __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const u
     uint4_t* lds_pairs = reinterpret_cast<uint4_t*>(smem);
     float* lds_corr = reinterpret_cast<float*>(smem + lds_pairs_bytes<F>(U, MB));
     float* lds_xsum = lds_corr + (size_t)MB * U * 4;
-    for (int b0 = batch_lo; b0 < batch_hi; b0 += MB) {
-        const int nb = batch_hi - b0 < MB ? batch_hi - b0 : MB;
-        if (b0 != batch_lo) __syncthreads();
-        stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum);
-        __syncthreads();
-        const float4_t* corr4 = reinterpret_cast<const float4_t*>(lds_corr);
-        const float4_t* xsum4 = reinterpret_cast<const float4_t*>(lds_xsum);
-        if (U > 32)
-            run_tiles<F, ScaleT, R, MB, NMAT, 64>(mats, rows, U, row_stride, gpr, gshift, b0, nb, lds_pairs, corr4, xsum4, epi);
-        else if (U > 16)
-            run_tiles<F, ScaleT, R, MB, NMAT, 32>(mats, rows, U, row_stride, gpr, gshift, b0, nb, lds_pairs, corr4, xsum4, epi);
-        else
-            run_tiles<F, ScaleT, R, MB, NMAT, 16>(mats, rows, U, row_stride, gpr, gshift, b0, nb, lds_pairs, corr4, xsum4, epi);
-    }
+    if (U > 32)
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 64>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, epi);
+    else if (U > 16)
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 32>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, epi);
+    else
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 16>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, epi);
 }
 
 template <class F>
