@@ -17,6 +17,7 @@ constexpr int kWave = 64;
 
 // Element types of activations / scales as stored in memory (raw 16-bit patterns).
 struct F16 {
+    static constexpr bool kIsF16 = true;
     static __device__ __forceinline__ float widen(uint16_t b) {
         return (float)__builtin_bit_cast(_Float16, b);
     }
@@ -29,6 +30,7 @@ struct F16 {
 };
 
 struct BF16 {
+    static constexpr bool kIsF16 = false;
     static __device__ __forceinline__ float widen(uint16_t b) {
         return __builtin_bit_cast(float, (uint32_t)b << 16);
     }

@@ -32,6 +32,8 @@ __device__ __forceinline__ uint32_t and_or(uint32_t c, uint32_t mask, uint32_t m
 // The semantic weight is kSemMul * (code + pair terms - offset) * scale.
 // ---------------------------------------------------------------------------------------
 struct FmtU4 {
+    static constexpr int kDwordsPerUnit = 4;
+    static constexpr bool kPerDwordScale = false;
     static constexpr int kBitsPerCode = 4;
     static constexpr int kPairsPerDword = 4;
     static constexpr bool kHasBias = true;
@@ -48,6 +50,8 @@ struct FmtU4 {
 };
 
 struct FmtTer2 {
+    static constexpr int kDwordsPerUnit = 4;
+    static constexpr bool kPerDwordScale = false;
     static constexpr int kBitsPerCode = 2;
     static constexpr int kPairsPerDword = 8;
     static constexpr bool kHasBias = false;
@@ -72,6 +76,8 @@ struct FmtTer2 {
 };
 
 struct FmtBin {
+    static constexpr int kDwordsPerUnit = 4;
+    static constexpr bool kPerDwordScale = false;
     static constexpr int kBitsPerCode = 1;
     static constexpr int kPairsPerDword = 16;
     static constexpr bool kHasBias = false;
@@ -103,19 +109,48 @@ struct FmtBin {
     }
 };
 
+// trit5: five base-3 digits per byte, decoded through a 243-entry table into the ternary2 bit
+// layout.  A 16-byte unit holds 80 columns = five 16-column dwords; a dword never straddles a
+// 128-column scale group, a unit can, so the scale is applied per dword.
+struct FmtTrit5 {
+    static constexpr int kDwordsPerUnit = 5;
+    static constexpr bool kPerDwordScale = true;
+    static constexpr int kBitsPerCode = 2;
+    static constexpr int kPairsPerDword = 8;
+    static constexpr bool kHasBias = false;
+    static constexpr float kSemMul = 1.0f;
+    static __device__ __forceinline__ float pair_offset(int i) { return FmtTer2::pair_offset(i); }
+    static __device__ __forceinline__ float dot(uint32_t c, const uint32_t* xp, float acc) {
+        return FmtTer2::dot(c, xp, acc);
+    }
+    static __device__ __forceinline__ void decode(const uint4_t& raw, const uint16_t* lut, uint32_t (&dw)[5]) {
+        uint32_t f[16];
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int k = 0; k < 16; ++k) f[k] = lut[(w[k >> 2] >> (8 * (k & 3))) & 0xFFu];
+        dw[0] = f[0] | (f[1] << 10) | (f[2] << 20) | (f[3] << 30);
+        dw[1] = (f[3] >> 2) | (f[4] << 8) | (f[5] << 18) | (f[6] << 28);
+        dw[2] = (f[6] >> 4) | (f[7] << 6) | (f[8] << 16) | (f[9] << 26);
+        dw[3] = (f[9] >> 6) | (f[10] << 4) | (f[11] << 14) | (f[12] << 24);
+        dw[4] = (f[12] >> 8) | (f[13] << 2) | (f[14] << 12) | (f[15] << 22);
+    }
+};
+
 template <class F>
 struct FmtGeom {
     static constexpr int kPPD = F::kPairsPerDword;
     static constexpr int kColsPerDword = 2 * kPPD;
-    static constexpr int kColsPerUnit = 4 * kColsPerDword;
+    static constexpr int kDPU = F::kDwordsPerUnit;         // code dwords per 16-byte unit after decode
+    static constexpr int kColsPerUnit = kDPU * kColsPerDword;
     static constexpr int kChunksPerDword = kPPD / 4;       // 16-byte LDS chunks (4 pairs each)
-    static constexpr int kChunksPerUnit = 4 * kChunksPerDword;
+    static constexpr int kChunksPerUnit = kDPU * kChunksPerDword;
+    static constexpr int kCorrStride = kDPU <= 4 ? 4 : 8;  // floats of per-dword corrections per unit
 };
 
 // LDS layout for one batch tile of MB activations over U units per row:
 //   pairs : [MB][kChunksPerUnit][U] x 16 B   (chunk-major so consecutive lanes hit consecutive 16 B)
-//   corr  : [MB][U] float4 (one float per dword of the unit)
-//   xsum  : [MB][U] float4 (affine only)
+//   corr  : [MB][U][kCorrStride] floats (one per dword of the unit)
+//   xsum  : [MB][U][kCorrStride] floats (affine only)
 template <class F>
 __device__ __forceinline__ size_t lds_pairs_bytes(int U, int MB) {
     return (size_t)MB * FmtGeom<F>::kChunksPerUnit * U * 16;
@@ -129,11 +164,12 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
     using G = FmtGeom<F>;
     constexpr int PPD = G::kPPD;
     constexpr int CPD = G::kColsPerDword;
-    const int dwords = U * 4;
+    constexpr int DPU = G::kDPU;
+    const int dwords = U * DPU;
     for (int item = threadIdx.x; item < MB * dwords; item += blockDim.x) {
         const int b = item / dwords;
         const int D = item - b * dwords;
-        const int u = D >> 2, d = D & 3;
+        const int u = D / DPU, d = D - u * DPU;
         const int col0 = D * CPD;
         uint16_t v[CPD];
         if (b < nb && col0 + CPD <= cols) {
@@ -171,8 +207,8 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
             ch.z = pairs[4 * j + 2]; ch.w = pairs[4 * j + 3];
             lds_pairs[((size_t)b * G::kChunksPerUnit + d * G::kChunksPerDword + j) * U + u] = ch;
         }
-        lds_corr[((size_t)b * U + u) * 4 + d] = corr;
-        if (F::kHasBias) lds_xsum[((size_t)b * U + u) * 4 + d] = xsum;
+        lds_corr[((size_t)b * U + u) * G::kCorrStride + d] = corr;
+        if (F::kHasBias) lds_xsum[((size_t)b * U + u) * G::kCorrStride + d] = xsum;
     }
 }
 
@@ -189,7 +225,7 @@ template <int R, int NMAT>
 struct ItemRegs {
     uint4_t c[NMAT][R];
     uint16_t s[NMAT][R];
-    uint16_t b[NMAT][R];
+    uint16_t b[NMAT][R];   // affine bias; for per-dword-scale formats the next group's scale
 };
 
 template <class F, int R, int NMAT>
@@ -204,17 +240,21 @@ __device__ __forceinline__ void load_item(const MatPtrs (&mats)[NMAT], const int
             it.c[m][r] = *reinterpret_cast<const uint4_t*>(mats[m].codes + (size_t)row[r] * row_stride + (size_t)u * 16);
             const size_t si = (size_t)row[r] * groups_per_row + g;
             it.s[m][r] = mats[m].scales[si];
-            it.b[m][r] = F::kHasBias ? mats[m].biases[si] : (uint16_t)0;
+            if (F::kHasBias) it.b[m][r] = mats[m].biases[si];
+            else if (F::kPerDwordScale) it.b[m][r] = mats[m].scales[g + 1 < groups_per_row ? si + 1 : si];
+            else it.b[m][r] = 0;
         }
 }
 
 // acc[m][r][b] += scale * (sum (base + code) * x  -  sum base * x) + bias * sum x   for unit u
 template <class F, class ScaleT, int R, int MB, int NMAT>
-__device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u, int U,
-                                             const uint4_t* lds_pairs, const float4_t* lds_corr,
-                                             const float4_t* lds_xsum, float (&acc)[NMAT][R][MB]) {
+__device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u, int U, int gshift,
+                                             const uint4_t* lds_pairs, const float* lds_corr,
+                                             const float* lds_xsum, const uint16_t* lut,
+                                             float (&acc)[NMAT][R][MB]) {
     using G = FmtGeom<F>;
     constexpr int NCH = G::kChunksPerUnit;
+    constexpr int DPU = G::kDPU;
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
         uint32_t xp[NCH * 4];
@@ -223,26 +263,53 @@ __device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u,
             const uint4_t t = lds_pairs[((size_t)b * NCH + q) * U + u];
             xp[4 * q + 0] = t.x; xp[4 * q + 1] = t.y; xp[4 * q + 2] = t.z; xp[4 * q + 3] = t.w;
         }
-        const float4_t cr = lds_corr[(size_t)b * U + u];
-        const float corr = (cr.x + cr.y) + (cr.z + cr.w);
-        float xsum = 0.0f;
-        if (F::kHasBias) {
-            const float4_t xs = lds_xsum[(size_t)b * U + u];
-            xsum = (xs.x + xs.y) + (xs.z + xs.w);
+        float cr[DPU];
+        {
+            const float4_t* c4 = reinterpret_cast<const float4_t*>(lds_corr + ((size_t)b * U + u) * G::kCorrStride);
+            const float4_t lo = c4[0];
+            cr[0] = lo.x; cr[1] = lo.y; cr[2] = lo.z; cr[3] = lo.w;
+            if constexpr (DPU > 4) cr[DPU - 1] = c4[1].x;
         }
+        if constexpr (F::kPerDwordScale) {
+            const int g0 = (u * G::kColsPerUnit) >> gshift;
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m)
+            for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                float d = -corr;
-                d = F::dot(it.c[m][r].x, xp + 0 * G::kPPD, d);
-                d = F::dot(it.c[m][r].y, xp + 1 * G::kPPD, d);
-                d = F::dot(it.c[m][r].z, xp + 2 * G::kPPD, d);
-                d = F::dot(it.c[m][r].w, xp + 3 * G::kPPD, d);
-                float a = acc[m][r][b];
-                if (F::kHasBias) a = __builtin_fmaf(ScaleT::widen(it.b[m][r]), xsum, a);
-                acc[m][r][b] = __builtin_fmaf(F::kSemMul * ScaleT::widen(it.s[m][r]), d, a);
+                for (int r = 0; r < R; ++r) {
+                    uint32_t dw[DPU];
+                    F::decode(it.c[m][r], lut, dw);
+                    const float s0 = F::kSemMul * ScaleT::widen(it.s[m][r]);
+                    const float s1 = F::kSemMul * ScaleT::widen(it.b[m][r]);
+                    float a = acc[m][r][b];
+#pragma unroll
+                    for (int j = 0; j < DPU; ++j) {
+                        const float d = F::dot(dw[j], xp + j * G::kPPD, -cr[j]);
+                        const int gj = (u * G::kColsPerUnit + j * G::kColsPerDword) >> gshift;
+                        a = __builtin_fmaf(gj == g0 ? s0 : s1, d, a);
+                    }
+                    acc[m][r][b] = a;
+                }
+        } else {
+            const float corr = (cr[0] + cr[1]) + (cr[2] + cr[3]);
+            float xsum = 0.0f;
+            if (F::kHasBias) {
+                const float4_t xs = *reinterpret_cast<const float4_t*>(lds_xsum + ((size_t)b * U + u) * G::kCorrStride);
+                xsum = (xs.x + xs.y) + (xs.z + xs.w);
             }
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    float d = -corr;
+                    d = F::dot(it.c[m][r].x, xp + 0 * G::kPPD, d);
+                    d = F::dot(it.c[m][r].y, xp + 1 * G::kPPD, d);
+                    d = F::dot(it.c[m][r].z, xp + 2 * G::kPPD, d);
+                    d = F::dot(it.c[m][r].w, xp + 3 * G::kPPD, d);
+                    float a = acc[m][r][b];
+                    if (F::kHasBias) a = __builtin_fmaf(ScaleT::widen(it.b[m][r]), xsum, a);
+                    acc[m][r][b] = __builtin_fmaf(F::kSemMul * ScaleT::widen(it.s[m][r]), d, a);
+                }
+        }
     }
 }
 

@@ -3,14 +3,21 @@
 // by ascending binding index), followed by the shape arguments the pipeline table appends.
 #pragma once
 #include "matvec.hpp"
+#include "misc_kernels.hpp"
 
 namespace smelt {
 
 // ---- epilogues ---------------------------------------------------------------------------
 // Each epilogue receives the reduced fp32 sums of one (batch, row) for NMAT matrices.
 
+// Epilogues may keep per-thread state; end_chunk() runs on every thread once all rows of a
+// batch chunk are done.
+struct EpiBase {
+    __device__ __forceinline__ void end_chunk(int, int) const {}
+};
+
 template <class ActT>
-struct EpiStore {
+struct EpiStore : EpiBase {
     uint16_t* y;
     int rows;
     __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
@@ -20,7 +27,7 @@ struct EpiStore {
 
 // project, round to the activation type, add the residual in that type
 template <class ActT>
-struct EpiAdd {
+struct EpiAdd : EpiBase {
     uint16_t* y;
     const uint16_t* residual;
     int rows;
@@ -33,7 +40,7 @@ struct EpiAdd {
 
 // affine SwiGLU: narrow(gate / (1 + exp(-gate)) * up) on the fp32 sums
 template <class ActT>
-struct EpiAffineSwiglu {
+struct EpiAffineSwiglu : EpiBase {
     uint16_t* y;
     int rows;
     __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
@@ -45,7 +52,7 @@ struct EpiAffineSwiglu {
 // signed SwiGLU: gate and up are first rounded to the activation type and every intermediate
 // (exp, 1+e, reciprocal, 1-tail, gate*sigmoid, *up) is materialised in that type
 template <class ActT>
-struct EpiSignedSwiglu {
+struct EpiSignedSwiglu : EpiBase {
     uint16_t* y;
     int rows;
     static __device__ __forceinline__ float rt(float v) { return ActT::widen(ActT::narrow(v)); }
@@ -61,7 +68,7 @@ struct EpiSignedSwiglu {
 };
 
 template <class ActT>
-struct EpiDual {
+struct EpiDual : EpiBase {
     uint16_t* y1;
     uint16_t* y2;
     int rows;
@@ -82,7 +89,8 @@ template <class F, class ActT, class ScaleT, int R, int MB, int NMAT, int L, cla
 __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uint16_t* x, int rows,
                                           int cols, int U, int row_stride, int gpr, int gshift,
                                           int batch_lo, int batch_hi, uint4_t* lds_pairs,
-                                          float* lds_corr, float* lds_xsum, const Epi& epi) {
+                                          float* lds_corr, float* lds_xsum, const uint16_t* lut,
+                                          const Epi& epi) {
     constexpr int S = kWave / L;
     constexpr int TILE = S * R;
     const int waves = blockDim.x / kWave;
@@ -96,8 +104,6 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
     const int stride = gridDim.x * waves;
     const int my_tiles = first < tiles ? (tiles - first + stride - 1) / stride : 0;
     const int nq = my_tiles * nit;
-    const float4_t* corr4 = reinterpret_cast<const float4_t*>(lds_corr);
-    const float4_t* xsum4 = reinterpret_cast<const float4_t*>(lds_xsum);
 
     for (int b0 = batch_lo; b0 < batch_hi; b0 += MB) {
         const int nb = batch_hi - b0 < MB ? batch_hi - b0 : MB;
@@ -134,7 +140,7 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
                         for (int b = 0; b < MB; ++b) acc[m][r][b] = 0.0f;
             }
             const int u = sub + L * it_c;
-            if (u < U) compute_item<F, ScaleT, R, MB, NMAT>(cur, u, U, lds_pairs, corr4, xsum4, acc);
+            if (u < U) compute_item<F, ScaleT, R, MB, NMAT>(cur, u, U, gshift, lds_pairs, lds_corr, lds_xsum, lut, acc);
             if (it_c == nit - 1) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
@@ -169,6 +175,7 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
             step(regs_a, regs_b, q);
             if (q + 1 < nq) step(regs_b, regs_a, q + 1);
         }
+        epi.end_chunk(b0, nb);
     }
 }
 
@@ -184,17 +191,21 @@ __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const u
     const int gpr = (cols + group - 1) / group;
     uint4_t* lds_pairs = reinterpret_cast<uint4_t*>(smem);
     float* lds_corr = reinterpret_cast<float*>(smem + lds_pairs_bytes<F>(U, MB));
-    float* lds_xsum = lds_corr + (size_t)MB * U * 4;
+    float* lds_xsum = lds_corr + (size_t)MB * U * FmtGeom<F>::kCorrStride;
+    uint16_t* lut = reinterpret_cast<uint16_t*>(lds_xsum + (size_t)MB * U * FmtGeom<F>::kCorrStride);
+    if (F::kPerDwordScale)  // decode table; visible to every wave after the staging barrier
+        for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) lut[i] = trit5_lut_entry(i);
     if (U > 32)
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 64>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, epi);
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 64>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
     else if (U > 16)
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 32>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, epi);
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 32>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
     else
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 16>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, epi);
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 16>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
 }
 
 template <class F>
 __device__ __forceinline__ int packed_row_stride(int cols, int group) {
+    if (F::kPerDwordScale) return (((cols + 4) / 5) + 15) & ~15;  // trit5: 5 digits per byte, 16-byte rows
     const int padded = F::kHasBias ? cols : (cols + group - 1) / group * group;
     return (padded * F::kBitsPerCode + 7) / 8;
 }
@@ -213,7 +224,7 @@ using u32 = uint32_t;
                                               u32 group) {                                        \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
-        EpiStore<ACT> epi{y, (int)rows};                                                          \
+        EpiStore<ACT> epi{{}, y, (int)rows};                                                          \
         matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
@@ -223,7 +234,7 @@ using u32 = uint32_t;
                                                   u32 cols, u32 group) {                          \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
-        EpiAdd<ACT> epi{y, res, (int)rows};                                                       \
+        EpiAdd<ACT> epi{{}, y, res, (int)rows};                                                       \
         matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
@@ -233,7 +244,7 @@ using u32 = uint32_t;
         const u16* x, u16* y, u32 rows, u32 cols, u32 group) {                                    \
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
-        EpiAffineSwiglu<ACT> epi{y, (int)rows};                                                   \
+        EpiAffineSwiglu<ACT> epi{{}, y, (int)rows};                                                   \
         matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
@@ -243,7 +254,7 @@ using u32 = uint32_t;
         const u16* x, u16* y1, u16* y2, u32 rows, u32 cols, u32 group) {                          \
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
-        EpiDual<ACT> epi{y1, y2, (int)rows};                                                      \
+        EpiDual<ACT> epi{{}, y1, y2, (int)rows};                                                      \
         matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
@@ -255,7 +266,7 @@ using u32 = uint32_t;
         u32 cols, u32 group, u32 batch_tile) {                                                    \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
-        EpiStore<ACT> epi{Y, (int)rows};                                                          \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                          \
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
@@ -268,7 +279,7 @@ using u32 = uint32_t;
         u32 rows, u32 cols, u32 group, u32 batch_tile) {                                          \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
-        EpiAdd<ACT> epi{Y, res, (int)rows};                                                       \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                       \
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
@@ -281,7 +292,7 @@ using u32 = uint32_t;
         const u16* X, u16* Y, u32 batch, u32 rows, u32 cols, u32 group, u32 batch_tile) {         \
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
-        EpiAffineSwiglu<ACT> epi{Y, (int)rows};                                                   \
+        EpiAffineSwiglu<ACT> epi{{}, Y, (int)rows};                                                   \
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
@@ -296,7 +307,7 @@ using u32 = uint32_t;
                                                      u16* Y, u32 rows, u32 cols) {                \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
-        EpiStore<ACT> epi{Y, (int)rows};                                                          \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                          \
         matvec_body<FMT, ACT, F16, 4, 1, 1>(mats, X, rows, cols,                                  \
                                             packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
                                             blockIdx.y + 1, epi);                                 \
@@ -306,7 +317,7 @@ using u32 = uint32_t;
                                                          u32 cols) {                              \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
-        EpiAdd<ACT> epi{Y, res, (int)rows};                                                       \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                       \
         matvec_body<FMT, ACT, F16, 4, 1, 1>(mats, X, rows, cols,                                  \
                                             packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
                                             blockIdx.y + 1, epi);                                 \
@@ -316,7 +327,7 @@ using u32 = uint32_t;
         u32 cols) {                                                                               \
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
-        EpiSignedSwiglu<ACT> epi{Y, (int)rows};                                                   \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                                   \
         matvec_body<FMT, ACT, F16, 2, 1, 2>(mats, X, rows, cols,                                  \
                                             packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
                                             blockIdx.y + 1, epi);                                 \
@@ -325,7 +336,7 @@ using u32 = uint32_t;
                                                         u16* Y, u32 rows, u32 cols, u32 batch) {  \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
-        EpiStore<ACT> epi{Y, (int)rows};                                                          \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                          \
         const u32 lo = blockIdx.y * 4;                                                            \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + 4 < batch ? lo + 4 : batch;                                           \
@@ -337,10 +348,120 @@ using u32 = uint32_t;
         u32 cols, u32 batch) {                                                                    \
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
-        EpiSignedSwiglu<ACT> epi{Y, (int)rows};                                                   \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                                   \
         const u32 lo = blockIdx.y * 4;                                                            \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + 4 < batch ? lo + 4 : batch;                                           \
         matvec_body<FMT, ACT, F16, 2, 2, 2>(mats, X, rows, cols,                                  \
                                             packed_row_stride<FMT>(cols, 128), 128, lo, hi, epi); \
+    }
+
+// ---- lm_head: matvec fused with argmax over the rounded logits -------------------------------
+namespace smelt {
+
+// Keeps the best (value, index) key per thread; end_chunk() reduces the workgroup and writes one
+// partial key for the batch row at partials[batch * gridDim.x + blockIdx.x].
+template <class ActT>
+struct EpiArgmax {
+    uint2_t* partials;
+    float logit_cap;
+    uint2_t* best;      // one per thread (register-resident in the caller)
+    uint2_t* lds_keys;  // blockDim.x / 64 entries
+    __device__ __forceinline__ void operator()(int, int row, const float* v) const {
+        float x = v[0];
+        if (logit_cap > 0.0f) x = logit_cap * tanhf(x / logit_cap);
+        *best = argmax_key_max(*best, argmax_pack_key(ActT::narrow(x), (uint32_t)row));
+    }
+    __device__ __forceinline__ void end_chunk(int b0, int) const {
+        const uint2_t k = wave_argmax_key(*best);
+        const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+        __syncthreads();
+        if (lane == 0) lds_keys[wave] = k;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint2_t b = lds_keys[0];
+            for (int w = 1; w < (int)(blockDim.x / kWave); ++w) b = argmax_key_max(b, lds_keys[w]);
+            partials[(size_t)b0 * gridDim.x + blockIdx.x] = b;
+        }
+        *best = uint2_t{0u, 0u};
+    }
+};
+
+// Projection bank: up to four members share the input and one contiguous slab of code rows and
+// scale rows; virtual row r belongs to the member whose row range contains it.
+template <class ActT>
+struct EpiBank4 : EpiBase {
+    uint16_t* y[4];
+    uint32_t rows_m[4];
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        uint32_t r = (uint32_t)row;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            if (r < rows_m[m]) { y[m][(size_t)b * rows_m[m] + r] = ActT::narrow(v[0]); return; }
+            r -= rows_m[m];
+        }
+    }
+};
+
+}  // namespace smelt
+
+#define SMELT_AFFINE_ARGMAX(T, ACT, SC)                                                           \
+    SMELT_KERNEL void smelt_affine_matvec_argmax_##T(                                             \
+        const u8* W, const u16* S, const u16* B, const u16* X, smelt::uint2_t* keys, u32 batch,   \
+        float logit_cap, u32 rows, u32 cols, u32 group, u32 batch_tile) {                         \
+        using namespace smelt;                                                                    \
+        __shared__ uint2_t wave_keys[4];                                                          \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        uint2_t best = {0u, 0u};                                                                  \
+        EpiArgmax<ACT> epi{keys, logit_cap, &best, wave_keys};                                    \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, X, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group, lo,    \
+                                             hi, epi);                                            \
+    }
+
+// The ternary "affine" pipelines bind the scale plane a second time where MLX binds a bias
+// plane (bias = -scale); the arithmetic here is scale * (code - 1), so it is ignored.
+#define SMELT_TERAFF_KERNELS(T, ACT)                                                              \
+    SMELT_KERNEL void smelt_teraff_matvec_##T(const u8* C, const u16* S, const u16*,              \
+                                              const u16* X, u16* Y, u32 rows, u32 cols) {         \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        matvec_body<FmtTer2, ACT, F16, 4, 1, 1>(mats, X, rows, cols,                              \
+                                                packed_row_stride<FmtTer2>(cols, 128), 128,       \
+                                                blockIdx.y, blockIdx.y + 1, epi);                 \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_teraff_matvec_add_##T(const u8* C, const u16* S, const u16*,          \
+                                                  const u16* X, u16* Y, const u16* res, u32 rows, \
+                                                  u32 cols) {                                     \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        matvec_body<FmtTer2, ACT, F16, 4, 1, 1>(mats, X, rows, cols,                              \
+                                                packed_row_stride<FmtTer2>(cols, 128), 128,       \
+                                                blockIdx.y, blockIdx.y + 1, epi);                 \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_teraff_gate_up_swiglu_##T(                                            \
+        const u8* gC, const u16* gS, const u16*, const u8* uC, const u16* uS, const u16*,         \
+        const u16* X, u16* Y, u32 rows, u32 cols) {                                               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        matvec_body<FmtTer2, ACT, F16, 2, 1, 2>(mats, X, rows, cols,                              \
+                                                packed_row_stride<FmtTer2>(cols, 128), 128,       \
+                                                blockIdx.y, blockIdx.y + 1, epi);                 \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_teraff_bank4_matvec_##T(                                              \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* y0, u16* y1, u16* y2, u16* y3,  \
+        u32 rows0, u32 rows1, u32 rows2, u32 rows3, u32 cols) {                                   \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        const u32 rows = rows0 + rows1 + rows2 + rows3;                                           \
+        matvec_body<FmtTer2, ACT, F16, 4, 1, 1>(mats, X, rows, cols,                              \
+                                                packed_row_stride<FmtTer2>(cols, 128), 128, 0, 1, \
+                                                epi);                                             \
     }

@@ -2,6 +2,7 @@
 // Built with:  hipcc --offload-arch=gfx950 --genco -O3 -Xclang -target-feature -Xclang -packed-fp32-ops
 #include "matvec_kernels.hpp"
 #include "misc_kernels.hpp"
+#include "qmm.hpp"
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
@@ -16,3 +17,10 @@ SMELT_SIGNED_KERNELS(binary, smelt::FmtBin, f16, smelt::F16)
 SMELT_SIGNED_KERNELS(binary, smelt::FmtBin, bf16, smelt::BF16)
 SMELT_SIGNED_KERNELS(ternary, smelt::FmtTer2, f16, smelt::F16)
 SMELT_SIGNED_KERNELS(ternary, smelt::FmtTer2, bf16, smelt::BF16)
+
+SMELT_AFFINE_ARGMAX(f16, smelt::F16, smelt::F16)
+SMELT_AFFINE_ARGMAX(bf16, smelt::BF16, smelt::BF16)
+SMELT_TERAFF_KERNELS(f16, smelt::F16)
+SMELT_TERAFF_KERNELS(bf16, smelt::BF16)
+SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, f16, smelt::F16)
+SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, bf16, smelt::BF16)

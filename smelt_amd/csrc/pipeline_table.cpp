@@ -47,9 +47,9 @@ bool is_pow2(uint32_t v) { return v && !(v & (v - 1)); }
 const char* act_suffix(ActDType a) { return a == kActBF16 ? "bf16" : "f16"; }
 
 // resident activation rows per pass for the batched matvec kernels, bounded by LDS
-uint32_t pick_mb(int bits, uint32_t row_stride, uint32_t want, size_t lds_limit) {
+uint32_t pick_mb(CodeLayout layout, uint32_t row_stride, uint32_t want, size_t lds_limit) {
     for (uint32_t mb = want; mb > 1; mb >>= 1)
-        if (matvec_lds_bytes(bits, true, row_stride, mb) <= lds_limit) return mb;
+        if (matvec_lds_bytes(layout, row_stride, mb) <= lds_limit) return mb;
     return 1;
 }
 
@@ -60,10 +60,35 @@ struct AffineName {
 
 }  // namespace
 
-size_t matvec_lds_bytes(int bits_per_code, bool, uint32_t row_stride_bytes, uint32_t mb) {
+CodeLayout code_layout(SignedFormat f) {
+    switch (f) {
+        case kFmtBinary1: return kCodesBinary1;
+        case kFmtTernary2: return kCodesTernary2;
+        case kFmtTrit5: return kCodesTrit5;
+        default: return kCodesU4;
+    }
+}
+
+size_t matvec_lds_bytes(CodeLayout layout, uint32_t row_stride_bytes, uint32_t mb) {
     const size_t U = row_stride_bytes / 16;
-    const size_t chunks = 16 / (size_t)bits_per_code;  // 16-byte LDS chunks of fp16 pairs per unit
-    return (size_t)mb * U * 16 * (chunks + 2);         // + per-dword corrections and sums
+    // 16-byte LDS chunks of fp16 pairs per unit, and floats of per-dword corrections per unit
+    size_t chunks = 4, corr = 4, extra = 0;
+    switch (layout) {
+        case kCodesU4: chunks = 4; break;
+        case kCodesTernary2: chunks = 8; break;
+        case kCodesBinary1: chunks = 16; break;
+        case kCodesTrit5: chunks = 10; corr = 8; extra = 512; break;  // + decode table
+    }
+    return (size_t)mb * U * (16 * chunks + 2 * 4 * corr) + extra;
+}
+
+size_t qmm_lds_bytes(uint32_t nmat, uint32_t mt) {
+    const size_t ld = 128 + 8;
+    return ((size_t)nmat * 64 + (size_t)mt * 16) * ld * 2;
+}
+
+size_t qmm_affine_lds_bytes(uint32_t nmat, uint32_t mt) {
+    return (size_t)nmat * (64 * 80 + 2 * 4 * 64 * 4) + (size_t)mt * (16 * (128 + 8) * 2 + 16 * 4 * 4);
 }
 
 uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
@@ -147,12 +172,16 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         else if (suffix == "_batched_tile4" || suffix == "_batched_ext_b4") bt = 4;
         else if (suffix == "_batched_ext_b5" || suffix == "_batched_sg4_bt5") bt = 5;
         else if (suffix == "_batched_full") { bt = 16; full = true; }
-        else if (suffix == "_batched_full_b8") { bt = 8; full = true; }
+        else if (starts_with(suffix, "_batched_full_b") && parse_uint(suffix.substr(15), &bt) && bt >= 1 && bt <= 4096) { full = true; }
         else if (!m1) { *why = "unknown kernel variant '" + suffix + "' in '" + entry + "'"; return kResolveUnknown; }
 
         if (a.m1 == kFamAffineArgmax) {
-            *why = "affine_matvec_argmax is not built yet";
-            return kResolveUnknown;
+            if (m1 || full) { *why = "affine_matvec_argmax exists only as '_batched'"; return kResolveUnknown; }
+            out->family = kFamAffineArgmax;
+            out->symbol = "smelt_affine_matvec_argmax_" + t;
+            out->kinds = "PPPPPUFUUUU";
+            out->appended = {rows, cols, group, bt};
+            return kResolveOk;
         }
         if (m1) {
             out->family = a.m1;
@@ -167,10 +196,17 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             return kResolveOk;
         }
         if (full) {
-            *why = "affine qmm (batched_full) is not built yet";
-            return kResolveUnknown;
+            const uint32_t mt = bt >= 64 ? 4 : 1;
+            out->lds_variant = mt;
+            const std::string mts = "mt" + std::to_string(mt) + "_" + t;
+            if (a.m1 == kFamAffineMatvec) { out->family = kFamAffineQmm; out->symbol = "smelt_affine_qmm_" + mts; out->kinds = "PPPPPUUUUU"; }
+            else if (a.m1 == kFamAffineAdd) { out->family = kFamAffineQmmAdd; out->symbol = "smelt_affine_qmm_add_" + mts; out->kinds = "PPPPPPPUUUUU"; }
+            else if (a.m1 == kFamAffineGateUp) { out->family = kFamAffineQmmGateUp; out->symbol = "smelt_affine_qmm_gate_up_swiglu_" + mts; out->kinds = "PPPPPPPPUUUUU"; }
+            else { *why = "no qmm HIP kernel for '" + entry + "'"; return kResolveUnknown; }
+            out->appended = {rows, cols, group, bt};
+            return kResolveOk;
         }
-        const uint32_t mb = pick_mb(4, row_stride, 4, lds_limit);
+        const uint32_t mb = pick_mb(kCodesU4, row_stride, 4, lds_limit);
         out->lds_variant = mb;
         const std::string mbs = "mb" + std::to_string(mb) + "_" + t;
         if (a.m1 == kFamAffineMatvec) { out->family = kFamAffineBatched; out->symbol = "smelt_affine_matvec_batched_" + mbs; out->kinds = "PPPPPUUUUU"; }
@@ -193,6 +229,16 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         {"signed_ternary_gate_up_swiglu_g128_rows8", kFamSignedGateUp, kFmtTernary2, "smelt_signed_ternary_gate_up_swiglu_", "PPPPPPUU"},
         {"signed_ternary_matvec_g128_rows8_batched_b4", kFamSignedB4, kFmtTernary2, "smelt_signed_ternary_matvec_b4_", "PPPPUUU"},
         {"signed_ternary_gate_up_swiglu_g128_rows8_batched_b4", kFamSignedGateUpB4, kFmtTernary2, "smelt_signed_ternary_gate_up_swiglu_b4_", "PPPPPPUUU"},
+        {"signed_trit5_matvec_g128_rows8", kFamSignedMatvec, kFmtTrit5, "smelt_signed_trit5_matvec_", "PPPPUU"},
+        {"signed_trit5_matvec_add_g128_rows8", kFamSignedAdd, kFmtTrit5, "smelt_signed_trit5_matvec_add_", "PPPPPUU"},
+        {"signed_trit5_gate_up_swiglu_g128_rows8", kFamSignedGateUp, kFmtTrit5, "smelt_signed_trit5_gate_up_swiglu_", "PPPPPPUU"},
+        {"signed_trit5_matvec_g128_rows8_batched_b4", kFamSignedB4, kFmtTrit5, "smelt_signed_trit5_matvec_b4_", "PPPPUUU"},
+        {"signed_trit5_gate_up_swiglu_g128_rows8_batched_b4", kFamSignedGateUpB4, kFmtTrit5, "smelt_signed_trit5_gate_up_swiglu_b4_", "PPPPPPUUU"},
+        {"signed_ternary_affine_matvec_g128_rows8", kFamTerAffMatvec, kFmtTernary2, "smelt_teraff_matvec_", "PPPPPUU"},
+        {"signed_ternary_affine_matvec_add_g128_rows8", kFamTerAffAdd, kFmtTernary2, "smelt_teraff_matvec_add_", "PPPPPPUU"},
+        {"signed_ternary_affine_gate_up_swiglu_g128_rows8", kFamTerAffGateUp, kFmtTernary2, "smelt_teraff_gate_up_swiglu_", "PPPPPPPPUU"},
+        {"signed_ternary_affine_bank4_matvec_g128_rows8", kFamTerAffBank4, kFmtTernary2, "smelt_teraff_bank4_matvec_", "PPPPPPPPUUUUU"},
+        {"signed_ternary_affine_qmm_g128_bm32_bn32_bk32", kFamTerAffQmm, kFmtTernary2, "smelt_ternary_qmm_mt2_", "PPPPPUUU"},
     };
     for (const SignedName& s : kSigned) {
         if (entry == s.name) {
@@ -211,6 +257,12 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
     if (entry == "signed_ternary_embedding_gather_g128") { out->family = kFamSignedGather; out->format = kFmtTernary2; out->symbol = "smelt_signed_ternary_embedding_gather_" + t; out->kinds = "PPPPU"; return kResolveOk; }
     if (entry == "signed_trit5_embedding_gather_g128") { out->family = kFamSignedGather; out->format = kFmtTrit5; out->symbol = "smelt_signed_trit5_embedding_gather_" + t; out->kinds = "PPPPU"; return kResolveOk; }
     if (entry == "argmax_fp16_partials") { out->family = kFamArgmaxPartials; out->symbol = "smelt_argmax16_partials"; out->kinds = "PPUU"; return kResolveOk; }
+    if (starts_with(entry, "lm_head_argmax_reduce_r")) {
+        uint32_t n = 0;
+        if (!parse_uint(entry.substr(23), &n) || n == 0) { *why = "Malformed pipeline entry: '" + entry_in + "'"; return kResolveMalformed; }
+        out->family = kFamLmHeadReduce; out->symbol = "smelt_lm_head_argmax_reduce"; out->kinds = "PPUU";
+        return kResolveOk;
+    }
     if (entry == "argmax_key_reduce") { out->family = kFamArgmaxReduce; out->symbol = "smelt_argmax_key_reduce"; out->kinds = "PPU"; return kResolveOk; }
 
     *why = "no HIP kernel named '" + entry + "'";

@@ -50,7 +50,8 @@ struct ResolvedPipeline {
     std::vector<uint32_t> appended;  // values appended after the record's own bindings
     ActDType act;
     SignedFormat format = kFmtNone;
-    uint32_t lds_variant = 0;        // batched families: activations resident per pass (1, 2, 4)
+    uint32_t lds_variant = 0;        // batched matvec: activation rows resident per pass (1, 2, 4);
+                                     // qmm: 16-token blocks per workgroup tile (1, 2, 4)
 };
 
 enum ResolveStatus { kResolveOk = 0, kResolveUnknown = 1, kResolveMalformed = 2 };
@@ -59,8 +60,16 @@ enum ResolveStatus { kResolveOk = 0, kResolveUnknown = 1, kResolveMalformed = 2 
 ResolveStatus resolve_pipeline(const std::string& entry, ActDType default_act, size_t lds_limit,
                                ResolvedPipeline* out, std::string* why);
 
-// LDS bytes the matvec kernels need for `cols` columns of a format with `mb` resident rows.
-size_t matvec_lds_bytes(int bits_per_code, bool has_bias, uint32_t row_stride_bytes, uint32_t mb);
+// Packed-code layouts the matvec kernels consume.
+enum CodeLayout { kCodesU4 = 0, kCodesBinary1 = 1, kCodesTernary2 = 2, kCodesTrit5 = 3 };
+CodeLayout code_layout(SignedFormat f);
+
+// LDS bytes the matvec kernels need for one packed row stride with `mb` resident activation rows.
+size_t matvec_lds_bytes(CodeLayout layout, uint32_t row_stride_bytes, uint32_t mb);
+// LDS bytes of the MFMA qmm kernels: nmat weight tiles of 64 x 128 fp16 plus 16*mt token rows.
+size_t qmm_lds_bytes(uint32_t nmat, uint32_t mt);
+// LDS bytes of the affine qmm kernels: packed code tiles, fp32 scale/bias tiles, token rows and sums.
+size_t qmm_affine_lds_bytes(uint32_t nmat, uint32_t mt);
 
 uint32_t signed_row_stride(SignedFormat f, uint32_t cols);
 

@@ -145,9 +145,12 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             return bad_geom("signed g128 kernels need rows > 0 and cols % 128 == 0");
         return 0;
     };
-    int bits = 4;
-    if (r.format == kFmtBinary1) bits = 1;
-    if (r.format == kFmtTernary2) bits = 2;
+    const CodeLayout layout = code_layout(r.format);
+    auto signed_lds = [&](size_t cols, uint32_t mb) { return matvec_lds_bytes(layout, signed_row_stride(r.format, (uint32_t)cols), mb); };
+    auto need_256 = [&]() -> int {
+        if (L.block[0] != 256) return bad_geom("MFMA qmm kernels run with 256-thread workgroups, got " + std::to_string(L.block[0]));
+        return 0;
+    };
     switch (r.family) {
         case kFamAffineMatvec:
         case kFamAffineAdd: {
@@ -158,7 +161,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[3] = gy * cols * 2; align[3] = 16;
             need[4] = gy * rows * 2; written[4] = true;
             if (r.family == kFamAffineAdd) need[5] = gy * rows * 2;
-            L.lds = matvec_lds_bytes(4, true, (uint32_t)(cols / 2), 1);
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
             break;
         }
         case kFamAffineGateUp:
@@ -171,7 +174,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[6] = gy * cols * 2; align[6] = 16;
             need[7] = gy * rows * 2; written[7] = true;
             if (r.family == kFamAffineDual) { need[8] = gy * rows * 2; written[8] = true; }
-            L.lds = matvec_lds_bytes(4, true, (uint32_t)(cols / 2), 1);
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
             break;
         }
         case kFamAffineBatched:
@@ -185,7 +188,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             if (r.family == kFamAffineGateUpBatched) { affine(3, 4, 5, rows, cols, group); xi = 6; yi = 7; }
             need[xi] = batch * cols * 2; align[xi] = 16;
             need[yi] = batch * rows * 2; written[yi] = true;
-            L.lds = matvec_lds_bytes(4, true, (uint32_t)(cols / 2), r.lds_variant);
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), r.lds_variant);
             break;
         }
         case kFamSignedMatvec:
@@ -197,7 +200,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[2] = gy * cols * 2; align[2] = 16;
             need[3] = gy * rows * 2; written[3] = true;
             if (r.family == kFamSignedAdd) need[4] = gy * rows * 2;
-            L.lds = matvec_lds_bytes(bits, false, signed_row_stride(r.format, (uint32_t)cols), 1);
+            L.lds = signed_lds(cols, 1);
             break;
         }
         case kFamSignedGateUp: {
@@ -207,7 +210,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             signed_w(2, 3, rows, cols);
             need[4] = gy * cols * 2; align[4] = 16;
             need[5] = gy * rows * 2; written[5] = true;
-            L.lds = matvec_lds_bytes(bits, false, signed_row_stride(r.format, (uint32_t)cols), 1);
+            L.lds = signed_lds(cols, 1);
             break;
         }
         case kFamSignedB4:
@@ -221,7 +224,90 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             if (r.family == kFamSignedGateUpB4) { signed_w(2, 3, rows, cols); xi = 4; yi = 5; }
             need[xi] = batch * cols * 2; align[xi] = 16;
             need[yi] = batch * rows * 2; written[yi] = true;
-            L.lds = matvec_lds_bytes(bits, false, signed_row_stride(r.format, (uint32_t)cols), 2);
+            L.lds = signed_lds(cols, 2);
+            break;
+        }
+        case kFamAffineArgmax: {
+            const size_t batch = U(5), rows = U(7), cols = U(8), group = U(9), bt = U(10);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (bt == 0 || gy * bt < batch) return bad_geom("grid height * batch tile does not cover the batch");
+            if (rows > (1u << 18)) return bad_geom("argmax keys hold 18 index bits");
+            affine(0, 1, 2, rows, cols, group);
+            need[3] = batch * cols * 2; align[3] = 16;
+            need[4] = batch * (size_t)L.grid[0] * 8; align[4] = 8; written[4] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamLmHeadReduce: {
+            const size_t batch = U(2), parts = U(3);
+            if ((size_t)L.grid[0] < batch) return bad_geom("one workgroup per batch row is required");
+            need[0] = batch * parts * 8; align[0] = 8;
+            need[1] = batch * 4; align[1] = 4; written[1] = true;
+            break;
+        }
+        case kFamAffineQmm:
+        case kFamAffineQmmAdd:
+        case kFamAffineQmmGateUp: {
+            if (int e = need_256()) return e;
+            const size_t o = r.family == kFamAffineQmm ? 5 : (r.family == kFamAffineQmmAdd ? 7 : 8);
+            const size_t batch = U(o), rows = U(o + 1), cols = U(o + 2), group = U(o + 3), bt = U(o + 4);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (bt == 0 || gy * bt < batch) return bad_geom("grid height * batch tile does not cover the batch");
+            affine(0, 1, 2, rows, cols, group);
+            if (r.family == kFamAffineQmmGateUp) {
+                affine(3, 4, 5, rows, cols, group);
+                need[6] = batch * cols * 2; align[6] = 16;
+                need[7] = batch * rows * 2; written[7] = true;
+            } else {
+                need[3] = batch * cols * 2; align[3] = 16;
+                need[4] = batch * rows * 2; written[4] = true;
+                if (r.family == kFamAffineQmmAdd) { need[5] = batch * rows * 2; need[6] = batch * rows * 2; written[6] = true; }
+            }
+            L.lds = qmm_affine_lds_bytes(r.family == kFamAffineQmmGateUp ? 2 : 1, r.lds_variant);
+            break;
+        }
+        case kFamTerAffMatvec:
+        case kFamTerAffAdd: {
+            const size_t o = r.family == kFamTerAffAdd ? 6 : 5;
+            const size_t rows = U(o), cols = U(o + 1);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            signed_w(0, 1, rows, cols);
+            need[2] = need[1];
+            need[3] = gy * cols * 2; align[3] = 16;
+            need[4] = gy * rows * 2; written[4] = true;
+            if (r.family == kFamTerAffAdd) need[5] = gy * rows * 2;
+            L.lds = signed_lds(cols, 1);
+            break;
+        }
+        case kFamTerAffGateUp: {
+            const size_t rows = U(8), cols = U(9);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            signed_w(0, 1, rows, cols); need[2] = need[1];
+            signed_w(3, 4, rows, cols); need[5] = need[4];
+            need[6] = gy * cols * 2; align[6] = 16;
+            need[7] = gy * rows * 2; written[7] = true;
+            L.lds = signed_lds(cols, 1);
+            break;
+        }
+        case kFamTerAffBank4: {
+            const size_t rows = U(8) + U(9) + U(10) + U(11), cols = U(12);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            if (gy != 1) return bad_geom("projection banks are batch-1 kernels");
+            signed_w(0, 1, rows, cols); need[2] = need[1];
+            need[3] = cols * 2; align[3] = 16;
+            for (size_t m = 0; m < 4; ++m) { need[4 + m] = U(8 + m) * 2; written[4 + m] = U(8 + m) > 0; }
+            L.lds = signed_lds(cols, 1);
+            break;
+        }
+        case kFamTerAffQmm: {
+            if (int e = need_256()) return e;
+            const size_t rows = U(5), cols = U(6), batch = U(7);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            if (gy * 32 < batch) return bad_geom("grid height * 32 does not cover the batch");
+            signed_w(0, 1, rows, cols); need[2] = need[1];
+            need[3] = batch * cols * 2; align[3] = 16;
+            need[4] = batch * rows * 2; written[4] = true;
+            L.lds = qmm_lds_bytes(1, 2);
             break;
         }
         case kFamAffineGather:
