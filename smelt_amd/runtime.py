@@ -143,11 +143,16 @@ def load_library() -> C.CDLL:
 
 
 def exported_symbols() -> list[str]:
-    """Names include/smelt_hip.h declares (parsed from the header)."""
+    """Function names the headers under include/ declare (parsed from the header text)."""
     import re
-    hdr = os.path.join(os.path.dirname(HERE), "include", "smelt_hip.h")
-    text = open(hdr).read()
-    return sorted(set(re.findall(r"\b(smelt_hip_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    inc = os.path.join(os.path.dirname(HERE), "include")
+    for hdr in sorted(os.listdir(inc)):
+        if hdr.endswith(".h"):
+            text = open(os.path.join(inc, hdr)).read()
+            text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+            names.update(re.findall(r"\b(smelt_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 class Context:

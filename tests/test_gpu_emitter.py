@@ -1,0 +1,155 @@
+"""GPU: records produced by the emitters, interpreted eagerly and replayed as a HIP graph,
+reproduce the oracle on a small decode-step-shaped table for each weight family."""
+import numpy as np
+import pytest
+
+import fixtures as fx
+import gpu_harness as gh
+from oracle import oracle as so
+from smelt_amd import compiler as cc
+from smelt_amd import runtime as rt
+
+pytestmark = pytest.mark.gpu
+
+H_SLOT, Q_SLOT, FFN_SLOT, OUT_SLOT, KEY_SLOT, TOK_SLOT, RES_SLOT = 1, 2, 3, 4, 5, 6, 7
+
+
+def build_affine_table(dtype):
+    hidden, qdim, ffn, vocab, group = 1024, 512, 3584, 4096, 64
+    lay = cc.Layout()
+    wq, wg, wu = lay.affine(qdim, hidden, group), lay.affine(ffn, hidden, group), lay.affine(ffn, hidden, group)
+    wd, wl = lay.affine(hidden, ffn, group), lay.affine(vocab, hidden, group)
+    image = np.zeros(lay.total_bytes, np.uint8)
+    tensors = {}
+    for i, (name, e) in enumerate((("q", wq), ("gate", wg), ("up", wu), ("down", wd), ("lm_head", wl))):
+        t = fx.synth_affine(e.rows, e.cols, group, dtype, config=1, tensor=20 + i)
+        cc.write_affine(image, e, *t)
+        tensors[name] = t
+    em = cc.Emitter(rt.ACT_BF16 if dtype == fx.BF16 else rt.ACT_F16)
+    em.matvec(0, wq, cc.bind(H_SLOT), cc.bind(Q_SLOT))
+    em.gate_up_swiglu(0, wg, wu, cc.bind(H_SLOT), cc.bind(FFN_SLOT))
+    em.matvec_add(0, wd, cc.bind(FFN_SLOT), cc.bind(OUT_SLOT), cc.bind(RES_SLOT))
+    em.lm_head_argmax(0, wl, cc.bind(OUT_SLOT), cc.bind(KEY_SLOT), cc.bind(TOK_SLOT))
+    return em, image, tensors, (hidden, qdim, ffn, vocab, group)
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_affine_decode_table_eager_and_graph(dtype):
+    em, image, tensors, (hidden, qdim, ffn, vocab, group) = build_affine_table(dtype)
+    ctx = rt.Context(act_dtype=rt.ACT_BF16 if dtype == fx.BF16 else rt.ACT_F16)
+    try:
+        em.install(ctx)
+        ctx.upload_weights(0, image)
+        x = fx.synth_activation(1, hidden, dtype, config=1, tensor=70)
+        res = fx.to_bits(fx.rng_for(1, 71).normal(0, 1, (1, hidden)).astype(np.float32), dtype)
+        ctx.put(H_SLOT, x)
+        ctx.put(RES_SLOT, res)
+        ctx.alloc(Q_SLOT, qdim * 2)
+        ctx.alloc(FFN_SLOT, ffn * 2)
+        ctx.alloc(OUT_SLOT, hidden * 2)
+        ctx.alloc(KEY_SLOT, max(em.argmax_partial_bytes, 8))
+        ctx.alloc(TOK_SLOT, 4)
+        table = em.records()
+        assert ctx.interpret_decode(table) == 5
+        ctx.submit()
+        ctx.wait()
+        assert ctx.last_gpu_ns() > 0
+
+        def outputs():
+            return (ctx.read(Q_SLOT, np.uint16, qdim), ctx.read(FFN_SLOT, np.uint16, ffn),
+                    ctx.read(OUT_SLOT, np.uint16, hidden), int(ctx.read(TOK_SLOT, np.int32, 1)[0]))
+
+        q, act, out, tok = outputs()
+        xf = fx.from_bits(x, dtype)
+        gh.check_outputs(q.reshape(1, -1), so.affine_matvec(*tensors["q"], xf, qdim, hidden, group, dtype), dtype, "q")
+        g = so.affine_matvec(*tensors["gate"], xf, ffn, hidden, group, dtype)
+        u = so.affine_matvec(*tensors["up"], xf, ffn, hidden, group, dtype)
+        act_ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, dtype), dtype)
+        gh.check_outputs(act.reshape(1, -1), act_ref, dtype, "gate_up", rel_tol=4e-3)
+        # downstream references consume the GPU's own upstream bits, as the next kernel does
+        d = so.affine_matvec(*tensors["down"], fx.from_bits(act.reshape(1, -1), dtype), hidden, ffn, group, dtype)
+        out_ref = fx.from_bits(so.epilogue_residual_add(d, res, dtype), dtype)
+        gh.check_outputs(out.reshape(1, -1), out_ref, dtype, "down+add")
+        logits = so.affine_matvec(*tensors["lm_head"], fx.from_bits(out.reshape(1, -1), dtype), vocab, hidden, group, dtype)
+        assert tok == so.argmax16(so.narrow(logits, dtype)[0])
+
+        # graph replays: eager work and synchronisation between replays, every replay checked
+        graph, launches = ctx.capture_decode(table)
+        assert launches == 5
+        for i in range(3):
+            ctx.write(Q_SLOT, np.zeros(qdim, np.uint16))
+            ctx.write(OUT_SLOT, np.zeros(hidden, np.uint16))
+            ctx.write(TOK_SLOT, np.full(1, -1, np.int32))
+            assert ctx.graph_launch(graph) == 5
+            ctx.wait()
+            q2, act2, out2, tok2 = outputs()
+            assert np.array_equal(q2, q) and np.array_equal(act2, act) and np.array_equal(out2, out) and tok2 == tok, i
+        ctx.graph_destroy(graph)
+    finally:
+        ctx.close()
+
+
+@pytest.mark.parametrize("wdtype", [cc.BINARY1, cc.TERNARY2, cc.TRIT5])
+def test_signed_layer_table_decode_and_prefill(wdtype):
+    fmt = {cc.BINARY1: fx.BINARY1, cc.TERNARY2: fx.TERNARY2, cc.TRIT5: fx.TRIT5}[wdtype]
+    base = fx.TERNARY2 if fmt == fx.TRIT5 else fmt
+    hidden, kv, ffn = 1280, 256, 2048
+    lay = cc.Layout()
+    wk = lay.signed(kv, hidden, wdtype)
+    wg, wu = lay.signed(ffn, hidden, wdtype), lay.signed(ffn, hidden, wdtype)
+    wd = lay.signed(hidden, ffn, wdtype)
+    image = np.zeros(lay.total_bytes, np.uint8)
+    t = {}
+    for i, (name, e) in enumerate((("k", wk), ("gate", wg), ("up", wu), ("down", wd))):
+        codes = fx.synth_signed_codes(base, e.rows, e.cols, config=2, tensor=30 + i)
+        scales = fx.synth_signed_scales(e.rows, e.cols, config=2, tensor=30 + i)
+        packed = fx.pack_signed_np(codes, fmt, e.packed_row_stride)
+        cc.write_signed(image, e, packed, scales)
+        t[name] = (packed, scales)
+    ctx = rt.Context()
+    try:
+        # decode table
+        em = cc.Emitter()
+        em.matvec(0, wk, cc.bind(H_SLOT), cc.bind(Q_SLOT))
+        em.gate_up_swiglu(0, wg, wu, cc.bind(H_SLOT), cc.bind(FFN_SLOT))
+        em.matvec_add(0, wd, cc.bind(FFN_SLOT), cc.bind(OUT_SLOT), cc.bind(RES_SLOT))
+        # prefill table appended to the same pipeline list: k projection over seqLen tokens
+        em.matvec(0, wk, cc.bind(H_SLOT), cc.bind(Q_SLOT), batch=1, dynamic=True)
+        em.install(ctx)
+        ctx.upload_weights(0, image)
+        batch = 9
+        x = fx.synth_activation(batch, hidden, fx.F16, config=2, tensor=72)
+        res = fx.to_bits(fx.rng_for(2, 73).normal(0, 1, (1, hidden)).astype(np.float32), fx.F16)
+        ctx.put(H_SLOT, x)
+        ctx.put(RES_SLOT, res)
+        ctx.alloc(Q_SLOT, batch * kv * 2)
+        ctx.alloc(FFN_SLOT, ffn * 2)
+        ctx.alloc(OUT_SLOT, hidden * 2)
+        recs = em.records()
+        decode = ctx.table(list(recs)[:3])
+        assert ctx.interpret_decode(decode) == 3
+        ctx.wait()
+        xf = fx.from_bits(x, fx.F16)
+        ofmt = {fx.BINARY1: so.BINARY1, fx.TERNARY2: so.TERNARY2, fx.TRIT5: so.TRIT5}[fmt]
+        k_ref = so.signed_matvec(ofmt, *t["k"], xf, kv, hidden, hidden, 128)
+        gh.check_outputs(ctx.read(Q_SLOT, np.uint16, kv).reshape(1, -1), k_ref[:1], fx.F16, "k")
+        g = so.narrow(so.signed_matvec(ofmt, *t["gate"], xf[:1], ffn, hidden, hidden, 128), fx.F16)
+        u = so.narrow(so.signed_matvec(ofmt, *t["up"], xf[:1], ffn, hidden, hidden, 128), fx.F16)
+        act = ctx.read(FFN_SLOT, np.uint16, ffn)
+        act_ref = fx.from_bits(so.epilogue_signed_swiglu(g, u, so.F16), fx.F16)
+        gh.check_outputs(act.reshape(1, -1), act_ref, fx.F16, "signed gate_up", rel_tol=6e-3)
+        d = so.signed_matvec(ofmt, *t["down"], fx.from_bits(act.reshape(1, -1), fx.F16), hidden, ffn, ffn, 128)
+        out_ref = fx.from_bits(so.epilogue_residual_add(d, res, so.F16), fx.F16)
+        gh.check_outputs(ctx.read(OUT_SLOT, np.uint16, hidden).reshape(1, -1), out_ref, fx.F16, "down+add")
+        # prefill records at several sequence lengths (ternary switches QMV -> QMM at 6)
+        prefill = ctx.table(list(recs)[3:])
+        for seq in (1, 4, 5, 6, 9):
+            ctx.write(Q_SLOT, np.zeros(batch * kv, np.uint16))
+            assert ctx.interpret_prefill(prefill, seq_len=seq) == 1
+            ctx.wait()
+            y = ctx.read(Q_SLOT, np.uint16, seq * kv).reshape(seq, kv)
+            gh.check_outputs(y, k_ref[:seq], fx.F16, f"prefill seq={seq}")
+            rest = ctx.read(Q_SLOT, np.uint16, (batch - seq) * kv, offset=seq * kv * 2) if seq < batch else np.zeros(0)
+            assert not rest.any(), "tokens past seqLen must not be written"
+    finally:
+        ctx.close()
