@@ -4,8 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one pass over the decode-step matvec set of a 24-layer Qwen3.5-0.8B-shaped stack
-(BASELINE configs[1]): q/k/v/o projections, fused gate+up, down (+residual) per layer and the
-tied lm_head with fused argmax; all affine 4-bit g64 weights, bf16 activations, seeded synthetic
+(BASELINE configs[1]): the q/k/v projection bank, o, fused gate+up, down (+residual) per layer and
+the tied lm_head with fused argmax; all affine 4-bit g64 weights, bf16 activations, seeded synthetic
 tensors resident in HBM before the timed region.  The records are emitted by the library's own
 emitters, captured once into a HIP graph and replayed; `value` is weight bytes (packed codes +
 scales + biases, counted once per step) divided by the step time.
@@ -65,9 +65,9 @@ def main() -> int:
     lay = cc.Layout()
     per_layer = []
     for _ in range(layers):
+        q, k, v = lay.affine_bank([2048, 512, 512], hidden, group)  # same-input projection bank
         per_layer.append({
-            "q": lay.affine(2048, hidden, group), "k": lay.affine(512, hidden, group),
-            "v": lay.affine(512, hidden, group), "o": lay.affine(1024, hidden, group),
+            "q": q, "k": k, "v": v, "o": lay.affine(1024, hidden, group),
             "gate": lay.affine(ffn, hidden, group), "up": lay.affine(ffn, hidden, group),
             "down": lay.affine(hidden, ffn, group)})
     lm_copies = 4  # copy 0 belongs to the step; 1..3 only rotate under the roofline measurement
@@ -92,9 +92,9 @@ def main() -> int:
     em = cc.Emitter(rt.ACT_BF16, cus)
     for L in per_layer:
         # cur = hidden state in, alt = hidden state out; swapped after every layer
-        em.matvec(W, L["q"], cc.bind(rt.SLOT_CUR), cc.bind(QKV, 0))
-        em.matvec(W, L["k"], cc.bind(rt.SLOT_CUR), cc.bind(QKV, 2048 * 2))
-        em.matvec(W, L["v"], cc.bind(rt.SLOT_CUR), cc.bind(QKV, 2560 * 2))
+        banked = em.bank_matvec(W, [L["q"], L["k"], L["v"]], cc.bind(rt.SLOT_CUR),
+                                [cc.bind(QKV, 0), cc.bind(QKV, 2048 * 2), cc.bind(QKV, 2560 * 2)])
+        assert banked
         em.matvec(W, L["o"], cc.bind(ATT), cc.bind(rt.SLOT_ALT))
         em.gate_up_swiglu(W, L["gate"], L["up"], cc.bind(rt.SLOT_ALT), cc.bind(ACT))
         em.matvec_add(W, L["down"], cc.bind(ACT), cc.bind(rt.SLOT_ALT), cc.bind(rt.SLOT_CUR))
@@ -299,7 +299,7 @@ def cpu_baseline(fx, per_layer, lm_head, group) -> dict:
         one_pass()
         passes += 1
         dt = time.perf_counter() - t0
-        if dt > 10.0 or passes >= 400:
+        if dt > 10.0:
             break
     gbs = nbytes * passes / dt / 1e9
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": cores, "kind": "port",

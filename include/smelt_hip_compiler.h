@@ -86,6 +86,12 @@ int smelt_layout_make_affine_entry(int rows, int cols, int group_size, uint64_t 
  * dtype is binary1, ternary2, or trit5 (16-byte-aligned rows of ceil(cols/5) bytes). */
 int smelt_layout_make_signed_entry(int rows, int cols, int dtype, int group_size,
                                    uint64_t *offset_io, SmeltWeightEntryC *out);
+/* Projection bank (SmeltWeightLayoutPlanner.swift:404-572): 2-4 same-input members are re-offset
+ * so their packed rows form one contiguous slab, followed by one 128-byte-aligned scale slab
+ * (and, for affine, one bias slab).  Byte counts are unchanged and every member keeps its own
+ * entry; a bank kernel then walks the members as one virtual row space. */
+int smelt_layout_make_affine_bank(const int *member_rows, int members, int cols, int group_size,
+                                  uint64_t *offset_io, SmeltWeightEntryC *out_members);
 /* dense fp16/bf16/fp32/int32 entry, 16-byte aligned (:700-737) */
 int smelt_layout_make_dense_entry(int rows, int cols, int dtype, uint64_t *offset_io,
                                   SmeltWeightEntryC *out);
@@ -135,6 +141,12 @@ int smelt_emit_gate_up_swiglu(smelt_emitter *e, int weights_slot, const SmeltWei
 int smelt_emit_dual_matvec(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w1,
                            const SmeltWeightEntryC *w2, SmeltBinding input, SmeltBinding output1,
                            SmeltBinding output2);
+/* Common-input projection bank (emitSignedPackedProjectionBankIfPossible,
+ * SmeltCodeEmitter.swift:1264-1340): one dispatch for 2-4 members whose slabs are contiguous.
+ * Returns 1 (nothing emitted) when the members do not form a bank, so callers keep
+ * independent matvecs. */
+int smelt_emit_bank_matvec(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *members,
+                           int count, SmeltBinding input, const SmeltBinding *outputs);
 /* lm_head: affine_matvec_argmax + lm_head_argmax_reduce (TopLevelEmitter.swift:907) */
 int smelt_emit_lm_head_argmax(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w,
                               SmeltBinding input, SmeltBinding partial_keys, SmeltBinding token_out,

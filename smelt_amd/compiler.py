@@ -65,6 +65,8 @@ def lib() -> C.CDLL:
         "smelt_layout_make_affine_entry": (i32, [i32, i32, i32, u64p, we]),
         "smelt_layout_make_signed_entry": (i32, [i32, i32, i32, i32, u64p, we]),
         "smelt_layout_make_dense_entry": (i32, [i32, i32, i32, u64p, we]),
+        "smelt_layout_make_affine_bank": (i32, [C.POINTER(i32), i32, i32, i32, u64p, we]),
+        "smelt_emit_bank_matvec": (i32, [vp, i32, we, i32, Binding, C.POINTER(Binding)]),
         "smelt_route_decode_affine": (i32, [i32, i32, i32, i32, i32, C.POINTER(Route)]),
         "smelt_route_prefill_affine": (i32, [i32, i32, i32, i32, i32, i32, C.POINTER(Route)]),
         "smelt_emitter_create": (i32, [i32, i32, C.POINTER(vp)]),
@@ -128,6 +130,15 @@ class Layout:
         self._check(lib().smelt_layout_make_signed_entry(rows, cols, dtype, group, C.byref(self.offset), C.byref(e)))
         self.entries.append(e)
         return e
+
+    def affine_bank(self, member_rows, cols, group) -> list[WeightEntry]:
+        n = len(member_rows)
+        rows = (C.c_int * n)(*member_rows)
+        out = (WeightEntry * n)()
+        self._check(lib().smelt_layout_make_affine_bank(rows, n, cols, group, C.byref(self.offset), out))
+        members = [WeightEntry.from_buffer_copy(bytes(out[i])) for i in range(n)]
+        self.entries.extend(members)
+        return members
 
     def dense(self, rows, cols, dtype) -> WeightEntry:
         e = WeightEntry()
@@ -223,6 +234,17 @@ class Emitter:
 
     def dual_matvec(self, weights_slot, w1, w2, x, y1, y2):
         self._check(self.l.smelt_emit_dual_matvec(self.h, weights_slot, C.byref(w1), C.byref(w2), x, y1, y2))
+
+    def bank_matvec(self, weights_slot, members, x, outputs) -> bool:
+        """One dispatch for 2-4 contiguous same-input members; False if they do not form a bank."""
+        n = len(members)
+        arr = (WeightEntry * n)(*members)
+        outs = (Binding * n)(*outputs)
+        rc = self.l.smelt_emit_bank_matvec(self.h, weights_slot, arr, n, x, outs)
+        if rc == 1:
+            return False
+        self._check(rc)
+        return True
 
     def lm_head_argmax(self, weights_slot, w, x, keys, out, batch=1, logit_cap=0.0):
         self._check(self.l.smelt_emit_lm_head_argmax(self.h, weights_slot, C.byref(w), x, keys, out, batch,

@@ -313,6 +313,38 @@ int smelt_layout_make_signed_entry(int rows, int cols, int dtype, int group_size
     return SMELT_HIP_OK;
 }
 
+int smelt_layout_make_affine_bank(const int* member_rows, int members, int cols, int group_size, uint64_t* offset_io, SmeltWeightEntryC* out) {
+    if (!member_rows || !offset_io || !out || members < 2 || members > 4 || cols <= 0 || group_size <= 0) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    const uint64_t stride = (uint64_t)((cols + 1) / 2);
+    const uint64_t groups = (uint64_t)((cols + group_size - 1) / group_size);
+    uint64_t total_rows = 0;
+    for (int m = 0; m < members; ++m) {
+        if (member_rows[m] <= 0) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+        total_rows += (uint64_t)member_rows[m];
+    }
+    const uint64_t packed0 = align_to(*offset_io, 128);
+    const uint64_t scales0 = align_to(packed0 + total_rows * stride, 128);
+    const uint64_t biases0 = align_to(scales0 + total_rows * groups * 2, 128);
+    *offset_io = biases0 + total_rows * groups * 2;
+    uint64_t before = 0;
+    for (int m = 0; m < members; ++m) {
+        SmeltWeightEntryC& e = out[m];
+        memset(&e, 0, sizeof(e));
+        e.rows = member_rows[m]; e.cols = cols;
+        e.dtype = SMELT_DTYPE_AFFINE_U4;
+        e.group_size = group_size;
+        e.packed_row_stride = (int32_t)stride;
+        e.padded_cols = cols;
+        e.offset = packed0 + before * stride;
+        e.size_bytes = (uint64_t)e.rows * stride;
+        e.scales_offset = scales0 + before * groups * 2;
+        e.biases_offset = biases0 + before * groups * 2;
+        e.scales_size_bytes = e.biases_size_bytes = (uint64_t)e.rows * groups * 2;
+        before += (uint64_t)e.rows;
+    }
+    return SMELT_HIP_OK;
+}
+
 int smelt_layout_make_dense_entry(int rows, int cols, int dtype, uint64_t* offset_io, SmeltWeightEntryC* out) {
     if (!offset_io || !out || rows <= 0 || cols <= 0) return SMELT_HIP_ERR_INVALID_ARGUMENT;
     int bpe = 0;
@@ -629,6 +661,53 @@ int smelt_emit_dual_matvec(smelt_emitter* e, int weights_slot, const SmeltWeight
     if (!route.specialized) rb.constant(9, (uint32_t)w1->rows);
     rb.grid((uint32_t)route.grid_w, 1, 1, 256);
     rb.r.pipeline = e->pipeline_index(route.pipeline);
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+int smelt_emit_bank_matvec(smelt_emitter* e, int weights_slot, const SmeltWeightEntryC* members, int count, SmeltBinding input, const SmeltBinding* outputs) {
+    if (!e || !members || !outputs || count < 2 || count > 4) return efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "a bank has 2 to 4 members");
+    int family = 0;
+    if (int rc = gateway(e, &members[0], SMELT_SHAPE_GEMV, SMELT_FUSION_NONE, &family)) return rc;
+    const SmeltWeightEntryC& first = members[0];
+    uint64_t rows = 0;
+    for (int m = 0; m < count; ++m) {
+        const SmeltWeightEntryC& w = members[m];
+        if (w.dtype != first.dtype || w.cols != first.cols || w.group_size != first.group_size) return 1;
+        if (m > 0) {
+            const SmeltWeightEntryC& p = members[m - 1];
+            if (w.offset != p.offset + p.size_bytes || w.scales_offset != p.scales_offset + p.scales_size_bytes) return 1;
+            if (family == SMELT_FAMILY_AFFINE_U4 && w.biases_offset != p.biases_offset + p.biases_size_bytes) return 1;
+        }
+        rows += (uint64_t)w.rows;
+    }
+    RecordBuilder rb;
+    if (family == SMELT_FAMILY_AFFINE_U4) {
+        for (int m = 0; m < count; ++m)
+            if (!affine_entry_ok(&members[m])) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "unsupported affine geometry");
+        const MatvecGeometry g = matvec_geometry((uint32_t)first.cols / 2, (int)rows, 4, e->compute_units);
+        bind_affine(rb, 0, weights_slot, &first);
+        rb.buffer(3, input);
+        for (int m = 0; m < 4; ++m) rb.buffer((uint8_t)(4 + m), outputs[m < count ? m : 0]);
+        for (int m = 0; m < 4; ++m) rb.constant((uint8_t)(8 + m), m < count ? (uint32_t)members[m].rows : 0u);
+        rb.grid((uint32_t)g.grid_w, 1, 1, 256);
+        rb.r.pipeline = e->pipeline_index("affine_bank4_matvec:" + std::to_string(first.cols) + ":" + std::to_string(first.group_size));
+        e->records.push_back(rb.r);
+        return SMELT_HIP_OK;
+    }
+    if (family != SMELT_FAMILY_TERNARY2) return 1;  // banks exist for affine and ternary members
+    for (int m = 0; m < count; ++m)
+        if (int rc = check_signed_entry(e, &members[m])) return rc;
+    const MatvecGeometry g = matvec_geometry(signed_row_stride(kFmtTernary2, (uint32_t)first.cols), (int)rows, 4, e->compute_units);
+    rb.buffer(0, weights_slot, first.offset);
+    rb.buffer(1, weights_slot, first.scales_offset);
+    rb.buffer(2, weights_slot, first.scales_offset);
+    rb.buffer(3, input);
+    for (int m = 0; m < 4; ++m) rb.buffer((uint8_t)(4 + m), outputs[m < count ? m : 0]);
+    for (int m = 0; m < 4; ++m) rb.constant((uint8_t)(8 + m), m < count ? (uint32_t)members[m].rows : 0u);
+    rb.constant(12, (uint32_t)first.cols);
+    rb.grid((uint32_t)g.grid_w, 1, 1, 256);
+    rb.r.pipeline = e->pipeline_index("signed_ternary_affine_bank4_matvec_g128_rows8");
     e->records.push_back(rb.r);
     return SMELT_HIP_OK;
 }

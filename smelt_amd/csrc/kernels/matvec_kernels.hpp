@@ -369,7 +369,11 @@ struct EpiArgmax {
     uint2_t* lds_keys;  // blockDim.x / 64 entries
     __device__ __forceinline__ void operator()(int, int row, const float* v) const {
         float x = v[0];
-        if (logit_cap > 0.0f) x = logit_cap * tanhf(x / logit_cap);
+        if (logit_cap > 0.0f) {
+            // cap * tanh(x / cap) as cap * (1 - 2 / (1 + exp(2x / cap))); exp overflow gives +-cap
+            const float e = expf(2.0f * x / logit_cap);
+            x = logit_cap * (1.0f - 2.0f / (1.0f + e));
+        }
         *best = argmax_key_max(*best, argmax_pack_key(ActT::narrow(x), (uint32_t)row));
     }
     __device__ __forceinline__ void end_chunk(int b0, int) const {
@@ -420,6 +424,21 @@ struct EpiBank4 : EpiBase {
         matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, X, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group, lo,    \
                                              hi, epi);                                            \
+    }
+
+// Affine projection bank: up to four same-input members whose packed rows, scale rows and bias
+// rows each form one contiguous slab in member order (q | k | v ...), driven as one matvec over
+// the virtual row space; member m's rows go to output m.
+#define SMELT_AFFINE_BANK(T, ACT, SC)                                                             \
+    SMELT_KERNEL void smelt_affine_bank4_matvec_##T(                                              \
+        const u8* W, const u16* S, const u16* B, const u16* x, u16* y0, u16* y1, u16* y2,         \
+        u16* y3, u32 rows0, u32 rows1, u32 rows2, u32 rows3, u32 cols, u32 group) {               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x, rows0 + rows1 + rows2 + rows3, cols,        \
+                                             packed_row_stride<FmtU4>(cols, group), group, 0, 1,  \
+                                             epi);                                                \
     }
 
 // The ternary "affine" pipelines bind the scale plane a second time where MLX binds a bias

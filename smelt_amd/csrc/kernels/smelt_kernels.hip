@@ -24,3 +24,5 @@ SMELT_TERAFF_KERNELS(f16, smelt::F16)
 SMELT_TERAFF_KERNELS(bf16, smelt::BF16)
 SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, f16, smelt::F16)
 SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, bf16, smelt::BF16)
+SMELT_AFFINE_BANK(f16, smelt::F16, smelt::F16)
+SMELT_AFFINE_BANK(bf16, smelt::BF16, smelt::BF16)

@@ -135,6 +135,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         else if (name == "fused_affine_matvec_add") { out->family = kFamAffineAdd; out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; }
         else if (name == "fused_affine_gate_up_swiglu") { out->family = kFamAffineGateUp; out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; }
         else if (name == "fused_dual_affine_matvec") { out->family = kFamAffineDual; out->symbol = "smelt_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; }
+        else if (name == "affine_bank4_matvec") { out->family = kFamAffineBank4; out->symbol = "smelt_affine_bank4_matvec_" + t; out->kinds = "PPPPPPPPUUUUUU"; }
         else { *why = "no HIP kernel for function-constant pipeline '" + name + "'"; return kResolveUnknown; }
         if (!is_pow2(group) || group < 32 || cols % 32 != 0 || cols == 0) {
             *why = "affine kernels need cols % 32 == 0 and a power-of-two group >= 32 (got cols " +

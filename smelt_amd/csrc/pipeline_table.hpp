@@ -33,6 +33,7 @@ enum FamilyId {
     kFamTerAffGateUp,         // gC gS gS2 uC uS uS2 X Y rows cols
     kFamTerAffBank4,          // C S S2 x y0 y1 y2 y3 rows0 rows1 rows2 rows3 cols
     kFamTerAffQmm,            // C S S2 X Y rows cols batch
+    kFamAffineBank4,          // W S B x y0 y1 y2 y3 rows0 rows1 rows2 rows3 | cols group
     kFamAffineGather,         // W S B id out cols group
     kFamAffineGatherBatched,  // W S B ids out cols batch group
     kFamSignedGather,         // C S ids out hidden

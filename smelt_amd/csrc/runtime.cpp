@@ -117,7 +117,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
     auto bad_geom = [&](const std::string& m) {
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
     };
-    const bool matvec_like = r.family <= kFamTerAffQmm;
+    const bool matvec_like = r.family <= kFamAffineBank4;
     if (matvec_like) {
         if (L.block[0] % 64 != 0 || L.block[0] == 0 || L.block[0] > 256 || L.block[1] != 1 || L.block[2] != 1)
             return bad_geom("threadgroup must be 64..256 threads in whole wavefronts, got " +
@@ -297,6 +297,16 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[3] = cols * 2; align[3] = 16;
             for (size_t m = 0; m < 4; ++m) { need[4 + m] = U(8 + m) * 2; written[4 + m] = U(8 + m) > 0; }
             L.lds = signed_lds(cols, 1);
+            break;
+        }
+        case kFamAffineBank4: {
+            const size_t rows = U(8) + U(9) + U(10) + U(11), cols = U(12), group = U(13);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (gy != 1) return bad_geom("projection banks are batch-1 kernels");
+            affine(0, 1, 2, rows, cols, group);
+            need[3] = cols * 2; align[3] = 16;
+            for (size_t m = 0; m < 4; ++m) { need[4 + m] = U(8 + m) * 2; written[4 + m] = U(8 + m) > 0; }
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
             break;
         }
         case kFamTerAffQmm: {

@@ -153,3 +153,39 @@ def test_signed_layer_table_decode_and_prefill(wdtype):
             assert not rest.any(), "tokens past seqLen must not be written"
     finally:
         ctx.close()
+
+
+def test_affine_projection_bank_equals_independent_matvecs():
+    """One bank dispatch over q|k|v gives the bits of three independent dispatches."""
+    hidden, group = 1024, 64
+    member_rows = [2048, 512, 520]
+    lay = cc.Layout()
+    members = lay.affine_bank(member_rows, hidden, group)
+    lone = lay.affine(64, hidden, group)
+    # slabs are contiguous per plane and 128-byte aligned; byte counts are unchanged
+    assert members[1].offset == members[0].offset + members[0].size_bytes
+    assert members[2].scales_offset == members[1].scales_offset + members[1].scales_size_bytes
+    assert members[0].offset % 128 == 0 and members[0].scales_offset % 128 == 0 and members[0].biases_offset % 128 == 0
+    image = np.zeros(lay.total_bytes, np.uint8)
+    for i, e in enumerate(members):
+        cc.write_affine(image, e, *fx.synth_affine(e.rows, e.cols, group, fx.F16, config=1, tensor=40 + i))
+    ctx = rt.Context()
+    try:
+        em = cc.Emitter()
+        outs = [cc.bind(2, 0), cc.bind(2, 2048 * 2), cc.bind(2, 2560 * 2)]
+        assert em.bank_matvec(0, members, cc.bind(1), outs)
+        for e, o in zip(members, [cc.bind(3, 0), cc.bind(3, 2048 * 2), cc.bind(3, 2560 * 2)]):
+            em.matvec(0, e, cc.bind(1), o)
+        assert not em.bank_matvec(0, [members[0], lone], cc.bind(1), outs[:2])   # not contiguous: no bank
+        em.install(ctx)
+        ctx.upload_weights(0, image)
+        ctx.put(1, fx.synth_activation(1, hidden, fx.F16, config=1, tensor=41))
+        total = sum(member_rows)
+        ctx.alloc(2, total * 2)
+        ctx.alloc(3, total * 2)
+        assert ctx.interpret_decode(em.records()) == 4
+        ctx.wait()
+        a, b = ctx.read(2, np.uint16, total), ctx.read(3, np.uint16, total)
+        assert a.any() and np.array_equal(a, b)
+    finally:
+        ctx.close()

@@ -199,6 +199,43 @@ def test_lm_head_argmax_fused_and_staged(ctx):
         assert int(ctx.read(gh.Y_SLOT, np.int32, 1)[0]) == want[0]
 
 
+def test_lm_head_argmax_logit_cap(ctx):
+    """cap * tanh(v / cap) is applied in fp32 before the fp16/bf16 rounding that forms the key
+    (lut_matvec.metal:4194-4199).  The cap compresses the top logits into a few representable
+    values, so the winner is checked by value: its capped, rounded logit equals the best capped,
+    rounded logit of the oracle (to one output ulp for the exp-vs-tanh formulation), and where
+    the oracle's top value is unique by more than that the index is identical."""
+    rows, cols, group = 6000, 1024, 64
+    for dtype in (fx.F16, fx.BF16):
+        w = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=8)
+        x = fx.synth_activation(1, cols, dtype, config=1, tensor=34)
+        ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, group, dtype)[0].astype(np.float64)
+        cap = float(np.abs(ref).max()) * 0.75
+        capped = fx.from_bits(so.narrow((cap * np.tanh(ref / cap)).astype(np.float32), dtype), dtype).astype(np.float64)
+        wf = gh.WeightFile()
+        offs = [wf.add(a) for a in w]
+        ctx.upload_weights(0, wf.image())
+        ctx.put(gh.X_SLOT, x)
+        grid_w = 96
+        ctx.alloc(gh.AUX_SLOT, grid_w * 8)
+        ctx.alloc(gh.Y_SLOT, 4)
+        p1 = ctx.pipeline(f"affine_matvec_argmax_c{cols}_r{rows}_g{group}_batched" + gh.t_suffix(dtype))
+        p2 = ctx.pipeline(f"lm_head_argmax_reduce_r{rows}")
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.AUX_SLOT, 4, 0)]
+        r1 = rt.make_record(p1, bufs, [(5, 1), (6, cap)], (grid_w, 1, 1), (256, 1, 1))
+        r2 = rt.make_record(p2, [(gh.AUX_SLOT, 0, 0), (gh.Y_SLOT, 1, 0)], [(2, 1), (3, grid_w)], (1, 1, 1), (256, 1, 1))
+        assert ctx.interpret_decode(ctx.table([r1, r2])) == 2
+        ctx.wait()
+        got = int(ctx.read(gh.Y_SLOT, np.int32, 1)[0])
+        top = capped.max()
+        ulp = top * (2.0 ** -10 if dtype == fx.F16 else 2.0 ** -7)
+        assert 0 <= got < rows and capped[got] >= top - ulp, (got, capped[got], top)
+        assert capped[got] < cap * 1.001
+        order = np.sort(capped)
+        if order[-1] - order[-2] > 2 * ulp:
+            assert got == int(np.argmax(capped))
+
+
 def test_argmax_ties_and_signed_zero(ctx):
     vals = np.zeros(5000, np.float16)
     vals[[17, 400, 4999]] = 3.5                  # ties -> lowest index
