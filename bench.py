@@ -149,6 +149,19 @@ def main() -> int:
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "bytes_per_launch": int(lm_bytes), "us_per_launch": round(lm_us, 3)}
     del rl_table
+    roofline["traffic"] = committed_traffic()
+
+    # One plain copy of known size: the calibration dispatch for HBM traffic counters (a counter
+    # run of this same command scales FETCH_SIZE / WRITE_SIZE of the lm_head kernel by what they
+    # read for this copy).
+    CAL_SRC, CAL_DST, cal_bytes = 8, 9, 256 << 20
+    ctx.alloc(CAL_SRC, cal_bytes)
+    ctx.alloc(CAL_DST, cal_bytes)
+    cp = ctx.pipeline("copy_u128")
+    cal = rt.make_record(cp, [(CAL_SRC, 0, 0), (CAL_DST, 1, 0)], [(2, cal_bytes // 16)], (cus * 16, 1, 1), (256, 1, 1))
+    for _ in range(2):
+        ctx.interpret_decode(ctx.table([cal]))
+    ctx.wait()
 
     extra = {}
     if not args.no_extra:
@@ -174,6 +187,19 @@ def main() -> int:
     print(json.dumps(out))
     ctx.close()
     return 0
+
+
+def committed_traffic():
+    """HBM bytes per lm_head launch from the committed counter summary (two rocprofv3 --pmc runs of
+    this command, scaled by the copy calibration); None when no summary is present."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "lm_head_argmax_bf16_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch"):
+                return int(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def side_measurements(ctx, fx, cc, rt, cus) -> dict:

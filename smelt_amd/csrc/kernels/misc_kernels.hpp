@@ -167,3 +167,12 @@ SMELT_MISC_KERNEL void smelt_lm_head_argmax_reduce(const smelt::uint2_t* partial
         output[blockIdx.x] = (int)(kArgmaxMaxIndex - best.y);
     }
 }
+
+// Plain device copy of n16 16-byte elements (grid-stride).  It moves a known number of bytes
+// each way, which makes it the calibration kernel for memory-traffic counters.
+extern "C" __global__ __launch_bounds__(256) void smelt_copy_u128(const smelt::uint4_t* __restrict__ src,
+                                                                  smelt::uint4_t* __restrict__ dst,
+                                                                  uint32_t n16) {
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}

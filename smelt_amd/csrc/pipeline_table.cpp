@@ -264,6 +264,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         out->family = kFamLmHeadReduce; out->symbol = "smelt_lm_head_argmax_reduce"; out->kinds = "PPUU";
         return kResolveOk;
     }
+    if (entry == "copy_u128") { out->family = kFamCopy; out->symbol = "smelt_copy_u128"; out->kinds = "PPU"; return kResolveOk; }
     if (entry == "argmax_key_reduce") { out->family = kFamArgmaxReduce; out->symbol = "smelt_argmax_key_reduce"; out->kinds = "PPU"; return kResolveOk; }
 
     *why = "no HIP kernel named '" + entry + "'";

@@ -39,6 +39,7 @@ enum FamilyId {
     kFamSignedGather,         // C S ids out hidden
     kFamArgmaxPartials,       // logits partials vocab chunk
     kFamArgmaxReduce,         // partials out num_partials
+    kFamCopy,                 // src dst n16
     kFamCount
 };
 

@@ -353,6 +353,11 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[1] = (size_t)L.grid[0] * 4; align[1] = 4; written[1] = true;
             break;
         }
+        case kFamCopy: {
+            need[0] = U(2) * 16; align[0] = 16;
+            need[1] = U(2) * 16; align[1] = 16; written[1] = true;
+            break;
+        }
         default:
             return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "pipeline '" + p.entry + "' has no launch validator");
     }
