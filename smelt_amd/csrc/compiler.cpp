@@ -396,6 +396,15 @@ int smelt_route_prefill_affine(int rows, int cols, int group, int fusion, int ma
         set_route(out, base + "_batched_tile4", true, g.rows_per_group, 4, 256, g.grid_w);
         return SMELT_HIP_OK;
     }
+    if (max_batch <= 32 && group == 64 && cols % 512 == 0) {
+        // skinny MFMA qmm: 32-row tiles, K split over enough workgroups to keep the whole matrix
+        // in flight (about ten 64-column windows per workgroup, at least three workgroups per CU)
+        const int nwin = cols / 64, tiles = (rows + 31) / 32;
+        int ksplit = std::max(1, nwin / 10);
+        while (tiles * ksplit < 3 * std::max(1, compute_units) && (nwin + ksplit) / (ksplit + 1) >= 4) ++ksplit;
+        set_route(out, base + "_batched_skinny", true, 32, 32, 256, tiles * ksplit);
+        return SMELT_HIP_OK;
+    }
     // MFMA qmm: 64-row slabs; 16-token tiles up to 32 tokens, 64-token tiles beyond
     const int bt = max_batch > 32 ? 64 : 16;
     const std::string suffix = bt == 16 ? "_batched_full" : "_batched_full_b64";

@@ -1,0 +1,331 @@
+// Skinny quantized matmul for gfx950: Y[M, N] = X[M, K] * W[N, K]^T with M <= 32 tokens per pass,
+// affine u4 weights with one scale group per 64 columns.
+//
+// At this batch the weights still stream from HBM once and the arithmetic is small, so the kernel is
+// organised around keeping every byte of W in flight rather than around tile reuse:
+//   * v_mfma_f32_32x32x16_f16 with the tokens as the A operand and 32 weight rows as the B operand.
+//     Lane (j = lane % 32, kb = lane / 32) loads 16 bytes = 32 codes of row j; dword t of those 16
+//     bytes holds exactly the eight k-values lane (j, kb) supplies to the t-th MFMA of a 64-column
+//     window, so a packed dword becomes a B operand with one shift, four v_bitop3 and four packed
+//     subtracts, with no shuffles and no LDS round trip for the weights.
+//   * The MFMA multiplies the exact integer codes; the per-(row, window) scale is applied in fp32
+//     on the 32x32 accumulator (each lane owns one weight row, so it is one scalar per lane).
+//   * The bias term  sum_g b[n, g] * xsum[m, g]  is itself a small matmul over scale groups and is
+//     fed through the same MFMA, with xsum split into fp16 high and low parts (22 significant bits).
+//   * K is split over the four waves of a workgroup and, for long rows, over `ksplit` workgroups
+//     (gridDim.x = row tiles * ksplit).  Wave partials meet in LDS; workgroup partials meet in a
+//     workspace where the last workgroup to arrive adds them in a fixed order, so results do not
+//     depend on arrival order.
+// Activations are staged once per workgroup into LDS as fp16 in the operand order of the code
+// pairs (every run of 8 columns permuted to 0,4,1,5,2,6,3,7).
+#pragma once
+#include "common.hpp"
+#include "matvec.hpp"
+#include "qmm.hpp"
+
+namespace smelt {
+
+typedef float float16v_t __attribute__((ext_vector_type(16)));
+
+constexpr int kSkRows = 32;  // weight rows per workgroup tile (MFMA N)
+constexpr int kSkTok = 32;   // tokens per pass (MFMA M)
+constexpr int kSkWB = 4;     // windows per register batch
+
+struct SkinnyWorkspace {
+    float* partial;      // [gridDim.y][tiles][ksplit][NMAT][32 tokens][32 rows]
+    uint32_t* counters;  // [gridDim.y][tiles], zero between launches
+};
+
+template <int NMAT>
+struct SkinnyBatch {
+    uint4_t c[NMAT][kSkWB];
+    uint16_t s[NMAT][kSkWB];
+};
+
+// eight codes of one dword -> fp16 values (0..15) in operand order (0,4,1,5,2,6,3,7)
+__device__ __forceinline__ half8_t skinny_codes(uint32_t c) {
+    const uint32_t c8 = c >> 8;
+    const half2_t o1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    const half2_t o64 = {(_Float16)64.0f, (_Float16)64.0f};
+    const half2_t a0 = as_half2(and_or(c, 0x000F000Fu, 0x64006400u)) - o1024;
+    const half2_t a1 = as_half2(and_or(c, 0x00F000F0u, 0x54005400u)) - o64;
+    const half2_t a2 = as_half2(and_or(c8, 0x000F000Fu, 0x64006400u)) - o1024;
+    const half2_t a3 = as_half2(and_or(c8, 0x00F000F0u, 0x54005400u)) - o64;
+    half8_t a;
+    a[0] = a0.x; a[1] = a0.y; a[2] = a1.x; a[3] = a1.y;
+    a[4] = a2.x; a[5] = a2.y; a[6] = a3.x; a[7] = a3.y;
+    return a;
+}
+
+// Windows per K chunk and LDS bytes; the host computes the same numbers to size the launch.
+__host__ __device__ inline int skinny_chunk_windows(int cols, int ksplit) {
+    const int nwin = cols / 64;
+    return (nwin + ksplit - 1) / ksplit;
+}
+__host__ __device__ inline int skinny_bias_blocks(int chunk_windows) { return (chunk_windows + 15) / 16 + 1; }
+__host__ __device__ inline size_t skinny_lds_bytes(int cols, int ksplit, int nmat) {
+    const int cw = skinny_chunk_windows(cols, ksplit);
+    const size_t stage = (size_t)cw * 4096 + (size_t)skinny_bias_blocks(cw) * 2048;
+    const size_t reduce = (size_t)4 * nmat * 4096;
+    return stage > reduce ? stage : reduce;
+}
+
+template <class ActT, class ScaleT, int NMAT, class Epi>
+__device__ __forceinline__ void qmm_skinny_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
+                                                const uint16_t* const (&B)[NMAT], const uint16_t* X,
+                                                int rows, int cols, int batch, int batch_tile,
+                                                SkinnyWorkspace ws, const Epi& epi) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ uint32_t last_flag;
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave, lane = tid % kWave;
+    const int lj = lane & 31, kb = lane >> 5;
+    const int tiles = (rows + kSkRows - 1) / kSkRows;
+    const int ksplit = gridDim.x / tiles;
+    const int tile = blockIdx.x / ksplit, ks = blockIdx.x % ksplit;
+    const int nwin = cols / 64;  // == scale groups per row
+    const int cw = skinny_chunk_windows(cols, ksplit);
+    const int W0 = ks * cw < nwin ? ks * cw : nwin;
+    const int W1 = W0 + cw < nwin ? W0 + cw : nwin;
+    const int m0 = blockIdx.y * batch_tile;
+    const int ntok = batch - m0 < batch_tile ? batch - m0 : batch_tile;  // <= 32
+    const int rs = cols / 2;
+
+    uint4_t* xs = reinterpret_cast<uint4_t*>(smem);                       // [cw][4][2][32] x 16 B
+    uint4_t* xsum_hi = xs + (size_t)cw * 256;                              // [blocks][2][32] x 16 B
+    uint4_t* xsum_lo = xsum_hi + (size_t)skinny_bias_blocks(cw) * 64;
+    float* red = reinterpret_cast<float*>(smem);                           // aliases the staging area
+    const int blk0 = W0 / 16, blk1 = (W1 + 15) / 16;
+
+    // this wave's windows of the chunk
+    const int pw = (W1 - W0 + 3) / 4;
+    const int w0 = W0 + wave * pw < W1 ? W0 + wave * pw : W1;
+    const int w1 = w0 + pw < W1 ? w0 + pw : W1;
+    int row = tile * kSkRows + lj;
+    if (row >= rows) row = rows - 1;  // clamped rows are computed and never stored
+
+    auto load = [&](SkinnyBatch<NMAT>& dst, int wb) {
+#pragma unroll
+        for (int i = 0; i < kSkWB; ++i) {
+            const int w = wb + i;
+            if (w < w1) {
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) {
+                    dst.c[m][i] = *reinterpret_cast<const uint4_t*>(W[m] + (size_t)row * rs + (size_t)w * 32 + kb * 16);
+                    dst.s[m][i] = S[m][(size_t)row * nwin + w];
+                }
+            }
+        }
+    };
+    SkinnyBatch<NMAT> bufa, bufb;
+    load(bufa, w0);  // in flight while the activations are staged
+
+    // ---- stage activations -------------------------------------------------------------------
+    for (int i = tid; i < (blk1 - blk0) * 128; i += blockDim.x) {
+        const uint4_t z = {0u, 0u, 0u, 0u};
+        (i < (blk1 - blk0) * 64 ? xsum_hi[i] : xsum_lo[i - (blk1 - blk0) * 64]) = z;
+    }
+    __syncthreads();
+    for (int item = tid; item < (W1 - W0) * kSkTok; item += blockDim.x) {
+        const int wl = item / kSkTok, tok = item % kSkTok;
+        const int w = W0 + wl;
+        float xsum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {  // run e of 8 columns belongs to lane half e / 4, MFMA e % 4
+            uint4_t v = {0u, 0u, 0u, 0u};
+            if (tok < ntok) v = *reinterpret_cast<const uint4_t*>(X + (size_t)(m0 + tok) * cols + (size_t)w * 64 + e * 8);
+            uint16_t h[8];
+            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                h[2 * q] = ActT::to_f16_bits((uint16_t)(d[q] & 0xFFFF));
+                h[2 * q + 1] = ActT::to_f16_bits((uint16_t)(d[q] >> 16));
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) xsum += F16::widen(h[q]);
+            uint4_t o;
+            o.x = h[0] | ((uint32_t)h[4] << 16);
+            o.y = h[1] | ((uint32_t)h[5] << 16);
+            o.z = h[2] | ((uint32_t)h[6] << 16);
+            o.w = h[3] | ((uint32_t)h[7] << 16);
+            xs[((size_t)(wl * 4 + (e & 3)) * 2 + (e >> 2)) * 32 + tok] = o;
+        }
+        const uint16_t hi = F16::narrow(xsum);
+        const uint16_t lo = F16::narrow(xsum - F16::widen(hi));
+        const size_t at = ((size_t)((w >> 4) - blk0) * 2 + ((w >> 3) & 1)) * 32 + tok;
+        reinterpret_cast<uint16_t*>(xsum_hi + at)[w & 7] = hi;
+        reinterpret_cast<uint16_t*>(xsum_lo + at)[w & 7] = lo;
+    }
+    __syncthreads();
+
+    // ---- main loop: windows of this wave, register batches double-buffered --------------------
+    float16v_t y[NMAT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) y[m][v] = 0.0f;
+
+    auto compute = [&](const SkinnyBatch<NMAT>& cur, int wb) {
+#pragma unroll
+        for (int i = 0; i < kSkWB; ++i) {
+            const int w = wb + i;
+            if (w < w1) {
+                float16v_t acc[NMAT];
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[m][v] = 0.0f;
+                const uint4_t* xw = xs + (size_t)(w - W0) * 256 + kb * 32 + lj;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const half8_t xa = *reinterpret_cast<const half8_t*>(xw + t * 64);
+#pragma unroll
+                    for (int m = 0; m < NMAT; ++m) {
+                        const uint32_t cd = t == 0 ? cur.c[m][i].x : (t == 1 ? cur.c[m][i].y : (t == 2 ? cur.c[m][i].z : cur.c[m][i].w));
+                        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa, skinny_codes(cd), acc[m], 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) {
+                    const float sv = ScaleT::widen(cur.s[m][i]);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) y[m][v] = __builtin_fmaf(sv, acc[m][v], y[m][v]);
+                }
+            }
+        }
+    };
+    for (int wb = w0; wb < w1; wb += 2 * kSkWB) {
+        if (wb + kSkWB < w1) load(bufb, wb + kSkWB);
+        compute(bufa, wb);
+        if (wb + kSkWB < w1) {
+            if (wb + 2 * kSkWB < w1) load(bufa, wb + 2 * kSkWB);
+            compute(bufb, wb + kSkWB);
+        }
+    }
+
+    // ---- bias term: blocks of 16 scale groups, one MFMA pair each, spread over the waves -------
+    for (int blk = blk0 + wave; blk < blk1; blk += 4) {
+        const int g = blk * 16 + kb * 8;
+        const half8_t ah = *reinterpret_cast<const half8_t*>(xsum_hi + ((size_t)(blk - blk0) * 2 + kb) * 32 + lj);
+        const half8_t al = *reinterpret_cast<const half8_t*>(xsum_lo + ((size_t)(blk - blk0) * 2 + kb) * 32 + lj);
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            uint4_t bv = {0u, 0u, 0u, 0u};
+            if (g < nwin) bv = *reinterpret_cast<const uint4_t*>(B[m] + (size_t)row * nwin + g);
+            const uint32_t d[4] = {bv.x, bv.y, bv.z, bv.w};
+            uint32_t p[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                p[q] = (uint32_t)ScaleT::to_f16_bits((uint16_t)(d[q] & 0xFFFF)) |
+                       ((uint32_t)ScaleT::to_f16_bits((uint16_t)(d[q] >> 16)) << 16);
+            half8_t bq;
+            {
+                const half2_t b0 = as_half2(p[0]), b1 = as_half2(p[1]), b2 = as_half2(p[2]), b3 = as_half2(p[3]);
+                bq[0] = b0.x; bq[1] = b0.y; bq[2] = b1.x; bq[3] = b1.y;
+                bq[4] = b2.x; bq[5] = b2.y; bq[6] = b3.x; bq[7] = b3.y;
+            }
+            y[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bq, y[m], 0, 0, 0);
+            y[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bq, y[m], 0, 0, 0);
+        }
+    }
+
+    // ---- reduce the four waves through LDS --------------------------------------------------------
+    __syncthreads();  // every wave is done with the staged activations
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int tok = 8 * (v >> 2) + 4 * kb + (v & 3);
+            red[((size_t)(wave * NMAT + m) * kSkTok + tok) * kSkRows + lj] = y[m][v];
+        }
+    __syncthreads();
+    const int tok = tid >> 3, r4 = (tid & 7) * 4;
+    float val[NMAT][4];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) {
+        float4_t sum = *reinterpret_cast<const float4_t*>(red + ((size_t)m * kSkTok + tok) * kSkRows + r4);
+#pragma unroll
+        for (int wv = 1; wv < 4; ++wv) {
+            const float4_t p = *reinterpret_cast<const float4_t*>(red + ((size_t)(wv * NMAT + m) * kSkTok + tok) * kSkRows + r4);
+            sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+        }
+        val[m][0] = sum.x; val[m][1] = sum.y; val[m][2] = sum.z; val[m][3] = sum.w;
+    }
+
+    if (ksplit > 1) {
+        // Workgroup partials meet in the workspace; the last to arrive adds them in chunk order.
+        const size_t slot = (size_t)blockIdx.y * tiles + tile;
+        float* mine = ws.partial + ((slot * ksplit + ks) * NMAT) * 1024;
+        if (tok < ntok) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                float4_t o = {val[m][0], val[m][1], val[m][2], val[m][3]};
+                *reinterpret_cast<float4_t*>(mine + (size_t)m * 1024 + tok * kSkRows + r4) = o;
+            }
+        }
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) last_flag = atomicAdd(ws.counters + slot, 1u) == (uint32_t)(ksplit - 1) ? 1u : 0u;
+        __syncthreads();
+        if (!last_flag) return;
+        __threadfence();
+        if (tok < ntok) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+                for (int c = 0; c < ksplit; ++c) {
+                    const float4_t p = *reinterpret_cast<const float4_t*>(
+                        ws.partial + ((slot * ksplit + c) * NMAT + m) * 1024 + tok * kSkRows + r4);
+                    sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+                }
+                val[m][0] = sum.x; val[m][1] = sum.y; val[m][2] = sum.z; val[m][3] = sum.w;
+            }
+        }
+        if (tid == 0) ws.counters[slot] = 0u;  // ready for the next launch on this stream
+    }
+    if (tok < ntok) epi(m0 + tok, tile * kSkRows + r4, rows, val);
+}
+
+}  // namespace smelt
+
+#define SMELT_AFFINE_QMM_SKINNY(T, ACT, SC)                                                        \
+    SMELT_QMM_KERNEL void smelt_affine_qmm_skinny_##T(                                             \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* Y,    \
+        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t group, uint32_t batch_tile,         \
+        float* ws_partial, uint32_t* ws_counters) {                                                \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        QEpiStore<ACT> epi{Y};                                                                     \
+        qmm_skinny_body<ACT, SC, 1>(w, s, b, X, rows, cols, batch, batch_tile,                     \
+                                    SkinnyWorkspace{ws_partial, ws_counters}, epi);                \
+    }                                                                                              \
+    SMELT_QMM_KERNEL void smelt_affine_qmm_add_skinny_##T(                                         \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* MV,   \
+        const uint16_t* RES, uint16_t* OUT, uint32_t batch, uint32_t rows, uint32_t cols,          \
+        uint32_t group, uint32_t batch_tile, float* ws_partial, uint32_t* ws_counters) {           \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        QEpiAdd<ACT> epi{MV, RES, OUT};                                                            \
+        qmm_skinny_body<ACT, SC, 1>(w, s, b, X, rows, cols, batch, batch_tile,                     \
+                                    SkinnyWorkspace{ws_partial, ws_counters}, epi);                \
+    }                                                                                              \
+    SMELT_QMM_KERNEL void smelt_affine_qmm_gate_up_swiglu_skinny_##T(                              \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t group, uint32_t batch_tile, float* ws_partial,      \
+        uint32_t* ws_counters) {                                                                   \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        QEpiSwiglu<ACT> epi{Y};                                                                    \
+        qmm_skinny_body<ACT, SC, 2>(w, s, b, X, rows, cols, batch, batch_tile,                     \
+                                    SkinnyWorkspace{ws_partial, ws_counters}, epi);                \
+    }
+
+SMELT_AFFINE_QMM_SKINNY(f16, smelt::F16, smelt::F16)
+SMELT_AFFINE_QMM_SKINNY(bf16, smelt::BF16, smelt::BF16)

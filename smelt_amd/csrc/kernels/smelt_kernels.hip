@@ -3,6 +3,7 @@
 #include "matvec_kernels.hpp"
 #include "misc_kernels.hpp"
 #include "qmm.hpp"
+#include "qmm_skinny.hpp"
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)

@@ -91,6 +91,15 @@ size_t qmm_affine_lds_bytes(uint32_t nmat, uint32_t mt) {
     return (size_t)nmat * (64 * 80 + 2 * 4 * 64 * 4) + (size_t)mt * (16 * (128 + 8) * 2 + 16 * 4 * 4);
 }
 
+size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat) {
+    // staged activations: 4 KB per 64-column window of a chunk, plus fp16 high/low activation sums
+    // in blocks of 16 groups; the wave reduction (4 waves x nmat x 4 KB) reuses the same bytes
+    const size_t nwin = cols / 64, cw = (nwin + ksplit - 1) / ksplit;
+    const size_t stage = cw * 4096 + ((cw + 15) / 16 + 1) * 2048;
+    const size_t reduce = (size_t)4 * nmat * 4096;
+    return stage > reduce ? stage : reduce;
+}
+
 uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
     const uint32_t padded = (cols + 127u) / 128u * 128u;
     switch (f) {
@@ -167,8 +176,9 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         const uint32_t row_stride = cols / 2;
         const bool m1 = suffix.empty() || suffix == "_rows4" || suffix == "_rows8" || suffix == "_rows4_sg1";
         uint32_t bt = 0;
-        bool full = false;
+        bool full = false, skinny = false;
         if (suffix == "_batched") bt = 8;
+        else if (suffix == "_batched_skinny") { bt = 32; full = true; skinny = true; }
         else if (suffix == "_batched_tile3") bt = 3;
         else if (suffix == "_batched_tile4" || suffix == "_batched_ext_b4") bt = 4;
         else if (suffix == "_batched_ext_b5" || suffix == "_batched_sg4_bt5") bt = 5;
@@ -194,6 +204,17 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                 default: break;
             }
             out->appended = {rows, cols, group};
+            return kResolveOk;
+        }
+        if (full && skinny) {
+            if (group != 64 || cols % 512 != 0) { *why = "skinny qmm needs group 64 and cols % 512 == 0: '" + entry + "'"; return kResolveMalformed; }
+            out->lds_variant = kSkinnyVariant;
+            out->workspace = true;
+            if (a.m1 == kFamAffineMatvec) { out->family = kFamAffineQmm; out->symbol = "smelt_affine_qmm_skinny_" + t; out->kinds = "PPPPPUUUUU"; }
+            else if (a.m1 == kFamAffineAdd) { out->family = kFamAffineQmmAdd; out->symbol = "smelt_affine_qmm_add_skinny_" + t; out->kinds = "PPPPPPPUUUUU"; }
+            else if (a.m1 == kFamAffineGateUp) { out->family = kFamAffineQmmGateUp; out->symbol = "smelt_affine_qmm_gate_up_swiglu_skinny_" + t; out->kinds = "PPPPPPPPUUUUU"; }
+            else { *why = "no skinny qmm HIP kernel for '" + entry + "'"; return kResolveUnknown; }
+            out->appended = {rows, cols, group, bt};
             return kResolveOk;
         }
         if (full) {

@@ -53,8 +53,14 @@ struct ResolvedPipeline {
     ActDType act;
     SignedFormat format = kFmtNone;
     uint32_t lds_variant = 0;        // batched matvec: activation rows resident per pass (1, 2, 4);
-                                     // qmm: 16-token blocks per workgroup tile (1, 2, 4)
+                                     // qmm: 16-token blocks per workgroup tile (1, 2, 4),
+                                     // or kSkinnyVariant for the split-K skinny kernels
+    bool workspace = false;          // kernel takes the context's (partials, counters) pointers last
 };
+
+constexpr uint32_t kSkinnyVariant = 32;
+// LDS bytes of the skinny qmm kernels for a K split into `ksplit` chunks.
+size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat);
 
 enum ResolveStatus { kResolveOk = 0, kResolveUnknown = 1, kResolveMalformed = 2 };
 

@@ -65,6 +65,11 @@ struct smelt_hip_context {
     int weights_slot = -1;
     ActDType default_act = kActF16;
     uint32_t cache_seq_capacity = 0;
+    // split-K workspace shared by every launch on the stream: partial sums and arrival counters
+    // (counters are zero between launches; the last workgroup of each tile resets its own)
+    void* ws_partial = nullptr;
+    void* ws_counters = nullptr;
+    size_t ws_partial_bytes = 0, ws_counter_bytes = 0;
     size_t lds_limit = 65536;
     hipDeviceProp_t props;
     mutable std::string error;
@@ -263,7 +268,21 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
                 need[4] = batch * rows * 2; written[4] = true;
                 if (r.family == kFamAffineQmmAdd) { need[5] = batch * rows * 2; need[6] = batch * rows * 2; written[6] = true; }
             }
-            L.lds = qmm_affine_lds_bytes(r.family == kFamAffineQmmGateUp ? 2 : 1, r.lds_variant);
+            const uint32_t nmat = r.family == kFamAffineQmmGateUp ? 2 : 1;
+            if (r.lds_variant == kSkinnyVariant) {
+                const size_t tiles = (rows + 31) / 32;
+                if (bt > 32) return bad_geom("skinny qmm handles at most 32 tokens per pass");
+                if (L.grid[0] < tiles || L.grid[0] % tiles != 0)
+                    return bad_geom("skinny qmm needs grid width = row tiles (" + std::to_string(tiles) + ") * k-splits");
+                const uint32_t ksplit = (uint32_t)(L.grid[0] / tiles);
+                L.lds = qmm_skinny_lds_bytes((uint32_t)cols, ksplit, nmat);
+                if (ksplit > 1) {
+                    if ((size_t)L.grid[0] * gy * nmat * 4096 > ctx->ws_partial_bytes || tiles * gy * 4 > ctx->ws_counter_bytes)
+                        return bad_geom("split-K partials exceed the context workspace");
+                }
+                break;
+            }
+            L.lds = qmm_affine_lds_bytes(nmat, r.lds_variant);
             break;
         }
         case kFamTerAffMatvec:
@@ -566,6 +585,12 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             pos += 4;
         }
     }
+    if (p->res.workspace) {
+        pos = (pos + 7) & ~(size_t)7;
+        memcpy(kernarg + pos, &ctx->ws_partial, 8);
+        memcpy(kernarg + pos + 8, &ctx->ws_counters, 8);
+        pos += 16;
+    }
     size_t kernarg_size = pos;
     void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, kernarg, HIP_LAUNCH_PARAM_BUFFER_SIZE, &kernarg_size, HIP_LAUNCH_PARAM_END};
     if (!ctx->batch_open) {
@@ -611,6 +636,8 @@ int smelt_hip_context_create(int device_index, smelt_hip_context** out) {
     ctx->slots.resize(64);
     auto bail = [&](hipError_t err, const char* what) {
         int rc = hip_fail(nullptr, err, what);
+        if (ctx->ws_partial) (void)hipFree(ctx->ws_partial);
+        if (ctx->ws_counters) (void)hipFree(ctx->ws_counters);
         delete ctx;
         return rc;
     };
@@ -620,6 +647,11 @@ int smelt_hip_context_create(int device_index, smelt_hip_context** out) {
     if ((e = hipEventCreate(&ctx->ev_start)) != hipSuccess) return bail(e, "hipEventCreate");
     if ((e = hipEventCreate(&ctx->ev_end)) != hipSuccess) return bail(e, "hipEventCreate");
     ctx->lds_limit = ctx->props.sharedMemPerBlock ? ctx->props.sharedMemPerBlock : 65536;
+    ctx->ws_partial_bytes = (size_t)64 << 20;
+    ctx->ws_counter_bytes = (size_t)256 << 10;
+    if ((e = hipMalloc(&ctx->ws_partial, ctx->ws_partial_bytes)) != hipSuccess) return bail(e, "hipMalloc(workspace)");
+    if ((e = hipMalloc(&ctx->ws_counters, ctx->ws_counter_bytes)) != hipSuccess) return bail(e, "hipMalloc(workspace counters)");
+    if ((e = hipMemset(ctx->ws_counters, 0, ctx->ws_counter_bytes)) != hipSuccess) return bail(e, "hipMemset(workspace counters)");
     *out = ctx;
     return SMELT_HIP_OK;
 }
@@ -630,6 +662,8 @@ void smelt_hip_context_destroy(smelt_hip_context* ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     for (SlotBuffer& s : ctx->slots)
         if (s.ptr) (void)hipFree(s.ptr);
+    if (ctx->ws_partial) (void)hipFree(ctx->ws_partial);
+    if (ctx->ws_counters) (void)hipFree(ctx->ws_counters);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
