@@ -65,7 +65,7 @@ __host__ __device__ inline int skinny_chunk_windows(int cols, int ksplit) {
 __host__ __device__ inline int skinny_bias_blocks(int chunk_windows) { return (chunk_windows + 15) / 16 + 1; }
 __host__ __device__ inline size_t skinny_lds_bytes(int cols, int ksplit, int nmat) {
     const int cw = skinny_chunk_windows(cols, ksplit);
-    const size_t stage = (size_t)cw * 4096 + (size_t)skinny_bias_blocks(cw) * 2048;
+    const size_t stage = (size_t)cw * (4096 + 1024) + (size_t)skinny_bias_blocks(cw) * 2048;
     const size_t reduce = (size_t)4 * nmat * 4096;
     return stage > reduce ? stage : reduce;
 }
@@ -92,7 +92,8 @@ __device__ __forceinline__ void qmm_skinny_body(const uint8_t* const (&W)[NMAT],
     const int rs = cols / 2;
 
     uint4_t* xs = reinterpret_cast<uint4_t*>(smem);                       // [cw][4][2][32] x 16 B
-    uint4_t* xsum_hi = xs + (size_t)cw * 256;                              // [blocks][2][32] x 16 B
+    float* psum = reinterpret_cast<float*>(xs + (size_t)cw * 256);         // [cw][8][32] run sums
+    uint4_t* xsum_hi = reinterpret_cast<uint4_t*>(psum + (size_t)cw * 256);  // [blocks][2][32] x 16 B
     uint4_t* xsum_lo = xsum_hi + (size_t)skinny_bias_blocks(cw) * 64;
     float* red = reinterpret_cast<float*>(smem);                           // aliases the staging area
     const int blk0 = W0 / 16, blk1 = (W1 + 15) / 16;
@@ -125,36 +126,68 @@ __device__ __forceinline__ void qmm_skinny_body(const uint8_t* const (&W)[NMAT],
         const uint4_t z = {0u, 0u, 0u, 0u};
         (i < (blk1 - blk0) * 64 ? xsum_hi[i] : xsum_lo[i - (blk1 - blk0) * 64]) = z;
     }
-    __syncthreads();
-    for (int item = tid; item < (W1 - W0) * kSkTok; item += blockDim.x) {
-        const int wl = item / kSkTok, tok = item % kSkTok;
-        const int w = W0 + wl;
-        float xsum = 0.0f;
+    // One item = one run of 8 columns of one live token: a 16-byte load, converted to fp16 in
+    // operand order.  Items are taken four at a time with the loads issued first, so a thread
+    // pays one memory latency per four items.  Slots of tokens beyond the batch stay unwritten:
+    // they only feed output rows that are never stored.
+    {
+        int tshift = 0;
+        while ((1 << tshift) < ntok) ++tshift;
+        const int nitems = ntok > 0 ? ((W1 - W0) * 8) << tshift : 0;
+        for (int base = tid; base < nitems; base += 4 * blockDim.x) {
+            uint4_t v[4];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {  // run e of 8 columns belongs to lane half e / 4, MFMA e % 4
-            uint4_t v = {0u, 0u, 0u, 0u};
-            if (tok < ntok) v = *reinterpret_cast<const uint4_t*>(X + (size_t)(m0 + tok) * cols + (size_t)w * 64 + e * 8);
-            uint16_t h[8];
-            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                h[2 * q] = ActT::to_f16_bits((uint16_t)(d[q] & 0xFFFF));
-                h[2 * q + 1] = ActT::to_f16_bits((uint16_t)(d[q] >> 16));
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * blockDim.x;
+                const int tok = idx & ((1 << tshift) - 1), rest = idx >> tshift;
+                const int e = rest & 7, wl = rest >> 3;
+                v[u] = uint4_t{0u, 0u, 0u, 0u};
+                if (idx < nitems && tok < ntok)
+                    v[u] = *reinterpret_cast<const uint4_t*>(X + (size_t)(m0 + tok) * cols + (size_t)(W0 + wl) * 64 + e * 8);
             }
 #pragma unroll
-            for (int q = 0; q < 8; ++q) xsum += F16::widen(h[q]);
-            uint4_t o;
-            o.x = h[0] | ((uint32_t)h[4] << 16);
-            o.y = h[1] | ((uint32_t)h[5] << 16);
-            o.z = h[2] | ((uint32_t)h[6] << 16);
-            o.w = h[3] | ((uint32_t)h[7] << 16);
-            xs[((size_t)(wl * 4 + (e & 3)) * 2 + (e >> 2)) * 32 + tok] = o;
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * blockDim.x;
+                const int tok = idx & ((1 << tshift) - 1), rest = idx >> tshift;
+                const int e = rest & 7, wl = rest >> 3;  // run e belongs to lane half e / 4, MFMA e % 4
+                if (idx < nitems && tok < ntok) {
+                    uint16_t h[8];
+                    const uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        h[2 * q] = ActT::to_f16_bits((uint16_t)(d[q] & 0xFFFF));
+                        h[2 * q + 1] = ActT::to_f16_bits((uint16_t)(d[q] >> 16));
+                    }
+                    float run = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) run += F16::widen(h[q]);
+                    uint4_t o;
+                    o.x = h[0] | ((uint32_t)h[4] << 16);
+                    o.y = h[1] | ((uint32_t)h[5] << 16);
+                    o.z = h[2] | ((uint32_t)h[6] << 16);
+                    o.w = h[3] | ((uint32_t)h[7] << 16);
+                    xs[((size_t)(wl * 4 + (e & 3)) * 2 + (e >> 2)) * 32 + tok] = o;
+                    psum[(size_t)(wl * 8 + e) * 32 + tok] = run;
+                }
+            }
         }
-        const uint16_t hi = F16::narrow(xsum);
-        const uint16_t lo = F16::narrow(xsum - F16::widen(hi));
-        const size_t at = ((size_t)((w >> 4) - blk0) * 2 + ((w >> 3) & 1)) * 32 + tok;
-        reinterpret_cast<uint16_t*>(xsum_hi + at)[w & 7] = hi;
-        reinterpret_cast<uint16_t*>(xsum_lo + at)[w & 7] = lo;
+        __syncthreads();
+        // per-(token, window) activation sum: the eight run sums in column order, split into fp16
+        // high and low parts for the bias MFMA
+        for (int idx = tid; idx < ((W1 - W0) << tshift); idx += blockDim.x) {
+            const int tok = idx & ((1 << tshift) - 1), wl = idx >> tshift;
+            if (tok < ntok) {
+                float xsum = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) xsum += psum[(size_t)(wl * 8 + e) * 32 + tok];
+                const int w = W0 + wl;
+                const uint16_t hi = F16::narrow(xsum);
+                const uint16_t lo = F16::narrow(xsum - F16::widen(hi));
+                const size_t at = ((size_t)((w >> 4) - blk0) * 2 + ((w >> 3) & 1)) * 32 + tok;
+                reinterpret_cast<uint16_t*>(xsum_hi + at)[w & 7] = hi;
+                reinterpret_cast<uint16_t*>(xsum_lo + at)[w & 7] = lo;
+            }
+        }
     }
     __syncthreads();
 
@@ -256,29 +289,33 @@ __device__ __forceinline__ void qmm_skinny_body(const uint8_t* const (&W)[NMAT],
         // Workgroup partials meet in the workspace; the last to arrive adds them in chunk order.
         const size_t slot = (size_t)blockIdx.y * tiles + tile;
         float* mine = ws.partial + ((slot * ksplit + ks) * NMAT) * 1024;
+        // Partials are written and read with agent-scope relaxed atomics (coherent across the
+        // compute dies without cache write-backs); a workgroup's stores are complete before its
+        // arrival is counted, and the last arrival reads only after its count returned.
         if (tok < ntok) {
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m) {
-                float4_t o = {val[m][0], val[m][1], val[m][2], val[m][3]};
-                *reinterpret_cast<float4_t*>(mine + (size_t)m * 1024 + tok * kSkRows + r4) = o;
-            }
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    __hip_atomic_store(mine + (size_t)m * 1024 + tok * kSkRows + r4 + i, val[m][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __threadfence();
+        __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's stores are acknowledged
         __syncthreads();
         if (tid == 0) last_flag = atomicAdd(ws.counters + slot, 1u) == (uint32_t)(ksplit - 1) ? 1u : 0u;
         __syncthreads();
         if (!last_flag) return;
-        __threadfence();
         if (tok < ntok) {
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) {
-                float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+                float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
                 for (int c = 0; c < ksplit; ++c) {
-                    const float4_t p = *reinterpret_cast<const float4_t*>(
-                        ws.partial + ((slot * ksplit + c) * NMAT + m) * 1024 + tok * kSkRows + r4);
-                    sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+                    const float* theirs = ws.partial + ((slot * ksplit + c) * NMAT + m) * 1024 + tok * kSkRows + r4;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        sum[i] += __hip_atomic_load(theirs + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
-                val[m][0] = sum.x; val[m][1] = sum.y; val[m][2] = sum.z; val[m][3] = sum.w;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) val[m][i] = sum[i];
             }
         }
         if (tid == 0) ws.counters[slot] = 0u;  // ready for the next launch on this stream

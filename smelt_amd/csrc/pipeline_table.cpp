@@ -92,10 +92,10 @@ size_t qmm_affine_lds_bytes(uint32_t nmat, uint32_t mt) {
 }
 
 size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat) {
-    // staged activations: 4 KB per 64-column window of a chunk, plus fp16 high/low activation sums
+    // staged activations: 4 KB (+1 KB of run sums) per 64-column window of a chunk, plus fp16 high/low activation sums
     // in blocks of 16 groups; the wave reduction (4 waves x nmat x 4 KB) reuses the same bytes
     const size_t nwin = cols / 64, cw = (nwin + ksplit - 1) / ksplit;
-    const size_t stage = cw * 4096 + ((cw + 15) / 16 + 1) * 2048;
+    const size_t stage = cw * (4096 + 1024) + ((cw + 15) / 16 + 1) * 2048;
     const size_t reduce = (size_t)4 * nmat * 4096;
     return stage > reduce ? stage : reduce;
 }
