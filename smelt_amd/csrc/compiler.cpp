@@ -397,11 +397,18 @@ int smelt_route_prefill_affine(int rows, int cols, int group, int fusion, int ma
         return SMELT_HIP_OK;
     }
     if (max_batch <= 32 && group == 64 && cols % 512 == 0) {
-        // skinny MFMA qmm: 32-row tiles, K split over enough workgroups to keep the whole matrix
-        // in flight (about ten 64-column windows per workgroup, at least three workgroups per CU)
+        // skinny MFMA qmm: 32-row tiles.  K is split over as few workgroups as keep the staged
+        // activations of a chunk within ~96 KB of LDS and give every CU a workgroup; each extra
+        // split costs a round trip through the split-K workspace.
         const int nwin = cols / 64, tiles = (rows + 31) / 32;
-        int ksplit = std::max(1, nwin / 10);
-        while (tiles * ksplit < 3 * std::max(1, compute_units) && (nwin + ksplit) / (ksplit + 1) >= 4) ++ksplit;
+        int tpad = 1;
+        while (tpad < max_batch) tpad *= 2;
+        const int nmat = fusion == SMELT_FUSION_GATE_UP_SWIGLU ? 2 : 1;
+        auto lds = [&](int ks) { return qmm_skinny_lds_bytes((uint32_t)cols, (uint32_t)ks, (uint32_t)nmat, (uint32_t)tpad, 4); };
+        int ksplit = 1;
+        while (ksplit < nwin && lds(ksplit) > (size_t)96 * 1024) ++ksplit;
+        const int want = (std::max(1, compute_units) + tiles / 2) / tiles;
+        while (ksplit < want && (nwin + ksplit) / (ksplit + 1) >= 8) ++ksplit;
         set_route(out, base + "_batched_skinny", true, 32, 32, 256, tiles * ksplit);
         return SMELT_HIP_OK;
     }

@@ -91,12 +91,16 @@ size_t qmm_affine_lds_bytes(uint32_t nmat, uint32_t mt) {
     return (size_t)nmat * (64 * 80 + 2 * 4 * 64 * 4) + (size_t)mt * (16 * (128 + 8) * 2 + 16 * 4 * 4);
 }
 
-size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat) {
-    // staged activations: 4 KB (+1 KB of run sums) per 64-column window of a chunk, plus fp16 high/low activation sums
-    // in blocks of 16 groups; the wave reduction (4 waves x nmat x 4 KB) reuses the same bytes
+size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat, uint32_t live_tokens, uint32_t waves) {
+    // staged activations: per 64-column window of a chunk, 8 operand rows of (tokens + 1) 16-byte
+    // slots and 8 rows of (tokens + 1) run sums (live tokens rounded up to a power of two), plus
+    // fp16 high/low activation sums in blocks of 16 groups; the wave reduction
+    // (waves x nmat x 4 KB) reuses the same bytes
+    uint32_t shift = 0;
+    while ((1u << shift) < live_tokens) ++shift;
     const size_t nwin = cols / 64, cw = (nwin + ksplit - 1) / ksplit;
-    const size_t stage = cw * (4096 + 1024) + ((cw + 15) / 16 + 1) * 2048;
-    const size_t reduce = (size_t)4 * nmat * 4096;
+    const size_t stage = cw * 8 * ((1u << shift) + 1) * 20 + ((cw + 15) / 16 + 1) * 2048;
+    const size_t reduce = (size_t)waves * nmat * 4096;
     return stage > reduce ? stage : reduce;
 }
 

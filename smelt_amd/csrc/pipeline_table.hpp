@@ -60,7 +60,7 @@ struct ResolvedPipeline {
 
 constexpr uint32_t kSkinnyVariant = 32;
 // LDS bytes of the skinny qmm kernels for a K split into `ksplit` chunks.
-size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat);
+size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat, uint32_t live_tokens, uint32_t waves);
 
 enum ResolveStatus { kResolveOk = 0, kResolveUnknown = 1, kResolveMalformed = 2 };
 

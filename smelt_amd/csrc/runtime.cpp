@@ -123,8 +123,10 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
     };
     const bool matvec_like = r.family <= kFamAffineBank4;
+    const bool skinny = r.lds_variant == kSkinnyVariant &&
+                        (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
     if (matvec_like) {
-        if (L.block[0] % 64 != 0 || L.block[0] == 0 || L.block[0] > 256 || L.block[1] != 1 || L.block[2] != 1)
+        if (L.block[0] % 64 != 0 || L.block[0] == 0 || (L.block[0] > 256 && !skinny) || L.block[1] != 1 || L.block[2] != 1)
             return bad_geom("threadgroup must be 64..256 threads in whole wavefronts, got " +
                             std::to_string(L.block[0]) + "x" + std::to_string(L.block[1]) + "x" + std::to_string(L.block[2]));
         if (L.grid[2] != 1) return bad_geom("grid depth must be 1");
@@ -253,7 +255,13 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
         case kFamAffineQmm:
         case kFamAffineQmmAdd:
         case kFamAffineQmmGateUp: {
-            if (int e = need_256()) return e;
+            if (skinny) {
+                const uint32_t max_threads = 512;
+                if (L.block[0] < 256 || L.block[0] % 64 != 0 || L.block[0] > max_threads || L.block[1] != 1 || L.block[2] != 1)
+                    return bad_geom("skinny qmm runs with 256.." + std::to_string(max_threads) + " threads in whole waves, got " + std::to_string(L.block[0]));
+            } else if (int e = need_256()) {
+                return e;
+            }
             const size_t o = r.family == kFamAffineQmm ? 5 : (r.family == kFamAffineQmmAdd ? 7 : 8);
             const size_t batch = U(o), rows = U(o + 1), cols = U(o + 2), group = U(o + 3), bt = U(o + 4);
             if (int e = check_affine_shape(rows, cols, group)) return e;
@@ -275,7 +283,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
                 if (L.grid[0] < tiles || L.grid[0] % tiles != 0)
                     return bad_geom("skinny qmm needs grid width = row tiles (" + std::to_string(tiles) + ") * k-splits");
                 const uint32_t ksplit = (uint32_t)(L.grid[0] / tiles);
-                L.lds = qmm_skinny_lds_bytes((uint32_t)cols, ksplit, nmat);
+                L.lds = qmm_skinny_lds_bytes((uint32_t)cols, ksplit, nmat, (uint32_t)std::min(batch, bt), L.block[0] / 64);
                 if (ksplit > 1) {
                     if ((size_t)L.grid[0] * gy * nmat * 4096 > ctx->ws_partial_bytes || tiles * gy * 4 > ctx->ws_counter_bytes)
                         return bad_geom("split-K partials exceed the context workspace");

@@ -96,9 +96,9 @@ def test_shape_routes():
     with pytest.raises(ValueError):
         cc.route_decode_affine(64, 1000, 64)                    # cols not a multiple of 32
     r = cc.route_prefill_affine(9216, 2560, 64, max_batch=8)     # 5..32 tokens, g64: split-K skinny MFMA kernel
-    assert r.pipeline == b"affine_matvec_c2560_r9216_g64_batched_skinny" and (r.batch_tile, r.grid_w) == (32, 288 * 4)
+    assert r.pipeline == b"affine_matvec_c2560_r9216_g64_batched_skinny" and (r.batch_tile, r.grid_w) == (32, 288)
     r = cc.route_prefill_affine(2560, 9216, 64, max_batch=32)
-    assert r.pipeline == b"affine_matvec_c9216_r2560_g64_batched_skinny" and r.grid_w % 80 == 0 and r.grid_w >= 768
+    assert r.pipeline == b"affine_matvec_c9216_r2560_g64_batched_skinny" and r.grid_w % 80 == 0 and r.grid_w >= 240
     r = cc.route_prefill_affine(9216, 2560, 128, max_batch=8)    # other group sizes keep the slab kernel
     assert r.pipeline == b"affine_matvec_c2560_r9216_g128_batched_full" and (r.batch_tile, r.grid_w) == (16, 144)
     r = cc.route_prefill_affine(9216, 2560, 64, max_batch=512)

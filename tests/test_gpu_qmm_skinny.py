@@ -20,7 +20,7 @@ def ctx():
     c.close()
 
 
-def skinny(ctx, w, x_bits, dtype, rows, cols, ksplit, group=64, bt=32):
+def skinny(ctx, w, x_bits, dtype, rows, cols, ksplit, group=64, bt=32, threads=256):
     batch = x_bits.shape[0]
     wf = gh.WeightFile()
     offs = [wf.add(a) for a in w]
@@ -30,7 +30,7 @@ def skinny(ctx, w, x_bits, dtype, rows, cols, ksplit, group=64, bt=32):
     pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g{group}_batched_skinny" + gh.t_suffix(dtype))
     bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
     tiles = (rows + 31) // 32
-    rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], (tiles * ksplit, bt, 1), (256, 1, 1),
+    rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], (tiles * ksplit, bt, 1), (threads, 1, 1),
                          grid_kinds=(0, rt.GRID_SEQ_LEN_CEIL_DIV, 0))
     assert ctx.encode_prefill(rec, seq_len=batch) == 1
     ctx.wait()
@@ -51,19 +51,19 @@ def test_skinny_qmm_4b_shapes(ctx, dtype, batch):
 
 
 def test_skinny_qmm_every_split_is_the_same_sum_within_tolerance(ctx):
-    """K = 1536 (24 windows) split 1, 2, 3, 5, 7 and 24 ways (uneven chunks, one-window chunks, waves
-    with no window): all within tolerance of the oracle, and a repeated launch is bit-identical
-    (fixed summation order, counters back at zero)."""
+    """K = 1536 (24 windows) split 1, 2, 3, 5, 7 and 24 ways over workgroups of 4 to 8 waves (uneven
+    chunks, one-window chunks, waves with no window): all within tolerance of the oracle, and a
+    repeated launch is bit-identical (fixed summation order, counters back at zero)."""
     dtype = fx.BF16
     rows, cols, batch = 100, 1536, 13        # 100 rows: the last tile has 4 live rows
     w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=11)
     x = fx.synth_activation(batch, cols, dtype, config=4, tensor=113, outlier_frac=0.01)
     ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
-    for ksplit in (1, 2, 3, 5, 7, 24):
-        y = skinny(ctx, w, x, dtype, rows, cols, ksplit)
-        gh.check_outputs(y, ref, dtype, f"skinny qmm ksplit={ksplit}")
-        again = skinny(ctx, w, x, dtype, rows, cols, ksplit)
-        assert np.array_equal(y, again), ksplit
+    for ksplit, threads in ((1, 256), (1, 512), (2, 512), (3, 256), (5, 448), (7, 320), (24, 256)):
+        y = skinny(ctx, w, x, dtype, rows, cols, ksplit, threads=threads)
+        gh.check_outputs(y, ref, dtype, f"skinny qmm ksplit={ksplit} threads={threads}")
+        again = skinny(ctx, w, x, dtype, rows, cols, ksplit, threads=threads)
+        assert np.array_equal(y, again), (ksplit, threads)
 
 
 def test_skinny_qmm_long_rows_and_token_blocks(ctx):
@@ -76,6 +76,8 @@ def test_skinny_qmm_long_rows_and_token_blocks(ctx):
     ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
     y = skinny(ctx, w, x, dtype, rows, cols, ksplit=12)
     gh.check_outputs(y, ref, dtype, "skinny qmm K=9216 M=40")
+    y = skinny(ctx, w, x, dtype, rows, cols, ksplit=6, threads=512)
+    gh.check_outputs(y, ref, dtype, "skinny qmm K=9216 M=40, 8 waves")
     y16 = skinny(ctx, w, x, dtype, rows, cols, ksplit=12, bt=16)
     gh.check_outputs(y16, ref, dtype, "skinny qmm K=9216 M=40 bt=16")
 
@@ -117,7 +119,7 @@ def test_skinny_qmm_fused_add_and_gate_up(ctx):
     assert np.array_equal(out, so.narrow(fx.from_bits(plain, dtype) + fx.from_bits(res, dtype), dtype))
     pipe = ctx.pipeline(f"fused_affine_gate_up_swiglu_c{cols}_r{rows}_g64_batched_skinny@bf16")
     bufs = [(0, i, offs[i]) for i in range(6)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
-    rec = rt.make_record(pipe, bufs, [(8, batch)], (tiles * ksplit, 1, 1), (256, 1, 1))
+    rec = rt.make_record(pipe, bufs, [(8, batch)], (tiles * ksplit, 1, 1), (512, 1, 1))
     assert ctx.encode_prefill(rec, seq_len=batch) == 1
     ctx.wait()
     y = ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
@@ -140,6 +142,9 @@ def test_skinny_qmm_rejects_bad_launches(ctx):
     pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g64_batched_skinny")
     bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
     bad = rt.make_record(pipe, bufs, [(5, 4)], (3, 1, 1), (256, 1, 1))       # 3 is not a multiple of 2 tiles
+    with pytest.raises(rt.SmeltHipError):
+        ctx.encode_prefill(bad, seq_len=4)
+    bad = rt.make_record(pipe, bufs, [(5, 4)], (2, 1, 1), (128, 1, 1))       # fewer than four waves
     with pytest.raises(rt.SmeltHipError):
         ctx.encode_prefill(bad, seq_len=4)
     with pytest.raises(rt.SmeltHipError):                                    # group 128 has no skinny kernel
