@@ -1,0 +1,77 @@
+// __global__ entry points of the matrix-core matvec.  Argument lists are those of the vector-ALU
+// kernels of the same pipelines followed by `kw`, the number of waves that share one row tile.
+#pragma once
+#include "matvec_kernels.hpp"
+#include "mfma_matvec.hpp"
+
+#define SMELT_AFFINE_MM_KERNELS(T, ACT, SC)                                                       \
+    SMELT_KERNEL void smelt_affine_mm_matvec_##T(const u8* W, const u16* S, const u16* B,         \
+                                                 const u16* x, u16* y, u32 rows, u32 cols,        \
+                                                 u32 group, u32 kw) {                             \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, y, (int)rows};                                                      \
+        mfma_matvec_body<MvU4, ACT, SC, 1>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+                                           blockIdx.y + 1, epi);                                  \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_mm_matvec_add_##T(const u8* W, const u16* S, const u16* B,     \
+                                                     const u16* x, u16* y, const u16* res,        \
+                                                     u32 rows, u32 cols, u32 group, u32 kw) {     \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiAdd<ACT> epi{{}, y, res, (int)rows};                                                   \
+        mfma_matvec_body<MvU4, ACT, SC, 1>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+                                           blockIdx.y + 1, epi);                                  \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_##T(                                         \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* x, u16* y, u32 rows, u32 cols, u32 group, u32 kw) {                            \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiAffineSwiglu<ACT> epi{{}, y, (int)rows};                                               \
+        mfma_matvec_body<MvU4, ACT, SC, 2>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+                                           blockIdx.y + 1, epi);                                  \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_mm_matvec_batched_##T(                                         \
+        const u8* W, const u16* S, const u16* B, const u16* X, u16* Y, u32 batch, u32 rows,       \
+        u32 cols, u32 group, u32 batch_tile, u32 kw) {                                            \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        mfma_matvec_body<MvU4, ACT, SC, 1>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_batched_##T(                                 \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* X, u16* Y, u32 batch, u32 rows, u32 cols, u32 group, u32 batch_tile,           \
+        u32 kw) {                                                                                 \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiAffineSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        mfma_matvec_body<MvU4, ACT, SC, 2>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_mm_matvec_argmax_##T(                                          \
+        const u8* W, const u16* S, const u16* B, const u16* X, smelt::uint2_t* keys, u32 batch,   \
+        float logit_cap, u32 rows, u32 cols, u32 group, u32 batch_tile, u32 kw) {                 \
+        using namespace smelt;                                                                    \
+        __shared__ uint2_t wave_keys[4];                                                          \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        uint2_t best = {0u, 0u};                                                                  \
+        EpiArgmax<ACT> epi{keys, logit_cap, &best, wave_keys};                                    \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        /* one key per token and workgroup: tokens take their own pass over the rows */           \
+        for (u32 b = lo; b < hi; ++b) {                                                           \
+            if (b != lo) __syncthreads();                                                         \
+            mfma_matvec_body<MvU4, ACT, SC, 1>(mats, X, rows, cols, cols / 2, kw, b, b + 1, epi); \
+        }                                                                                         \
+    }
+
+SMELT_AFFINE_MM_KERNELS(f16, smelt::F16, smelt::F16)
+SMELT_AFFINE_MM_KERNELS(bf16, smelt::BF16, smelt::BF16)

@@ -1,6 +1,7 @@
 // Single translation unit for the gfx950 code object (smelt_kernels.hsaco).
 // Built with:  hipcc --offload-arch=gfx950 --genco -O3 -Xclang -target-feature -Xclang -packed-fp32-ops
 #include "matvec_kernels.hpp"
+#include "mfma_matvec_kernels.hpp"
 #include "misc_kernels.hpp"
 #include "qmm.hpp"
 #include "qmm_skinny.hpp"

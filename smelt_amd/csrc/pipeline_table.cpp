@@ -104,6 +104,31 @@ size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat, uint3
     return stage > reduce ? stage : reduce;
 }
 
+size_t mfma_matvec_lds_bytes(CodeLayout layout, uint32_t cols, uint32_t tokens, uint32_t nmat, uint32_t waves, uint32_t kw) {
+    // operand fragments [windows][8 * MFMAs per dword][tokens] x 16 B (tokens rounded up to a power
+    // of two, at most 8), one zero slot, per-window corrections (and activation sums for affine)
+    // for 8 token slots, and wave partials when K is split over waves
+    const uint32_t window = layout == kCodesU4 ? 64 : 128, frags = layout == kCodesU4 ? 8 : 16;
+    uint32_t shift = 0;
+    while ((1u << shift) < tokens && shift < 3) ++shift;
+    const size_t nwin = cols / window;
+    size_t bytes = ((nwin * frags * 16) << shift) + 16 + nwin * 32 * (layout == kCodesU4 ? 2 : 1);
+    if (kw > 1) bytes += (size_t)waves * nmat * 1024;
+    return bytes;
+}
+
+uint32_t mfma_matvec_kw(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t tokens, uint32_t nmat, size_t lds_limit) {
+    // Matrices that stream from HBM (8M weights and up) with one scale group per window and whole
+    // batches of four windows per row; smaller ones are latency-bound and stay on the vector ALU.
+    const uint32_t window = layout == kCodesU4 ? 64 : 128;
+    if (layout != kCodesU4 && layout != kCodesTernary2) return 0;
+    if (group != window || cols % (4 * window) != 0 || (uint64_t)rows * cols < (8u << 20)) return 0;
+    const uint32_t tiles = (rows + 31) / 32;
+    const uint32_t kw = tiles >= 2048 ? 1 : (tiles >= 1024 ? 2 : 4);
+    if (mfma_matvec_lds_bytes(layout, cols, tokens, nmat, 4, kw) > lds_limit) return 0;
+    return kw;
+}
+
 uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
     const uint32_t padded = (cols + 127u) / 128u * 128u;
     switch (f) {
@@ -196,6 +221,12 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->symbol = "smelt_affine_matvec_argmax_" + t;
             out->kinds = "PPPPPUFUUUU";
             out->appended = {rows, cols, group, bt};
+            if (const uint32_t kw = mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 1, lds_limit)) {
+                out->mfma_kw = kw;
+                out->symbol = "smelt_affine_mm_matvec_argmax_" + t;
+                out->kinds += "U";
+                out->appended.push_back(kw);
+            }
             return kResolveOk;
         }
         if (m1) {
@@ -208,6 +239,14 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                 default: break;
             }
             out->appended = {rows, cols, group};
+            const uint32_t nmat = a.m1 == kFamAffineGateUp ? 2 : 1;
+            if (a.m1 != kFamAffineDual)
+                if (const uint32_t kw = mfma_matvec_kw(kCodesU4, rows, cols, group, 1, nmat, lds_limit)) {
+                    out->mfma_kw = kw;
+                    out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_" : (a.m1 == kFamAffineAdd ? "smelt_affine_mm_matvec_add_" : "smelt_affine_mm_gate_up_swiglu_")) + t;
+                    out->kinds += "U";
+                    out->appended.push_back(kw);
+                }
             return kResolveOk;
         }
         if (full && skinny) {
@@ -239,6 +278,12 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         else if (a.m1 == kFamAffineGateUp) { out->family = kFamAffineGateUpBatched; out->symbol = "smelt_affine_gate_up_swiglu_batched_" + mbs; out->kinds = "PPPPPPPPUUUUU"; }
         else { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
         out->appended = {rows, cols, group, bt};
+        if (const uint32_t kw = mfma_matvec_kw(kCodesU4, rows, cols, group, std::min(bt, 8u), a.m1 == kFamAffineGateUp ? 2 : 1, lds_limit)) {
+            out->mfma_kw = kw;
+            out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_batched_" : "smelt_affine_mm_gate_up_swiglu_batched_") + t;
+            out->kinds += "U";
+            out->appended.push_back(kw);
+        }
         return kResolveOk;
     }
 

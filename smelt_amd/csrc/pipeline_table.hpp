@@ -55,6 +55,7 @@ struct ResolvedPipeline {
     uint32_t lds_variant = 0;        // batched matvec: activation rows resident per pass (1, 2, 4);
                                      // qmm: 16-token blocks per workgroup tile (1, 2, 4),
                                      // or kSkinnyVariant for the split-K skinny kernels
+    uint32_t mfma_kw = 0;            // > 0: matrix-core matvec variant, waves that share a row tile
     bool workspace = false;          // kernel takes the context's (partials, counters) pointers last
 };
 
@@ -71,6 +72,11 @@ ResolveStatus resolve_pipeline(const std::string& entry, ActDType default_act, s
 // Packed-code layouts the matvec kernels consume.
 enum CodeLayout { kCodesU4 = 0, kCodesBinary1 = 1, kCodesTernary2 = 2, kCodesTrit5 = 3 };
 CodeLayout code_layout(SignedFormat f);
+
+// LDS bytes of the matrix-core matvec kernels (affine u4, 64-column windows).
+size_t mfma_matvec_lds_bytes(CodeLayout layout, uint32_t cols, uint32_t tokens, uint32_t nmat, uint32_t waves, uint32_t kw);
+// waves per row tile the matrix-core matvec uses for a shape; 0 when the shape stays on the vector-ALU kernels
+uint32_t mfma_matvec_kw(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t tokens, uint32_t nmat, size_t lds_limit);
 
 // LDS bytes the matvec kernels need for one packed row stride with `mb` resident activation rows.
 size_t matvec_lds_bytes(CodeLayout layout, uint32_t row_stride_bytes, uint32_t mb);

@@ -158,6 +158,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
         if (L.block[0] != 256) return bad_geom("MFMA qmm kernels run with 256-thread workgroups, got " + std::to_string(L.block[0]));
         return 0;
     };
+    size_t mm_cols = 0, mm_tokens = 1, mm_nmat = 1;  // matrix-core matvec variants: LDS is sized after the switch
     switch (r.family) {
         case kFamAffineMatvec:
         case kFamAffineAdd: {
@@ -169,6 +170,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[4] = gy * rows * 2; written[4] = true;
             if (r.family == kFamAffineAdd) need[5] = gy * rows * 2;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            mm_cols = cols;
             break;
         }
         case kFamAffineGateUp:
@@ -182,6 +184,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[7] = gy * rows * 2; written[7] = true;
             if (r.family == kFamAffineDual) { need[8] = gy * rows * 2; written[8] = true; }
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            mm_cols = cols; mm_nmat = 2;
             break;
         }
         case kFamAffineBatched:
@@ -196,6 +199,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[xi] = batch * cols * 2; align[xi] = 16;
             need[yi] = batch * rows * 2; written[yi] = true;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), r.lds_variant);
+            mm_cols = cols; mm_tokens = std::min<size_t>(8, std::min(batch, bt)); mm_nmat = r.family == kFamAffineGateUpBatched ? 2 : 1;
             break;
         }
         case kFamSignedMatvec:
@@ -243,6 +247,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[3] = batch * cols * 2; align[3] = 16;
             need[4] = batch * (size_t)L.grid[0] * 8; align[4] = 8; written[4] = true;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            mm_cols = cols;  // one token per pass
             break;
         }
         case kFamLmHeadReduce: {
@@ -387,6 +392,10 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
         }
         default:
             return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "pipeline '" + p.entry + "' has no launch validator");
+    }
+    if (r.mfma_kw > 0) {
+        if (L.block[0] != 256) return bad_geom("matrix-core matvec kernels run with 256-thread workgroups, got " + std::to_string(L.block[0]));
+        L.lds = mfma_matvec_lds_bytes(layout, (uint32_t)mm_cols, (uint32_t)std::max<size_t>(mm_tokens, 1), (uint32_t)mm_nmat, 4, r.mfma_kw);
     }
     if (L.lds > ctx->lds_limit)
         return bad_geom("needs " + std::to_string(L.lds) + " bytes of LDS, device allows " + std::to_string(ctx->lds_limit));

@@ -1,0 +1,102 @@
+"""GPU parity: the matrix-core matvec variants the pipeline table selects for matrices of 8M weights
+and more (affine u4 g64): every K-split (1, 2, 4 waves per row tile), ragged row tiles, 1..8 and
+more than 8 tokens, the fused epilogues, and agreement with the vector-ALU kernels."""
+import numpy as np
+import pytest
+
+import fixtures as fx
+import gpu_harness as gh
+from oracle import oracle as so
+from smelt_amd import compiler as cc
+from smelt_amd import runtime as rt
+from test_gpu_matvec import run_affine
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = rt.Context()
+    yield c
+    c.close()
+
+
+def mm_symbol(entry):
+    rc, sym, kinds = cc.resolve_pipeline_name(entry)
+    assert rc == 0, entry
+    return sym
+
+
+# rows chosen so that the row-tile count selects 4, 2 and 1 waves per tile; none is a multiple of 32
+SHAPES = [(8200, 1024, 4), (33000, 256, 2), (70001, 256, 1), (5000, 2560, 4)]
+
+
+@pytest.mark.parametrize("rows,cols,kw", SHAPES)
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_mfma_matvec_matches_oracle(ctx, rows, cols, kw, dtype):
+    entry = f"affine_matvec_c{cols}_r{rows}_g64"
+    assert mm_symbol(entry) == "smelt_affine_mm_matvec_f16"
+    w = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=60 + kw)
+    x = fx.synth_activation(1, cols, dtype, config=1, tensor=61, outlier_frac=0.01)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
+    y = run_affine(ctx, *w, x, dtype, entry, grid=1024)
+    worst = gh.check_outputs(y, ref, dtype, f"mfma matvec {rows}x{cols}")
+    print(f"\n  mfma matvec {rows}x{cols} kw={kw} dtype={dtype}: max rel err {worst:.2e}")
+    # any grid covers every row; the generic entry runs the vector-ALU kernel on the same bytes
+    y_small = run_affine(ctx, *w, x, dtype, entry, grid=7)
+    assert np.array_equal(y, y_small)
+    y_valu = run_affine(ctx, *w, x, dtype, f"affine_matvec:{cols}:64", generic=True)
+    gh.check_outputs(y_valu, ref, dtype, "vector-ALU matvec")
+
+
+@pytest.mark.parametrize("batch,tile,suffix", [(1, 8, "_batched"), (3, 3, "_batched_tile3"), (8, 8, "_batched"),
+                                               (11, 8, "_batched"), (13, 4, "_batched_tile4")])
+def test_mfma_small_batch(ctx, batch, tile, suffix):
+    rows, cols = 8300, 1024
+    dtype = fx.BF16
+    entry = f"affine_matvec_c{cols}_r{rows}_g64{suffix}"
+    assert mm_symbol(entry + "@bf16") == "smelt_affine_mm_matvec_batched_bf16"
+    w = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=70)
+    x = fx.synth_activation(batch, cols, dtype, config=1, tensor=71 + batch, outlier_frac=0.01)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
+    y = run_affine(ctx, *w, x, dtype, entry, batched=True, batch_tile=tile)
+    gh.check_outputs(y, ref, dtype, f"mfma batched M={batch}")
+    # per-token results do not depend on the batch they ride in
+    y1 = run_affine(ctx, *w, x[batch - 1:batch], dtype, f"affine_matvec_c{cols}_r{rows}_g64")
+    assert np.array_equal(y[batch - 1], y1[0])
+
+
+def test_mfma_fused_add_and_gate_up(ctx):
+    rows, cols = 8192, 1024
+    dtype = fx.F16
+    gw = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=80)
+    uw = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=81)
+    x = fx.synth_activation(1, cols, dtype, config=1, tensor=82)
+    res = fx.to_bits(fx.rng_for(1, 83).normal(0, 1, (1, rows)).astype(np.float32), dtype)
+    assert mm_symbol(f"fused_affine_matvec_add_c{cols}_r{rows}_g64") == "smelt_affine_mm_matvec_add_f16"
+    y = run_affine(ctx, *gw, x, dtype, f"affine_matvec_c{cols}_r{rows}_g64")
+    fused = run_affine(ctx, *gw, x, dtype, f"fused_affine_matvec_add_c{cols}_r{rows}_g64", residual=res)
+    assert np.array_equal(fused, so.narrow(fx.from_bits(y, dtype) + fx.from_bits(res, dtype), dtype))
+    entry = f"fused_affine_gate_up_swiglu_c{cols}_r{rows}_g64"
+    assert mm_symbol(entry) == "smelt_affine_mm_gate_up_swiglu_f16"
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*gw, *uw)]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(gh.X_SLOT, x)
+    ctx.alloc(gh.Y_SLOT, rows * 2)
+    bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
+    ctx.encode_decode(rt.make_record(ctx.pipeline(entry), bufs, [], (256, 1, 1), (256, 1, 1)))
+    ctx.wait()
+    got = ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+    xf = fx.from_bits(x, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, 64, dtype)
+    u = so.affine_matvec(*uw, xf, rows, cols, 64, dtype)
+    ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, so.F16), fx.F16)
+    gh.check_outputs(got, ref, dtype, "mfma gate_up_swiglu", rel_tol=4e-3)
+
+
+def test_small_and_odd_shapes_stay_on_the_vector_alu():
+    assert mm_symbol("affine_matvec_c1024_r3584_g64") == "smelt_affine_matvec_f16"          # under 8M weights
+    assert mm_symbol("affine_matvec_c1024_r16384_g128") == "smelt_affine_matvec_f16"        # group != window
+    assert mm_symbol("affine_matvec_c1088_r16384_g64") == "smelt_affine_matvec_f16"         # cols % 256 != 0
+    assert mm_symbol("affine_matvec_c1024_r151936_g64@bf16") == "smelt_affine_mm_matvec_bf16"
