@@ -366,15 +366,26 @@ struct EpiArgmax {
     uint2_t* partials;
     float logit_cap;
     uint2_t* best;      // one per thread (register-resident in the caller)
+    float* best_raw;    // unrounded sum of the row that holds `best`; NaN while there is none
     uint2_t* lds_keys;  // blockDim.x / 64 entries
+    // A thread sees its rows in increasing order, and capping and rounding are monotonic, so a row
+    // whose raw sum does not exceed the raw sum of the current best can at most tie with it and
+    // lose on the index.  Only rows that pass this one comparison (and NaNs) form a key.
     __device__ __forceinline__ void operator()(int, int row, const float* v) const {
         float x = v[0];
-        if (logit_cap > 0.0f) {
-            // cap * tanh(x / cap) as cap * (1 - 2 / (1 + exp(2x / cap))); exp overflow gives +-cap
-            const float e = expf(2.0f * x / logit_cap);
-            x = logit_cap * (1.0f - 2.0f / (1.0f + e));
+        if (!(x <= *best_raw)) {
+            const float raw = x;
+            if (logit_cap > 0.0f) {
+                // cap * tanh(x / cap) as cap * (1 - 2 / (1 + exp(2x / cap))); exp overflow gives +-cap
+                const float e = expf(2.0f * x / logit_cap);
+                x = logit_cap * (1.0f - 2.0f / (1.0f + e));
+            }
+            const uint2_t key = argmax_pack_key(ActT::narrow(x), (uint32_t)row);
+            if (argmax_key_gt(key, *best)) {
+                *best = key;
+                *best_raw = raw;  // a NaN keeps every later row on this path, where keys decide
+            }
         }
-        *best = argmax_key_max(*best, argmax_pack_key(ActT::narrow(x), (uint32_t)row));
     }
     __device__ __forceinline__ void end_chunk(int b0, int) const {
         const uint2_t k = wave_argmax_key(*best);
@@ -388,6 +399,7 @@ struct EpiArgmax {
             partials[(size_t)b0 * gridDim.x + blockIdx.x] = b;
         }
         *best = uint2_t{0u, 0u};
+        *best_raw = __builtin_nanf("");
     }
 };
 
@@ -415,15 +427,43 @@ struct EpiBank4 : EpiBase {
         float logit_cap, u32 rows, u32 cols, u32 group, u32 batch_tile) {                         \
         using namespace smelt;                                                                    \
         __shared__ uint2_t wave_keys[4];                                                          \
-        const MatPtrs mats[1] = {{W, S, B}};                                                      \
         uint2_t best = {0u, 0u};                                                                  \
-        EpiArgmax<ACT> epi{keys, logit_cap, &best, wave_keys};                                    \
+        float best_raw = __builtin_nanf("");                                                      \
+        EpiArgmax<ACT> epi{keys, logit_cap, &best, &best_raw, wave_keys};                                    \
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        /* One key per token and workgroup: tokens take their own pass over the rows.  The        \
+           arguments are re-read as opaque values in every pass: otherwise everything derived     \
+           from them is hoisted out of the token loop and kept live, which halves the occupancy. */ \
+        for (u32 b = lo; b < hi; ++b) {                                                           \
+            if (b != lo) __syncthreads();                                                         \
+            const u8* w2 = W;                                                                     \
+            const u16 *s2 = S, *b2 = B, *x2 = X;                                                  \
+            u32 r2 = rows, c2 = cols, g2 = group;                                                 \
+            asm volatile("" : "+s"(w2), "+s"(s2), "+s"(b2), "+s"(x2), "+s"(r2), "+s"(c2), "+s"(g2)); \
+            const MatPtrs mats[1] = {{w2, s2, b2}};                                               \
+            matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x2, r2, c2,                                \
+                                                 packed_row_stride<FmtU4>(c2, g2), g2, b, b + 1,  \
+                                                 epi);                                            \
+        }                                                                                         \
+    }
+
+// Decode form of the fused argmax: exactly one token (batch == 1, one grid row), so no token loop
+// and the register footprint of the plain matvec.
+#define SMELT_AFFINE_ARGMAX_SINGLE(T, ACT, SC)                                                    \
+    SMELT_KERNEL void smelt_affine_matvec_argmax_single_##T(                                      \
+        const u8* W, const u16* S, const u16* B, const u16* X, smelt::uint2_t* keys, u32,         \
+        float logit_cap, u32 rows, u32 cols, u32 group, u32) {                                    \
+        using namespace smelt;                                                                    \
+        __shared__ uint2_t wave_keys[4];                                                          \
+        uint2_t best = {0u, 0u};                                                                  \
+        float best_raw = __builtin_nanf("");                                                      \
+        EpiArgmax<ACT> epi{keys, logit_cap, &best, &best_raw, wave_keys};                         \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
         matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, X, rows, cols,                                 \
-                                             packed_row_stride<FmtU4>(cols, group), group, lo,    \
-                                             hi, epi);                                            \
+                                             packed_row_stride<FmtU4>(cols, group), group, 0, 1,  \
+                                             epi);                                                \
     }
 
 // Affine projection bank: up to four same-input members whose packed rows, scale rows and bias

@@ -97,7 +97,7 @@ struct MvBatch {
     uint2_t b[NMAT];  // four 16-bit group biases (affine)
 };
 
-template <class F, class ActT, class ScaleT, int NMAT, class Epi>
+template <class F, class ActT, class ScaleT, int NMAT, bool STREAM, class Epi>
 __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], const uint16_t* x, int rows,
                                                  int cols, int row_stride, int kw, int batch_lo,
                                                  int batch_hi, const Epi& epi) {
@@ -185,6 +185,9 @@ __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], co
                     y[m].w = __builtin_fmaf(bv, xs4.w, y[m].w);
                 }
             }
+            // keep one window's fragments and operands live at a time: without this fence the
+            // scheduler hoists all sixteen operand sets of a batch and halves the occupancy
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -237,7 +240,7 @@ __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], co
         }
         __syncthreads();
 
-        if (kw == 1) {
+        if constexpr (STREAM) {
             // ---- streaming: every wave owns whole tiles; (tile, batch) items two deep ----------
             const int first = blockIdx.x * nwaves + wave, stride = gridDim.x * nwaves;
             const int my_tiles = first < tiles ? (tiles - first + stride - 1) / stride : 0;

@@ -4,35 +4,37 @@
 #include "matvec_kernels.hpp"
 #include "mfma_matvec.hpp"
 
-#define SMELT_AFFINE_MM_KERNELS(T, ACT, SC)                                                       \
-    SMELT_KERNEL void smelt_affine_mm_matvec_##T(const u8* W, const u16* S, const u16* B,         \
+// Two kernels per pipeline: `stream` (kw == 1, every wave streams whole rows) and `split` (K split
+// over kw waves of a workgroup), so that each keeps only its own registers live.
+#define SMELT_AFFINE_MM_KERNELS(T, ACT, SC, MODE, STREAMV)                                                       \
+    SMELT_KERNEL void smelt_affine_mm_matvec_##MODE##_##T(const u8* W, const u16* S, const u16* B,         \
                                                  const u16* x, u16* y, u32 rows, u32 cols,        \
                                                  u32 group, u32 kw) {                             \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         EpiStore<ACT> epi{{}, y, (int)rows};                                                      \
-        mfma_matvec_body<MvU4, ACT, SC, 1>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
                                            blockIdx.y + 1, epi);                                  \
     }                                                                                             \
-    SMELT_KERNEL void smelt_affine_mm_matvec_add_##T(const u8* W, const u16* S, const u16* B,     \
+    SMELT_KERNEL void smelt_affine_mm_matvec_add_##MODE##_##T(const u8* W, const u16* S, const u16* B,     \
                                                      const u16* x, u16* y, const u16* res,        \
                                                      u32 rows, u32 cols, u32 group, u32 kw) {     \
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         EpiAdd<ACT> epi{{}, y, res, (int)rows};                                                   \
-        mfma_matvec_body<MvU4, ACT, SC, 1>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
                                            blockIdx.y + 1, epi);                                  \
     }                                                                                             \
-    SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_##T(                                         \
+    SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_##MODE##_##T(                                         \
         const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
         const u16* x, u16* y, u32 rows, u32 cols, u32 group, u32 kw) {                            \
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
         EpiAffineSwiglu<ACT> epi{{}, y, (int)rows};                                               \
-        mfma_matvec_body<MvU4, ACT, SC, 2>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+        mfma_matvec_body<MvU4, ACT, SC, 2, STREAMV>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
                                            blockIdx.y + 1, epi);                                  \
     }                                                                                             \
-    SMELT_KERNEL void smelt_affine_mm_matvec_batched_##T(                                         \
+    SMELT_KERNEL void smelt_affine_mm_matvec_batched_##MODE##_##T(                                         \
         const u8* W, const u16* S, const u16* B, const u16* X, u16* Y, u32 batch, u32 rows,       \
         u32 cols, u32 group, u32 batch_tile, u32 kw) {                                            \
         using namespace smelt;                                                                    \
@@ -41,9 +43,9 @@
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
-        mfma_matvec_body<MvU4, ACT, SC, 1>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
+        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
     }                                                                                             \
-    SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_batched_##T(                                 \
+    SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_batched_##MODE##_##T(                                 \
         const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
         const u16* X, u16* Y, u32 batch, u32 rows, u32 cols, u32 group, u32 batch_tile,           \
         u32 kw) {                                                                                 \
@@ -53,25 +55,28 @@
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
-        mfma_matvec_body<MvU4, ACT, SC, 2>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
+        mfma_matvec_body<MvU4, ACT, SC, 2, STREAMV>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
     }                                                                                             \
-    SMELT_KERNEL void smelt_affine_mm_matvec_argmax_##T(                                          \
+    SMELT_KERNEL void smelt_affine_mm_matvec_argmax_##MODE##_##T(                                          \
         const u8* W, const u16* S, const u16* B, const u16* X, smelt::uint2_t* keys, u32 batch,   \
         float logit_cap, u32 rows, u32 cols, u32 group, u32 batch_tile, u32 kw) {                 \
         using namespace smelt;                                                                    \
         __shared__ uint2_t wave_keys[4];                                                          \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         uint2_t best = {0u, 0u};                                                                  \
-        EpiArgmax<ACT> epi{keys, logit_cap, &best, wave_keys};                                    \
+        float best_raw = __builtin_nanf("");                                                      \
+        EpiArgmax<ACT> epi{keys, logit_cap, &best, &best_raw, wave_keys};                                    \
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
         /* one key per token and workgroup: tokens take their own pass over the rows */           \
         for (u32 b = lo; b < hi; ++b) {                                                           \
             if (b != lo) __syncthreads();                                                         \
-            mfma_matvec_body<MvU4, ACT, SC, 1>(mats, X, rows, cols, cols / 2, kw, b, b + 1, epi); \
+            mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, X, rows, cols, cols / 2, kw, b, b + 1, epi); \
         }                                                                                         \
     }
 
-SMELT_AFFINE_MM_KERNELS(f16, smelt::F16, smelt::F16)
-SMELT_AFFINE_MM_KERNELS(bf16, smelt::BF16, smelt::BF16)
+SMELT_AFFINE_MM_KERNELS(f16, smelt::F16, smelt::F16, stream, true)
+SMELT_AFFINE_MM_KERNELS(f16, smelt::F16, smelt::F16, split, false)
+SMELT_AFFINE_MM_KERNELS(bf16, smelt::BF16, smelt::BF16, stream, true)
+SMELT_AFFINE_MM_KERNELS(bf16, smelt::BF16, smelt::BF16, split, false)

@@ -21,7 +21,9 @@ SMELT_SIGNED_KERNELS(ternary, smelt::FmtTer2, f16, smelt::F16)
 SMELT_SIGNED_KERNELS(ternary, smelt::FmtTer2, bf16, smelt::BF16)
 
 SMELT_AFFINE_ARGMAX(f16, smelt::F16, smelt::F16)
+SMELT_AFFINE_ARGMAX_SINGLE(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_ARGMAX(bf16, smelt::BF16, smelt::BF16)
+SMELT_AFFINE_ARGMAX_SINGLE(bf16, smelt::BF16, smelt::BF16)
 SMELT_TERAFF_KERNELS(f16, smelt::F16)
 SMELT_TERAFF_KERNELS(bf16, smelt::BF16)
 SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, f16, smelt::F16)

@@ -118,8 +118,8 @@ size_t mfma_matvec_lds_bytes(CodeLayout layout, uint32_t cols, uint32_t tokens, 
 }
 
 uint32_t mfma_matvec_kw(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t tokens, uint32_t nmat, size_t lds_limit) {
-    // Matrices that stream from HBM (8M weights and up) with one scale group per window and whole
-    // batches of four windows per row; smaller ones are latency-bound and stay on the vector ALU.
+    // One scale group per window and whole batches of four windows per row; matrices under 8M
+    // weights are latency-bound and gain nothing from it.
     const uint32_t window = layout == kCodesU4 ? 64 : 128;
     if (layout != kCodesU4 && layout != kCodesTernary2) return 0;
     if (group != window || cols % (4 * window) != 0 || (uint64_t)rows * cols < (8u << 20)) return 0;
@@ -203,7 +203,17 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             return kResolveMalformed;
         }
         const uint32_t row_stride = cols / 2;
+        // "_mfma" after the variant suffix asks for the matrix-core matvec of the same pipeline
+        bool want_mfma = false;
+        if (suffix.size() >= 5 && suffix.compare(suffix.size() - 5, 5, "_mfma") == 0) {
+            want_mfma = true;
+            suffix.resize(suffix.size() - 5);
+        }
         const bool m1 = suffix.empty() || suffix == "_rows4" || suffix == "_rows8" || suffix == "_rows4_sg1";
+        if (want_mfma && mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 2, lds_limit) == 0) {
+            *why = "matrix-core matvec needs group 64, cols % 256 == 0 and at least 8M weights: '" + entry + "'";
+            return kResolveMalformed;
+        }
         uint32_t bt = 0;
         bool full = false, skinny = false;
         if (suffix == "_batched") bt = 8;
@@ -219,11 +229,15 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             if (m1 || full) { *why = "affine_matvec_argmax exists only as '_batched'"; return kResolveUnknown; }
             out->family = kFamAffineArgmax;
             out->symbol = "smelt_affine_matvec_argmax_" + t;
+            out->symbol_single = "smelt_affine_matvec_argmax_single_" + t;  // decode: one token, no token loop
+            out->single_arg = 5;
             out->kinds = "PPPPPUFUUUU";
             out->appended = {rows, cols, group, bt};
-            if (const uint32_t kw = mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 1, lds_limit)) {
+            if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 1, lds_limit) : 0) {
                 out->mfma_kw = kw;
-                out->symbol = "smelt_affine_mm_matvec_argmax_" + t;
+                out->symbol_single.clear();
+                out->single_arg = -1;
+                out->symbol = std::string("smelt_affine_mm_matvec_argmax_") + (kw == 1 ? "stream_" : "split_") + t;
                 out->kinds += "U";
                 out->appended.push_back(kw);
             }
@@ -241,9 +255,9 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->appended = {rows, cols, group};
             const uint32_t nmat = a.m1 == kFamAffineGateUp ? 2 : 1;
             if (a.m1 != kFamAffineDual)
-                if (const uint32_t kw = mfma_matvec_kw(kCodesU4, rows, cols, group, 1, nmat, lds_limit)) {
+                if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, 1, nmat, lds_limit) : 0) {
                     out->mfma_kw = kw;
-                    out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_" : (a.m1 == kFamAffineAdd ? "smelt_affine_mm_matvec_add_" : "smelt_affine_mm_gate_up_swiglu_")) + t;
+                    out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_" : (a.m1 == kFamAffineAdd ? "smelt_affine_mm_matvec_add_" : "smelt_affine_mm_gate_up_swiglu_")) + (kw == 1 ? "stream_" : "split_") + t;
                     out->kinds += "U";
                     out->appended.push_back(kw);
                 }
@@ -278,9 +292,9 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         else if (a.m1 == kFamAffineGateUp) { out->family = kFamAffineGateUpBatched; out->symbol = "smelt_affine_gate_up_swiglu_batched_" + mbs; out->kinds = "PPPPPPPPUUUUU"; }
         else { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
         out->appended = {rows, cols, group, bt};
-        if (const uint32_t kw = mfma_matvec_kw(kCodesU4, rows, cols, group, std::min(bt, 8u), a.m1 == kFamAffineGateUp ? 2 : 1, lds_limit)) {
+        if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, std::min(bt, 8u), a.m1 == kFamAffineGateUp ? 2 : 1, lds_limit) : 0) {
             out->mfma_kw = kw;
-            out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_batched_" : "smelt_affine_mm_gate_up_swiglu_batched_") + t;
+            out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_batched_" : "smelt_affine_mm_gate_up_swiglu_batched_") + (kw == 1 ? "stream_" : "split_") + t;
             out->kinds += "U";
             out->appended.push_back(kw);
         }

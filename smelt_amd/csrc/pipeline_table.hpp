@@ -55,6 +55,8 @@ struct ResolvedPipeline {
     uint32_t lds_variant = 0;        // batched matvec: activation rows resident per pass (1, 2, 4);
                                      // qmm: 16-token blocks per workgroup tile (1, 2, 4),
                                      // or kSkinnyVariant for the split-K skinny kernels
+    std::string symbol_single;       // optional kernel for launches whose batch argument is 1
+    int single_arg = -1;             // index of that batch argument
     uint32_t mfma_kw = 0;            // > 0: matrix-core matvec variant, waves that share a row tile
     bool workspace = false;          // kernel takes the context's (partials, counters) pointers last
 };

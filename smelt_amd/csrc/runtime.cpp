@@ -39,6 +39,7 @@ struct Pipeline {
     std::string entry;
     bool ready = false;
     hipFunction_t fn = nullptr;
+    hipFunction_t fn_single = nullptr;  // used when the record's batch argument is 1
     ResolvedPipeline res;
 };
 
@@ -615,7 +616,9 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         ctx->batch_open = true;
         ctx->timing_valid = false;
     }
-    HIP_TRY(ctx, hipModuleLaunchKernel(p->fn, L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2],
+    hipFunction_t fn = p->fn;
+    if (p->fn_single && p->res.single_arg >= 0 && L.args[(size_t)p->res.single_arg].value == 1 && L.grid[1] == 1) fn = p->fn_single;
+    HIP_TRY(ctx, hipModuleLaunchKernel(fn, L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2],
                                        (unsigned)L.lds, ctx->stream, nullptr, config));
     return 1;
 }
@@ -732,6 +735,9 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
                 return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "code object has no kernel '" + p.res.symbol + "' for pipeline '" + p.entry + "': " + hipGetErrorString(e));
         } else {
             p.ready = true;
+            if (!p.res.symbol_single.empty() &&
+                hipModuleGetFunction(&p.fn_single, ctx->module, p.res.symbol_single.c_str()) != hipSuccess)
+                p.fn_single = nullptr;
         }
     }
     std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);

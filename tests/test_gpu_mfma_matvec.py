@@ -1,5 +1,5 @@
-"""GPU parity: the matrix-core matvec variants the pipeline table selects for matrices of 8M weights
-and more (affine u4 g64): every K-split (1, 2, 4 waves per row tile), ragged row tiles, 1..8 and
+"""GPU parity: the matrix-core matvec variants ("_mfma" pipeline names, affine u4 g64, matrices of 8M
+weights and more): every K-split (1, 2, 4 waves per row tile), ragged row tiles, 1..8 and
 more than 8 tokens, the fused epilogues, and agreement with the vector-ALU kernels."""
 import numpy as np
 import pytest
@@ -34,8 +34,8 @@ SHAPES = [(8200, 1024, 4), (33000, 256, 2), (70001, 256, 1), (5000, 2560, 4)]
 @pytest.mark.parametrize("rows,cols,kw", SHAPES)
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 def test_mfma_matvec_matches_oracle(ctx, rows, cols, kw, dtype):
-    entry = f"affine_matvec_c{cols}_r{rows}_g64"
-    assert mm_symbol(entry) == "smelt_affine_mm_matvec_f16"
+    entry = f"affine_matvec_c{cols}_r{rows}_g64_mfma"
+    assert mm_symbol(entry) == f"smelt_affine_mm_matvec_{'stream' if kw == 1 else 'split'}_f16"
     w = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=60 + kw)
     x = fx.synth_activation(1, cols, dtype, config=1, tensor=61, outlier_frac=0.01)
     ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
@@ -54,15 +54,15 @@ def test_mfma_matvec_matches_oracle(ctx, rows, cols, kw, dtype):
 def test_mfma_small_batch(ctx, batch, tile, suffix):
     rows, cols = 8300, 1024
     dtype = fx.BF16
-    entry = f"affine_matvec_c{cols}_r{rows}_g64{suffix}"
-    assert mm_symbol(entry + "@bf16") == "smelt_affine_mm_matvec_batched_bf16"
+    entry = f"affine_matvec_c{cols}_r{rows}_g64{suffix}_mfma"
+    assert mm_symbol(entry + "@bf16") == "smelt_affine_mm_matvec_batched_split_bf16"
     w = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=70)
     x = fx.synth_activation(batch, cols, dtype, config=1, tensor=71 + batch, outlier_frac=0.01)
     ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
     y = run_affine(ctx, *w, x, dtype, entry, batched=True, batch_tile=tile)
     gh.check_outputs(y, ref, dtype, f"mfma batched M={batch}")
     # per-token results do not depend on the batch they ride in
-    y1 = run_affine(ctx, *w, x[batch - 1:batch], dtype, f"affine_matvec_c{cols}_r{rows}_g64")
+    y1 = run_affine(ctx, *w, x[batch - 1:batch], dtype, f"affine_matvec_c{cols}_r{rows}_g64_mfma")
     assert np.array_equal(y[batch - 1], y1[0])
 
 
@@ -73,12 +73,12 @@ def test_mfma_fused_add_and_gate_up(ctx):
     uw = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=81)
     x = fx.synth_activation(1, cols, dtype, config=1, tensor=82)
     res = fx.to_bits(fx.rng_for(1, 83).normal(0, 1, (1, rows)).astype(np.float32), dtype)
-    assert mm_symbol(f"fused_affine_matvec_add_c{cols}_r{rows}_g64") == "smelt_affine_mm_matvec_add_f16"
-    y = run_affine(ctx, *gw, x, dtype, f"affine_matvec_c{cols}_r{rows}_g64")
-    fused = run_affine(ctx, *gw, x, dtype, f"fused_affine_matvec_add_c{cols}_r{rows}_g64", residual=res)
+    assert mm_symbol(f"fused_affine_matvec_add_c{cols}_r{rows}_g64_mfma") == "smelt_affine_mm_matvec_add_split_f16"
+    y = run_affine(ctx, *gw, x, dtype, f"affine_matvec_c{cols}_r{rows}_g64_mfma")
+    fused = run_affine(ctx, *gw, x, dtype, f"fused_affine_matvec_add_c{cols}_r{rows}_g64_mfma", residual=res)
     assert np.array_equal(fused, so.narrow(fx.from_bits(y, dtype) + fx.from_bits(res, dtype), dtype))
-    entry = f"fused_affine_gate_up_swiglu_c{cols}_r{rows}_g64"
-    assert mm_symbol(entry) == "smelt_affine_mm_gate_up_swiglu_f16"
+    entry = f"fused_affine_gate_up_swiglu_c{cols}_r{rows}_g64_mfma"
+    assert mm_symbol(entry) == "smelt_affine_mm_gate_up_swiglu_split_f16"
     wf = gh.WeightFile()
     offs = [wf.add(a) for a in (*gw, *uw)]
     ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
@@ -95,8 +95,34 @@ def test_mfma_fused_add_and_gate_up(ctx):
     gh.check_outputs(got, ref, dtype, "mfma gate_up_swiglu", rel_tol=4e-3)
 
 
-def test_small_and_odd_shapes_stay_on_the_vector_alu():
-    assert mm_symbol("affine_matvec_c1024_r3584_g64") == "smelt_affine_matvec_f16"          # under 8M weights
-    assert mm_symbol("affine_matvec_c1024_r16384_g128") == "smelt_affine_matvec_f16"        # group != window
-    assert mm_symbol("affine_matvec_c1088_r16384_g64") == "smelt_affine_matvec_f16"         # cols % 256 != 0
-    assert mm_symbol("affine_matvec_c1024_r151936_g64@bf16") == "smelt_affine_mm_matvec_bf16"
+def test_mfma_argmax_and_selection_rules(ctx):
+    """Fused lm_head argmax through the matrix-core kernel equals the oracle's argmax; the default
+    names stay on the vector-ALU kernels and ineligible shapes are refused."""
+    rows, cols, batch = 20000, 1024, 3
+    dtype = fx.BF16
+    w = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=7)
+    x = fx.synth_activation(batch, cols, dtype, config=1, tensor=33)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
+    want = [so.argmax16(so.narrow(ref, dtype)[b]) for b in range(batch)]
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in w]
+    ctx.upload_weights(0, wf.image())
+    ctx.put(gh.X_SLOT, x)
+    grid_w = 160
+    ctx.alloc(gh.AUX_SLOT, batch * grid_w * 8)
+    ctx.alloc(gh.Y_SLOT, batch * 4)
+    entry = f"affine_matvec_argmax_c{cols}_r{rows}_g64_batched_mfma@bf16"
+    assert mm_symbol(entry) == "smelt_affine_mm_matvec_argmax_split_bf16"
+    p1, p2 = ctx.pipeline(entry), ctx.pipeline(f"lm_head_argmax_reduce_r{rows}")
+    bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.AUX_SLOT, 4, 0)]
+    r1 = rt.make_record(p1, bufs, [(5, batch), (6, 0.0)], (grid_w, 1, 1), (256, 1, 1))
+    r2 = rt.make_record(p2, [(gh.AUX_SLOT, 0, 0), (gh.Y_SLOT, 1, 0)], [(2, batch), (3, grid_w)], (batch, 1, 1), (256, 1, 1))
+    assert ctx.interpret_decode(ctx.table([r1, r2])) == 2
+    ctx.wait()
+    assert ctx.read(gh.Y_SLOT, np.int32, batch).tolist() == want
+    assert mm_symbol("affine_matvec_c1024_r151936_g64@bf16") == "smelt_affine_matvec_bf16"
+    assert mm_symbol("affine_matvec_c1024_r151936_g64_mfma@bf16") == "smelt_affine_mm_matvec_stream_bf16"
+    for bad in ("affine_matvec_c1024_r3584_g64_mfma",        # under 8M weights
+                "affine_matvec_c1024_r16384_g128_mfma",      # group != window
+                "affine_matvec_c1088_r16384_g64_mfma"):      # cols % 256 != 0
+        assert cc.resolve_pipeline_name(bad)[0] != 0
