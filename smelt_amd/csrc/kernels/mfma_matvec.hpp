@@ -66,6 +66,8 @@ struct MvTer2 {
     }
 };
 
+constexpr int kMvRing = 2;  // items of packed codes a streaming wave keeps in its LDS ring
+
 template <class F>
 struct MvGeom {
     static constexpr int kWindowCols = 8 * F::kCPD;  // 2 halves x 4 dwords: one scale group
@@ -81,6 +83,7 @@ __host__ __device__ inline size_t mfma_matvec_lds_bytes(int cols, int token_shif
     size_t bytes = ((nwin * MvGeom<F>::kFragsPerWindow * 16) << token_shift) + 16;
     bytes += nwin * 32 * (F::kHasBias ? 2 : 1);
     if (kw > 1) bytes += (size_t)waves * nmat * 1024;
+    else bytes = ((bytes + 1023) & ~(size_t)1023) + (size_t)waves * nmat * kMvRing * 4096;  // code rings of the streaming form
     return bytes;
 }
 
@@ -97,7 +100,8 @@ struct MvBatch {
     uint2_t b[NMAT];  // four 16-bit group biases (affine)
 };
 
-template <class F, class ActT, class ScaleT, int NMAT, bool STREAM, class Epi>
+// ONE: the launch carries a single activation row (decode): only token slot 0 is formed and used.
+template <class F, class ActT, class ScaleT, int NMAT, bool STREAM, bool ONE, class Epi>
 __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], const uint16_t* x, int rows,
                                                  int cols, int row_stride, int kw, int batch_lo,
                                                  int batch_hi, const Epi& epi) {
@@ -120,7 +124,7 @@ __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], co
     float* red = xsum + (F::kHasBias ? (size_t)nwin * 8 : 0);  // [nwaves][NMAT][8][32], kw > 1 only
 
     // A-operand lane (token slot i = lane % 16, kb): live where the slot's row half matches kb's
-    const bool a_live = ((lj >> 3) == rsel) && ((lj & 7) <= tmask);
+    const bool a_live = ((lj >> 3) == rsel) && ((lj & 7) <= tmask) && (!ONE || (lj & 7) == 0);
     const int a_tok = lj & 7;
 
     const int tpw = nwaves / kw;         // tiles a workgroup covers per step
@@ -139,55 +143,87 @@ __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], co
             if (F::kHasBias) dst.b[m] = *reinterpret_cast<const uint2_t*>(mats[m].biases + (size_t)row * nwin + w0);
         }
     };
+    uint4_t fr[4 * MPD];  // activation fragments of the window in hand
+#pragma unroll
+    for (int k = 0; k < 4 * MPD; ++k) fr[k] = uint4_t{0u, 0u, 0u, 0u};
     // y[m][v] += scale * (sum (base + code) * x - sum base * x) + bias * sum x  for four windows
-    auto compute = [&](const MvBatch<F, NMAT>& cur, int batch, float4_t (&y)[NMAT]) {
+    auto compute = [&](const MvBatch<F, NMAT>& cur, int batch, float4_t (&y)[NMAT], auto&& codes_of) {
         const int w0 = batch * WB;
 #pragma unroll
         for (int i = 0; i < WB; ++i) {
             const int w = w0 + i;
-            const uint4_t* fw = a_live ? frags + (((size_t)w * FPW + half) << tshift) + a_tok : zero_slot;
-            const size_t fstep = a_live ? ((size_t)2 << tshift) : 0;
+            // activation fragments: dead lanes hold zeros (ONE: registers that are never written;
+            // otherwise a zero slot in LDS)
+            if constexpr (ONE) {
+                if (a_live) {
+#pragma unroll
+                    for (int k = 0; k < 4 * MPD; ++k) fr[k] = frags[(size_t)w * FPW + half + 2 * k];
+                }
+            } else {
+                const uint4_t* fw = a_live ? frags + (((size_t)w * FPW + half) << tshift) + a_tok : zero_slot;
+                const size_t fstep = a_live ? ((size_t)2 << tshift) : 0;
+#pragma unroll
+                for (int k = 0; k < 4 * MPD; ++k) fr[k] = fw[(size_t)k * fstep];
+            }
             float4_t acc[NMAT];
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) acc[m] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            uint4_t cw[NMAT];
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) cw[m] = codes_of(m, i);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 uint4_t ops[NMAT][MPD];
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
-                    F::operands(t == 0 ? cur.c[m][i].x : (t == 1 ? cur.c[m][i].y : (t == 2 ? cur.c[m][i].z : cur.c[m][i].w)), ops[m]);
+                    F::operands(t == 0 ? cw[m].x : (t == 1 ? cw[m].y : (t == 2 ? cw[m].z : cw[m].w)), ops[m]);
 #pragma unroll
                 for (int q = 0; q < MPD; ++q) {
-                    const half8_t xa = *reinterpret_cast<const half8_t*>(fw + (size_t)(t * MPD + q) * fstep);
+                    const half8_t xa = __builtin_bit_cast(half8_t, fr[t * MPD + q]);
 #pragma unroll
                     for (int m = 0; m < NMAT; ++m)
                         acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8_t, ops[m][q]), acc[m], 0, 0, 0);
                 }
             }
             // D lane (row j, ib = kb): tokens 4 * (kb % 2) + v of row half kb / 2
-            const float4_t cr = *reinterpret_cast<const float4_t*>(corr + (size_t)w * 8 + 4 * half);
-            float4_t xs4 = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-            if (F::kHasBias) xs4 = *reinterpret_cast<const float4_t*>(xsum + (size_t)w * 8 + 4 * half);
+            if constexpr (ONE) {
+                const float cr = corr[(size_t)w * 8];
+                const float xs1 = F::kHasBias ? xsum[(size_t)w * 8] : 0.0f;
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m) {
-                const uint32_t sp = i < 2 ? cur.s[m].x : cur.s[m].y;
-                const float sv = F::kSemMul * ScaleT::widen((uint16_t)((i & 1) ? sp >> 16 : sp & 0xFFFFu));
-                y[m].x = __builtin_fmaf(sv, acc[m].x - cr.x, y[m].x);
-                y[m].y = __builtin_fmaf(sv, acc[m].y - cr.y, y[m].y);
-                y[m].z = __builtin_fmaf(sv, acc[m].z - cr.z, y[m].z);
-                y[m].w = __builtin_fmaf(sv, acc[m].w - cr.w, y[m].w);
-                if (F::kHasBias) {
-                    const uint32_t bp = i < 2 ? cur.b[m].x : cur.b[m].y;
-                    const float bv = ScaleT::widen((uint16_t)((i & 1) ? bp >> 16 : bp & 0xFFFFu));
-                    y[m].x = __builtin_fmaf(bv, xs4.x, y[m].x);
-                    y[m].y = __builtin_fmaf(bv, xs4.y, y[m].y);
-                    y[m].z = __builtin_fmaf(bv, xs4.z, y[m].z);
-                    y[m].w = __builtin_fmaf(bv, xs4.w, y[m].w);
+                for (int m = 0; m < NMAT; ++m) {
+                    const uint32_t sp = i < 2 ? cur.s[m].x : cur.s[m].y;
+                    const float sv = F::kSemMul * ScaleT::widen((uint16_t)((i & 1) ? sp >> 16 : sp & 0xFFFFu));
+                    y[m].x = __builtin_fmaf(sv, acc[m].x - cr, y[m].x);
+                    if (F::kHasBias) {
+                        const uint32_t bp = i < 2 ? cur.b[m].x : cur.b[m].y;
+                        y[m].x = __builtin_fmaf(ScaleT::widen((uint16_t)((i & 1) ? bp >> 16 : bp & 0xFFFFu)), xs1, y[m].x);
+                    }
+                }
+            } else {
+                const float4_t cr = *reinterpret_cast<const float4_t*>(corr + (size_t)w * 8 + 4 * half);
+                float4_t xs4 = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                if (F::kHasBias) xs4 = *reinterpret_cast<const float4_t*>(xsum + (size_t)w * 8 + 4 * half);
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) {
+                    const uint32_t sp = i < 2 ? cur.s[m].x : cur.s[m].y;
+                    const float sv = F::kSemMul * ScaleT::widen((uint16_t)((i & 1) ? sp >> 16 : sp & 0xFFFFu));
+                    y[m].x = __builtin_fmaf(sv, acc[m].x - cr.x, y[m].x);
+                    y[m].y = __builtin_fmaf(sv, acc[m].y - cr.y, y[m].y);
+                    y[m].z = __builtin_fmaf(sv, acc[m].z - cr.z, y[m].z);
+                    y[m].w = __builtin_fmaf(sv, acc[m].w - cr.w, y[m].w);
+                    if (F::kHasBias) {
+                        const uint32_t bp = i < 2 ? cur.b[m].x : cur.b[m].y;
+                        const float bv = ScaleT::widen((uint16_t)((i & 1) ? bp >> 16 : bp & 0xFFFFu));
+                        y[m].x = __builtin_fmaf(bv, xs4.x, y[m].x);
+                        y[m].y = __builtin_fmaf(bv, xs4.y, y[m].y);
+                        y[m].z = __builtin_fmaf(bv, xs4.z, y[m].z);
+                        y[m].w = __builtin_fmaf(bv, xs4.w, y[m].w);
+                    }
                 }
             }
             // keep one window's fragments and operands live at a time: without this fence the
             // scheduler hoists all sixteen operand sets of a batch and halves the occupancy
-            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (!STREAM) __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -242,27 +278,59 @@ __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], co
 
         if constexpr (STREAM) {
             // ---- streaming: every wave owns whole tiles; (tile, batch) items two deep ----------
+            // The packed codes of an item go straight from global memory into a wave-private LDS
+            // ring (128-bit loads to LDS), eight consecutive lanes per 128-byte row segment, so
+            // every load instruction reads whole cache lines.  Lane l of load i lands in slot
+            // (row 8i + l/8, l%8) and fetches piece (l%8) ^ f(row), f(row) = (row/2) % 8; the MFMA
+            // lane of row r then finds piece q in slot q ^ f(r), and the sixteen rows a 16-lane
+            // group reads fall in sixteen different bank groups.
             const int first = blockIdx.x * nwaves + wave, stride = gridDim.x * nwaves;
             const int my_tiles = first < tiles ? (tiles - first + stride - 1) / stride : 0;
             const int nq = my_tiles * nbatch;
-            MvBatch<F, NMAT> regs_a, regs_b;
+            unsigned char* ring = smem + (((size_t)(reinterpret_cast<unsigned char*>(red) - smem) + 1023) & ~(size_t)1023) +
+                                  (size_t)wave * NMAT * kMvRing * 4096;
+            const int my_r = lj + 16 * rsel;                      // row of the tile this lane feeds to the MFMA
+            const int my_f = (my_r >> 1) & 7;
+            MvBatch<F, NMAT> regs_a, regs_b;                      // scales and biases only; codes live in the ring
             int tile_c = first, bat_c = 0, tile_n = first, bat_n = 0;
-            auto row_of = [&](int tile) {
-                const int r = tile * 32 + lj + 16 * rsel;
-                return r < rows ? r : rows - 1;  // clamped rows are computed, never stored
-            };
-            auto fetch = [&](MvBatch<F, NMAT>& dst) {
-                load(dst, row_of(tile_n), bat_n);
+            auto fetch = [&](MvBatch<F, NMAT>& dst, int slot) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0): reads of this ring slot have returned
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int rt = 8 * i + (lane >> 3);
+                        int row = tile_n * 32 + rt;
+                        if (row >= rows) row = rows - 1;         // clamped rows are computed, never stored
+                        const int piece = (lane & 7) ^ ((rt >> 1) & 7);
+                        const uint8_t* src = mats[m].codes + (size_t)row * row_stride + (size_t)bat_n * 128 + piece * 16;
+                        __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(ring + ((size_t)(slot * NMAT + m) * 4 + i) * 1024), 16, 0, 0);
+                    }
+                    int row = tile_n * 32 + my_r;
+                    if (row >= rows) row = rows - 1;
+                    dst.s[m] = *reinterpret_cast<const uint2_t*>(mats[m].scales + (size_t)row * nwin + bat_n * WB);
+                    if (F::kHasBias) dst.b[m] = *reinterpret_cast<const uint2_t*>(mats[m].biases + (size_t)row * nwin + bat_n * WB);
+                }
                 if (++bat_n == nbatch) { bat_n = 0; tile_n += stride; }
             };
+            constexpr int kLoadsPerItem = NMAT * (4 + 1 + (F::kHasBias ? 1 : 0));
+            constexpr int kAhead = kMvRing - 1;                   // items in flight beyond the one computed
             float4_t y[NMAT];
-            auto step = [&](const MvBatch<F, NMAT>& cur, MvBatch<F, NMAT>& nxt, int q) {
-                if (q + 1 < nq) fetch(nxt);
+            // item q lives in ring slot q % kMvRing and register set q % kMvRing
+            auto step = [&](const MvBatch<F, NMAT>& cur, MvBatch<F, NMAT>& ahead, int slot, int q) {
+                int newer = nq - 1 - q;                           // items requested after q
+                if (q + kAhead < nq) fetch(ahead, (slot + kAhead) % kMvRing);
+                if (newer > kAhead) newer = kAhead;
+                // item q has arrived once at most the loads of the newer items are outstanding
+                if (newer == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (kLoadsPerItem & 15) | ((kLoadsPerItem >> 4) << 14));
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
                 if (bat_c == 0) {
 #pragma unroll
                     for (int m = 0; m < NMAT; ++m) y[m] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
                 }
-                compute(cur, bat_c, y);
+                compute(cur, bat_c, y, [&](int m, int i) {
+                    return *reinterpret_cast<const uint4_t*>(ring + (size_t)(slot * NMAT + m) * 4096 + ((size_t)my_r * 8 + ((2 * i + half) ^ my_f)) * 16);
+                });
                 if (++bat_c == nbatch) {
                     const int row = tile_c * 32 + lj + 16 * rsel;
                     if (row < rows) {
@@ -281,10 +349,11 @@ __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], co
                     tile_c += stride;
                 }
             };
-            if (nq > 0) fetch(regs_a);
+            static_assert(kMvRing == 2, "the item loop below is unrolled for a ring of two");
+            if (nq > 0) fetch(regs_a, 0);
             for (int q = 0; q < nq; q += 2) {
-                step(regs_a, regs_b, q);
-                if (q + 1 < nq) step(regs_b, regs_a, q + 1);
+                step(regs_a, regs_b, 0, q);
+                if (q + 1 < nq) step(regs_b, regs_a, 1, q + 1);
             }
         } else {
             // ---- K split over kw waves: per tile, load everything, compute, meet in LDS --------
@@ -300,8 +369,8 @@ __device__ __forceinline__ void mfma_matvec_body(const MatPtrs (&mats)[NMAT], co
                         MvBatch<F, NMAT> ra, rb;
                         load(ra, row, kwi + g0 * kw);
                         if (g0 + 1 < my_batches) load(rb, row, kwi + (g0 + 1) * kw);
-                        compute(ra, kwi + g0 * kw, y);
-                        if (g0 + 1 < my_batches) compute(rb, kwi + (g0 + 1) * kw, y);
+                        compute(ra, kwi + g0 * kw, y, [&](int m, int i) { return ra.c[m][i]; });
+                        if (g0 + 1 < my_batches) compute(rb, kwi + (g0 + 1) * kw, y, [&](int m, int i) { return rb.c[m][i]; });
                     }
                 }
 #pragma unroll

@@ -13,7 +13,7 @@
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         EpiStore<ACT> epi{{}, y, (int)rows};                                                      \
-        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV, true>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
                                            blockIdx.y + 1, epi);                                  \
     }                                                                                             \
     SMELT_KERNEL void smelt_affine_mm_matvec_add_##MODE##_##T(const u8* W, const u16* S, const u16* B,     \
@@ -22,7 +22,7 @@
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         EpiAdd<ACT> epi{{}, y, res, (int)rows};                                                   \
-        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV, true>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
                                            blockIdx.y + 1, epi);                                  \
     }                                                                                             \
     SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_##MODE##_##T(                                         \
@@ -31,7 +31,7 @@
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
         EpiAffineSwiglu<ACT> epi{{}, y, (int)rows};                                               \
-        mfma_matvec_body<MvU4, ACT, SC, 2, STREAMV>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
+        mfma_matvec_body<MvU4, ACT, SC, 2, STREAMV, true>(mats, x, rows, cols, cols / 2, kw, blockIdx.y,         \
                                            blockIdx.y + 1, epi);                                  \
     }                                                                                             \
     SMELT_KERNEL void smelt_affine_mm_matvec_batched_##MODE##_##T(                                         \
@@ -43,7 +43,7 @@
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
-        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
+        mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV, false>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
     }                                                                                             \
     SMELT_KERNEL void smelt_affine_mm_gate_up_swiglu_batched_##MODE##_##T(                                 \
         const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
@@ -55,7 +55,7 @@
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
-        mfma_matvec_body<MvU4, ACT, SC, 2, STREAMV>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
+        mfma_matvec_body<MvU4, ACT, SC, 2, STREAMV, false>(mats, X, rows, cols, cols / 2, kw, lo, hi, epi);       \
     }                                                                                             \
     SMELT_KERNEL void smelt_affine_mm_matvec_argmax_##MODE##_##T(                                          \
         const u8* W, const u16* S, const u16* B, const u16* X, smelt::uint2_t* keys, u32 batch,   \
@@ -72,7 +72,7 @@
         /* one key per token and workgroup: tokens take their own pass over the rows */           \
         for (u32 b = lo; b < hi; ++b) {                                                           \
             if (b != lo) __syncthreads();                                                         \
-            mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV>(mats, X, rows, cols, cols / 2, kw, b, b + 1, epi); \
+            mfma_matvec_body<MvU4, ACT, SC, 1, STREAMV, true>(mats, X, rows, cols, cols / 2, kw, b, b + 1, epi); \
         }                                                                                         \
     }
 

@@ -114,6 +114,7 @@ size_t mfma_matvec_lds_bytes(CodeLayout layout, uint32_t cols, uint32_t tokens, 
     const size_t nwin = cols / window;
     size_t bytes = ((nwin * frags * 16) << shift) + 16 + nwin * 32 * (layout == kCodesU4 ? 2 : 1);
     if (kw > 1) bytes += (size_t)waves * nmat * 1024;
+    else bytes = ((bytes + 1023) & ~(size_t)1023) + (size_t)waves * nmat * 2 * 4096;  // code rings of the streaming form (two items per wave)
     return bytes;
 }
 
