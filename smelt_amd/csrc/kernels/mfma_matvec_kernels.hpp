@@ -80,3 +80,58 @@ SMELT_AFFINE_MM_KERNELS(f16, smelt::F16, smelt::F16, stream, true)
 SMELT_AFFINE_MM_KERNELS(f16, smelt::F16, smelt::F16, split, false)
 SMELT_AFFINE_MM_KERNELS(bf16, smelt::BF16, smelt::BF16, stream, true)
 SMELT_AFFINE_MM_KERNELS(bf16, smelt::BF16, smelt::BF16, split, false)
+
+// Signed g128 formats (scales are fp16; no bias plane).  Same argument lists as the vector-ALU
+// kernels of the pipelines, followed by kw.  The ternary "affine" pipelines bind the scale plane
+// a second time where MLX binds a bias plane; it is ignored as in the vector-ALU kernels.
+#define SMELT_SIGNED_MM_KERNELS(FN, FMT, T, ACT, MODE, STREAMV)                                   \
+    SMELT_KERNEL void smelt_signed_##FN##_mm_matvec_##MODE##_##T(                                 \
+        const u8* C, const u16* S, const u16* X, u16* Y, u32 rows, u32 cols, u32 kw) {            \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mfma_matvec_body<FMT, ACT, F16, 1, STREAMV, true>(mats, X, rows, cols,                    \
+                                                          packed_row_stride<typename FMT::Valu>(cols, 128), kw, \
+                                                          blockIdx.y, blockIdx.y + 1, epi);       \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_mm_matvec_add_##MODE##_##T(                             \
+        const u8* C, const u16* S, const u16* X, u16* Y, const u16* res, u32 rows, u32 cols,      \
+        u32 kw) {                                                                                 \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        mfma_matvec_body<FMT, ACT, F16, 1, STREAMV, true>(mats, X, rows, cols,                    \
+                                                          packed_row_stride<typename FMT::Valu>(cols, 128), kw, \
+                                                          blockIdx.y, blockIdx.y + 1, epi);       \
+    }
+
+#define SMELT_TERAFF_MM_KERNELS(T, ACT, MODE, STREAMV)                                            \
+    SMELT_KERNEL void smelt_teraff_mm_matvec_##MODE##_##T(                                        \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* Y, u32 rows, u32 cols,          \
+        u32 kw) {                                                                                 \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mfma_matvec_body<MvTer2, ACT, F16, 1, STREAMV, true>(mats, X, rows, cols, cols / 4, kw,   \
+                                                             blockIdx.y, blockIdx.y + 1, epi);    \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_teraff_mm_matvec_add_##MODE##_##T(                                    \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* Y, const u16* res, u32 rows,    \
+        u32 cols, u32 kw) {                                                                       \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        mfma_matvec_body<MvTer2, ACT, F16, 1, STREAMV, true>(mats, X, rows, cols, cols / 4, kw,   \
+                                                             blockIdx.y, blockIdx.y + 1, epi);    \
+    }
+
+#define SMELT_SIGNED_MM_ALL(T, ACT)                                                               \
+    SMELT_SIGNED_MM_KERNELS(binary, smelt::MvBin, T, ACT, stream, true)                           \
+    SMELT_SIGNED_MM_KERNELS(binary, smelt::MvBin, T, ACT, split, false)                           \
+    SMELT_SIGNED_MM_KERNELS(ternary, smelt::MvTer2, T, ACT, stream, true)                         \
+    SMELT_SIGNED_MM_KERNELS(ternary, smelt::MvTer2, T, ACT, split, false)                         \
+    SMELT_TERAFF_MM_KERNELS(T, ACT, stream, true)                                                 \
+    SMELT_TERAFF_MM_KERNELS(T, ACT, split, false)
+
+SMELT_SIGNED_MM_ALL(f16, smelt::F16)
+SMELT_SIGNED_MM_ALL(bf16, smelt::BF16)

@@ -105,27 +105,29 @@ size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat, uint3
 }
 
 size_t mfma_matvec_lds_bytes(CodeLayout layout, uint32_t cols, uint32_t tokens, uint32_t nmat, uint32_t waves, uint32_t kw) {
-    // operand fragments [windows][8 * MFMAs per dword][tokens] x 16 B (tokens rounded up to a power
-    // of two, at most 8), one zero slot, per-window corrections (and activation sums for affine)
-    // for 8 token slots, and wave partials when K is split over waves
+    // operand fragments [windows][fragments per window][tokens] x 16 B (tokens rounded up to a
+    // power of two, at most 8), one zero slot, per-window corrections (and activation sums for
+    // affine) for 8 token slots, wave partials when K is split over waves, then (1 KB aligned) the
+    // code rings: two 4 KB items per wave and matrix
     const uint32_t window = layout == kCodesU4 ? 64 : 128, frags = layout == kCodesU4 ? 8 : 16;
     uint32_t shift = 0;
     while ((1u << shift) < tokens && shift < 3) ++shift;
     const size_t nwin = cols / window;
     size_t bytes = ((nwin * frags * 16) << shift) + 16 + nwin * 32 * (layout == kCodesU4 ? 2 : 1);
     if (kw > 1) bytes += (size_t)waves * nmat * 1024;
-    else bytes = ((bytes + 1023) & ~(size_t)1023) + (size_t)waves * nmat * 2 * 4096;  // code rings of the streaming form (two items per wave)
-    return bytes;
+    return ((bytes + 1023) & ~(size_t)1023) + (size_t)waves * nmat * 2 * 4096;
 }
 
 uint32_t mfma_matvec_kw(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t tokens, uint32_t nmat, size_t lds_limit) {
-    // One scale group per window and whole batches of four windows per row; matrices under 8M
-    // weights are latency-bound and gain nothing from it.
+    // One scale group per window and whole ring items (128 bytes per row) along K; matrices under
+    // 8M weights are latency-bound and gain nothing from it.
+    if (layout != kCodesU4 && layout != kCodesTernary2 && layout != kCodesBinary1) return 0;
     const uint32_t window = layout == kCodesU4 ? 64 : 128;
-    if (layout != kCodesU4 && layout != kCodesTernary2) return 0;
-    if (group != window || cols % (4 * window) != 0 || (uint64_t)rows * cols < (8u << 20)) return 0;
-    const uint32_t tiles = (rows + 31) / 32;
-    const uint32_t kw = tiles >= 2048 ? 1 : (tiles >= 1024 ? 2 : 4);
+    const uint32_t item_cols = layout == kCodesU4 ? 256 : (layout == kCodesTernary2 ? 512 : 1024);
+    if (group != window || cols == 0 || cols % item_cols != 0 || (uint64_t)rows * cols < (8u << 20)) return 0;
+    const uint32_t tiles = (rows + 31) / 32, items = cols / item_cols;
+    uint32_t kw = tiles >= 2048 ? 1 : (tiles >= 1024 ? 2 : 4);
+    while (kw > items) kw /= 2;  // every wave of a tile needs at least one item
     if (mfma_matvec_lds_bytes(layout, cols, tokens, nmat, 4, kw) > lds_limit) return 0;
     return kw;
 }
@@ -332,6 +334,18 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->format = s.fmt;
             out->symbol = std::string(s.sym) + t;
             out->kinds = s.kinds;
+            // matrix-core variants, chosen per launch from the record's rows and cols
+            const bool add = s.fam == kFamSignedAdd || s.fam == kFamTerAffAdd;
+            if ((s.fam == kFamSignedMatvec || add || s.fam == kFamTerAffMatvec) && s.fmt != kFmtTrit5) {
+                const std::string stem = (s.fam == kFamTerAffMatvec || s.fam == kFamTerAffAdd)
+                                             ? "smelt_teraff_mm_matvec_"
+                                             : std::string("smelt_signed_") + (s.fmt == kFmtBinary1 ? "binary" : "ternary") + "_mm_matvec_";
+                out->symbol_mm_stream = stem + (add ? "add_stream_" : "stream_") + t;
+                out->symbol_mm_split = stem + (add ? "add_split_" : "split_") + t;
+                const int first_const = (int)std::string(s.kinds).find('U');
+                out->rows_arg = first_const;
+                out->cols_arg = first_const + 1;
+            }
             return kResolveOk;
         }
     }

@@ -57,6 +57,8 @@ struct ResolvedPipeline {
                                      // or kSkinnyVariant for the split-K skinny kernels
     std::string symbol_single;       // optional kernel for launches whose batch argument is 1
     int single_arg = -1;             // index of that batch argument
+    std::string symbol_mm_stream, symbol_mm_split;  // optional matrix-core kernels picked per launch by shape
+    int rows_arg = -1, cols_arg = -1;               // where that launch finds rows and cols
     uint32_t mfma_kw = 0;            // > 0: matrix-core matvec variant, waves that share a row tile
     bool workspace = false;          // kernel takes the context's (partials, counters) pointers last
 };

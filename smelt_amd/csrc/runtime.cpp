@@ -40,6 +40,7 @@ struct Pipeline {
     bool ready = false;
     hipFunction_t fn = nullptr;
     hipFunction_t fn_single = nullptr;  // used when the record's batch argument is 1
+    hipFunction_t fn_mm_stream = nullptr, fn_mm_split = nullptr;  // matrix-core variants picked by shape
     ResolvedPipeline res;
 };
 
@@ -588,6 +589,20 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     if ((size_t)L.block[0] * L.block[1] * L.block[2] > 1024)
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "threadgroup exceeds 1024 threads");
     if (int e = validate_launch(ctx, *p, L)) return e;
+    hipFunction_t fn = p->fn;
+    if (p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
+        // signed g128 matvec: large matrices run on the matrix cores (same bytes, same arguments + kw)
+        const uint32_t rows = L.args[(size_t)p->res.rows_arg].value, cols = L.args[(size_t)p->res.cols_arg].value;
+        const CodeLayout layout = code_layout(p->res.format);
+        if (const uint32_t kw = mfma_matvec_kw(layout, rows, cols, 128, 1, 1, ctx->lds_limit)) {
+            fn = kw == 1 ? p->fn_mm_stream : p->fn_mm_split;
+            L.lds = mfma_matvec_lds_bytes(layout, cols, 1, 1, 4, kw);
+            Arg a;
+            a.kind = 'U';
+            a.value = kw;
+            L.args.push_back(a);
+        }
+    }
 
     // kernarg block: natural alignment in argument order
     alignas(16) unsigned char kernarg[512];
@@ -616,7 +631,6 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         ctx->batch_open = true;
         ctx->timing_valid = false;
     }
-    hipFunction_t fn = p->fn;
     if (p->fn_single && p->res.single_arg >= 0 && L.args[(size_t)p->res.single_arg].value == 1 && L.grid[1] == 1) fn = p->fn_single;
     HIP_TRY(ctx, hipModuleLaunchKernel(fn, L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2],
                                        (unsigned)L.lds, ctx->stream, nullptr, config));
@@ -738,6 +752,10 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
             if (!p.res.symbol_single.empty() &&
                 hipModuleGetFunction(&p.fn_single, ctx->module, p.res.symbol_single.c_str()) != hipSuccess)
                 p.fn_single = nullptr;
+            if (!p.res.symbol_mm_stream.empty() &&
+                (hipModuleGetFunction(&p.fn_mm_stream, ctx->module, p.res.symbol_mm_stream.c_str()) != hipSuccess ||
+                 hipModuleGetFunction(&p.fn_mm_split, ctx->module, p.res.symbol_mm_split.c_str()) != hipSuccess))
+                p.fn_mm_stream = p.fn_mm_split = nullptr;
         }
     }
     std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);

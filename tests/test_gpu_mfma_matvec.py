@@ -28,7 +28,7 @@ def mm_symbol(entry):
 
 
 # rows chosen so that the row-tile count selects 4, 2 and 1 waves per tile; none is a multiple of 32
-SHAPES = [(8200, 1024, 4), (33000, 256, 2), (70001, 256, 1), (5000, 2560, 4)]
+SHAPES = [(8200, 1024, 4), (33000, 512, 2), (70001, 256, 1), (5000, 2560, 4)]
 
 
 @pytest.mark.parametrize("rows,cols,kw", SHAPES)
@@ -126,3 +126,52 @@ def test_mfma_argmax_and_selection_rules(ctx):
                 "affine_matvec_c1024_r16384_g128_mfma",      # group != window
                 "affine_matvec_c1088_r16384_g64_mfma"):      # cols % 256 != 0
         assert cc.resolve_pipeline_name(bad)[0] != 0
+
+
+# ---- signed g128 formats: the runtime moves large matrices to the matrix cores per launch ---------
+from test_gpu_matvec import run_signed  # noqa: E402
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")])
+@pytest.mark.parametrize("shape", [(2050, 5120), (1030, 17408), (40010, 1024), (70001, 1024)])
+def test_signed_large_matrices_match_oracle(ctx, fmt, name, dtype, shape):
+    """27B-layer-like shapes of 8M weights and more (row counts off the 32-row tile, K split 4, 2 and 1
+    ways): same pipeline names, same records, matrix-core kernels underneath."""
+    rows, cols = shape
+    codes = fx.synth_signed_codes(fmt, rows, cols, config=2 + fmt, tensor=rows % 7)
+    scales = fx.synth_signed_scales(rows, cols, config=2 + fmt, tensor=rows % 7)
+    packed = fx.pack_signed_np(codes, fmt)
+    x = fx.synth_activation(2, cols, dtype, config=2 + fmt, outlier_frac=0.01)
+    ref = so.signed_matvec(fmt, packed, scales, fx.from_bits(x, dtype), rows, cols, cols, 128)
+    y = run_signed(ctx, name, packed, scales, x, dtype, rows, cols)
+    w = gh.check_outputs(y, ref, dtype, f"signed {name} {shape}")
+    print(f"\n  mfma {name} {shape} dtype={dtype} max rel err {w:.2e}")
+    y_small = run_signed(ctx, name, packed, scales, x, dtype, rows, cols, grid=5)
+    assert np.array_equal(y, y_small)
+
+
+def test_signed_large_fused_add_and_ternary_affine_names(ctx):
+    rows, cols = 2048, 5120
+    dtype = fx.BF16
+    for fmt, name in ((fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")):
+        codes = fx.synth_signed_codes(fmt, rows, cols, config=2 + fmt, tensor=3)
+        scales = fx.synth_signed_scales(rows, cols, config=2 + fmt, tensor=3)
+        packed = fx.pack_signed_np(codes, fmt)
+        x = fx.synth_activation(1, cols, dtype, config=2 + fmt)
+        res = fx.to_bits(fx.rng_for(2, 90).normal(0, 1, (1, rows)).astype(np.float32), dtype)
+        y = run_signed(ctx, name, packed, scales, x, dtype, rows, cols)
+        fused = run_signed(ctx, name, packed, scales, x, dtype, rows, cols, kind="add", residual=res)
+        assert np.array_equal(fused, so.narrow(fx.from_bits(y, dtype) + fx.from_bits(res, dtype), dtype))
+        if fmt == fx.TERNARY2:
+            # production ternary pipeline name: scales bound twice, same arithmetic
+            wf = gh.WeightFile()
+            oc, os_ = wf.add(packed), wf.add(scales)
+            ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+            ctx.put(gh.X_SLOT, x)
+            ctx.alloc(gh.Y_SLOT, rows * 2)
+            pipe = ctx.pipeline("signed_ternary_affine_matvec_g128_rows8@bf16")
+            bufs = [(0, 0, oc), (0, 1, os_), (0, 2, os_), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+            ctx.encode_decode(rt.make_record(pipe, bufs, [(5, rows), (6, cols)], (256, 1, 1), (256, 1, 1)))
+            ctx.wait()
+            assert np.array_equal(ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows), y)
