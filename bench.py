@@ -146,7 +146,7 @@ def main() -> int:
     lm_us = ctx.graph_time(g2, reps) / (reps * n2)
     ctx.graph_destroy(g2)
     achieved = lm_bytes / lm_us / 1e3
-    roofline = {"bound": "hbm", "kernel": "smelt_affine_matvec_argmax_bf16 (lm_head 151936x1024 u4 g64)",
+    roofline = {"bound": "hbm", "kernel": "smelt_affine_matvec_argmax_single_bf16 (lm_head 151936x1024 u4 g64, fused argmax)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "bytes_per_launch": int(lm_bytes), "us_per_launch": round(lm_us, 3)}
