@@ -121,15 +121,19 @@ struct MatvecGeometry {
 
 // Rows one 256-thread workgroup walks per step and the workgroup count: four waves, each owning
 // R rows per 64/L row groups (L = lanes a row's 16-byte units occupy), capped at 4 workgroups
-// per compute unit (rows beyond that are covered by the kernels' grid-stride loop).
+// per compute unit (rows beyond that are covered by the kernels' grid-stride loop).  A matrix too
+// small to give every compute unit two such workgroups is launched one row per wave slot instead:
+// the kernels switch to single-row work items when the grid holds more waves than R-row tiles.
 MatvecGeometry matvec_geometry(uint32_t row_stride, int rows, int rows_per_wave, int compute_units) {
     const int U = (int)(row_stride / 16);
     const int L = U > 32 ? 64 : (U > 16 ? 32 : 16);
-    const int tile = (64 / L) * rows_per_wave;
+    const int cus = std::max(1, compute_units);
+    int tile = (64 / L) * rows_per_wave;
+    if ((rows + tile * 4 - 1) / (tile * 4) < 2 * cus) tile = 64 / L;
     MatvecGeometry g;
     g.rows_per_group = tile * 4;
     const int want = (rows + g.rows_per_group - 1) / g.rows_per_group;
-    g.grid_w = std::max(1, std::min(want, std::max(1, compute_units) * 4));
+    g.grid_w = std::max(1, std::min(want, cus * 4));
     return g;
 }
 

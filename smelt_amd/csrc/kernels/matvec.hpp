@@ -226,6 +226,7 @@ struct ItemRegs {
     uint4_t c[NMAT][R];
     uint16_t s[NMAT][R];
     uint16_t b[NMAT][R];   // affine bias; for per-dword-scale formats the next group's scale
+    uint16_t res[R];       // epilogue operand fetched ahead with a row's last item (when the epilogue asks)
 };
 
 template <class F, int R, int NMAT>

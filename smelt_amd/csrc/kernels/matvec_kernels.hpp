@@ -2,6 +2,7 @@
 // the binding order of the Smelt dispatch record that drives it (buffers and 4-byte constants
 // by ascending binding index), followed by the shape arguments the pipeline table appends.
 #pragma once
+#include <type_traits>
 #include "matvec.hpp"
 #include "misc_kernels.hpp"
 
@@ -13,6 +14,9 @@ namespace smelt {
 // Epilogues may keep per-thread state; end_chunk() runs on every thread once all rows of a
 // batch chunk are done.
 struct EpiBase {
+    // An epilogue that reads one 16-bit operand per output row can have it fetched together with
+    // the row's last weight item instead of after the reduction (single-token launches only).
+    static constexpr bool kPrefetch = false;
     __device__ __forceinline__ void end_chunk(int, int) const {}
 };
 
@@ -31,10 +35,14 @@ struct EpiAdd : EpiBase {
     uint16_t* y;
     const uint16_t* residual;
     int rows;
-    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
-        const size_t i = (size_t)b * rows + row;
+    static constexpr bool kPrefetch = true;
+    __device__ __forceinline__ uint16_t prefetch(int b, int row) const { return residual[(size_t)b * rows + row]; }
+    __device__ __forceinline__ void finish(int b, int row, const float* v, uint16_t res) const {
         const float projected = ActT::widen(ActT::narrow(v[0]));
-        y[i] = ActT::narrow(projected + ActT::widen(residual[i]));
+        y[(size_t)b * rows + row] = ActT::narrow(projected + ActT::widen(res));
+    }
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        finish(b, row, v, residual[(size_t)b * rows + row]);
     }
 };
 
@@ -81,9 +89,9 @@ struct EpiDual : EpiBase {
 // ---- workgroup body ------------------------------------------------------------------------
 //
 // A wave walks its row tiles (grid-stride, so any grid covers every row) as a flat sequence of
-// work items (tile, unit step).  Items are software-pipelined two deep: the loads of item q+1
-// are issued before item q is computed, and the loads of the very first item are issued before
-// the activations are staged, so a small matrix pays one memory latency, not two.
+// work items (tile, unit step).  Items are software-pipelined two deep: the loads of items q+1
+// and q+2 are in flight while item q is computed, and the loads of the first two items are issued
+// before the activations are staged, so a small matrix pays one memory latency, not two.
 
 template <class F, class ActT, class ScaleT, int R, int MB, int NMAT, int L, class Epi>
 __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uint16_t* x, int rows,
@@ -112,25 +120,29 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
         int tile_c = first, it_c = 0, tile_n = first, it_n = 0;
         auto load = [&](ItemRegs<R, NMAT>& dst) {
             const int u = sub + L * it_n;
-            if (u < U) {
-                int row[R];
+            int row[R];
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const int rr = tile_n * TILE + side * R + r;
-                    row[r] = rr < rows ? rr : rows - 1;  // clamped rows are computed, never stored
+            for (int r = 0; r < R; ++r) {
+                const int rr = tile_n * TILE + side * R + r;
+                row[r] = rr < rows ? rr : rows - 1;  // clamped rows are computed, never stored
+            }
+            if (u < U) load_item<F, R, NMAT>(mats, row, u, row_stride, gpr, gshift, dst);
+            if constexpr (Epi::kPrefetch && MB == 1) {
+                if (it_n == nit - 1 && sub == L - 1) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) dst.res[r] = epi.prefetch(b0, row[r]);
                 }
-                load_item<F, R, NMAT>(mats, row, u, row_stride, gpr, gshift, dst);
             }
             if (++it_n == nit) { it_n = 0; tile_n += stride; }
         };
         if (nq > 0) load(regs_a);
+        if (nq > 1) load(regs_b);
         if (b0 != batch_lo) __syncthreads();
         stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum);
         __syncthreads();
 
         float acc[NMAT][R][MB];
-        auto step = [&](const ItemRegs<R, NMAT>& cur, ItemRegs<R, NMAT>& nxt, int q) {
-            if (q + 1 < nq) load(nxt);
+        auto step = [&](ItemRegs<R, NMAT>& cur, int q) {
             if (it_c == 0) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
@@ -159,7 +171,8 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
                                     float v[NMAT];
 #pragma unroll
                                     for (int m = 0; m < NMAT; ++m) v[m] = acc[m][r][b];
-                                    epi(b0 + b, row, v);
+                                    if constexpr (Epi::kPrefetch && MB == 1) epi.finish(b0 + b, row, v, cur.res[r]);
+                                    else epi(b0 + b, row, v);
                                 }
                             }
                         }
@@ -170,10 +183,11 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
             } else {
                 ++it_c;
             }
+            if (q + 2 < nq) load(cur);  // refill the registers just consumed: two items stay in flight
         };
         for (int q = 0; q < nq; q += 2) {
-            step(regs_a, regs_b, q);
-            if (q + 1 < nq) step(regs_b, regs_a, q + 1);
+            step(regs_a, q);
+            if (q + 1 < nq) step(regs_b, q + 1);
         }
         epi.end_chunk(b0, nb);
     }
@@ -195,12 +209,24 @@ __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const u
     uint16_t* lut = reinterpret_cast<uint16_t*>(lds_xsum + (size_t)MB * U * FmtGeom<F>::kCorrStride);
     if (F::kPerDwordScale)  // decode table; visible to every wave after the staging barrier
         for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) lut[i] = trit5_lut_entry(i);
-    if (U > 32)
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 64>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
-    else if (U > 16)
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 32>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
-    else
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, 16>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
+    // A grid with more waves than there are R-row tiles asks for finer work items: such launches
+    // (small matrices, where one wave per SIMD would otherwise chew through R rows serially) run
+    // one row per wave slot, which shortens the latency-bound tail of the kernel.
+    const int total_waves = (int)(gridDim.x * (blockDim.x / kWave));
+    auto go = [&](auto lanes) {
+        constexpr int L = decltype(lanes)::value;
+        if constexpr (R > 1 && MB == 1) {
+            const int tiles = (rows + (kWave / L) * R - 1) / ((kWave / L) * R);
+            if (tiles < total_waves) {
+                run_tiles<F, ActT, ScaleT, 1, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
+                return;
+            }
+        }
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
+    };
+    if (U > 32) go(std::integral_constant<int, 64>{});
+    else if (U > 16) go(std::integral_constant<int, 32>{});
+    else go(std::integral_constant<int, 16>{});
 }
 
 template <class F>
@@ -214,12 +240,14 @@ __device__ __forceinline__ int packed_row_stride(int cols, int group) {
 
 // ---- entry points ---------------------------------------------------------------------------
 #define SMELT_KERNEL extern "C" __global__ __launch_bounds__(256)
+// single-token streaming kernels: registers are held to what five waves per SIMD allow
+#define SMELT_KERNEL_W5 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5)))
 using u16 = uint16_t;
 using u8 = uint8_t;
 using u32 = uint32_t;
 
 #define SMELT_AFFINE_KERNELS(T, ACT, SC)                                                          \
-    SMELT_KERNEL void smelt_affine_matvec_##T(const u8* W, const u16* S, const u16* B,            \
+    SMELT_KERNEL_W5 void smelt_affine_matvec_##T(const u8* W, const u16* S, const u16* B,            \
                                               const u16* x, u16* y, u32 rows, u32 cols,           \
                                               u32 group) {                                        \
         using namespace smelt;                                                                    \
@@ -229,7 +257,7 @@ using u32 = uint32_t;
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
     }                                                                                             \
-    SMELT_KERNEL void smelt_affine_matvec_add_##T(const u8* W, const u16* S, const u16* B,        \
+    SMELT_KERNEL_W5 void smelt_affine_matvec_add_##T(const u8* W, const u16* S, const u16* B,        \
                                                   const u16* x, u16* y, const u16* res, u32 rows, \
                                                   u32 cols, u32 group) {                          \
         using namespace smelt;                                                                    \
@@ -239,7 +267,7 @@ using u32 = uint32_t;
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
     }                                                                                             \
-    SMELT_KERNEL void smelt_affine_gate_up_swiglu_##T(                                            \
+    SMELT_KERNEL_W5 void smelt_affine_gate_up_swiglu_##T(                                         \
         const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
         const u16* x, u16* y, u32 rows, u32 cols, u32 group) {                                    \
         using namespace smelt;                                                                    \
@@ -363,6 +391,7 @@ namespace smelt {
 // partial key for the batch row at partials[batch * gridDim.x + blockIdx.x].
 template <class ActT>
 struct EpiArgmax {
+    static constexpr bool kPrefetch = false;
     uint2_t* partials;
     float logit_cap;
     uint2_t* best;      // one per thread (register-resident in the caller)
@@ -452,7 +481,7 @@ struct EpiBank4 : EpiBase {
 // Decode form of the fused argmax: exactly one token (batch == 1, one grid row), so no token loop
 // and the register footprint of the plain matvec.
 #define SMELT_AFFINE_ARGMAX_SINGLE(T, ACT, SC)                                                    \
-    SMELT_KERNEL void smelt_affine_matvec_argmax_single_##T(                                      \
+    SMELT_KERNEL_W5 void smelt_affine_matvec_argmax_single_##T(                                      \
         const u8* W, const u16* S, const u16* B, const u16* X, smelt::uint2_t* keys, u32,         \
         float logit_cap, u32 rows, u32 cols, u32 group, u32) {                                    \
         using namespace smelt;                                                                    \
