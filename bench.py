@@ -205,8 +205,8 @@ def committed_traffic():
 
 
 def side_measurements(ctx, fx, cc, rt, cus) -> dict:
-    """27B-layer binary / ternary / trit5 matvec sets and the 4B FFN qmm at M in {7,8,9,32,512}.
-    Reported beside the headline; not part of `value`."""
+    """27B-layer binary / ternary / trit5 matvec sets, the 4B FFN qmm at M in {7,8,9,32,512} and the
+    affine 4-bit quantiser.  Reported beside the headline; not part of `value`."""
     out = {}
     W, X, Y, ACT = 20, 21, 22, 23
     shapes = [(17408, 5120), (17408, 5120), (5120, 17408), (5120, 5120), (5120, 5120), (1024, 5120), (1024, 5120)]
@@ -299,6 +299,31 @@ def side_measurements(ctx, fx, cc, rt, cus) -> dict:
                          "weight_GBps": round(layer_bytes / us / 1e3, 1)}
         pipes_installed += len(names)
     out["qwen35_4b_ffn_qmm"] = qmm
+    c.close()
+    # weight import: affine 4-bit quantiser over a 9216 x 2560 tensor resident in HBM
+    # (algorithmic bytes = source read + packed codes, scales and biases written)
+    c = rt.Context(act_dtype=rt.ACT_BF16)
+    rows, cols, group = 9216, 2560, 64
+    gpr = cols // group
+    quant = {}
+    for src_name, src_dtype, esize in (("f32", 0, 4), ("bf16", 2, 2)):
+        w = fx.rng_for(5, src_dtype).normal(0, 0.05, (rows, cols)).astype(np.float32)
+        c.put(1, w if esize == 4 else fx.bf16_bits(w))
+        c.alloc(2, rows * cols // 2)
+        c.alloc(3, rows * gpr * 2)
+        c.alloc(4, rows * gpr * 2)
+        pipe = c.pipeline(f"affine_quantize_u4:{cols}:{group}")
+        moved = rows * cols * esize + rows * cols // 2 + 2 * rows * gpr * 2
+        for clip_name, clip in (("min_max", 0), ("mse_optimal", 1)):
+            rec = rt.make_record(pipe, [(1, 0, 0), (2, 1, 0), (3, 2, 0), (4, 3, 0)],
+                                 [(5, rows), (6, src_dtype), (7, clip)], (cus * 16, 1, 1), (128, 1, 1))
+            g, n = c.capture_decode(c.table([rec] * 4))
+            c.graph_time(g, 1)
+            us = c.graph_time(g, 3) / (3 * n)
+            c.graph_destroy(g)
+            quant[f"{src_name}_{clip_name}"] = {"us": round(us, 1), "GBps": round(moved / us / 1e3, 1),
+                                               "Gweights_per_s": round(rows * cols / us / 1e3, 2)}
+    out["affine_quantize_u4_9216x2560_g64"] = quant
     c.close()
     return out
 

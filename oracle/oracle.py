@@ -205,6 +205,26 @@ def affine_matvec_f64(packed, scales, biases, x_f32, rows, cols, group, dtype=F1
 # signed codec
 # ---------------------------------------------------------------------------
 
+
+def signed_validate(codes: np.ndarray, logical_count: int, fmt: int):
+    """(status, index of the first invalid code or -1) — SmeltSignedQuantCodec.swift:128-145"""
+    codes = np.ascontiguousarray(codes, np.uint8)
+    bad = C.c_int64(-1)
+    rc = lib().so_signed_validate_codes(_p(codes, np.uint8), codes.size, logical_count, fmt, C.byref(bad))
+    return rc, bad.value
+
+
+def signed_normalize_mlx(fmt: int, scales: np.ndarray, biases: np.ndarray):
+    """(status, canonical scale bits, failing group or -1) — SmeltSignedQuantCodec.swift:154-215"""
+    scales = np.ascontiguousarray(scales, np.uint16)
+    biases = np.ascontiguousarray(biases, np.uint16)
+    out = np.zeros(scales.shape, np.uint16)
+    bad = C.c_int(-1)
+    rc = lib().so_signed_normalize_mlx_scales(fmt, _p(scales, np.uint16), _p(biases, np.uint16), scales.size,
+                                              _p(out, np.uint16), C.byref(bad))
+    return rc, out, bad.value
+
+
 def signed_row_stride(padded_cols: int, fmt: int, align: int = 1) -> int:
     n = int(lib().so_signed_packed_byte_count(padded_cols, fmt))
     return (n + align - 1) // align * align

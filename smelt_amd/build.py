@@ -22,7 +22,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 instructions are switched off for all device code
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-HOST_SOURCES = ["runtime.cpp", "pipeline_table.cpp", "compiler.cpp"]
+HOST_SOURCES = ["runtime.cpp", "pipeline_table.cpp", "compiler.cpp", "import.cpp"]
 
 
 def _run(cmd: list[str]) -> None:

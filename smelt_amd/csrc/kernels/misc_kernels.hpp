@@ -129,13 +129,31 @@ SMELT_MISC_KERNEL void smelt_argmax16_partials(const uint16_t* logits, smelt::ui
     }
 }
 
+// Best key of row[0 .. n) over the workgroup's threads, four independent loads in flight per
+// thread (a one-load-per-iteration loop pays a full memory round trip per iteration).
+namespace smelt {
+__device__ __forceinline__ uint2_t strided_key_max(const uint2_t* row, uint32_t n) {
+    uint2_t best = {0u, 0u};
+    for (uint32_t base = threadIdx.x; base < n; base += 4 * blockDim.x) {
+        uint2_t v[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t i = base + j * blockDim.x;
+            v[j] = i < n ? row[i] : uint2_t{0u, 0u};
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) best = argmax_key_max(best, v[j]);
+    }
+    return best;
+}
+}  // namespace smelt
+
 // one block per batch row (blockIdx.x); partials are [batch, num_partials]
 SMELT_MISC_KERNEL void smelt_argmax_key_reduce(const smelt::uint2_t* partials, int* output,
                                                uint32_t num_partials) {
     using namespace smelt;
     const uint2_t* row = partials + (size_t)blockIdx.x * num_partials;
-    uint2_t best = {0u, 0u};
-    for (uint32_t i = threadIdx.x; i < num_partials; i += blockDim.x) best = argmax_key_max(best, row[i]);
+    uint2_t best = strided_key_max(row, num_partials);
     best = wave_argmax_key(best);
     __shared__ uint2_t wave_best[16];
     const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -154,8 +172,7 @@ SMELT_MISC_KERNEL void smelt_lm_head_argmax_reduce(const smelt::uint2_t* partial
     using namespace smelt;
     if (blockIdx.x >= batch) return;
     const uint2_t* row = partials + (size_t)blockIdx.x * num_partials;
-    uint2_t best = {0u, 0u};
-    for (uint32_t i = threadIdx.x; i < num_partials; i += blockDim.x) best = argmax_key_max(best, row[i]);
+    uint2_t best = strided_key_max(row, num_partials);
     best = wave_argmax_key(best);
     __shared__ uint2_t wave_best[16];
     const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;

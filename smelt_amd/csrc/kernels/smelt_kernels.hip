@@ -5,6 +5,7 @@
 #include "misc_kernels.hpp"
 #include "qmm.hpp"
 #include "qmm_skinny.hpp"
+#include "import_kernels.hpp"
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
@@ -30,3 +31,10 @@ SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, f16, smelt::F16)
 SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, bf16, smelt::BF16)
 SMELT_AFFINE_BANK(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_BANK(bf16, smelt::BF16, smelt::BF16)
+
+SMELT_AFFINE_QUANTIZE(f16, smelt::F16, 32)
+SMELT_AFFINE_QUANTIZE(f16, smelt::F16, 64)
+SMELT_AFFINE_QUANTIZE(f16, smelt::F16, 128)
+SMELT_AFFINE_QUANTIZE(bf16, smelt::BF16, 32)
+SMELT_AFFINE_QUANTIZE(bf16, smelt::BF16, 64)
+SMELT_AFFINE_QUANTIZE(bf16, smelt::BF16, 128)

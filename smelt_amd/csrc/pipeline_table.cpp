@@ -172,6 +172,20 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             *why = "Malformed specialized pipeline entry: '" + entry_in + "'";
             return kResolveMalformed;
         }
+        if (name == "affine_quantize_u4" || name == "affine_quantize_u4_weighted") {
+            // producer of the affine 4-bit layout: one kernel per group size, scales in the tagged type
+            if (cols == 0 || (group != 32 && group != 64 && group != 128)) {
+                *why = "affine quantiser kernels exist for groups of 32, 64 and 128 (got cols " +
+                       std::to_string(cols) + ", group " + std::to_string(group) + ")";
+                return kResolveMalformed;
+            }
+            out->family = kFamAffineQuantize;
+            out->symbol = "smelt_affine_quantize_g" + std::to_string(group) + "_" + t;
+            out->kinds = name == "affine_quantize_u4" ? "PPPPZUUU" : "PPPPPUUU";
+            out->appended = {cols, group};
+            out->kinds += "UU";
+            return kResolveOk;
+        }
         if (name == "affine_matvec") { out->family = kFamAffineMatvec; out->symbol = "smelt_affine_matvec_" + t; out->kinds = "PPPPPUUU"; }
         else if (name == "fused_affine_matvec_add") { out->family = kFamAffineAdd; out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; }
         else if (name == "fused_affine_gate_up_swiglu") { out->family = kFamAffineGateUp; out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; }
@@ -363,6 +377,8 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         out->family = kFamLmHeadReduce; out->symbol = "smelt_lm_head_argmax_reduce"; out->kinds = "PPUU";
         return kResolveOk;
     }
+    if (entry == "signed_validate_codes") { out->family = kFamSignedValidate; out->symbol = "smelt_signed_validate_codes"; out->kinds = "PPUUU"; return kResolveOk; }
+    if (entry == "signed_normalize_mlx_scales") { out->family = kFamSignedMlxScales; out->symbol = "smelt_signed_normalize_mlx_scales"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "copy_u128") { out->family = kFamCopy; out->symbol = "smelt_copy_u128"; out->kinds = "PPU"; return kResolveOk; }
     if (entry == "argmax_key_reduce") { out->family = kFamArgmaxReduce; out->symbol = "smelt_argmax_key_reduce"; out->kinds = "PPU"; return kResolveOk; }
 

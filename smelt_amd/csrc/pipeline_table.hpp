@@ -40,6 +40,9 @@ enum FamilyId {
     kFamArgmaxPartials,       // logits partials vocab chunk
     kFamArgmaxReduce,         // partials out num_partials
     kFamCopy,                 // src dst n16
+    kFamAffineQuantize,       // src packed scales biases [importance] rows src_dtype clip | cols group
+    kFamSignedValidate,       // codes status count_lo count_hi format
+    kFamSignedMlxScales,      // scales biases out status groups format
     kFamCount
 };
 
@@ -48,7 +51,8 @@ enum SignedFormat { kFmtNone = -1, kFmtBinary1 = 0, kFmtTernary2 = 1, kFmtTrit5 
 struct ResolvedPipeline {
     FamilyId family;
     std::string symbol;              // kernel symbol in the code object
-    std::string kinds;               // final argument kinds: 'P' pointer, 'U' u32, 'F' f32
+    std::string kinds;               // final argument kinds: 'P' pointer, 'U' u32, 'F' f32,
+                                     // 'Z' pointer the record does not bind (passed as null)
     std::vector<uint32_t> appended;  // values appended after the record's own bindings
     ActDType act;
     SignedFormat format = kFmtNone;

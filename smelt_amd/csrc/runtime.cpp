@@ -392,6 +392,43 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[1] = U(2) * 16; align[1] = 16; written[1] = true;
             break;
         }
+        case kFamAffineQuantize: {
+            // src packed scales biases importance rows src_dtype clip cols group
+            const size_t rows = U(5), dt = U(6), clip = U(7), cols = U(8), group = U(9);
+            if (dt > 2) return bad_geom("source dtype must be 0 (fp32), 1 (fp16) or 2 (bf16)");
+            if (clip > 1) return bad_geom("clip mode must be 0 (min/max) or 1 (least reconstruction error)");
+            if (rows == 0) return bad_geom("rows must be positive");
+            const size_t gpr = cdiv(cols, group);
+            if (rows * gpr >= ((size_t)1 << 31)) return bad_geom("more than 2^31 groups in one tensor");
+            const size_t waves = 128 / group;  // about 34 KB of staging per workgroup
+            if (L.block[0] != waves * 64 || L.block[1] != 1 || L.block[2] != 1 || L.grid[1] != 1 || L.grid[2] != 1)
+                return bad_geom("group " + std::to_string(group) + " quantiser runs with " + std::to_string(waves * 64) + "-thread workgroups in a 1-D grid");
+            need[0] = rows * cols * (dt == 0 ? 4 : 2); align[0] = dt == 0 ? 4 : 2;
+            need[1] = rows * cdiv(cols, 2); align[1] = 1; written[1] = true;
+            need[2] = rows * gpr * 2; written[2] = true;
+            need[3] = rows * gpr * 2; written[3] = true;
+            if (L.args[4].kind == 'P') { need[4] = cols * 4; align[4] = 4; }
+            L.lds = waves * (64 * (group + 1) + 128) * 4;
+            break;
+        }
+        case kFamSignedValidate: {
+            // codes status count_lo count_hi format
+            const size_t count = ((size_t)U(3) << 32) | U(2);
+            if (U(4) != 1 && U(4) != 2) return bad_geom("format must be 1 (ternary2) or 2 (trit5)");
+            need[0] = U(4) == 2 ? cdiv(count, 5) : cdiv(count * 2, 8); align[0] = 1;
+            need[1] = 8; align[1] = 8; written[1] = true;
+            if (L.grid[1] != 1 || L.grid[2] != 1 || L.block[1] != 1 || L.block[2] != 1) return bad_geom("1-D launch expected");
+            break;
+        }
+        case kFamSignedMlxScales: {
+            // scales biases out status groups format
+            if (U(5) > 1) return bad_geom("format must be 0 (binary1) or 1 (ternary2)");
+            need[0] = U(4) * 2; need[1] = U(4) * 2;
+            need[2] = U(4) * 2; written[2] = true;
+            need[3] = 8; align[3] = 8; written[3] = true;
+            if (L.grid[1] != 1 || L.grid[2] != 1 || L.block[1] != 1 || L.block[2] != 1) return bad_geom("1-D launch expected");
+            break;
+        }
         default:
             return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "pipeline '" + p.entry + "' has no launch validator");
     }
@@ -566,6 +603,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         a.value = p->res.appended[i];
     }
     for (size_t i = 0; i < L.args.size(); ++i)
+        if (L.args[i].kind == 0 && kinds[i] == 'Z') L.args[i].kind = 'Z';  // optional pointer: null
+    for (size_t i = 0; i < L.args.size(); ++i)
         if (L.args[i].kind == 0)
             return fail(ctx, SMELT_HIP_ERR_BINDING_MISMATCH, "pipeline '" + p->entry + "': argument " + std::to_string(i) + " is not bound by the record");
 
@@ -608,7 +647,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     alignas(16) unsigned char kernarg[512];
     size_t pos = 0;
     for (const Arg& a : L.args) {
-        if (a.kind == 'P') {
+        if (a.kind == 'P' || a.kind == 'Z') {
             pos = (pos + 7) & ~(size_t)7;
             void* ptr = a.ptr;
             memcpy(kernarg + pos, &ptr, 8);
