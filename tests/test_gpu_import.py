@@ -244,3 +244,66 @@ def test_device_resident_quantiser_pipeline_and_bad_launches():
             ctx.pipeline(f"affine_quantize_u4:{cols}:48")
     finally:
         ctx.close()
+
+
+def test_package_built_on_the_gpu_reads_back_and_decodes(imp, tmp_path):
+    """checkpoint tensors -> GPU producers -> weights.bin + manifest.json -> reader -> upload ->
+    matvec records: every stage against the oracle."""
+    import gpu_harness as gh
+    from smelt_amd import compiler as cc
+    from smelt_amd import package as pk
+    rows, cols = 96, 512
+    w = weights(21, rows, cols)
+    rng = fx.rng_for(84, 0)
+    codes = rng.integers(0, 3, (rows, cols)).astype(np.uint8)
+    ter_packed = so.signed_pack(codes, so.TERNARY2)
+    mlx_scale = so.narrow(np.abs(rng.normal(0, 0.03, (rows, cols // 128))).astype(np.float32) + 1e-3, so.F16)
+    mlx_bias = so.narrow(-so.widen(mlx_scale, so.F16), so.F16)
+    b = pk.PackageBuilder()
+    b.add_affine_u4("layers.0.q_proj.weight", imp, w, im.SRC_F32, rows, cols, 64)
+    b.add_signed("layers.0.o_proj.weight", imp, ter_packed, mlx_scale, mlx_bias, rows, cols, cc.TERNARY2)
+    b.add_dense("norm.weight", np.ones(cols, np.float16), cc.FP16)
+    b.write(str(tmp_path))
+    pw = pk.PackageWeights(str(tmp_path))
+    ref_q = so.affine_quantize(w, 64, 0, None, so.F16)
+    assert np.array_equal(pw.region("layers.0.q_proj.weight").reshape(rows, -1), ref_q[0])
+    assert np.array_equal(pw.region("layers.0.q_proj.weight", "scales").view(np.uint16).reshape(rows, -1), ref_q[1])
+    assert np.array_equal(pw.region("layers.0.q_proj.weight", "biases").view(np.uint16).reshape(rows, -1), ref_q[2])
+    assert np.array_equal(pw.region("layers.0.o_proj.weight", "scales").view(np.uint16).reshape(rows, -1), mlx_scale)
+    # a ternary tensor with a forbidden code never reaches the file
+    bad = ter_packed.copy()
+    bad[5, 7] |= 0xC0
+    with pytest.raises(im.ImportError_) as e:
+        pk.PackageBuilder().add_signed("x", imp, bad, mlx_scale, mlx_bias, rows, cols, cc.TERNARY2)
+    assert e.value.index == 5 * cols + 7 * 4 + 3
+    ctx = rt.Context()
+    try:
+        pw.upload(ctx, gh.WEIGHTS_SLOT)
+        x = so.narrow(rng.normal(0, 1, (1, cols)).astype(np.float32), so.F16)
+        ctx.put(gh.X_SLOT, x)
+        ctx.alloc(gh.Y_SLOT, rows * 2)
+        em = cc.Emitter(rt.ACT_F16, ctx.device_info()["compute_units"])
+        eq, eo = pw.entry("layers.0.q_proj.weight"), pw.entry("layers.0.o_proj.weight")
+        em.matvec(gh.WEIGHTS_SLOT, eq, cc.bind(gh.X_SLOT), cc.bind(gh.Y_SLOT))
+        em.install(ctx)
+        ctx.interpret_decode(em.records())
+        ctx.wait()
+        got = ctx.read(gh.Y_SLOT, np.uint16, rows)
+        gh.check_outputs(got, so.affine_matvec(*ref_q, so.widen(x, so.F16)[0], rows, cols, 64, so.F16), so.F16, "q_proj from package")
+    finally:
+        ctx.close()
+    ctx = rt.Context()
+    try:
+        pw.upload(ctx, gh.WEIGHTS_SLOT)
+        ctx.put(gh.X_SLOT, x)
+        ctx.alloc(gh.Y_SLOT, rows * 2)
+        em = cc.Emitter(rt.ACT_F16, ctx.device_info()["compute_units"])
+        em.matvec(gh.WEIGHTS_SLOT, eo, cc.bind(gh.X_SLOT), cc.bind(gh.Y_SLOT))
+        em.install(ctx)
+        ctx.interpret_decode(em.records())
+        ctx.wait()
+        got = ctx.read(gh.Y_SLOT, np.uint16, rows)
+        ref = so.signed_matvec(so.TERNARY2, ter_packed, mlx_scale, so.widen(x, so.F16)[0], rows, cols, cols, 128)
+        gh.check_outputs(got, ref, so.F16, "o_proj from package")
+    finally:
+        ctx.close()
