@@ -151,6 +151,20 @@ int smelt_emit_bank_matvec(smelt_emitter *e, int weights_slot, const SmeltWeight
 int smelt_emit_lm_head_argmax(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w,
                               SmeltBinding input, SmeltBinding partial_keys, SmeltBinding token_out,
                               int batch_size, float logit_cap);
+/* emitRMSNorm1PW (SmeltCodeEmitter.swift:2837-2872) and its batched / residual forms: one
+ * threadgroup per token.  eps == 1e-6 selects the fixed-dimension pipeline
+ * "rms_norm_1pw_d{dim}[_add][_batched]" (no constants); any other eps the generic
+ * "rms_norm_1pw[_batched]" with dim and eps as constants 3 and 4 (no residual form exists for it).
+ * `weight` is [dim] 16-bit values (a delta from 1); residual may be NULL. */
+int smelt_emit_rms_norm_1pw(smelt_emitter *e, SmeltBinding input, SmeltBinding weight,
+                            SmeltBinding output, const SmeltBinding *residual, int dim, float eps,
+                            int batch_size);
+/* emitElementwiseAdd (SmeltCodeEmitter.swift:2944-2966) / elementwise_mul: dispatchThreads over count */
+int smelt_emit_elementwise(smelt_emitter *e, int multiply, SmeltBinding a, SmeltBinding b,
+                           SmeltBinding output, int count);
+/* staged swiglu_fused over `count` gate / up values (DenseTrunkEmitter.swift:209) */
+int smelt_emit_swiglu_fused(smelt_emitter *e, SmeltBinding gate, SmeltBinding up,
+                            SmeltBinding output, int count);
 /* swap cur/alt (SmeltDispatchRecord.swap) */
 int smelt_emit_swap(smelt_emitter *e);
 

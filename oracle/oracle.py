@@ -88,6 +88,10 @@ def _declare(l: C.CDLL) -> None:
         "so_epilogue_residual_add": (u16, [f32, u16, i32]),
         "so_epilogue_affine_swiglu": (u16, [f32, f32, i32]),
         "so_epilogue_signed_swiglu": (u16, [u16, u16, i32]),
+        "so_rms_scale": (f32, [vp, i32, f32, i32]),
+        "so_rms_norm_1pw": (None, [vp, vp, vp, i32, f32, i32, i32, vp]),
+        "so_swiglu_fused": (None, [vp, vp, i32, i32, vp]),
+        "so_elementwise": (None, [vp, vp, i32, i32, i32, vp]),
         "so_argmax_ordered_key16": (u32, [u16]),
         "so_argmax_pack_key": (C.c_uint64, [u16, u32]),
         "so_argmax16": (i32, [vp, i32]),
@@ -328,3 +332,38 @@ def epilogue_signed_swiglu(gate_bits: np.ndarray, up_bits: np.ndarray, dtype: in
     return np.array([l.so_epilogue_signed_swiglu(int(g), int(u), dtype)
                      for g, u in zip(np.ravel(gate_bits), np.ravel(up_bits))],
                     dtype=np.uint16).reshape(np.shape(gate_bits))
+
+
+# ---------------------------------------------------------------------------
+# layer ops between the matvecs (norms.metal, activations_precise.metal, activations.metal)
+# ---------------------------------------------------------------------------
+
+def rms_scale(x_bits: np.ndarray, eps: float, dtype: int) -> float:
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    return float(lib().so_rms_scale(_p(x, np.uint16), x.size, eps, dtype))
+
+
+def rms_norm_1pw(x_bits, w_bits, eps: float, dtype: int, two_step: bool, residual_bits=None) -> np.ndarray:
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    w = np.ascontiguousarray(w_bits, np.uint16)
+    out = np.zeros(x.size, np.uint16)
+    res = None if residual_bits is None else np.ascontiguousarray(residual_bits, np.uint16)
+    lib().so_rms_norm_1pw(_p(x, np.uint16), _p(w, np.uint16), None if res is None else _p(res, np.uint16),
+                          x.size, eps, dtype, int(two_step), _p(out, np.uint16))
+    return out
+
+
+def swiglu_fused(gate_bits, up_bits, dtype: int) -> np.ndarray:
+    g = np.ascontiguousarray(gate_bits, np.uint16)
+    u = np.ascontiguousarray(up_bits, np.uint16)
+    out = np.zeros(g.size, np.uint16)
+    lib().so_swiglu_fused(_p(g, np.uint16), _p(u, np.uint16), g.size, dtype, _p(out, np.uint16))
+    return out
+
+
+def elementwise(a_bits, b_bits, dtype: int, multiply: bool = False) -> np.ndarray:
+    a = np.ascontiguousarray(a_bits, np.uint16)
+    b = np.ascontiguousarray(b_bits, np.uint16)
+    out = np.zeros(a.size, np.uint16)
+    lib().so_elementwise(_p(a, np.uint16), _p(b, np.uint16), a.size, dtype, int(multiply), _p(out, np.uint16))
+    return out

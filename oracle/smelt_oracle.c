@@ -623,6 +623,56 @@ SO_EXPORT uint16_t so_epilogue_signed_swiglu(uint16_t gate_bits, uint16_t up_bit
 }
 
 /* ------------------------------------------------------------------------- */
+/* Layer ops between the matvecs                                               */
+/* ------------------------------------------------------------------------- */
+
+/* 1 / sqrt(mean(x^2) + eps), fp32, summed in index order
+ * (CPU mirror: Tests/SmeltCompilerTests/Helpers/MetalKernelTestSupport.swift:233-235;
+ *  kernels: Resources/Shaders/norms.metal:991-1020). */
+SO_EXPORT float so_rms_scale(const uint16_t *x, int n, float eps, int dtype) {
+    float sum = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        float v = widen(x[i], dtype);
+        sum += v * v;
+    }
+    return 1.0f / sqrtf(sum / (float)n + eps);
+}
+
+/* rms_norm_1pw: x * rs * (1 + w) in the 16-bit type.
+ * two_step != 0: half(1 + w) * half(x * rs) (norms.metal:54-62, 1537-1545);
+ * two_step == 0: half(x * (rs * (1 + w))) (the fixed-dimension kernels, norms.metal:164-170).
+ * residual (may be NULL) is added to the rounded result in the 16-bit type (norms.metal:412-445). */
+SO_EXPORT void so_rms_norm_1pw(const uint16_t *x, const uint16_t *w, const uint16_t *residual, int n,
+                               float eps, int dtype, int two_step, uint16_t *out) {
+    float rs = so_rms_scale(x, n, eps, dtype);
+    for (int i = 0; i < n; ++i) {
+        float v = widen(x[i], dtype), wt = widen(w[i], dtype);
+        uint16_t y;
+        if (two_step) {
+            float normalized = so_round_through(v * rs, dtype);
+            float direct = so_round_through(1.0f + wt, dtype);
+            y = narrow(direct * normalized, dtype);
+        } else {
+            float scale = rs * (1.0f + wt);
+            y = narrow(v * scale, dtype);
+        }
+        if (residual) y = narrow(widen(y, dtype) + widen(residual[i], dtype), dtype);
+        out[i] = y;
+    }
+}
+
+/* swiglu_fused (activations_precise.metal:9-22), elementwise_add / _mul (activations.metal:56-66, 85-95) */
+SO_EXPORT void so_swiglu_fused(const uint16_t *gate, const uint16_t *up, int n, int dtype, uint16_t *out) {
+    for (int i = 0; i < n; ++i) out[i] = so_epilogue_signed_swiglu(gate[i], up[i], dtype);
+}
+SO_EXPORT void so_elementwise(const uint16_t *a, const uint16_t *b, int n, int dtype, int multiply, uint16_t *out) {
+    for (int i = 0; i < n; ++i) {
+        float x = widen(a[i], dtype), y = widen(b[i], dtype);
+        out[i] = narrow(multiply ? x * y : x + y, dtype);
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* Argmax key — lut_matvec.metal:4045-4074                                     */
 /* ------------------------------------------------------------------------- */
 

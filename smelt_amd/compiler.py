@@ -78,6 +78,9 @@ def lib() -> C.CDLL:
         "smelt_emit_dual_matvec": (i32, [vp, i32, we, we, Binding, Binding, Binding]),
         "smelt_emit_lm_head_argmax": (i32, [vp, i32, we, Binding, Binding, Binding, i32, C.c_float]),
         "smelt_emit_swap": (i32, [vp]),
+        "smelt_emit_rms_norm_1pw": (i32, [vp, Binding, Binding, Binding, C.POINTER(Binding), i32, C.c_float, i32]),
+        "smelt_emit_elementwise": (i32, [vp, i32, Binding, Binding, Binding, i32]),
+        "smelt_emit_swiglu_fused": (i32, [vp, Binding, Binding, Binding, i32]),
         "smelt_emitter_record_count": (sz, [vp]),
         "smelt_emitter_records": (C.POINTER(rt.DispatchRecord), [vp]),
         "smelt_emitter_pipeline_count": (sz, [vp]),
@@ -249,6 +252,19 @@ class Emitter:
     def lm_head_argmax(self, weights_slot, w, x, keys, out, batch=1, logit_cap=0.0):
         self._check(self.l.smelt_emit_lm_head_argmax(self.h, weights_slot, C.byref(w), x, keys, out, batch,
                                                      C.c_float(logit_cap)))
+
+    def rms_norm_1pw(self, x, weight, y, dim, eps=1e-6, batch=1, residual=None):
+        res = None if residual is None else C.byref(residual)
+        self._check(self.l.smelt_emit_rms_norm_1pw(self.h, x, weight, y, res, dim, C.c_float(eps), batch))
+
+    def elementwise_add(self, a, b, y, count):
+        self._check(self.l.smelt_emit_elementwise(self.h, 0, a, b, y, count))
+
+    def elementwise_mul(self, a, b, y, count):
+        self._check(self.l.smelt_emit_elementwise(self.h, 1, a, b, y, count))
+
+    def swiglu_fused(self, gate, up, y, count):
+        self._check(self.l.smelt_emit_swiglu_fused(self.h, gate, up, y, count))
 
     def swap(self):
         self._check(self.l.smelt_emit_swap(self.h))

@@ -436,6 +436,60 @@ void smelt_emitter_destroy(smelt_emitter* e) { delete e; }
 
 const char* smelt_emitter_last_error(const smelt_emitter* e) { return e ? e->error.c_str() : ""; }
 
+int smelt_emit_rms_norm_1pw(smelt_emitter* e, SmeltBinding input, SmeltBinding weight, SmeltBinding output,
+                            const SmeltBinding* residual, int dim, float eps, int batch_size) {
+    if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (dim <= 0 || batch_size <= 0) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "rms norm needs positive dim and batch");
+    const bool fixed = eps == 1e-6f;
+    if (residual && !fixed) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "the residual form of rms_norm_1pw exists for eps 1e-6 only");
+    RecordBuilder rb;
+    rb.buffer(0, input);
+    rb.buffer(1, weight);
+    std::string name = "rms_norm_1pw";
+    if (fixed) name += "_d" + std::to_string(dim);
+    if (residual) {
+        rb.buffer(2, *residual);
+        rb.buffer(3, output);
+        name += "_add";
+    } else {
+        rb.buffer(2, output);
+    }
+    if (batch_size > 1) name += "_batched";
+    if (!fixed) {
+        rb.constant(3, (uint32_t)dim);
+        rb.constant_f32(4, eps);
+    }
+    // whole waves, eight elements per thread, at most 1024 threads
+    const int threads = std::min(1024, std::max(64, ((dim + 7) / 8 + 63) / 64 * 64));
+    rb.grid((uint32_t)batch_size, 1, 1, (uint32_t)threads);
+    rb.r.pipeline = e->pipeline_index(name);
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+static int emit_pointwise(smelt_emitter* e, const char* name, SmeltBinding a, SmeltBinding b, SmeltBinding output, int count) {
+    if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (count <= 0) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "element count must be positive");
+    RecordBuilder rb;
+    rb.buffer(0, a);
+    rb.buffer(1, b);
+    rb.buffer(2, output);
+    rb.constant(3, (uint32_t)count);
+    rb.r.style = SMELT_STYLE_THREADS;   // the grid counts threads (dispatchThreads)
+    rb.grid((uint32_t)count, 1, 1, (uint32_t)std::min(count, 1024));
+    rb.r.pipeline = e->pipeline_index(name);
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+int smelt_emit_elementwise(smelt_emitter* e, int multiply, SmeltBinding a, SmeltBinding b, SmeltBinding output, int count) {
+    return emit_pointwise(e, multiply ? "elementwise_mul" : "elementwise_add", a, b, output, count);
+}
+
+int smelt_emit_swiglu_fused(smelt_emitter* e, SmeltBinding gate, SmeltBinding up, SmeltBinding output, int count) {
+    return emit_pointwise(e, "swiglu_fused", gate, up, output, count);
+}
+
 int smelt_emit_swap(smelt_emitter* e) {
     if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
     RecordBuilder rb;

@@ -6,6 +6,7 @@
 #include "qmm.hpp"
 #include "qmm_skinny.hpp"
 #include "import_kernels.hpp"
+#include "layer_kernels.hpp"
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
@@ -38,3 +39,6 @@ SMELT_AFFINE_QUANTIZE(f16, smelt::F16, 128)
 SMELT_AFFINE_QUANTIZE(bf16, smelt::BF16, 32)
 SMELT_AFFINE_QUANTIZE(bf16, smelt::BF16, 64)
 SMELT_AFFINE_QUANTIZE(bf16, smelt::BF16, 128)
+
+SMELT_LAYER_KERNELS(f16, smelt::F16)
+SMELT_LAYER_KERNELS(bf16, smelt::BF16)

@@ -377,6 +377,54 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         out->family = kFamLmHeadReduce; out->symbol = "smelt_lm_head_argmax_reduce"; out->kinds = "PPUU";
         return kResolveOk;
     }
+    // ---- layer ops between the matvecs: norms.metal, activations_precise.metal, activations.metal ----
+    {
+        auto eps_bits = [](float e) { uint32_t b; memcpy(&b, &e, 4); return b; };
+        auto strip = [](std::string& s, const char* suffix) {
+            const size_t n = strlen(suffix);
+            if (s.size() >= n && s.compare(s.size() - n, n, suffix) == 0) { s.resize(s.size() - n); return true; }
+            return false;
+        };
+        if (starts_with(entry, "rms_norm_1pw")) {
+            std::string rest = entry.substr(12);
+            strip(rest, "_batched");            // batch rows are the grid width either way
+            const bool add = strip(rest, "_add");
+            uint32_t dim = 0;
+            bool ok = rest.empty();
+            if (!ok && starts_with(rest, "_d") && parse_uint(rest.substr(2), &dim) && dim > 0) ok = true;
+            if (ok && !(add && dim == 0)) {
+                out->family = add ? kFamRmsNormAdd : kFamRmsNorm;
+                out->symbol = std::string(add ? "smelt_rms_norm_1pw_add_" : "smelt_rms_norm_1pw_") + t;
+                if (dim == 0) { out->kinds = "PPPUFU"; out->appended = {1u}; }                  // dim, eps from the record
+                else { out->kinds = add ? "PPPPUUU" : "PPPUUU"; out->appended = {dim, eps_bits(1e-6f), 0u}; }
+                return kResolveOk;
+            }
+        }
+        if (starts_with(entry, "rms_norm_scale_only")) {
+            std::string rest = entry.substr(19);
+            strip(rest, "_batched");
+            const bool eps5 = strip(rest, "_eps1e5");
+            uint32_t dim = 0;
+            if (rest.empty() || rest == "_precise") {
+                out->family = kFamRmsScale; out->symbol = "smelt_rms_norm_scale_only_" + t; out->kinds = "PPUF";
+                return kResolveOk;
+            }
+            if (starts_with(rest, "_d") && parse_uint(rest.substr(2), &dim) && dim > 0) {
+                out->family = kFamRmsScale; out->symbol = "smelt_rms_norm_scale_only_" + t; out->kinds = "PPUU";
+                out->appended = {dim, eps_bits(eps5 ? 1e-5f : 1e-6f)};
+                return kResolveOk;
+            }
+        }
+        if (entry == "residual_add_rms_norm_scale_only_precise") {
+            out->family = kFamResidualAddRmsScale; out->symbol = "smelt_residual_add_rms_norm_scale_only_" + t; out->kinds = "PPPPUF";
+            return kResolveOk;
+        }
+        if (entry == "swiglu_fused" || entry == "elementwise_add" || entry == "elementwise_mul") {
+            out->family = kFamElementwise; out->symbol = "smelt_" + entry + "_" + t; out->kinds = "PPPU";
+            return kResolveOk;
+        }
+        if (entry == "buffer_copy") { out->family = kFamCopy16; out->symbol = "smelt_buffer_copy16"; out->kinds = "PPU"; return kResolveOk; }
+    }
     if (entry == "signed_validate_codes") { out->family = kFamSignedValidate; out->symbol = "smelt_signed_validate_codes"; out->kinds = "PPUUU"; return kResolveOk; }
     if (entry == "signed_normalize_mlx_scales") { out->family = kFamSignedMlxScales; out->symbol = "smelt_signed_normalize_mlx_scales"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "copy_u128") { out->family = kFamCopy; out->symbol = "smelt_copy_u128"; out->kinds = "PPU"; return kResolveOk; }

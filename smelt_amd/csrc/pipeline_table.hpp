@@ -43,6 +43,12 @@ enum FamilyId {
     kFamAffineQuantize,       // src packed scales biases [importance] rows src_dtype clip | cols group
     kFamSignedValidate,       // codes status count_lo count_hi format
     kFamSignedMlxScales,      // scales biases out status groups format
+    kFamRmsNorm,              // x w y | dim eps two_step            (grid.x = token row)
+    kFamRmsNormAdd,           // x w res y | dim eps two_step
+    kFamRmsScale,             // x scale | dim eps
+    kFamResidualAddRmsScale,  // a b out scale dim eps
+    kFamElementwise,          // a b out count
+    kFamCopy16,               // src dst count
     kFamCount
 };
 

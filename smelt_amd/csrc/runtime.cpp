@@ -392,6 +392,41 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[1] = U(2) * 16; align[1] = 16; written[1] = true;
             break;
         }
+        case kFamRmsNorm:
+        case kFamRmsNormAdd:
+        case kFamRmsScale:
+        case kFamResidualAddRmsScale: {
+            // one workgroup per token row; the row is staged in LDS
+            const bool norm = r.family == kFamRmsNorm || r.family == kFamRmsNormAdd;
+            const size_t first_u = r.family == kFamRmsNorm ? 3 : (r.family == kFamRmsScale ? 2 : 4);
+            const size_t dim = U(first_u), tokens = L.grid[0];
+            if (dim == 0) return bad_geom("dim must be positive");
+            if (L.block[0] % 64 != 0 || L.block[1] != 1 || L.block[2] != 1 || L.grid[1] != 1 || L.grid[2] != 1)
+                return bad_geom("norm kernels run whole waves in a 1-D launch, one workgroup per token");
+            const size_t row = tokens * dim * 2;
+            if (norm) {
+                need[0] = row; need[1] = dim * 2;
+                if (r.family == kFamRmsNormAdd) { need[2] = row; need[3] = row; written[3] = true; }
+                else { need[2] = row; written[2] = true; }
+            } else if (r.family == kFamRmsScale) {
+                need[0] = row; need[1] = tokens * 4; align[1] = 4; written[1] = true;
+            } else {
+                need[0] = row; need[1] = row; need[2] = row; written[2] = true;
+                need[3] = tokens * 4; align[3] = 4; written[3] = true;
+            }
+            L.lds = 64 + dim * 2;
+            break;
+        }
+        case kFamElementwise:
+        case kFamCopy16: {
+            const size_t ci = r.family == kFamCopy16 ? 2 : 3;
+            const size_t count = U(ci);
+            if (L.block[1] != 1 || L.block[2] != 1 || L.grid[1] != 1 || L.grid[2] != 1) return bad_geom("1-D launch expected");
+            if ((size_t)L.grid[0] * L.block[0] < count) return bad_geom("grid covers " + std::to_string((size_t)L.grid[0] * L.block[0]) + " of " + std::to_string(count) + " elements");
+            for (size_t i = 0; i < ci; ++i) need[i] = count * 2;
+            written[ci - 1] = true;
+            break;
+        }
         case kFamAffineQuantize: {
             // src packed scales biases importance rows src_dtype clip cols group
             const size_t rows = U(5), dt = U(6), clip = U(7), cols = U(8), group = U(9);

@@ -131,6 +131,16 @@ def test_pipeline_names_resolve_to_kernels_with_the_reference_binding_counts():
         "signed_ternary_affine_bank4_matvec_g128_rows8": ("smelt_teraff_bank4_matvec_f16", 8, 5),
         "signed_binary_embedding_gather_g128": ("smelt_signed_binary_embedding_gather_f16", 4, 1),
         "affine_matvec_argmax_c2560_r262144_g128_batched": ("smelt_affine_matvec_argmax_f16", 5, 2),
+        # layer ops between the matvecs (SmeltKernelCatalog.swift:630, 700-707, 964, 1312, 1966, 3004-3014)
+        "rms_norm_1pw": ("smelt_rms_norm_1pw_f16", 3, 2),
+        "rms_norm_1pw_batched": ("smelt_rms_norm_1pw_f16", 3, 2),
+        "rms_norm_1pw_d1024": ("smelt_rms_norm_1pw_f16", 3, 0),
+        "rms_norm_1pw_d1536_add_batched": ("smelt_rms_norm_1pw_add_f16", 4, 0),
+        "rms_norm_scale_only_precise": ("smelt_rms_norm_scale_only_f16", 2, 2),
+        "rms_norm_scale_only_d2048_eps1e5_batched": ("smelt_rms_norm_scale_only_f16", 2, 0),
+        "residual_add_rms_norm_scale_only_precise": ("smelt_residual_add_rms_norm_scale_only_f16", 4, 2),
+        "swiglu_fused": ("smelt_swiglu_fused_f16", 3, 1),
+        "elementwise_add": ("smelt_elementwise_add_f16", 3, 1),
     }
     for entry, (symbol, nbuf, nconst) in cases.items():
         rc, sym, kinds = cc.resolve_pipeline_name(entry)
@@ -142,7 +152,8 @@ def test_pipeline_names_resolve_to_kernels_with_the_reference_binding_counts():
     assert cc.resolve_pipeline_name("affine_matvec:1024")[0] == -3        # malformed entry
     assert cc.resolve_pipeline_name("affine_matvec:10:64")[0] == -3       # cols not a multiple of 32
     assert cc.resolve_pipeline_name("fused_lut_matvec:1024:64")[0] == -4  # u4_lut is out of scope
-    assert cc.resolve_pipeline_name("rms_norm_1pw")[0] == -4
+    assert cc.resolve_pipeline_name("rms_norm_1pw_from_fp32")[0] == -4     # fp32 hidden states are out of scope
+    assert cc.resolve_pipeline_name("rope_apply")[0] == -4
 
 
 def test_emitters_bind_what_the_reference_emitters_bind():

@@ -1,0 +1,89 @@
+"""Pins of the oracle's layer ops (RMS norm with the 1 + weight convention, staged SwiGLU,
+elementwise add / multiply): closed forms, invariants and an independent restatement in numpy's
+own float16 arithmetic, chosen so that a dropped eps, a missing "1 +", a wrong mean or a moved
+rounding point fails at least one of them."""
+import numpy as np
+
+import fixtures as fx
+from oracle import oracle as so
+
+
+def f16(v):
+    return so.narrow(np.asarray(v, np.float32), so.F16)
+
+
+def test_rms_scale_closed_forms():
+    assert so.rms_scale(f16(np.ones(64)), 0.0, so.F16) == 1.0
+    assert so.rms_scale(f16(np.full(48, -4.0)), 0.0, so.F16) == 0.25                 # 1 / sqrt(mean(16))
+    x = np.zeros(100, np.float32); x[0] = 10.0                                       # mean = 100 / 100
+    assert so.rms_scale(f16(x), 0.0, so.F16) == 1.0
+    assert so.rms_scale(f16(np.zeros(8)), 0.25, so.F16) == 2.0                       # eps is under the root
+    assert abs(so.rms_scale(f16(np.ones(8)), 3.0, so.F16) - 0.5) < 1e-7              # ... and added to the mean
+    assert so.rms_scale(so.narrow(np.full(16, 2.0, np.float32), so.BF16), 0.0, so.BF16) == 0.5
+
+
+def test_rms_norm_closed_forms_and_invariants():
+    n = 256
+    x = np.where(np.arange(n) % 2 == 0, 0.5, -0.5).astype(np.float32)
+    zero = f16(np.zeros(n))
+    for two_step in (False, True):
+        out = so.widen(so.rms_norm_1pw(f16(x), zero, 0.0, so.F16, two_step), so.F16)
+        assert np.array_equal(out, np.sign(x))                                       # unit RMS, weight 1 + 0
+        out = so.widen(so.rms_norm_1pw(f16(x), f16(np.ones(n)), 0.0, so.F16, two_step), so.F16)
+        assert np.array_equal(out, 2 * np.sign(x))                                   # the stored weight is a delta from 1
+        out = so.widen(so.rms_norm_1pw(f16(x), f16(np.full(n, -1.0)), 0.0, so.F16, two_step), so.F16)
+        assert not out.any()
+        rng = fx.rng_for(90, int(two_step))
+        r = rng.normal(0, 1, n).astype(np.float32)
+        w = rng.normal(0, 0.2, n).astype(np.float32)
+        a = so.rms_norm_1pw(f16(r), f16(w), 0.0, so.F16, two_step)
+        b = so.rms_norm_1pw(f16(4 * so.widen(f16(r), so.F16)), f16(w), 0.0, so.F16, two_step)
+        assert np.array_equal(a, b)                                                  # scale invariance for powers of two
+        res = f16(rng.normal(0, 1, n))
+        with_res = so.rms_norm_1pw(f16(r), f16(w), 1e-6, so.F16, two_step, res)
+        plain = so.rms_norm_1pw(f16(r), f16(w), 1e-6, so.F16, two_step)
+        assert np.array_equal(with_res.view(np.float16), (plain.view(np.float16) + res.view(np.float16)))
+
+
+def test_rms_norm_against_numpy_float16_arithmetic():
+    """Independent restatement: numpy's float16 type performs the half multiplies and roundings."""
+    rng = fx.rng_for(91, 0)
+    for n in (64, 1000, 2560):
+        xb, wb = f16(rng.normal(0, 2, n)), f16(rng.normal(0, 0.3, n))
+        x32, w32 = xb.view(np.float16).astype(np.float32), wb.view(np.float16).astype(np.float32)
+        rs = np.float32(so.rms_scale(xb, 1e-6, so.F16))
+        exact = 1.0 / np.sqrt(np.mean(x32.astype(np.float64) ** 2) + 1e-6)
+        assert abs(float(rs) - exact) <= 2e-6 * exact                             # fp32 running sum
+        two = (np.float32(1.0) + w32).astype(np.float16) * (x32 * rs).astype(np.float16)
+        assert np.array_equal(so.rms_norm_1pw(xb, wb, 1e-6, so.F16, True), two.view(np.uint16))
+        one = (x32 * (rs * (np.float32(1.0) + w32))).astype(np.float16)
+        assert np.array_equal(so.rms_norm_1pw(xb, wb, 1e-6, so.F16, False), one.view(np.uint16))
+        # the two rounding conventions stay within two 16-bit ulps of each other
+        d = np.abs(two.astype(np.float64) - one.astype(np.float64))
+        assert np.all(d <= 2 * np.spacing(np.abs(one).astype(np.float16)).astype(np.float64))
+
+
+def test_swiglu_fused_closed_forms_and_numpy_float16():
+    assert so.swiglu_fused(f16([0.0]), f16([3.0]), so.F16)[0] == 0                    # silu(0) = 0
+    big = so.widen(so.swiglu_fused(f16([12.0, -12.0]), f16([0.5, 0.5]), so.F16), so.F16)
+    assert big[0] == 6.0 and abs(big[1]) < 1e-3                                      # sigmoid saturates to 1 / ~0
+    one = so.widen(so.swiglu_fused(f16([1.0]), f16([1.0]), so.F16), so.F16)[0]
+    assert abs(one - 0.7310585786) < 1e-3                                            # 1 * sigmoid(1)
+    rng = fx.rng_for(92, 0)
+    g, u = f16(rng.normal(0, 3, 4096)), f16(rng.normal(0, 1, 4096))
+    gh, uh = g.view(np.float16), u.view(np.float16)
+    h1 = np.float16(1.0)
+    tail = h1 / (h1 + np.exp(np.abs(gh)))            # float16 in, float16 out at every step
+    sig = np.where(gh < 0, tail, h1 - tail).astype(np.float16)
+    ref = ((gh * sig).astype(np.float16) * uh).astype(np.float16)
+    got = so.swiglu_fused(g, u, so.F16).view(np.float16)
+    ulp = np.spacing(np.abs(ref)).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - ref.astype(np.float64)) <= ulp)    # exp may differ in its last bit
+    assert np.mean(got.view(np.uint16) == ref.view(np.uint16)) > 0.995
+
+
+def test_elementwise_matches_numpy_float16():
+    rng = fx.rng_for(93, 0)
+    a, b = f16(rng.normal(0, 100, 5000)), f16(rng.normal(0, 0.01, 5000))
+    assert np.array_equal(so.elementwise(a, b, so.F16).view(np.float16), a.view(np.float16) + b.view(np.float16))
+    assert np.array_equal(so.elementwise(a, b, so.F16, True).view(np.float16), a.view(np.float16) * b.view(np.float16))
