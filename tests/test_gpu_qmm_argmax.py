@@ -379,7 +379,7 @@ def test_bad_records_are_rejected_before_launch(ctx):
         ctx.pipeline("causal_gqa_attn_cached_f32")
     assert e.value.code == -4
     # a missing function becomes a fallback-to-previous slot when the package allows it
-    idx = ctx.pipeline("rms_norm_1pw", allow_missing=True)
+    idx = ctx.pipeline("rope_apply_f32", allow_missing=True)
     assert not ctx.pipeline_ready(idx)
     # everything still works afterwards
     assert ctx.encode_decode(rt.make_record(pipe, good, [(5, rows)], (8, 1, 1), (256, 1, 1))) == 1
