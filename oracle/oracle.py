@@ -92,6 +92,11 @@ def _declare(l: C.CDLL) -> None:
         "so_rms_norm_1pw": (None, [vp, vp, vp, i32, f32, i32, i32, vp]),
         "so_swiglu_fused": (None, [vp, vp, i32, i32, vp]),
         "so_elementwise": (None, [vp, vp, i32, i32, i32, vp]),
+        "so_bitplane_max_q": (i32, [i32]),
+        "so_signed_activation_bitplanes": (None, [vp, i32, i32, i32, vp, vp, vp]),
+        "so_swiglu_signed_activation_bitplanes": (None, [vp, vp, i32, i32, i32, vp, vp]),
+        "so_norm_scale_signed_activation_bitplanes": (None, [f32, vp, vp, i32, i32, i32, vp, vp]),
+        "so_signed_bitplane_matvec": (None, [i32, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
         "so_argmax_ordered_key16": (u32, [u16]),
         "so_argmax_pack_key": (C.c_uint64, [u16, u32]),
         "so_argmax16": (i32, [vp, i32]),
@@ -366,4 +371,51 @@ def elementwise(a_bits, b_bits, dtype: int, multiply: bool = False) -> np.ndarra
     b = np.ascontiguousarray(b_bits, np.uint16)
     out = np.zeros(a.size, np.uint16)
     lib().so_elementwise(_p(a, np.uint16), _p(b, np.uint16), a.size, dtype, int(multiply), _p(out, np.uint16))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# signed activation views (bit planes) — signed_quant.metal:746-2260
+# ---------------------------------------------------------------------------
+
+def activation_bitplanes(x_bits, planes: int, dtype: int):
+    """(planes [groups, planes, 4] u32, scales [groups] u16, q [cols] int32)"""
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    groups = x.size // 128
+    out = np.zeros((groups, planes, 4), np.uint32)
+    scales = np.zeros(groups, np.uint16)
+    q = np.zeros(x.size, np.int32)
+    lib().so_signed_activation_bitplanes(_p(x, np.uint16), x.size, planes, dtype, _p(out, np.uint32),
+                                         _p(scales, np.uint16), _p(q, np.int32))
+    return out, scales, q
+
+
+def swiglu_activation_bitplanes(gate_bits, up_bits, planes: int, dtype: int):
+    g = np.ascontiguousarray(gate_bits, np.uint16)
+    u = np.ascontiguousarray(up_bits, np.uint16)
+    out = np.zeros((g.size // 128, planes, 4), np.uint32)
+    scales = np.zeros(g.size // 128, np.uint16)
+    lib().so_swiglu_signed_activation_bitplanes(_p(g, np.uint16), _p(u, np.uint16), g.size, planes, dtype,
+                                                _p(out, np.uint32), _p(scales, np.uint16))
+    return out, scales
+
+
+def norm_scale_activation_bitplanes(rs: float, x_bits, w_bits, planes: int, dtype: int):
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    w = np.ascontiguousarray(w_bits, np.uint16)
+    out = np.zeros((x.size // 128, planes, 4), np.uint32)
+    scales = np.zeros(x.size // 128, np.uint16)
+    lib().so_norm_scale_signed_activation_bitplanes(rs, _p(x, np.uint16), _p(w, np.uint16), x.size, planes, dtype,
+                                                    _p(out, np.uint32), _p(scales, np.uint16))
+    return out, scales
+
+
+def signed_bitplane_matvec(fmt, packed, weight_scales, planes_arr, act_scales, rows, cols, dtype):
+    packed = np.ascontiguousarray(packed, np.uint8)
+    ws = np.ascontiguousarray(weight_scales, np.uint16)
+    pl = np.ascontiguousarray(planes_arr, np.uint32)
+    sc = np.ascontiguousarray(act_scales, np.uint16)
+    out = np.zeros(rows, np.float32)
+    lib().so_signed_bitplane_matvec(fmt, _p(packed, np.uint8), _p(ws, np.uint16), _p(pl, np.uint32), _p(sc, np.uint16),
+                                    rows, cols, pl.shape[1], dtype, _p(out, np.float32))
     return out

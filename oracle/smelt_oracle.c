@@ -673,6 +673,136 @@ SO_EXPORT void so_elementwise(const uint16_t *a, const uint16_t *b, int n, int d
 }
 
 /* ------------------------------------------------------------------------- */
+/* Signed activation views (bit planes) — signed_quant.metal:746-2260          */
+/* ------------------------------------------------------------------------- */
+
+/* Largest magnitude of an i{planes} view: i2 keeps {-1, 0, +1} (signed_quant.metal:848-858),
+ * the others 2^(planes-1) - 1 (:757-775, 836-846, 860-872, 918-930). */
+SO_EXPORT int so_bitplane_max_q(int planes) { return planes == 2 ? 1 : (1 << (planes - 1)) - 1; }
+
+/* One group of 128 values -> scale bits + quantised integers (signed_quant.metal:797-834).
+ * i2 and i3 quantise with the unrounded scale, i4..i6 with the stored 16-bit scale. */
+static uint16_t bitplane_quantize_group(const float *v, int planes, int dtype, int *q) {
+    int max_q = so_bitplane_max_q(planes);
+    float max_abs = 0.0f;
+    for (int i = 0; i < 128; ++i) max_abs = fmaxf(max_abs, fabsf(v[i]));
+    float producer = max_abs > 0.0f ? max_abs / (float)max_q : 1.0f;
+    uint16_t stored = narrow(producer, dtype);
+    float scale = planes >= 4 ? widen(stored, dtype) : producer;
+    for (int i = 0; i < 128; ++i) {
+        float t = v[i] / scale;
+        t = fminf(fmaxf(t, -(float)max_q), (float)max_q);
+        q[i] = (int)roundf(t);
+    }
+    return stored;
+}
+
+/* Plane p < planes-1 holds bit p of |q|, plane planes-1 the sign; word w, bit l = value w*32+l;
+ * out_planes is [groups][planes][4] (signed_quant.metal:751-755, 786-794). */
+static void bitplane_pack_group(const int *q, int planes, uint32_t *out) {
+    for (int p = 0; p < planes; ++p)
+        for (int w = 0; w < 4; ++w) {
+            uint32_t word = 0;
+            for (int l = 0; l < 32; ++l) {
+                int v = q[w * 32 + l];
+                uint32_t bit = p == planes - 1 ? (v < 0 ? 1u : 0u) : (((uint32_t)abs(v) >> p) & 1u);
+                word |= bit << l;
+            }
+            out[p * 4 + w] = word;
+        }
+}
+
+/* signed_activation_bitplanes_i{2..6}_g128: cols a multiple of 128. q_out (may be NULL) receives
+ * the integers the planes encode. */
+SO_EXPORT void so_signed_activation_bitplanes(const uint16_t *x, int cols, int planes, int dtype,
+                                              uint32_t *out_planes, uint16_t *out_scales, int *q_out) {
+    int groups = cols / 128;
+    for (int g = 0; g < groups; ++g) {
+        float v[128];
+        int q[128];
+        for (int i = 0; i < 128; ++i) v[i] = widen(x[g * 128 + i], dtype);
+        out_scales[g] = bitplane_quantize_group(v, planes, dtype, q);
+        bitplane_pack_group(q, planes, out_planes + (size_t)g * planes * 4);
+        if (q_out) memcpy(q_out + g * 128, q, sizeof(q));
+    }
+}
+
+/* swiglu_signed_activation_bitplanes_i5_g128 (:876-916): the staged SwiGLU value, then the view. */
+SO_EXPORT void so_swiglu_signed_activation_bitplanes(const uint16_t *gate, const uint16_t *up, int cols,
+                                                     int planes, int dtype, uint32_t *out_planes,
+                                                     uint16_t *out_scales) {
+    int groups = cols / 128;
+    for (int g = 0; g < groups; ++g) {
+        float v[128];
+        int q[128];
+        for (int i = 0; i < 128; ++i)
+            v[i] = widen(so_epilogue_signed_swiglu(gate[g * 128 + i], up[g * 128 + i], dtype), dtype);
+        out_scales[g] = bitplane_quantize_group(v, planes, dtype, q);
+        bitplane_pack_group(q, planes, out_planes + (size_t)g * planes * 4);
+    }
+}
+
+/* norm_scale_signed_activation_bitplanes_i{2..6}_g128 (:1175-1223): rms_norm_1pw's two-step value
+ * half(x * rs) * half(1 + w) from a precomputed scale, then the view. */
+SO_EXPORT void so_norm_scale_signed_activation_bitplanes(float rs, const uint16_t *x, const uint16_t *w,
+                                                         int cols, int planes, int dtype,
+                                                         uint32_t *out_planes, uint16_t *out_scales) {
+    int groups = cols / 128;
+    for (int g = 0; g < groups; ++g) {
+        float v[128];
+        int q[128];
+        for (int i = 0; i < 128; ++i) {
+            float normalized = so_round_through(widen(x[g * 128 + i], dtype) * rs, dtype);
+            float direct = so_round_through(1.0f + widen(w[g * 128 + i], dtype), dtype);
+            v[i] = so_round_through(normalized * direct, dtype);
+        }
+        out_scales[g] = bitplane_quantize_group(v, planes, dtype, q);
+        bitplane_pack_group(q, planes, out_planes + (size_t)g * planes * 4);
+    }
+}
+
+static int popc32(uint32_t v) { return __builtin_popcount(v); }
+
+/* signed_{binary,ternary}_bitplane_i{N}_matvec_g128_rows8 (:1564-1636, 2054-2104): per (row, group)
+ * an integer dot of signed weights with the quantised activations, formed from popcounts
+ * (:1300-1348), times activation scale, times weight scale; fp32 sum over groups in group order. */
+SO_EXPORT void so_signed_bitplane_matvec(int format, const uint8_t *codes, const uint16_t *weight_scales,
+                                         const uint32_t *act_planes, const uint16_t *act_scales, int rows,
+                                         int cols, int planes, int dtype, float *out) {
+    int groups = cols / 128;
+    int row_bytes = format == SO_BINARY1 ? cols / 8 : cols / 4;
+    for (int r = 0; r < rows; ++r) {
+        float acc = 0.0f;
+        for (int g = 0; g < groups; ++g) {
+            uint32_t pos[4] = {0, 0, 0, 0}, neg[4] = {0, 0, 0, 0};
+            for (int c = 0; c < 128; ++c) {
+                int code = so_signed_code_at((int64_t)g * 128 + c, codes + (size_t)r * row_bytes, row_bytes, format);
+                int sem = 0;
+                so_signed_semantic(format, code, &sem);
+                if (sem > 0) pos[c >> 5] |= 1u << (c & 31);
+                if (sem < 0) neg[c >> 5] |= 1u << (c & 31);
+            }
+            const uint32_t *pl = act_planes + (size_t)g * planes * 4;
+            const uint32_t *sign = pl + (planes - 1) * 4;
+            int dot = 0;
+            for (int b = 0; b < planes - 1; ++b) {
+                int agreement = 0, active = 0;
+                for (int w = 0; w < 4; ++w) {
+                    uint32_t mask = (pos[w] & ~sign[w]) | (neg[w] & sign[w]);
+                    agreement += popc32(mask & pl[b * 4 + w]);
+                    active += popc32((pos[w] | neg[w]) & pl[b * 4 + w]);
+                }
+                dot += (1 << b) * (2 * agreement - active);
+            }
+            volatile float scaled = (float)dot * widen(act_scales[g], dtype);
+            volatile float term = scaled * so_f16_to_f32(weight_scales[(size_t)r * groups + g]);
+            acc += term;
+        }
+        out[r] = acc;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* Argmax key — lut_matvec.metal:4045-4074                                     */
 /* ------------------------------------------------------------------------- */
 

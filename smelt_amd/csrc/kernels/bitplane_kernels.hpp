@@ -1,0 +1,104 @@
+// Producers of signed activation views (signed_quant.metal:746-1298): every group of 128
+// activations becomes a 16-bit scale (largest magnitude / largest integer) and sign-magnitude
+// integers stored as bit planes, [group][plane][4 words], word w bit l = value 32 w + l.
+//   values   plain input, the staged SwiGLU of (gate, up), or rms_norm_1pw's two-step value
+//            half(x * rs) * half(1 + w) from a precomputed scale
+//   scale    i2 and i3 views quantise with the unrounded fp32 scale, i4..i6 with the stored one
+//   integer  round-half-away(clamp(value / scale, -max, +max)), max = 1 (i2) or 2^(planes-1) - 1
+// One wave per group, grid-strided; a 32-thread workgroup (the reference's launch shape) works too.
+#pragma once
+#include "common.hpp"
+
+namespace smelt {
+
+enum BitplaneSource : int { kPlaneSrcPlain = 0, kPlaneSrcSwiglu = 1, kPlaneSrcNormScale = 2 };
+
+template <class ActT, int SRC>
+__device__ __forceinline__ float bitplane_value(const float* norm_scale, const uint16_t* a, const uint16_t* b, size_t i) {
+    if constexpr (SRC == kPlaneSrcPlain) {
+        return ActT::widen(a[i]);
+    } else if constexpr (SRC == kPlaneSrcSwiglu) {
+        auto rt = [](float v) { return ActT::widen(ActT::narrow(v)); };
+        const float g = ActT::widen(a[i]), u = ActT::widen(b[i]);
+        const float e = rt(expf(fabsf(g)));
+        const float tail = rt(1.0f / rt(1.0f + e));
+        const float sig = g < 0.0f ? tail : rt(1.0f - tail);
+        return rt(rt(g * sig) * u);
+    } else {
+        const float normalized = ActT::widen(ActT::narrow(ActT::widen(a[i]) * norm_scale[0]));
+        const float direct = ActT::widen(ActT::narrow(1.0f + ActT::widen(b[i])));
+        return ActT::widen(ActT::narrow(normalized * direct));
+    }
+}
+
+template <class ActT, int SRC>
+__device__ __forceinline__ void activation_bitplanes_body(const float* norm_scale, const uint16_t* a, const uint16_t* b,
+                                                          uint32_t* planes, uint16_t* scales, uint32_t cols,
+                                                          uint32_t nplanes) {
+    const uint32_t groups = cols / 128;
+    const uint32_t width = blockDim.x < 64u ? blockDim.x : 64u;      // 32 or 64 live lanes per wave
+    const uint32_t lane = threadIdx.x % 64u;
+    const uint32_t waves = (blockDim.x + 63u) / 64u;
+    const uint32_t batch = blockIdx.y;
+    a += (size_t)batch * cols;
+    if (SRC == kPlaneSrcSwiglu) b += (size_t)batch * cols;           // the norm weight is shared by every token
+    planes += (size_t)batch * groups * nplanes * 4;
+    scales += (size_t)batch * groups;
+    const int max_q = nplanes == 2 ? 1 : (1 << (nplanes - 1)) - 1;
+    const uint32_t per_lane = 128u / width;
+    for (uint32_t g = blockIdx.x * waves + threadIdx.x / 64u; g < groups; g += gridDim.x * waves) {
+        float v[4];
+        float max_abs = 0.0f;
+        for (uint32_t k = 0; k < per_lane; ++k) {
+            v[k] = bitplane_value<ActT, SRC>(norm_scale, a, b, (size_t)g * 128 + k * width + lane);
+            max_abs = __builtin_fmaxf(max_abs, __builtin_fabsf(v[k]));
+        }
+        for (uint32_t off = width / 2; off > 0; off >>= 1) max_abs = __builtin_fmaxf(max_abs, __shfl_xor(max_abs, (int)off));
+        const float producer = max_abs > 0.0f ? max_abs / (float)max_q : 1.0f;
+        const uint16_t stored = ActT::narrow(producer);
+        const float scale = nplanes >= 4 ? ActT::widen(stored) : producer;
+        if (lane == 0) scales[g] = stored;
+        for (uint32_t k = 0; k < per_lane; ++k) {
+            float t = v[k] / scale;
+            t = __builtin_fminf(__builtin_fmaxf(t, -(float)max_q), (float)max_q);
+            const int q = (int)__builtin_roundf(t);
+            const uint32_t mag = (uint32_t)(q < 0 ? -q : q);
+            for (uint32_t p = 0; p < nplanes; ++p) {
+                const bool bit = p == nplanes - 1 ? q < 0 : ((mag >> p) & 1u) != 0;
+                const unsigned long long mask = __ballot(bit);
+                if (lane == 0) {
+                    uint32_t* dst = planes + ((size_t)g * nplanes + p) * 4;
+                    if (width == 64u) {
+                        dst[2 * k] = (uint32_t)mask;
+                        dst[2 * k + 1] = (uint32_t)(mask >> 32);
+                    } else {
+                        dst[k] = (uint32_t)mask;
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace smelt
+
+#define SMELT_PLANE_KERNEL extern "C" __global__ __launch_bounds__(1024)
+
+#define SMELT_ACTIVATION_BITPLANE_KERNELS(T, ACT)                                                  \
+    SMELT_PLANE_KERNEL void smelt_signed_activation_bitplanes_##T(                                 \
+        const uint16_t* x, uint32_t* planes, uint16_t* scales, uint32_t cols, uint32_t nplanes) {  \
+        smelt::activation_bitplanes_body<ACT, smelt::kPlaneSrcPlain>(nullptr, x, nullptr, planes,  \
+                                                                     scales, cols, nplanes);       \
+    }                                                                                              \
+    SMELT_PLANE_KERNEL void smelt_swiglu_signed_activation_bitplanes_##T(                          \
+        const uint16_t* gate, const uint16_t* up, uint32_t* planes, uint16_t* scales,              \
+        uint32_t cols, uint32_t nplanes) {                                                         \
+        smelt::activation_bitplanes_body<ACT, smelt::kPlaneSrcSwiglu>(nullptr, gate, up, planes,   \
+                                                                      scales, cols, nplanes);      \
+    }                                                                                              \
+    SMELT_PLANE_KERNEL void smelt_norm_scale_signed_activation_bitplanes_##T(                      \
+        const float* norm_scale, const uint16_t* x, const uint16_t* w, uint32_t* planes,           \
+        uint16_t* scales, uint32_t cols, uint32_t nplanes) {                                       \
+        smelt::activation_bitplanes_body<ACT, smelt::kPlaneSrcNormScale>(norm_scale, x, w, planes, \
+                                                                         scales, cols, nplanes);   \
+    }

@@ -32,6 +32,7 @@ __device__ __forceinline__ uint32_t and_or(uint32_t c, uint32_t mask, uint32_t m
 // The semantic weight is kSemMul * (code + pair terms - offset) * scale.
 // ---------------------------------------------------------------------------------------
 struct FmtU4 {
+    static constexpr bool kBitplanes = false;
     static constexpr int kDwordsPerUnit = 4;
     static constexpr bool kPerDwordScale = false;
     static constexpr int kBitsPerCode = 4;
@@ -50,6 +51,7 @@ struct FmtU4 {
 };
 
 struct FmtTer2 {
+    static constexpr bool kBitplanes = false;
     static constexpr int kDwordsPerUnit = 4;
     static constexpr bool kPerDwordScale = false;
     static constexpr int kBitsPerCode = 2;
@@ -76,6 +78,7 @@ struct FmtTer2 {
 };
 
 struct FmtBin {
+    static constexpr bool kBitplanes = false;
     static constexpr int kDwordsPerUnit = 4;
     static constexpr bool kPerDwordScale = false;
     static constexpr int kBitsPerCode = 1;
@@ -113,6 +116,7 @@ struct FmtBin {
 // layout.  A 16-byte unit holds 80 columns = five 16-column dwords; a dword never straddles a
 // 128-column scale group, a unit can, so the scale is applied per dword.
 struct FmtTrit5 {
+    static constexpr bool kBitplanes = false;
     static constexpr int kDwordsPerUnit = 5;
     static constexpr bool kPerDwordScale = true;
     static constexpr int kBitsPerCode = 2;
@@ -136,6 +140,34 @@ struct FmtTrit5 {
     }
 };
 
+// Signed activation views (signed_quant.metal:746-755): the activations of a 128-column group
+// arrive as a 16-bit scale and sign-magnitude integers stored as bit planes (plane p < P-1 = bit p of
+// |q|, plane P-1 = sign; word w, bit l = column 32 w + l).  A unit's dot product is then integer:
+//     sum_p 2^p * (2 * popcount(agree & plane_p) - popcount(nonzero & plane_p))
+// with `agree` the columns where weight and activation signs give a positive product.  Codes keep
+// the binary1 / ternary2 layouts and geometry; only staging and the per-unit arithmetic differ.
+struct FmtBinPlanes : FmtBin {
+    static constexpr bool kBitplanes = true;
+    static constexpr bool kTernaryPlanes = false;
+};
+struct FmtTerPlanes : FmtTer2 {
+    static constexpr bool kBitplanes = true;
+    static constexpr bool kTernaryPlanes = true;
+};
+
+// 16 bits -> the even bit positions of 32 (bit i -> bit 2 i)
+__device__ __forceinline__ uint32_t spread16(uint32_t v) {
+    v = (v | (v << 8)) & 0x00FF00FFu;
+    v = (v | (v << 4)) & 0x0F0F0F0Fu;
+    v = (v | (v << 2)) & 0x33333333u;
+    v = (v | (v << 1)) & 0x55555555u;
+    return v;
+}
+
+__device__ __forceinline__ int popcount128(const uint4_t& v) {
+    return __builtin_popcount(v.x) + __builtin_popcount(v.y) + __builtin_popcount(v.z) + __builtin_popcount(v.w);
+}
+
 template <class F>
 struct FmtGeom {
     static constexpr int kPPD = F::kPairsPerDword;
@@ -157,10 +189,55 @@ __device__ __forceinline__ size_t lds_pairs_bytes(int U, int MB) {
 }
 
 // Stage x[b0 .. b0+nb) (nb <= MB, rows of `cols` elements of ActT) into LDS.
+// Activation-view staging: plane p of unit u goes to lds_pairs[p * U + u] (binary: the group's four
+// words; ternary: the unit's 64 columns spread to the even bits of four dwords, the layout of the
+// 2-bit codes); lds_corr holds per unit the activation scale, the binary correction
+// sum_p 2^p popcount(plane_p) and the plane count.
+template <class F, class ActT>
+__device__ __forceinline__ void stage_planes(const uint32_t* __restrict__ planes, const uint16_t* __restrict__ act_scales,
+                                             int nplanes, int U, int batch_row, uint4_t* lds_pairs, float* lds_corr) {
+    constexpr bool TER = F::kTernaryPlanes;
+    const int groups = TER ? U / 2 : U;
+    planes += (size_t)batch_row * groups * nplanes * 4;
+    act_scales += (size_t)batch_row * groups;
+    for (int item = threadIdx.x; item < U * nplanes; item += blockDim.x) {
+        const int u = item / nplanes, p = item - u * nplanes;
+        uint4_t v;
+        if constexpr (!TER) {
+            v = *reinterpret_cast<const uint4_t*>(planes + ((size_t)u * nplanes + p) * 4);
+        } else {
+            const uint2_t w = *reinterpret_cast<const uint2_t*>(planes + ((size_t)(u >> 1) * nplanes + p) * 4 + 2 * (u & 1));
+            v.x = spread16(w.x & 0xFFFFu); v.y = spread16(w.x >> 16);
+            v.z = spread16(w.y & 0xFFFFu); v.w = spread16(w.y >> 16);
+        }
+        lds_pairs[(size_t)p * U + u] = v;
+    }
+    for (int u = threadIdx.x; u < U; u += blockDim.x) {
+        const int g = TER ? u >> 1 : u;
+        int bias = 0;
+        if constexpr (!TER) {
+            for (int p = 0; p < nplanes - 1; ++p)
+                bias += popcount128(*reinterpret_cast<const uint4_t*>(planes + ((size_t)g * nplanes + p) * 4)) << p;
+        }
+        float4_t c;
+        c.x = ActT::widen(act_scales[g]);
+        c.y = __builtin_bit_cast(float, bias);
+        c.z = __builtin_bit_cast(float, nplanes);
+        c.w = 0.0f;
+        *reinterpret_cast<float4_t*>(lds_corr + (size_t)u * 4) = c;
+    }
+}
+
 template <class F, class ActT, int MB>
 __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x, int cols, int U,
                                                   int b0, int nb, uint4_t* lds_pairs,
-                                                  float* lds_corr, float* lds_xsum) {
+                                                  float* lds_corr, float* lds_xsum,
+                                                  const uint16_t* x2 = nullptr, int nplanes = 0) {
+    if constexpr (F::kBitplanes) {
+        static_assert(MB == 1, "activation views are consumed one token per launch row");
+        stage_planes<F, ActT>(reinterpret_cast<const uint32_t*>(x), x2, nplanes, U, b0, lds_pairs, lds_corr);
+        return;
+    }
     using G = FmtGeom<F>;
     constexpr int PPD = G::kPPD;
     constexpr int CPD = G::kColsPerDword;
@@ -253,6 +330,51 @@ __device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u,
                                              const uint4_t* lds_pairs, const float* lds_corr,
                                              const float* lds_xsum, const uint16_t* lut,
                                              float (&acc)[NMAT][R][MB]) {
+    if constexpr (F::kBitplanes) {
+        const float4_t c4 = *reinterpret_cast<const float4_t*>(lds_corr + (size_t)u * 4);
+        // (elements are copied out before the bit casts: a bit cast applied directly to a vector
+        //  element reads the vector's first lane)
+        const float act_scale = c4.x, bias_bits = c4.y, nplanes_bits = c4.z;
+        const int bias = __builtin_bit_cast(int, bias_bits);
+        const int nplanes = __builtin_bit_cast(int, nplanes_bits);
+        const uint4_t sign = lds_pairs[(size_t)(nplanes - 1) * U + u];
+        uint4_t agree[NMAT][R], nonzero[NMAT][R];
+        int weighted[NMAT][R], active[NMAT][R];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint4_t c = it.c[m][r];
+                if constexpr (!F::kTernaryPlanes) {
+                    agree[m][r] = c ^ sign;          // weight +1 and activation >= 0, or -1 and < 0
+                } else {
+                    const uint4_t even = {0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u};
+                    const uint4_t pos = (c >> 1) & even;   // code 2 = +1
+                    nonzero[m][r] = ~c & even;             // code 1 = 0 has its low bit set
+                    agree[m][r] = nonzero[m][r] & (pos ^ sign);
+                }
+                weighted[m][r] = 0;
+                active[m][r] = 0;
+            }
+        for (int p = 0; p < nplanes - 1; ++p) {
+            const uint4_t plane = lds_pairs[(size_t)p * U + u];
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    weighted[m][r] += popcount128(agree[m][r] & plane) << p;
+                    if constexpr (F::kTernaryPlanes) active[m][r] += popcount128(nonzero[m][r] & plane) << p;
+                }
+        }
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int dot = 2 * weighted[m][r] - (F::kTernaryPlanes ? active[m][r] : bias);
+                acc[m][r][0] = __builtin_fmaf((float)dot * act_scale, ScaleT::widen(it.s[m][r]), acc[m][r][0]);
+            }
+        return;
+    }
     using G = FmtGeom<F>;
     constexpr int NCH = G::kChunksPerUnit;
     constexpr int DPU = G::kDPU;

@@ -98,7 +98,7 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
                                           int cols, int U, int row_stride, int gpr, int gshift,
                                           int batch_lo, int batch_hi, uint4_t* lds_pairs,
                                           float* lds_corr, float* lds_xsum, const uint16_t* lut,
-                                          const Epi& epi) {
+                                          const Epi& epi, const uint16_t* x2 = nullptr, int nplanes = 0) {
     constexpr int S = kWave / L;
     constexpr int TILE = S * R;
     const int waves = blockDim.x / kWave;
@@ -138,7 +138,7 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
         if (nq > 0) load(regs_a);
         if (nq > 1) load(regs_b);
         if (b0 != batch_lo) __syncthreads();
-        stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum);
+        stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum, x2, nplanes);
         __syncthreads();
 
         float acc[NMAT][R][MB];
@@ -198,7 +198,8 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
 template <class F, class ActT, class ScaleT, int R, int MB, int NMAT, class Epi>
 __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const uint16_t* x,
                                             int rows, int cols, int row_stride, int group,
-                                            int batch_lo, int batch_hi, const Epi& epi) {
+                                            int batch_lo, int batch_hi, const Epi& epi,
+                                            const uint16_t* x2 = nullptr, int nplanes = 0) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int U = row_stride / 16;
     const int gshift = ilog2((uint32_t)group);
@@ -218,11 +219,11 @@ __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const u
         if constexpr (R > 1 && MB == 1) {
             const int tiles = (rows + (kWave / L) * R - 1) / ((kWave / L) * R);
             if (tiles < total_waves) {
-                run_tiles<F, ActT, ScaleT, 1, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
+                run_tiles<F, ActT, ScaleT, 1, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi, x2, nplanes);
                 return;
             }
         }
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi);
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi, x2, nplanes);
     };
     if (U > 32) go(std::integral_constant<int, 64>{});
     else if (U > 16) go(std::integral_constant<int, 32>{});
@@ -382,6 +383,41 @@ using u32 = uint32_t;
         const u32 hi = lo + 4 < batch ? lo + 4 : batch;                                           \
         matvec_body<FMT, ACT, F16, 2, 2, 2>(mats, X, rows, cols,                                  \
                                             packed_row_stride<FMT>(cols, 128), 128, lo, hi, epi); \
+    }
+
+// Signed activation views: the activation operand is (planes, scales) instead of x
+// (signed_{binary,ternary}_bitplane_i{N}_{matvec,matvec_add,gate_up_swiglu}_g128_rows8,
+//  signed_quant.metal:1564-2260); batch row = blockIdx.y.
+#define SMELT_BITPLANE_KERNELS(FN, FMT, T, ACT)                                                   \
+    SMELT_KERNEL void smelt_signed_##FN##_bitplane_matvec_##T(                                    \
+        const u8* C, const u16* S, const u32* P, const u16* AS, u16* Y, u32 rows, u32 cols,       \
+        u32 nplanes) {                                                                            \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        matvec_body<FMT, ACT, F16, 4, 1, 1>(mats, reinterpret_cast<const u16*>(P), rows, cols,    \
+                                            packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
+                                            blockIdx.y + 1, epi, AS, (int)nplanes);               \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_bitplane_matvec_add_##T(                                \
+        const u8* C, const u16* S, const u32* P, const u16* AS, u16* Y, const u16* res, u32 rows, \
+        u32 cols, u32 nplanes) {                                                                  \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        matvec_body<FMT, ACT, F16, 4, 1, 1>(mats, reinterpret_cast<const u16*>(P), rows, cols,    \
+                                            packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
+                                            blockIdx.y + 1, epi, AS, (int)nplanes);               \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_bitplane_gate_up_swiglu_##T(                            \
+        const u8* gC, const u16* gS, const u8* uC, const u16* uS, const u32* P, const u16* AS,    \
+        u16* Y, u32 rows, u32 cols, u32 nplanes) {                                                \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        matvec_body<FMT, ACT, F16, 2, 1, 2>(mats, reinterpret_cast<const u16*>(P), rows, cols,    \
+                                            packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
+                                            blockIdx.y + 1, epi, AS, (int)nplanes);               \
     }
 
 // ---- lm_head: matvec fused with argmax over the rounded logits -------------------------------

@@ -7,6 +7,7 @@
 #include "qmm_skinny.hpp"
 #include "import_kernels.hpp"
 #include "layer_kernels.hpp"
+#include "bitplane_kernels.hpp"
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
@@ -42,3 +43,10 @@ SMELT_AFFINE_QUANTIZE(bf16, smelt::BF16, 128)
 
 SMELT_LAYER_KERNELS(f16, smelt::F16)
 SMELT_LAYER_KERNELS(bf16, smelt::BF16)
+
+SMELT_BITPLANE_KERNELS(binary, smelt::FmtBinPlanes, f16, smelt::F16)
+SMELT_BITPLANE_KERNELS(binary, smelt::FmtBinPlanes, bf16, smelt::BF16)
+SMELT_BITPLANE_KERNELS(ternary, smelt::FmtTerPlanes, f16, smelt::F16)
+SMELT_BITPLANE_KERNELS(ternary, smelt::FmtTerPlanes, bf16, smelt::BF16)
+SMELT_ACTIVATION_BITPLANE_KERNELS(f16, smelt::F16)
+SMELT_ACTIVATION_BITPLANE_KERNELS(bf16, smelt::BF16)

@@ -425,6 +425,55 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         }
         if (entry == "buffer_copy") { out->family = kFamCopy16; out->symbol = "smelt_buffer_copy16"; out->kinds = "PPU"; return kResolveOk; }
     }
+    // ---- signed activation views (bit planes): signed_quant.metal:746-2260 ----------------------
+    {
+        // "..._i{N}_..." with N planes, 2 <= N <= 6
+        auto planes_of = [](const std::string& s, size_t at, uint32_t* n, size_t* after) {
+            if (at + 2 > s.size() || s[at] != 'i' || s[at + 1] < '2' || s[at + 1] > '6') return false;
+            *n = (uint32_t)(s[at + 1] - '0');
+            *after = at + 2;
+            return true;
+        };
+        uint32_t n = 0;
+        size_t after = 0;
+        if (starts_with(entry, "signed_activation_bitplanes_") && planes_of(entry, 28, &n, &after) &&
+            (entry.substr(after) == "_g128" || entry.substr(after) == "_g128_batched")) {
+            out->family = kFamActivationPlanes; out->symbol = "smelt_signed_activation_bitplanes_" + t;
+            out->kinds = "PPPUU"; out->appended = {n};
+            return kResolveOk;
+        }
+        if (entry == "swiglu_signed_activation_bitplanes_i5_g128") {
+            out->family = kFamSwigluPlanes; out->symbol = "smelt_swiglu_signed_activation_bitplanes_" + t;
+            out->kinds = "PPPPUU"; out->appended = {5u};
+            return kResolveOk;
+        }
+        if (starts_with(entry, "norm_scale_signed_activation_bitplanes_") && planes_of(entry, 39, &n, &after) &&
+            entry.substr(after) == "_g128") {
+            out->family = kFamNormScalePlanes; out->symbol = "smelt_norm_scale_signed_activation_bitplanes_" + t;
+            out->kinds = "PPPPPUU"; out->appended = {n};
+            return kResolveOk;
+        }
+        for (const char* fmt : {"binary", "ternary"}) {
+            const std::string head = std::string("signed_") + fmt + "_bitplane_";
+            if (!starts_with(entry, head.c_str()) || !planes_of(entry, head.size(), &n, &after)) continue;
+            const std::string tail = entry.substr(after);
+            const std::string stem = std::string("smelt_signed_") + fmt + "_bitplane_";
+            out->format = fmt[0] == 'b' ? kFmtBinary1 : kFmtTernary2;
+            out->appended = {n};
+            if (tail == "_matvec_g128_rows8" || tail == "_matvec_g128_rows2_wide") {
+                out->family = kFamPlaneMatvec; out->symbol = stem + "matvec_" + t; out->kinds = "PPPPPUUU";
+                return kResolveOk;
+            }
+            if (tail == "_matvec_add_g128_rows8") {
+                out->family = kFamPlaneAdd; out->symbol = stem + "matvec_add_" + t; out->kinds = "PPPPPPUUU";
+                return kResolveOk;
+            }
+            if (tail == "_gate_up_swiglu_g128_rows8") {
+                out->family = kFamPlaneGateUp; out->symbol = stem + "gate_up_swiglu_" + t; out->kinds = "PPPPPPPUUU";
+                return kResolveOk;
+            }
+        }
+    }
     if (entry == "signed_validate_codes") { out->family = kFamSignedValidate; out->symbol = "smelt_signed_validate_codes"; out->kinds = "PPUUU"; return kResolveOk; }
     if (entry == "signed_normalize_mlx_scales") { out->family = kFamSignedMlxScales; out->symbol = "smelt_signed_normalize_mlx_scales"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "copy_u128") { out->family = kFamCopy; out->symbol = "smelt_copy_u128"; out->kinds = "PPU"; return kResolveOk; }

@@ -48,6 +48,12 @@ enum FamilyId {
     kFamRmsScale,             // x scale | dim eps
     kFamResidualAddRmsScale,  // a b out scale dim eps
     kFamElementwise,          // a b out count
+    kFamActivationPlanes,     // x planes scales cols | nplanes             (grid.y = token)
+    kFamSwigluPlanes,         // gate up planes scales cols | nplanes
+    kFamNormScalePlanes,      // norm_scale x w planes scales cols | nplanes
+    kFamPlaneMatvec,          // C S planes ascales Y rows cols | nplanes   (grid.y = token)
+    kFamPlaneAdd,             // C S planes ascales Y res rows cols | nplanes
+    kFamPlaneGateUp,          // gC gS uC uS planes ascales Y rows cols | nplanes
     kFamCopy16,               // src dst count
     kFamCount
 };

@@ -124,7 +124,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
     auto bad_geom = [&](const std::string& m) {
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
     };
-    const bool matvec_like = r.family <= kFamAffineBank4;
+    const bool plane_matvec = r.family == kFamPlaneMatvec || r.family == kFamPlaneAdd || r.family == kFamPlaneGateUp;
+    const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
     if (matvec_like) {
@@ -425,6 +426,47 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             if ((size_t)L.grid[0] * L.block[0] < count) return bad_geom("grid covers " + std::to_string((size_t)L.grid[0] * L.block[0]) + " of " + std::to_string(count) + " elements");
             for (size_t i = 0; i < ci; ++i) need[i] = count * 2;
             written[ci - 1] = true;
+            break;
+        }
+        case kFamPlaneMatvec:
+        case kFamPlaneAdd:
+        case kFamPlaneGateUp: {
+            // C S [uC uS] planes ascales Y [res] rows cols nplanes
+            const size_t pi = r.family == kFamPlaneGateUp ? 4 : 2;               // planes argument
+            const size_t ri = r.family == kFamPlaneMatvec ? 5 : (r.family == kFamPlaneAdd ? 6 : 7);
+            const size_t rows = U(ri), cols = U(ri + 1), nplanes = U(ri + 2);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            if (nplanes < 2 || nplanes > 6) return bad_geom("activation views hold 2 to 6 planes");
+            signed_w(0, 1, rows, cols);
+            if (r.family == kFamPlaneGateUp) signed_w(2, 3, rows, cols);
+            const size_t groups = cols / 128;
+            need[pi] = gy * groups * nplanes * 16; align[pi] = 16;
+            need[pi + 1] = gy * groups * 2;
+            need[pi + 2] = gy * rows * 2; written[pi + 2] = true;
+            if (r.family == kFamPlaneAdd) need[pi + 3] = gy * rows * 2;
+            L.lds = signed_lds(cols, 1);
+            break;
+        }
+        case kFamActivationPlanes:
+        case kFamSwigluPlanes:
+        case kFamNormScalePlanes: {
+            // [norm_scale] a [b] planes scales cols nplanes; one wave per 128-value group, grid.y = token
+            const size_t ai = r.family == kFamNormScalePlanes ? 1 : 0;
+            const size_t pl = r.family == kFamActivationPlanes ? 1 : (r.family == kFamSwigluPlanes ? 2 : 3);
+            const size_t cols = U(pl + 2), nplanes = U(pl + 3), tokens = gy;
+            if (cols == 0 || cols % 128 != 0) return bad_geom("activation views need cols % 128 == 0");
+            if (nplanes < 2 || nplanes > 6) return bad_geom("activation views hold 2 to 6 planes");
+            if ((L.block[0] != 32 && L.block[0] % 64 != 0) || L.block[1] != 1 || L.block[2] != 1 || L.grid[2] != 1)
+                return bad_geom("activation-view producers run 32 threads or whole waves per workgroup");
+            if (r.family == kFamNormScalePlanes) {
+                if (tokens != 1) return bad_geom("the norm-scale producer takes one token");
+                need[0] = 4; align[0] = 4;
+                need[2] = cols * 2;
+            }
+            need[ai] = tokens * cols * 2;
+            if (r.family == kFamSwigluPlanes) need[1] = tokens * cols * 2;
+            need[pl] = tokens * (cols / 128) * nplanes * 16; align[pl] = 16; written[pl] = true;
+            need[pl + 1] = tokens * (cols / 128) * 2; written[pl + 1] = true;
             break;
         }
         case kFamAffineQuantize: {
