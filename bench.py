@@ -254,10 +254,33 @@ def side_measurements(ctx, fx, cc, rt, cus) -> dict:
             b = e.size_bytes + e.scales_size_bytes
             per_kernel[f"{r}x{k}"] = {"us_warm_median": round(float(np.median(t)), 2), "weight_bytes": int(b)}
         c.graph_destroy(g)
+        views = None
+        if fmt in (fx.BINARY1, fx.TERNARY2):
+            # the same layer through signed activation views (i5): one view per distinct input
+            # (q/k/v share one, gate/up share one), every projection an integer popcount matvec
+            VP, VS = 24, 25
+            c.alloc(VP, 17408 // 128 * 5 * 16)
+            c.alloc(VS, 17408 // 128 * 2)
+            em2 = cc.Emitter(rt.ACT_BF16, cus)
+            for layer in ents:
+                for i, e in enumerate(layer):
+                    if i in (0, 2, 3, 5):   # gate (up shares it), down, q (k/v share it), o: a new input
+                        em2.activation_view(5, cc.bind(X), cc.bind(VP), cc.bind(VS), e.cols)
+                    em2.view_matvec(W, e, 5, cc.bind(VP), cc.bind(VS), cc.bind(Y))
+            remap = {i: c.pipeline(nm) for i, nm in enumerate(em2.pipelines)}
+            recs2 = list(em2.records())
+            for r in recs2:
+                r.pipeline = remap[r.pipeline]
+            g2, n2 = c.capture_decode(c.table(recs2))
+            c.graph_time(g2, 3)
+            us2 = c.graph_time(g2, reps) / (reps * copies)
+            c.graph_destroy(g2)
+            views = {"us_per_layer": round(us2, 2), "launches": n2 // copies, "planes": 5,
+                     "GBps": round(layer_bytes / us2 / 1e3, 1)}
         out[f"bonsai27b_layer_{name}"] = {
             "us_per_layer": round(us, 2), "weight_bytes": int(layer_bytes),
             "GBps": round(layer_bytes / us / 1e3, 1), "pct_of_hbm_peak": round(100 * layer_bytes / us / 1e3 / HBM_PEAK_GBS, 2),
-            "launches": len(shapes), "kernels": per_kernel}
+            "launches": len(shapes), "kernels": per_kernel, "activation_views_i5": views}
         c.close()
     # qmm: Qwen3.5-4B FFN (gate/up 2560->9216, down 9216->2560), affine u4 g64
     c = rt.Context(act_dtype=rt.ACT_BF16)

@@ -165,6 +165,22 @@ int smelt_emit_elementwise(smelt_emitter *e, int multiply, SmeltBinding a, Smelt
 /* staged swiglu_fused over `count` gate / up values (DenseTrunkEmitter.swift:209) */
 int smelt_emit_swiglu_fused(smelt_emitter *e, SmeltBinding gate, SmeltBinding up,
                             SmeltBinding output, int count);
+/* Signed activation views (emitSignedActivationBitplanes / emitSignedBitplane*IfPossible,
+ * SmeltCodeEmitter.swift; kernels signed_quant.metal:746-2260).  A view is `planes` bit planes
+ * (2..6) of [cols / 128] groups plus one 16-bit scale per group, built once per projection-bank
+ * input and consumed by every binary1 / ternary2 member of the bank.
+ *   smelt_emit_activation_view     signed_activation_bitplanes_i{N}_g128[_batched]
+ *   smelt_emit_view_matvec         signed_{binary,ternary}_bitplane_i{N}_matvec[_add]_g128_rows8
+ *   smelt_emit_view_gate_up_swiglu signed_{binary,ternary}_bitplane_i{N}_gate_up_swiglu_g128_rows8 */
+int smelt_emit_activation_view(smelt_emitter *e, int planes, SmeltBinding input,
+                               SmeltBinding view_planes, SmeltBinding view_scales, int cols,
+                               int batch_size);
+int smelt_emit_view_matvec(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w, int planes,
+                           SmeltBinding view_planes, SmeltBinding view_scales, SmeltBinding output,
+                           const SmeltBinding *residual, int batch_size);
+int smelt_emit_view_gate_up_swiglu(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *gate,
+                                   const SmeltWeightEntryC *up, int planes, SmeltBinding view_planes,
+                                   SmeltBinding view_scales, SmeltBinding output, int batch_size);
 /* swap cur/alt (SmeltDispatchRecord.swap) */
 int smelt_emit_swap(smelt_emitter *e);
 

@@ -78,6 +78,9 @@ def lib() -> C.CDLL:
         "smelt_emit_dual_matvec": (i32, [vp, i32, we, we, Binding, Binding, Binding]),
         "smelt_emit_lm_head_argmax": (i32, [vp, i32, we, Binding, Binding, Binding, i32, C.c_float]),
         "smelt_emit_swap": (i32, [vp]),
+        "smelt_emit_activation_view": (i32, [vp, i32, Binding, Binding, Binding, i32, i32]),
+        "smelt_emit_view_matvec": (i32, [vp, i32, we, i32, Binding, Binding, Binding, C.POINTER(Binding), i32]),
+        "smelt_emit_view_gate_up_swiglu": (i32, [vp, i32, we, we, i32, Binding, Binding, Binding, i32]),
         "smelt_emit_rms_norm_1pw": (i32, [vp, Binding, Binding, Binding, C.POINTER(Binding), i32, C.c_float, i32]),
         "smelt_emit_elementwise": (i32, [vp, i32, Binding, Binding, Binding, i32]),
         "smelt_emit_swiglu_fused": (i32, [vp, Binding, Binding, Binding, i32]),
@@ -265,6 +268,17 @@ class Emitter:
 
     def swiglu_fused(self, gate, up, y, count):
         self._check(self.l.smelt_emit_swiglu_fused(self.h, gate, up, y, count))
+
+    def activation_view(self, planes, x, view_planes, view_scales, cols, batch=1):
+        self._check(self.l.smelt_emit_activation_view(self.h, planes, x, view_planes, view_scales, cols, batch))
+
+    def view_matvec(self, weights_slot, w, planes, view_planes, view_scales, y, residual=None, batch=1):
+        res = None if residual is None else C.byref(residual)
+        self._check(self.l.smelt_emit_view_matvec(self.h, weights_slot, C.byref(w), planes, view_planes, view_scales, y, res, batch))
+
+    def view_gate_up_swiglu(self, weights_slot, gate, up, planes, view_planes, view_scales, y, batch=1):
+        self._check(self.l.smelt_emit_view_gate_up_swiglu(self.h, weights_slot, C.byref(gate), C.byref(up), planes,
+                                                          view_planes, view_scales, y, batch))
 
     def swap(self):
         self._check(self.l.smelt_emit_swap(self.h))

@@ -490,6 +490,85 @@ int smelt_emit_swiglu_fused(smelt_emitter* e, SmeltBinding gate, SmeltBinding up
     return emit_pointwise(e, "swiglu_fused", gate, up, output, count);
 }
 
+static int check_view(smelt_emitter* e, int planes, int cols, int batch_size) {
+    if (planes < 2 || planes > 6) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "activation views hold 2 to 6 planes");
+    if (cols <= 0 || cols % 128 != 0 || batch_size <= 0) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "activation views need cols % 128 == 0 and a positive batch");
+    return 0;
+}
+
+int smelt_emit_activation_view(smelt_emitter* e, int planes, SmeltBinding input, SmeltBinding view_planes,
+                               SmeltBinding view_scales, int cols, int batch_size) {
+    if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (int rc = check_view(e, planes, cols, batch_size)) return rc;
+    RecordBuilder rb;
+    rb.buffer(0, input);
+    rb.buffer(1, view_planes);
+    rb.buffer(2, view_scales);
+    rb.constant(3, (uint32_t)cols);
+    // one wave per group, four groups per workgroup
+    rb.grid((uint32_t)((cols / 128 + 3) / 4), (uint32_t)batch_size, 1, 256);
+    rb.r.pipeline = e->pipeline_index("signed_activation_bitplanes_i" + std::to_string(planes) + "_g128" + (batch_size > 1 ? "_batched" : ""));
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+static const char* view_weight_stem(smelt_emitter* e, const SmeltWeightEntryC* w) {
+    if (!w || (w->dtype != SMELT_DTYPE_BINARY1 && w->dtype != SMELT_DTYPE_TERNARY2)) {
+        efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "activation views are consumed by binary1 and ternary2 weights");
+        return nullptr;
+    }
+    if (check_signed_entry(e, w)) return nullptr;
+    return w->dtype == SMELT_DTYPE_BINARY1 ? "signed_binary_bitplane_i" : "signed_ternary_bitplane_i";
+}
+
+int smelt_emit_view_matvec(smelt_emitter* e, int weights_slot, const SmeltWeightEntryC* w, int planes, SmeltBinding view_planes,
+                           SmeltBinding view_scales, SmeltBinding output, const SmeltBinding* residual, int batch_size) {
+    if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    const char* stem = view_weight_stem(e, w);
+    if (!stem) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (int rc = check_view(e, planes, w->cols, batch_size)) return rc;
+    const MatvecGeometry g = matvec_geometry(signed_row_stride(to_format(w->dtype), (uint32_t)w->cols), w->rows, 4, e->compute_units);
+    RecordBuilder rb;
+    rb.buffer(0, weights_slot, w->offset);
+    rb.buffer(1, weights_slot, w->scales_offset);
+    rb.buffer(2, view_planes);
+    rb.buffer(3, view_scales);
+    rb.buffer(4, output);
+    uint8_t next = 5;
+    if (residual) rb.buffer(next++, *residual);
+    rb.constant(next, (uint32_t)w->rows);
+    rb.constant((uint8_t)(next + 1), (uint32_t)w->cols);
+    rb.grid((uint32_t)g.grid_w, (uint32_t)batch_size, 1, 256);
+    rb.r.pipeline = e->pipeline_index(std::string(stem) + std::to_string(planes) + (residual ? "_matvec_add_g128_rows8" : "_matvec_g128_rows8"));
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+int smelt_emit_view_gate_up_swiglu(smelt_emitter* e, int weights_slot, const SmeltWeightEntryC* gate, const SmeltWeightEntryC* up,
+                                   int planes, SmeltBinding view_planes, SmeltBinding view_scales, SmeltBinding output, int batch_size) {
+    if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    const char* stem = view_weight_stem(e, gate);
+    if (!stem || !view_weight_stem(e, up)) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (gate->dtype != up->dtype || gate->rows != up->rows || gate->cols != up->cols)
+        return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "gate and up must share format and shape");
+    if (int rc = check_view(e, planes, gate->cols, batch_size)) return rc;
+    const MatvecGeometry g = matvec_geometry(signed_row_stride(to_format(gate->dtype), (uint32_t)gate->cols), gate->rows, 2, e->compute_units);
+    RecordBuilder rb;
+    rb.buffer(0, weights_slot, gate->offset);
+    rb.buffer(1, weights_slot, gate->scales_offset);
+    rb.buffer(2, weights_slot, up->offset);
+    rb.buffer(3, weights_slot, up->scales_offset);
+    rb.buffer(4, view_planes);
+    rb.buffer(5, view_scales);
+    rb.buffer(6, output);
+    rb.constant(7, (uint32_t)gate->rows);
+    rb.constant(8, (uint32_t)gate->cols);
+    rb.grid((uint32_t)g.grid_w, (uint32_t)batch_size, 1, 256);
+    rb.r.pipeline = e->pipeline_index(std::string(stem) + std::to_string(planes) + "_gate_up_swiglu_g128_rows8");
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
 int smelt_emit_swap(smelt_emitter* e) {
     if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
     RecordBuilder rb;

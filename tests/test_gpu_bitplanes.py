@@ -190,3 +190,55 @@ def test_bad_view_records_are_refused(env):
     with pytest.raises(rt.SmeltHipError):
         ctx.interpret_decode(ctx.table([rt.make_record(ctx.pipeline("signed_activation_bitplanes_i4_g128"), [(X, 0, 0), (PL, 1, 0), (AS, 2, 0)],
                                                        [(3, 200)], (2, 1, 1), (32, 1, 1))]))
+
+
+def test_view_emitters_replay_a_signed_layer():
+    """One view per projection-bank input, every binary member consumes it: q/k/v from the hidden
+    view, gate+up+SwiGLU from the same view, down + residual from the activation's view."""
+    from smelt_amd import compiler as cc
+    hidden, ffn, planes = 1024, 2560, 5
+    ctx = rt.Context()
+    try:
+        lay = cc.Layout()
+        q, k = lay.signed(512, hidden, cc.BINARY1), lay.signed(256, hidden, cc.BINARY1)
+        gate, up = lay.signed(ffn, hidden, cc.BINARY1), lay.signed(ffn, hidden, cc.BINARY1)
+        down = lay.signed(hidden, ffn, cc.TERNARY2)
+        image = np.zeros(lay.total_bytes, np.uint8)
+        tensors = {}
+        for i, (name, e) in enumerate((("q", q), ("k", k), ("gate", gate), ("up", up), ("down", down))):
+            fmt = so.BINARY1 if e.dtype == cc.BINARY1 else so.TERNARY2
+            tensors[name] = signed_weights(50 + i, e.rows, e.cols, fmt) + (fmt,)
+            cc.write_signed(image, e, tensors[name][0], tensors[name][1])
+        H, V0P, V0S, Q, K, ACTB, V1P, V1S, OUT = 1, 2, 3, 4, 5, 6, 7, 8, 9
+        ctx.upload_weights(W, image)
+        h = fx.f16_bits(fx.rng_for(126, 0).normal(0, 1, hidden).astype(np.float32))
+        ctx.put(H, h)
+        for slot, size in ((V0P, hidden // 128 * planes * 16), (V0S, hidden // 128 * 2), (Q, 512 * 2), (K, 256 * 2), (ACTB, ffn * 2),
+                           (V1P, ffn // 128 * planes * 16), (V1S, ffn // 128 * 2), (OUT, hidden * 2)):
+            ctx.alloc(slot, size)
+        em = cc.Emitter(rt.ACT_F16, ctx.device_info()["compute_units"])
+        em.activation_view(planes, cc.bind(H), cc.bind(V0P), cc.bind(V0S), hidden)
+        em.view_matvec(W, q, planes, cc.bind(V0P), cc.bind(V0S), cc.bind(Q))
+        em.view_matvec(W, k, planes, cc.bind(V0P), cc.bind(V0S), cc.bind(K))
+        em.view_gate_up_swiglu(W, gate, up, planes, cc.bind(V0P), cc.bind(V0S), cc.bind(ACTB))
+        em.activation_view(planes, cc.bind(ACTB), cc.bind(V1P), cc.bind(V1S), ffn)
+        em.view_matvec(W, down, planes, cc.bind(V1P), cc.bind(V1S), cc.bind(OUT), residual=cc.bind(H))
+        assert em.pipelines == ["signed_activation_bitplanes_i5_g128", "signed_binary_bitplane_i5_matvec_g128_rows8",
+                                "signed_binary_bitplane_i5_gate_up_swiglu_g128_rows8", "signed_ternary_bitplane_i5_matvec_add_g128_rows8"]
+        em.install(ctx)
+        assert ctx.interpret_decode(em.records()) == 6
+        ctx.wait()
+        pl0, sc0, _ = so.activation_bitplanes(h, planes, so.F16)
+        mv = lambda n, pl, sc: so.signed_bitplane_matvec(tensors[n][2], tensors[n][0], tensors[n][1], pl, sc, tensors[n][0].shape[0],
+                                                         pl.shape[0] * 128, so.F16)
+        gh.check_outputs(ctx.read(Q, np.uint16, 512), mv("q", pl0, sc0), fx.F16, "q from the view")
+        gh.check_outputs(ctx.read(K, np.uint16, 256), mv("k", pl0, sc0), fx.F16, "k from the view")
+        act = ctx.read(ACTB, np.uint16, ffn)
+        ref_act = so.epilogue_signed_swiglu(so.narrow(mv("gate", pl0, sc0), so.F16), so.narrow(mv("up", pl0, sc0), so.F16), so.F16)
+        gh.check_outputs(act, so.widen(ref_act, so.F16), fx.F16, "gate+up+SwiGLU from the view", rel_tol=8e-3)
+        pl1, sc1, _ = so.activation_bitplanes(act, planes, so.F16)      # the device's own activations feed the second view
+        assert np.array_equal(ctx.read(V1P, np.uint32, pl1.size), pl1.reshape(-1)) and np.array_equal(ctx.read(V1S, np.uint16, sc1.size), sc1)
+        ref_out = so.epilogue_residual_add(mv("down", pl1, sc1), h, so.F16)
+        gh.check_outputs(ctx.read(OUT, np.uint16, hidden), so.widen(ref_out, so.F16), fx.F16, "down + residual from the view")
+    finally:
+        ctx.close()
