@@ -143,13 +143,17 @@ def main() -> int:
     g2, n2 = ctx.capture_decode(rl_only, cur=H0, alt=H1)
     ctx.graph_time(g2, 5)
     reps = 10
-    lm_us = ctx.graph_time(g2, reps) / (reps * n2)
+    # five timed series of ten replays each; the median series is reported (clock ramps and other
+    # tenants of the memory system move single series by a few percent)
+    series = sorted(ctx.graph_time(g2, reps) / (reps * n2) for _ in range(5))
+    lm_us = series[2]
     ctx.graph_destroy(g2)
     achieved = lm_bytes / lm_us / 1e3
     roofline = {"bound": "hbm", "kernel": "smelt_affine_matvec_argmax_single_bf16 (lm_head 151936x1024 u4 g64, fused argmax)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "bytes_per_launch": int(lm_bytes), "us_per_launch": round(lm_us, 3)}
+                "bytes_per_launch": int(lm_bytes), "us_per_launch": round(lm_us, 3),
+                "us_per_launch_series": [round(v, 3) for v in series]}
     del rl_table
     roofline["traffic"] = committed_traffic()
 
