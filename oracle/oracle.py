@@ -97,6 +97,9 @@ def _declare(l: C.CDLL) -> None:
         "so_swiglu_signed_activation_bitplanes": (None, [vp, vp, i32, i32, i32, vp, vp]),
         "so_norm_scale_signed_activation_bitplanes": (None, [f32, vp, vp, i32, i32, i32, vp, vp]),
         "so_signed_bitplane_matvec": (None, [i32, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+        "so_lut_matvec": (None, [vp, vp, vp, i32, i32, i32, vp]),
+        "so_epilogue_lut_add": (u16, [f32, u16, i32]),
+        "so_lut_gather": (None, [vp, vp, i32, i32, i32, vp]),
         "so_argmax_ordered_key16": (u32, [u16]),
         "so_argmax_pack_key": (C.c_uint64, [u16, u32]),
         "so_argmax16": (i32, [vp, i32]),
@@ -418,4 +421,31 @@ def signed_bitplane_matvec(fmt, packed, weight_scales, planes_arr, act_scales, r
     out = np.zeros(rows, np.float32)
     lib().so_signed_bitplane_matvec(fmt, _p(packed, np.uint8), _p(ws, np.uint16), _p(pl, np.uint32), _p(sc, np.uint16),
                                     rows, cols, pl.shape[1], dtype, _p(out, np.float32))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# u4_lut — lut_matvec.metal:28-790, 967-992
+# ---------------------------------------------------------------------------
+
+def lut_matvec(indices, lut_bits, x_f32, rows, cols, group) -> np.ndarray:
+    idx = np.ascontiguousarray(indices, np.uint8)
+    lut = np.ascontiguousarray(lut_bits, np.uint16)
+    x = np.ascontiguousarray(x_f32, np.float32)
+    out = np.zeros(rows, np.float32)
+    lib().so_lut_matvec(_p(idx, np.uint8), _p(lut, np.uint16), _p(x, np.float32), rows, cols, group, _p(out, np.float32))
+    return out
+
+
+def epilogue_lut_add(acc: np.ndarray, residual_bits: np.ndarray, dtype: int) -> np.ndarray:
+    l = lib()
+    return np.array([l.so_epilogue_lut_add(float(a), int(r), dtype) for a, r in zip(np.ravel(acc), np.ravel(residual_bits))],
+                    dtype=np.uint16)
+
+
+def lut_gather(indices, lut_bits, row, cols, group) -> np.ndarray:
+    idx = np.ascontiguousarray(indices, np.uint8)
+    lut = np.ascontiguousarray(lut_bits, np.uint16)
+    out = np.zeros(cols, np.uint16)
+    lib().so_lut_gather(_p(idx, np.uint8), _p(lut, np.uint16), row, cols, group, _p(out, np.uint16))
     return out

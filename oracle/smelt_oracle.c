@@ -803,6 +803,45 @@ SO_EXPORT void so_signed_bitplane_matvec(int format, const uint8_t *codes, const
 }
 
 /* ------------------------------------------------------------------------- */
+/* u4_lut — lut_matvec.metal:28-790, 967-992                                   */
+/* ------------------------------------------------------------------------- */
+
+/* y[r] = sum_c lut[r / group][index(r, c)] * x[c]: fp32, products accumulated in column order
+ * (lut_matvec.metal:86-140; the kernel's lanes each take every 32nd 16-column run, the scalar
+ * restatement keeps one running sum). lut is fp16 [ceil(rows / group), 16]. */
+SO_EXPORT void so_lut_matvec(const uint8_t *indices, const uint16_t *lut, const float *x, int rows,
+                             int cols, int group, float *out) {
+    int half_cols = cols / 2;
+    for (int r = 0; r < rows; ++r) {
+        const uint16_t *table = lut + (size_t)(r / group) * 16;
+        float acc = 0.0f;
+        for (int c = 0; c < cols; ++c) {
+            uint8_t byte = indices[(size_t)r * half_cols + (c >> 1)];
+            uint8_t idx = (c & 1) ? (byte >> 4) : (byte & 0x0F);
+            volatile float prod = so_f16_to_f32(table[idx]) * x[c];
+            acc += prod;
+        }
+        out[r] = acc;
+    }
+}
+
+/* fused_lut_matvec_add: half(float(residual) + acc) (lut_matvec.metal:334-340) */
+SO_EXPORT uint16_t so_epilogue_lut_add(float acc, uint16_t residual, int dtype) {
+    return narrow(widen(residual, dtype) + acc, dtype);
+}
+
+/* lut_embedding_gather (lut_matvec.metal:967-992) */
+SO_EXPORT void so_lut_gather(const uint8_t *indices, const uint16_t *lut, int row, int cols, int group,
+                             uint16_t *out) {
+    const uint16_t *table = lut + (size_t)(row / group) * 16;
+    for (int i = 0; i < cols / 2; ++i) {
+        uint8_t byte = indices[(size_t)row * (cols / 2) + i];
+        out[2 * i] = table[byte & 0x0F];
+        out[2 * i + 1] = table[byte >> 4];
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* Argmax key — lut_matvec.metal:4045-4074                                     */
 /* ------------------------------------------------------------------------- */
 

@@ -90,6 +90,9 @@ bool family_for(int weight, int* family) {
 bool hip_has_kernel(const SmeltMatvecCell& c, int family) {
     const bool quant = family == SMELT_FAMILY_AFFINE_U4 || family == SMELT_FAMILY_BINARY1 ||
                        family == SMELT_FAMILY_TERNARY2 || family == SMELT_FAMILY_TRIT5;
+    // u4_lut: single-token matvec, dual and gate+up+SwiGLU kernels (no batched / qmm form)
+    if (family == SMELT_FAMILY_LUT_U4)
+        return c.activation != SMELT_ACT_FP32 && c.shape == SMELT_SHAPE_GEMV && c.fusion != SMELT_FUSION_GATE_UP_GEGLU;
     if (!quant) return false;
     if (c.activation == SMELT_ACT_FP32) return false;
     if (c.fusion == SMELT_FUSION_GATE_UP_GEGLU) return false;

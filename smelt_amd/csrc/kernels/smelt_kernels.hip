@@ -8,6 +8,7 @@
 #include "import_kernels.hpp"
 #include "layer_kernels.hpp"
 #include "bitplane_kernels.hpp"
+#include "lut_kernels.hpp"
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
@@ -50,3 +51,5 @@ SMELT_BITPLANE_KERNELS(ternary, smelt::FmtTerPlanes, f16, smelt::F16)
 SMELT_BITPLANE_KERNELS(ternary, smelt::FmtTerPlanes, bf16, smelt::BF16)
 SMELT_ACTIVATION_BITPLANE_KERNELS(f16, smelt::F16)
 SMELT_ACTIVATION_BITPLANE_KERNELS(bf16, smelt::BF16)
+SMELT_LUT_KERNELS(f16, smelt::F16)
+SMELT_LUT_KERNELS(bf16, smelt::BF16)

@@ -186,6 +186,24 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->kinds += "UU";
             return kResolveOk;
         }
+        // u4_lut family (lut_matvec.metal:28-790): the second constant is the number of rows that share a table
+        {
+            const char* lut_symbol = nullptr;
+            if (name == "fused_lut_matvec") { out->family = kFamLutMatvec; lut_symbol = "smelt_lut_matvec_"; out->kinds = "PPPPUUU"; }
+            else if (name == "fused_lut_matvec_add") { out->family = kFamLutAdd; lut_symbol = "smelt_lut_matvec_add_"; out->kinds = "PPPPPUUU"; }
+            else if (name == "fused_dual_lut_matvec") { out->family = kFamLutDual; lut_symbol = "smelt_dual_lut_matvec_"; out->kinds = "PPPPPPPUUU"; }
+            else if (name == "fused_gate_up_swiglu") { out->family = kFamLutGateUp; lut_symbol = "smelt_lut_gate_up_swiglu_"; out->kinds = "PPPPPPUUU"; }
+            if (lut_symbol) {
+                if (cols == 0 || cols % 32 != 0 || group < 8) {
+                    *why = "u4_lut kernels need cols % 32 == 0 and at least 8 rows per table (got cols " +
+                           std::to_string(cols) + ", group " + std::to_string(group) + ")";
+                    return kResolveMalformed;
+                }
+                out->symbol = lut_symbol + t;
+                out->appended = {cols, group};
+                return kResolveOk;
+            }
+        }
         if (name == "affine_matvec") { out->family = kFamAffineMatvec; out->symbol = "smelt_affine_matvec_" + t; out->kinds = "PPPPPUUU"; }
         else if (name == "fused_affine_matvec_add") { out->family = kFamAffineAdd; out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; }
         else if (name == "fused_affine_gate_up_swiglu") { out->family = kFamAffineGateUp; out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; }
@@ -474,6 +492,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             }
         }
     }
+    if (entry == "lut_embedding_gather") { out->family = kFamLutGather; out->symbol = "smelt_lut_embedding_gather"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "signed_validate_codes") { out->family = kFamSignedValidate; out->symbol = "smelt_signed_validate_codes"; out->kinds = "PPUUU"; return kResolveOk; }
     if (entry == "signed_normalize_mlx_scales") { out->family = kFamSignedMlxScales; out->symbol = "smelt_signed_normalize_mlx_scales"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "copy_u128") { out->family = kFamCopy; out->symbol = "smelt_copy_u128"; out->kinds = "PPU"; return kResolveOk; }

@@ -48,6 +48,11 @@ enum FamilyId {
     kFamRmsScale,             // x scale | dim eps
     kFamResidualAddRmsScale,  // a b out scale dim eps
     kFamElementwise,          // a b out count
+    kFamLutMatvec,            // W lut x y rows | cols group                 (group = rows per table)
+    kFamLutAdd,               // W lut x y res rows | cols group
+    kFamLutDual,              // W1 lut1 W2 lut2 x y1 y2 rows | cols group
+    kFamLutGateUp,            // gW glut uW ulut x y rows | cols group
+    kFamLutGather,            // W lut token out cols group
     kFamActivationPlanes,     // x planes scales cols | nplanes             (grid.y = token)
     kFamSwigluPlanes,         // gate up planes scales cols | nplanes
     kFamNormScalePlanes,      // norm_scale x w planes scales cols | nplanes

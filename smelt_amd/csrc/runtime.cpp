@@ -124,8 +124,9 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
     auto bad_geom = [&](const std::string& m) {
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
     };
+    const bool lut_matvec = r.family == kFamLutMatvec || r.family == kFamLutAdd || r.family == kFamLutDual || r.family == kFamLutGateUp;
     const bool plane_matvec = r.family == kFamPlaneMatvec || r.family == kFamPlaneAdd || r.family == kFamPlaneGateUp;
-    const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec;
+    const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
     if (matvec_like) {
@@ -426,6 +427,40 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             if ((size_t)L.grid[0] * L.block[0] < count) return bad_geom("grid covers " + std::to_string((size_t)L.grid[0] * L.block[0]) + " of " + std::to_string(count) + " elements");
             for (size_t i = 0; i < ci; ++i) need[i] = count * 2;
             written[ci - 1] = true;
+            break;
+        }
+        case kFamLutMatvec:
+        case kFamLutAdd:
+        case kFamLutDual:
+        case kFamLutGateUp: {
+            // [W lut]+ x y [y2 | res] rows cols group
+            const size_t nmat = (r.family == kFamLutDual || r.family == kFamLutGateUp) ? 2 : 1;
+            const size_t xi = 2 * nmat;
+            const size_t ri = r.family == kFamLutMatvec ? 4 : (r.family == kFamLutAdd ? 5 : (r.family == kFamLutDual ? 7 : 6));
+            const size_t rows = U(ri), cols = U(ri + 1), group = U(ri + 2);
+            if (rows == 0 || cols == 0 || cols % 32 != 0 || group < 8) return bad_geom("u4_lut kernels need rows > 0, cols % 32 == 0 and at least 8 rows per table");
+            if (gy != 1) return bad_geom("u4_lut kernels take one token");
+            for (size_t m = 0; m < nmat; ++m) {
+                need[2 * m] = rows * (cols / 2); align[2 * m] = 16;
+                need[2 * m + 1] = cdiv(rows, group) * 32;
+            }
+            need[xi] = cols * 2; align[xi] = 16;
+            need[xi + 1] = rows * 2; written[xi + 1] = true;
+            if (r.family == kFamLutDual) { need[xi + 2] = rows * 2; written[xi + 2] = true; }
+            if (r.family == kFamLutAdd) need[xi + 2] = rows * 2;
+            L.lds = cols * 2 + (L.block[0] / 64) * nmat * 4 * 1024;
+            break;
+        }
+        case kFamLutGather: {
+            // W lut token out cols group
+            const size_t cols = U(4), group = U(5);
+            if (cols == 0 || cols % 2 != 0 || group == 0) return bad_geom("gather needs an even hidden size and a positive group");
+            if ((size_t)L.grid[0] * L.block[0] < cols / 2) return bad_geom("grid does not cover hidden / 2 threads");
+            if (L.grid[1] != 1 || L.grid[2] != 1 || L.block[1] != 1 || L.block[2] != 1) return bad_geom("1-D launch expected");
+            need[2] = 4; align[2] = 4;
+            need[3] = cols * 2; written[3] = true;
+            // rows are data (the token id): the table must at least hold one row and one table
+            need[0] = cols / 2; need[1] = 32;
             break;
         }
         case kFamPlaneMatvec:
