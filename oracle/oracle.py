@@ -100,6 +100,9 @@ def _declare(l: C.CDLL) -> None:
         "so_lut_matvec": (None, [vp, vp, vp, i32, i32, i32, vp]),
         "so_epilogue_lut_add": (u16, [f32, u16, i32]),
         "so_lut_gather": (None, [vp, vp, i32, i32, i32, vp]),
+        "so_tqh_prepare": (None, [vp, i32, i32, vp]),
+        "so_tqh_matvec": (None, [vp, vp, vp, i32, i32, vp]),
+        "so_tqh_dequantize_row": (None, [vp, vp, i32, vp]),
         "so_argmax_ordered_key16": (u32, [u16]),
         "so_argmax_pack_key": (C.c_uint64, [u16, u32]),
         "so_argmax16": (i32, [vp, i32]),
@@ -448,4 +451,32 @@ def lut_gather(indices, lut_bits, row, cols, group) -> np.ndarray:
     lut = np.ascontiguousarray(lut_bits, np.uint16)
     out = np.zeros(cols, np.uint16)
     lib().so_lut_gather(_p(idx, np.uint8), _p(lut, np.uint16), row, cols, group, _p(out, np.uint16))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# turbo_quant_h — lut_matvec.metal:1045-1079, 9207-9355
+# ---------------------------------------------------------------------------
+
+def tqh_prepare(x_bits, dtype: int) -> np.ndarray:
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    out = np.zeros((x.size + 127) // 128 * 128, np.float32)
+    lib().so_tqh_prepare(_p(x, np.uint16), x.size, dtype, _p(out, np.float32))
+    return out
+
+
+def tqh_matvec(codes, codebook_bits, xhat, rows, cols) -> np.ndarray:
+    c = np.ascontiguousarray(codes, np.uint8)
+    cb = np.ascontiguousarray(codebook_bits, np.uint16)
+    xh = np.ascontiguousarray(xhat, np.float32)
+    out = np.zeros(rows, np.float32)
+    lib().so_tqh_matvec(_p(c, np.uint8), _p(cb, np.uint16), _p(xh, np.float32), rows, cols, _p(out, np.float32))
+    return out
+
+
+def tqh_dequantize_row(row_codes, codebook_bits, cols) -> np.ndarray:
+    c = np.ascontiguousarray(row_codes, np.uint8)
+    cb = np.ascontiguousarray(codebook_bits, np.uint16)
+    out = np.zeros(cols, np.float32)
+    lib().so_tqh_dequantize_row(_p(c, np.uint8), _p(cb, np.uint16), cols, _p(out, np.float32))
     return out

@@ -842,6 +842,63 @@ SO_EXPORT void so_lut_gather(const uint8_t *indices, const uint16_t *lut, int ro
 }
 
 /* ------------------------------------------------------------------------- */
+/* turbo_quant_h — lut_matvec.metal:1045-1079, 9207-9355                       */
+/* ------------------------------------------------------------------------- */
+
+#define SO_TQH_INV_SQRT_G 0.0883883476483184405f
+
+static int tqh_code(const uint8_t *row_codes, int g, int j) {
+    return (row_codes[g * 32 + (j >> 2)] >> ((j & 3) * 2)) & 3;
+}
+
+/* tqh_matvec_prepare_input (:9222-9244): xhat[g, j] = sum_p (-1)^popcount(p & j) x[g*128 + p], fp32,
+ * p increasing, columns beyond cols skipped. xhat is [ceil(cols/128) * 128]. */
+SO_EXPORT void so_tqh_prepare(const uint16_t *x, int cols, int dtype, float *xhat) {
+    int groups = (cols + 127) / 128;
+    for (int g = 0; g < groups; ++g)
+        for (int j = 0; j < 128; ++j) {
+            float acc = 0.0f;
+            for (int p = 0; p < 128 && g * 128 + p < cols; ++p) {
+                float xp = widen(x[g * 128 + p], dtype);
+                acc += (__builtin_popcount((unsigned)(p & j)) & 1) ? -xp : xp;
+            }
+            xhat[g * 128 + j] = acc;
+        }
+}
+
+/* tqh_matvec (:9250-9343): acc = sum_{g, j} cb[g][code] * xhat[g, j] (fp32), out = acc / sqrt(128). */
+SO_EXPORT void so_tqh_matvec(const uint8_t *codes, const uint16_t *codebook, const float *xhat, int rows,
+                             int cols, float *out) {
+    int groups = (cols + 127) / 128;
+    int codes_per_row = groups * 32;
+    for (int r = 0; r < rows; ++r) {
+        float acc = 0.0f;
+        for (int g = 0; g < groups; ++g)
+            for (int j = 0; j < 128; ++j) {
+                volatile float prod = so_f16_to_f32(codebook[g * 4 + tqh_code(codes + (size_t)r * codes_per_row, g, j)]) * xhat[g * 128 + j];
+                acc += prod;
+            }
+        volatile float scaled = acc * SO_TQH_INV_SQRT_G;
+        out[r] = scaled;
+    }
+}
+
+/* tqh_embedding_gather (:1045-1079): one dequantised row in fp32 before the final rounding:
+ * W[p] = (sum_j (-1)^popcount(p & j) cb[g][code_j]) / sqrt(128). */
+SO_EXPORT void so_tqh_dequantize_row(const uint8_t *row_codes, const uint16_t *codebook, int cols, float *out) {
+    for (int c = 0; c < cols; ++c) {
+        int g = c / 128, p = c % 128;
+        float acc = 0.0f;
+        for (int j = 0; j < 128; ++j) {
+            float v = so_f16_to_f32(codebook[g * 4 + tqh_code(row_codes, g, j)]);
+            acc += (__builtin_popcount((unsigned)(p & j)) & 1) ? -v : v;
+        }
+        volatile float scaled = acc * SO_TQH_INV_SQRT_G;
+        out[c] = scaled;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* Argmax key — lut_matvec.metal:4045-4074                                     */
 /* ------------------------------------------------------------------------- */
 

@@ -93,6 +93,8 @@ bool hip_has_kernel(const SmeltMatvecCell& c, int family) {
     // u4_lut: single-token matvec, dual and gate+up+SwiGLU kernels (no batched / qmm form)
     if (family == SMELT_FAMILY_LUT_U4)
         return c.activation != SMELT_ACT_FP32 && c.shape == SMELT_SHAPE_GEMV && c.fusion != SMELT_FUSION_GATE_UP_GEGLU;
+    // turbo_quant_h: prepare + matvec pair (the batched names cover prefill rows), no fused forms
+    if (family == SMELT_FAMILY_TQH) return c.activation != SMELT_ACT_FP32 && c.fusion == SMELT_FUSION_NONE;
     if (!quant) return false;
     if (c.activation == SMELT_ACT_FP32) return false;
     if (c.fusion == SMELT_FUSION_GATE_UP_GEGLU) return false;

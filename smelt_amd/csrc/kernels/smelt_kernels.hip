@@ -9,6 +9,7 @@
 #include "layer_kernels.hpp"
 #include "bitplane_kernels.hpp"
 #include "lut_kernels.hpp"
+#include "tqh_kernels.hpp"
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
@@ -53,3 +54,5 @@ SMELT_ACTIVATION_BITPLANE_KERNELS(f16, smelt::F16)
 SMELT_ACTIVATION_BITPLANE_KERNELS(bf16, smelt::BF16)
 SMELT_LUT_KERNELS(f16, smelt::F16)
 SMELT_LUT_KERNELS(bf16, smelt::BF16)
+SMELT_TQH_KERNELS(f16, smelt::F16)
+SMELT_TQH_KERNELS(bf16, smelt::BF16)

@@ -492,6 +492,14 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             }
         }
     }
+    // turbo_quant_h (lut_matvec.metal:1045-1079, 9207-9486); the batched names differ only in the grid height
+    if (entry == "tqh_matvec_prepare_input" || entry == "tqh_matvec_prepare_input_batched") {
+        out->family = kFamTqhPrepare; out->symbol = "smelt_tqh_matvec_prepare_input_" + t; out->kinds = "PPU"; return kResolveOk;
+    }
+    if (entry == "tqh_matvec" || entry == "tqh_matvec_batched") {
+        out->family = kFamTqhMatvec; out->symbol = "smelt_tqh_matvec_" + t; out->kinds = "PPPPUUU"; return kResolveOk;
+    }
+    if (entry == "tqh_embedding_gather") { out->family = kFamTqhGather; out->symbol = "smelt_tqh_embedding_gather_" + t; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "lut_embedding_gather") { out->family = kFamLutGather; out->symbol = "smelt_lut_embedding_gather"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "signed_validate_codes") { out->family = kFamSignedValidate; out->symbol = "smelt_signed_validate_codes"; out->kinds = "PPUUU"; return kResolveOk; }
     if (entry == "signed_normalize_mlx_scales") { out->family = kFamSignedMlxScales; out->symbol = "smelt_signed_normalize_mlx_scales"; out->kinds = "PPPPUU"; return kResolveOk; }

@@ -53,6 +53,9 @@ enum FamilyId {
     kFamLutDual,              // W1 lut1 W2 lut2 x y1 y2 rows | cols group
     kFamLutGateUp,            // gW glut uW ulut x y rows | cols group
     kFamLutGather,            // W lut token out cols group
+    kFamTqhPrepare,           // x xhat cols                                 (grid.y = token)
+    kFamTqhMatvec,            // codes codebook xhat y rows cols codes_per_row (grid.y = token)
+    kFamTqhGather,            // codes codebook token out codes_per_row cols
     kFamActivationPlanes,     // x planes scales cols | nplanes             (grid.y = token)
     kFamSwigluPlanes,         // gate up planes scales cols | nplanes
     kFamNormScalePlanes,      // norm_scale x w planes scales cols | nplanes

@@ -463,6 +463,41 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[0] = cols / 2; need[1] = 32;
             break;
         }
+        case kFamTqhPrepare: {
+            // x xhat cols; dispatchThreads over groups * 128, grid.y = token
+            const size_t cols = U(2), groups = cdiv(cols, 128);
+            if (cols == 0) return bad_geom("cols must be positive");
+            if ((size_t)L.grid[0] * L.block[0] < groups * 128) return bad_geom("grid does not cover groups * 128 threads");
+            if (L.grid[2] != 1 || L.block[1] != 1 || L.block[2] != 1) return bad_geom("1-D workgroups expected");
+            need[0] = gy * cols * 2;
+            need[1] = gy * groups * 128 * 4; align[1] = 16; written[1] = true;
+            break;
+        }
+        case kFamTqhMatvec: {
+            // codes codebook xhat y rows cols codes_per_row; grid.y = token
+            const size_t rows = U(4), cols = U(5), cpr = U(6), groups = cdiv(cols, 128);
+            if (rows == 0 || cols == 0) return bad_geom("rows and cols must be positive");
+            if (cpr != groups * 32) return bad_geom("codes_per_row must be 32 bytes per 128-column group");
+            if (L.block[0] % 64 != 0 || L.block[0] > 256 || L.block[1] != 1 || L.block[2] != 1 || L.grid[2] != 1)
+                return bad_geom("tqh_matvec runs 64..256 threads in whole waves");
+            need[0] = rows * cpr; align[0] = 16;
+            need[1] = groups * 8;
+            need[2] = gy * groups * 128 * 4; align[2] = 16;
+            need[3] = gy * rows * 2; written[3] = true;
+            L.lds = groups * 128 * 4;
+            break;
+        }
+        case kFamTqhGather: {
+            // codes codebook token out codes_per_row cols
+            const size_t cpr = U(4), cols = U(5), groups = cdiv(cols, 128);
+            if (cols == 0 || cpr != groups * 32) return bad_geom("codes_per_row must be 32 bytes per 128-column group");
+            if ((size_t)L.grid[0] * L.block[0] < cols) return bad_geom("grid does not cover the row");
+            if (L.grid[1] != 1 || L.grid[2] != 1 || L.block[1] != 1 || L.block[2] != 1) return bad_geom("1-D launch expected");
+            need[0] = cpr; need[1] = groups * 8;
+            need[2] = 4; align[2] = 4;
+            need[3] = cols * 2; written[3] = true;
+            break;
+        }
         case kFamPlaneMatvec:
         case kFamPlaneAdd:
         case kFamPlaneGateUp: {

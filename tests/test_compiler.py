@@ -44,7 +44,7 @@ def test_gateway_has_no_holes_and_never_defaults():
     assert cc.select(cc.ACT_FP16, cc.FP16, hip_backend=True)[0] == cc.SELECT_MISSING
     assert cc.select(cc.ACT_FP16, cc.U4_LUT, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.U4_LUT, cc.GEMM, hip_backend=True)[0] == cc.SELECT_MISSING      # no batched u4_lut kernel
-    assert cc.select(cc.ACT_FP16, cc.TURBO_QUANT_H, hip_backend=True)[0] == cc.SELECT_MISSING
+    assert cc.select(cc.ACT_FP16, cc.TURBO_QUANT_H, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_MISSING
 
 
@@ -156,7 +156,8 @@ def test_pipeline_names_resolve_to_kernels_with_the_reference_binding_counts():
     assert cc.resolve_pipeline_name("fused_lut_matvec:1024:16")[1:] == ("smelt_lut_matvec_f16", "PPPPUUU")
     assert cc.resolve_pipeline_name("fused_gate_up_swiglu:1024:16")[1] == "smelt_lut_gate_up_swiglu_f16"
     assert cc.resolve_pipeline_name("fused_lut_matvec:1024:4")[0] == -3    # fewer than 8 rows per table
-    assert cc.resolve_pipeline_name("tqh_matvec")[0] == -4                 # turbo_quant_h is not built
+    assert cc.resolve_pipeline_name("tqh_matvec_batched")[1:] == ("smelt_tqh_matvec_f16", "PPPPUUU")
+    assert cc.resolve_pipeline_name("u4_lut_qmm")[0] == -4
     assert cc.resolve_pipeline_name("rms_norm_1pw_from_fp32")[0] == -4     # fp32 hidden states are out of scope
     assert cc.resolve_pipeline_name("rope_apply")[0] == -4
 
