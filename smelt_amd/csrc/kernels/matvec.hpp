@@ -183,8 +183,11 @@ struct FmtGeom {
 //   pairs : [MB][kChunksPerUnit][U] x 16 B   (chunk-major so consecutive lanes hit consecutive 16 B)
 //   corr  : [MB][U][kCorrStride] floats (one per dword of the unit)
 //   xsum  : [MB][U][kCorrStride] floats (affine only)
+constexpr int kPlaneSlots = 8;   // 16-byte plane slots per token and unit for activation views (2..6 used)
+
 template <class F>
 __device__ __forceinline__ size_t lds_pairs_bytes(int U, int MB) {
+    if constexpr (F::kBitplanes) return (size_t)MB * kPlaneSlots * U * 16;
     return (size_t)MB * FmtGeom<F>::kChunksPerUnit * U * 16;
 }
 
@@ -193,38 +196,47 @@ __device__ __forceinline__ size_t lds_pairs_bytes(int U, int MB) {
 // words; ternary: the unit's 64 columns spread to the even bits of four dwords, the layout of the
 // 2-bit codes); lds_corr holds per unit the activation scale, the binary correction
 // sum_p 2^p popcount(plane_p) and the plane count.
-template <class F, class ActT>
+template <class F, class ActT, int MB>
 __device__ __forceinline__ void stage_planes(const uint32_t* __restrict__ planes, const uint16_t* __restrict__ act_scales,
-                                             int nplanes, int U, int batch_row, uint4_t* lds_pairs, float* lds_corr) {
+                                             int nplanes, int U, int b0, int nb, uint4_t* lds_pairs, float* lds_corr) {
     constexpr bool TER = F::kTernaryPlanes;
+    constexpr int NCH = kPlaneSlots;
     const int groups = TER ? U / 2 : U;
-    planes += (size_t)batch_row * groups * nplanes * 4;
-    act_scales += (size_t)batch_row * groups;
-    for (int item = threadIdx.x; item < U * nplanes; item += blockDim.x) {
-        const int u = item / nplanes, p = item - u * nplanes;
-        uint4_t v;
-        if constexpr (!TER) {
-            v = *reinterpret_cast<const uint4_t*>(planes + ((size_t)u * nplanes + p) * 4);
-        } else {
-            const uint2_t w = *reinterpret_cast<const uint2_t*>(planes + ((size_t)(u >> 1) * nplanes + p) * 4 + 2 * (u & 1));
-            v.x = spread16(w.x & 0xFFFFu); v.y = spread16(w.x >> 16);
-            v.z = spread16(w.y & 0xFFFFu); v.w = spread16(w.y >> 16);
+    for (int item = threadIdx.x; item < MB * U * nplanes; item += blockDim.x) {
+        const int b = item / (U * nplanes), rest = item - b * U * nplanes;
+        const int u = rest / nplanes, p = rest - u * nplanes;
+        uint4_t v = {0u, 0u, 0u, 0u};
+        if (b < nb) {
+            const uint32_t* src = planes + (size_t)(b0 + b) * groups * nplanes * 4;
+            if constexpr (!TER) {
+                v = *reinterpret_cast<const uint4_t*>(src + ((size_t)u * nplanes + p) * 4);
+            } else {
+                const uint2_t w = *reinterpret_cast<const uint2_t*>(src + ((size_t)(u >> 1) * nplanes + p) * 4 + 2 * (u & 1));
+                v.x = spread16(w.x & 0xFFFFu); v.y = spread16(w.x >> 16);
+                v.z = spread16(w.y & 0xFFFFu); v.w = spread16(w.y >> 16);
+            }
         }
-        lds_pairs[(size_t)p * U + u] = v;
+        lds_pairs[((size_t)b * NCH + p) * U + u] = v;
     }
-    for (int u = threadIdx.x; u < U; u += blockDim.x) {
+    for (int item = threadIdx.x; item < MB * U; item += blockDim.x) {
+        const int b = item / U, u = item - b * U;
         const int g = TER ? u >> 1 : u;
         int bias = 0;
-        if constexpr (!TER) {
-            for (int p = 0; p < nplanes - 1; ++p)
-                bias += popcount128(*reinterpret_cast<const uint4_t*>(planes + ((size_t)g * nplanes + p) * 4)) << p;
+        float scale = 0.0f;
+        if (b < nb) {
+            const uint32_t* src = planes + (size_t)(b0 + b) * groups * nplanes * 4;
+            if constexpr (!TER) {
+                for (int p = 0; p < nplanes - 1; ++p)
+                    bias += popcount128(*reinterpret_cast<const uint4_t*>(src + ((size_t)g * nplanes + p) * 4)) << p;
+            }
+            scale = ActT::widen(act_scales[(size_t)(b0 + b) * groups + g]);
         }
         float4_t c;
-        c.x = ActT::widen(act_scales[g]);
+        c.x = scale;
         c.y = __builtin_bit_cast(float, bias);
         c.z = __builtin_bit_cast(float, nplanes);
         c.w = 0.0f;
-        *reinterpret_cast<float4_t*>(lds_corr + (size_t)u * 4) = c;
+        *reinterpret_cast<float4_t*>(lds_corr + ((size_t)b * U + u) * 4) = c;
     }
 }
 
@@ -234,8 +246,7 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
                                                   float* lds_corr, float* lds_xsum,
                                                   const uint16_t* x2 = nullptr, int nplanes = 0) {
     if constexpr (F::kBitplanes) {
-        static_assert(MB == 1, "activation views are consumed one token per launch row");
-        stage_planes<F, ActT>(reinterpret_cast<const uint32_t*>(x), x2, nplanes, U, b0, lds_pairs, lds_corr);
+        stage_planes<F, ActT, MB>(reinterpret_cast<const uint32_t*>(x), x2, nplanes, U, b0, nb, lds_pairs, lds_corr);
         return;
     }
     using G = FmtGeom<F>;
@@ -294,6 +305,11 @@ struct MatPtrs {
     const uint8_t* codes;
     const uint16_t* scales;
     const uint16_t* biases;  // affine only
+    // Optional second physical matrix that continues the row space at row `split` (two projections
+    // driven as one matvec without moving their weights); split == 0 means there is none.
+    const uint8_t* codes_hi = nullptr;
+    const uint16_t* scales_hi = nullptr;
+    int split = 0;
 };
 
 // Registers of one work item: the 16-byte unit `u` of R rows of NMAT matrices plus the group
@@ -315,11 +331,19 @@ __device__ __forceinline__ void load_item(const MatPtrs (&mats)[NMAT], const int
     for (int m = 0; m < NMAT; ++m)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            it.c[m][r] = *reinterpret_cast<const uint4_t*>(mats[m].codes + (size_t)row[r] * row_stride + (size_t)u * 16);
-            const size_t si = (size_t)row[r] * groups_per_row + g;
-            it.s[m][r] = mats[m].scales[si];
+            const uint8_t* codes = mats[m].codes;
+            const uint16_t* scales = mats[m].scales;
+            int rr = row[r];
+            if (mats[m].split > 0 && rr >= mats[m].split) {
+                codes = mats[m].codes_hi;
+                scales = mats[m].scales_hi;
+                rr -= mats[m].split;
+            }
+            it.c[m][r] = *reinterpret_cast<const uint4_t*>(codes + (size_t)rr * row_stride + (size_t)u * 16);
+            const size_t si = (size_t)rr * groups_per_row + g;
+            it.s[m][r] = scales[si];
             if (F::kHasBias) it.b[m][r] = mats[m].biases[si];
-            else if (F::kPerDwordScale) it.b[m][r] = mats[m].scales[g + 1 < groups_per_row ? si + 1 : si];
+            else if (F::kPerDwordScale) it.b[m][r] = scales[g + 1 < groups_per_row ? si + 1 : si];
             else it.b[m][r] = 0;
         }
 }
@@ -331,48 +355,53 @@ __device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u,
                                              const float* lds_xsum, const uint16_t* lut,
                                              float (&acc)[NMAT][R][MB]) {
     if constexpr (F::kBitplanes) {
-        const float4_t c4 = *reinterpret_cast<const float4_t*>(lds_corr + (size_t)u * 4);
-        // (elements are copied out before the bit casts: a bit cast applied directly to a vector
-        //  element reads the vector's first lane)
-        const float act_scale = c4.x, bias_bits = c4.y, nplanes_bits = c4.z;
-        const int bias = __builtin_bit_cast(int, bias_bits);
-        const int nplanes = __builtin_bit_cast(int, nplanes_bits);
-        const uint4_t sign = lds_pairs[(size_t)(nplanes - 1) * U + u];
-        uint4_t agree[NMAT][R], nonzero[NMAT][R];
-        int weighted[NMAT][R], active[NMAT][R];
+        constexpr int PCH = kPlaneSlots;
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const uint4_t c = it.c[m][r];
-                if constexpr (!F::kTernaryPlanes) {
-                    agree[m][r] = c ^ sign;          // weight +1 and activation >= 0, or -1 and < 0
-                } else {
-                    const uint4_t even = {0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u};
-                    const uint4_t pos = (c >> 1) & even;   // code 2 = +1
-                    nonzero[m][r] = ~c & even;             // code 1 = 0 has its low bit set
-                    agree[m][r] = nonzero[m][r] & (pos ^ sign);
-                }
-                weighted[m][r] = 0;
-                active[m][r] = 0;
-            }
-        for (int p = 0; p < nplanes - 1; ++p) {
-            const uint4_t plane = lds_pairs[(size_t)p * U + u];
+        for (int b = 0; b < MB; ++b) {
+            const float4_t c4 = *reinterpret_cast<const float4_t*>(lds_corr + ((size_t)b * U + u) * 4);
+            // (elements are copied out before the bit casts: a bit cast applied directly to a vector
+            //  element reads the vector's first lane)
+            const float act_scale = c4.x, bias_bits = c4.y, nplanes_bits = c4.z;
+            const int bias = __builtin_bit_cast(int, bias_bits);
+            const int nplanes = __builtin_bit_cast(int, nplanes_bits);
+            const uint4_t* my_planes = lds_pairs + (size_t)b * PCH * U + u;
+            const uint4_t sign = my_planes[(size_t)(nplanes - 1) * U];
+            uint4_t agree[NMAT][R], nonzero[NMAT][R];
+            int weighted[NMAT][R], active[NMAT][R];
 #pragma unroll
             for (int m = 0; m < NMAT; ++m)
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    weighted[m][r] += popcount128(agree[m][r] & plane) << p;
-                    if constexpr (F::kTernaryPlanes) active[m][r] += popcount128(nonzero[m][r] & plane) << p;
+                    const uint4_t c = it.c[m][r];
+                    if constexpr (!F::kTernaryPlanes) {
+                        agree[m][r] = c ^ sign;          // weight +1 and activation >= 0, or -1 and < 0
+                    } else {
+                        const uint4_t even = {0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u};
+                        const uint4_t pos = (c >> 1) & even;   // code 2 = +1
+                        nonzero[m][r] = ~c & even;             // code 1 = 0 has its low bit set
+                        agree[m][r] = nonzero[m][r] & (pos ^ sign);
+                    }
+                    weighted[m][r] = 0;
+                    active[m][r] = 0;
+                }
+            for (int p = 0; p < nplanes - 1; ++p) {
+                const uint4_t plane = my_planes[(size_t)p * U];
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        weighted[m][r] += popcount128(agree[m][r] & plane) << p;
+                        if constexpr (F::kTernaryPlanes) active[m][r] += popcount128(nonzero[m][r] & plane) << p;
+                    }
+            }
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int dot = 2 * weighted[m][r] - (F::kTernaryPlanes ? active[m][r] : bias);
+                    acc[m][r][b] = __builtin_fmaf((float)dot * act_scale, ScaleT::widen(it.s[m][r]), acc[m][r][b]);
                 }
         }
-#pragma unroll
-        for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int dot = 2 * weighted[m][r] - (F::kTernaryPlanes ? active[m][r] : bias);
-                acc[m][r][0] = __builtin_fmaf((float)dot * act_scale, ScaleT::widen(it.s[m][r]), acc[m][r][0]);
-            }
         return;
     }
     using G = FmtGeom<F>;

@@ -409,6 +409,32 @@ using u32 = uint32_t;
                                             packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
                                             blockIdx.y + 1, epi, AS, (int)nplanes);               \
     }                                                                                             \
+    /* prompt rows: `tile` tokens per grid row, four at a time share every weight load          \
+       (signed_binary_bitplane_i{N}_matvec_g128_rows8_batched_b{4,8,16}, :1350-1562) */          \
+    SMELT_KERNEL void smelt_signed_##FN##_bitplane_matvec_batched_##T(                            \
+        const u8* C, const u16* S, const u32* P, const u16* AS, u16* Y, u32 rows, u32 cols,       \
+        u32 batch, u32 nplanes, u32 tile) {                                                       \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        const u32 lo = blockIdx.y * tile;                                                         \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + tile < batch ? lo + tile : batch;                                     \
+        matvec_body<FMT, ACT, F16, 4, 4, 1>(mats, reinterpret_cast<const u16*>(P), rows, cols,    \
+                                            packed_row_stride<FMT>(cols, 128), 128, lo, hi, epi,  \
+                                            AS, (int)nplanes);                                    \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_##FN##_bitplane_bank4_matvec_##T(                              \
+        const u8* C, const u16* S, const u32* P, const u16* AS, u16* y0, u16* y1, u16* y2,        \
+        u16* y3, u32 rows0, u32 rows1, u32 rows2, u32 rows3, u32 cols, u32 nplanes) {             \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        matvec_body<FMT, ACT, F16, 4, 1, 1>(mats, reinterpret_cast<const u16*>(P),                \
+                                            rows0 + rows1 + rows2 + rows3, cols,                  \
+                                            packed_row_stride<FMT>(cols, 128), 128, 0, 1, epi,    \
+                                            AS, (int)nplanes);                                    \
+    }                                                                                             \
     SMELT_KERNEL void smelt_signed_##FN##_bitplane_gate_up_swiglu_##T(                            \
         const u8* gC, const u16* gS, const u8* uC, const u16* uS, const u32* P, const u16* AS,    \
         u16* Y, u32 rows, u32 cols, u32 nplanes) {                                                \
@@ -418,6 +444,41 @@ using u32 = uint32_t;
         matvec_body<FMT, ACT, F16, 2, 1, 2>(mats, reinterpret_cast<const u16*>(P), rows, cols,    \
                                             packed_row_stride<FMT>(cols, 128), 128, blockIdx.y,   \
                                             blockIdx.y + 1, epi, AS, (int)nplanes);               \
+    }
+
+// Binary projection banks on the direct (fp16 activation) path, signed_quant.metal:2638-2935:
+//   packed bank   one code slab whose rows belong to 2 or 4 consumers in order
+//   dual/virtual  two separate matrices driven as one row space (rows of the first, then the second)
+#define SMELT_BINARY_BANK_KERNELS(T, ACT)                                                         \
+    SMELT_KERNEL void smelt_signed_binary_packed_bank_matvec_##T(                                 \
+        const u8* C, const u16* S, const u16* X, u16* y0, u16* y1, u32 rows0, u32 rows1,          \
+        u32 cols) {                                                                               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, nullptr, nullptr}, {rows0, rows1, 0u, 0u}};                \
+        matvec_body<FmtBin, ACT, F16, 4, 1, 1>(mats, X, rows0 + rows1, cols,                      \
+                                               packed_row_stride<FmtBin>(cols, 128), 128, 0, 1,   \
+                                               epi);                                              \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_binary_packed_bank4_matvec_##T(                                \
+        const u8* C, const u16* S, const u16* X, u16* y0, u16* y1, u16* y2, u16* y3, u32 rows0,   \
+        u32 rows1, u32 rows2, u32 rows3, u32 cols) {                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        matvec_body<FmtBin, ACT, F16, 4, 1, 1>(mats, X, rows0 + rows1 + rows2 + rows3, cols,      \
+                                               packed_row_stride<FmtBin>(cols, 128), 128, 0, 1,   \
+                                               epi);                                              \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_signed_binary_two_matrix_matvec_##T(                                  \
+        const u8* C1, const u16* S1, const u8* C2, const u16* S2, const u16* X, u16* y1, u16* y2, \
+        u32 rows1, u32 rows2, u32 cols) {                                                         \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C1, S1, nullptr, C2, S2, (int)rows1}};                          \
+        EpiBank4<ACT> epi{{}, {y1, y2, nullptr, nullptr}, {rows1, rows2, 0u, 0u}};                \
+        matvec_body<FmtBin, ACT, F16, 4, 1, 1>(mats, X, rows1 + rows2, cols,                      \
+                                               packed_row_stride<FmtBin>(cols, 128), 128, 0, 1,   \
+                                               epi);                                              \
     }
 
 // ---- lm_head: matvec fused with argmax over the rounded logits -------------------------------

@@ -56,3 +56,5 @@ SMELT_LUT_KERNELS(f16, smelt::F16)
 SMELT_LUT_KERNELS(bf16, smelt::BF16)
 SMELT_TQH_KERNELS(f16, smelt::F16)
 SMELT_TQH_KERNELS(bf16, smelt::BF16)
+SMELT_BINARY_BANK_KERNELS(f16, smelt::F16)
+SMELT_BINARY_BANK_KERNELS(bf16, smelt::BF16)

@@ -82,6 +82,11 @@ size_t matvec_lds_bytes(CodeLayout layout, uint32_t row_stride_bytes, uint32_t m
     return (size_t)mb * U * (16 * chunks + 2 * 4 * corr) + extra;
 }
 
+size_t plane_matvec_lds_bytes(uint32_t row_stride_bytes, uint32_t mb) {
+    const size_t U = row_stride_bytes / 16;
+    return (size_t)mb * U * (16 * 8 + 2 * 4 * 4);
+}
+
 size_t qmm_lds_bytes(uint32_t nmat, uint32_t mt) {
     const size_t ld = 128 + 8;
     return ((size_t)nmat * 64 + (size_t)mt * 16) * ld * 2;
@@ -486,6 +491,18 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                 out->family = kFamPlaneAdd; out->symbol = stem + "matvec_add_" + t; out->kinds = "PPPPPPUUU";
                 return kResolveOk;
             }
+            for (uint32_t tile : {4u, 8u, 16u}) {
+                if (tail == "_matvec_g128_rows8_batched_b" + std::to_string(tile)) {
+                    out->family = kFamPlaneBatched; out->symbol = stem + "matvec_batched_" + t; out->kinds = "PPPPPUUUUU";
+                    out->appended = {n, tile};
+                    out->lds_variant = 4;
+                    return kResolveOk;
+                }
+            }
+            if (tail == "_bank4_matvec_g128_rows8") {
+                out->family = kFamPlaneBank4; out->symbol = stem + "bank4_matvec_" + t; out->kinds = "PPPPPPPPUUUUUU";
+                return kResolveOk;
+            }
             if (tail == "_gate_up_swiglu_g128_rows8") {
                 out->family = kFamPlaneGateUp; out->symbol = stem + "gate_up_swiglu_" + t; out->kinds = "PPPPPPPUUU";
                 return kResolveOk;
@@ -501,6 +518,16 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
     }
     if (entry == "tqh_embedding_gather") { out->family = kFamTqhGather; out->symbol = "smelt_tqh_embedding_gather_" + t; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "lut_embedding_gather") { out->family = kFamLutGather; out->symbol = "smelt_lut_embedding_gather"; out->kinds = "PPPPUU"; return kResolveOk; }
+    // binary projection banks on the direct path (signed_quant.metal:2638-2935)
+    if (entry == "signed_binary_packed_bank_matvec_g128_rows8") {
+        out->family = kFamBinaryPackedBank; out->format = kFmtBinary1; out->symbol = "smelt_signed_binary_packed_bank_matvec_" + t; out->kinds = "PPPPPUUU"; return kResolveOk;
+    }
+    if (entry == "signed_binary_packed_bank4_matvec_g128_rows8") {
+        out->family = kFamBinaryPackedBank4; out->format = kFmtBinary1; out->symbol = "smelt_signed_binary_packed_bank4_matvec_" + t; out->kinds = "PPPPPPPUUUUU"; return kResolveOk;
+    }
+    if (entry == "signed_binary_dual_matvec_g128_rows8" || entry == "signed_binary_virtual_bank_matvec_g128_rows8") {
+        out->family = kFamBinaryTwoMatrix; out->format = kFmtBinary1; out->symbol = "smelt_signed_binary_two_matrix_matvec_" + t; out->kinds = "PPPPPPPUUU"; return kResolveOk;
+    }
     if (entry == "signed_validate_codes") { out->family = kFamSignedValidate; out->symbol = "smelt_signed_validate_codes"; out->kinds = "PPUUU"; return kResolveOk; }
     if (entry == "signed_normalize_mlx_scales") { out->family = kFamSignedMlxScales; out->symbol = "smelt_signed_normalize_mlx_scales"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "copy_u128") { out->family = kFamCopy; out->symbol = "smelt_copy_u128"; out->kinds = "PPU"; return kResolveOk; }

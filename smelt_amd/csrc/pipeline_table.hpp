@@ -62,6 +62,11 @@ enum FamilyId {
     kFamPlaneMatvec,          // C S planes ascales Y rows cols | nplanes   (grid.y = token)
     kFamPlaneAdd,             // C S planes ascales Y res rows cols | nplanes
     kFamPlaneGateUp,          // gC gS uC uS planes ascales Y rows cols | nplanes
+    kFamPlaneBatched,         // C S planes ascales Y rows cols batch | nplanes tile   (grid.y = token tile)
+    kFamPlaneBank4,           // C S planes ascales y0 y1 y2 y3 rows0 rows1 rows2 rows3 cols | nplanes
+    kFamBinaryPackedBank,     // C S x y0 y1 rows0 rows1 cols
+    kFamBinaryPackedBank4,    // C S x y0 y1 y2 y3 rows0 rows1 rows2 rows3 cols
+    kFamBinaryTwoMatrix,      // C1 S1 C2 S2 x y1 y2 rows1 rows2 cols
     kFamCopy16,               // src dst count
     kFamCount
 };
@@ -108,6 +113,8 @@ uint32_t mfma_matvec_kw(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_
 
 // LDS bytes the matvec kernels need for one packed row stride with `mb` resident activation rows.
 size_t matvec_lds_bytes(CodeLayout layout, uint32_t row_stride_bytes, uint32_t mb);
+// LDS bytes of the activation-view consumers: eight 16-byte plane slots and four floats per token and unit.
+size_t plane_matvec_lds_bytes(uint32_t row_stride_bytes, uint32_t mb);
 // LDS bytes of the MFMA qmm kernels: nmat weight tiles of 64 x 128 fp16 plus 16*mt token rows.
 size_t qmm_lds_bytes(uint32_t nmat, uint32_t mt);
 // LDS bytes of the affine qmm kernels: packed code tiles, fp32 scale/bias tiles, token rows and sums.

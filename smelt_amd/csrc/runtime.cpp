@@ -125,7 +125,9 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
     };
     const bool lut_matvec = r.family == kFamLutMatvec || r.family == kFamLutAdd || r.family == kFamLutDual || r.family == kFamLutGateUp;
-    const bool plane_matvec = r.family == kFamPlaneMatvec || r.family == kFamPlaneAdd || r.family == kFamPlaneGateUp;
+    const bool plane_matvec = r.family == kFamPlaneMatvec || r.family == kFamPlaneAdd || r.family == kFamPlaneGateUp ||
+                              r.family == kFamPlaneBank4 || r.family == kFamPlaneBatched || r.family == kFamBinaryPackedBank || r.family == kFamBinaryPackedBank4 ||
+                              r.family == kFamBinaryTwoMatrix;
     const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
@@ -158,6 +160,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
     };
     const CodeLayout layout = code_layout(r.format);
     auto signed_lds = [&](size_t cols, uint32_t mb) { return matvec_lds_bytes(layout, signed_row_stride(r.format, (uint32_t)cols), mb); };
+    auto plane_lds = [&](size_t cols, uint32_t mb) { return plane_matvec_lds_bytes(signed_row_stride(r.format, (uint32_t)cols), mb); };
     auto need_256 = [&]() -> int {
         if (L.block[0] != 256) return bad_geom("MFMA qmm kernels run with 256-thread workgroups, got " + std::to_string(L.block[0]));
         return 0;
@@ -498,6 +501,60 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[3] = cols * 2; written[3] = true;
             break;
         }
+        case kFamPlaneBatched: {
+            // C S planes ascales Y rows cols batch nplanes tile
+            const size_t rows = U(5), cols = U(6), batch = U(7), nplanes = U(8), tile = U(9);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            if (nplanes < 2 || nplanes > 6) return bad_geom("activation views hold 2 to 6 planes");
+            if (batch == 0 || gy * tile < batch) return bad_geom("grid height * token tile does not cover the batch");
+            signed_w(0, 1, rows, cols);
+            need[2] = batch * (cols / 128) * nplanes * 16; align[2] = 16;
+            need[3] = batch * (cols / 128) * 2;
+            need[4] = batch * rows * 2; written[4] = true;
+            L.lds = plane_lds(cols, 4);
+            break;
+        }
+        case kFamPlaneBank4:
+        case kFamBinaryPackedBank:
+        case kFamBinaryPackedBank4: {
+            // C S (planes ascales | x) y0 .. y{n-1} rows0 .. rows{n-1} cols [nplanes]; one token
+            const bool view = r.family == kFamPlaneBank4;
+            const size_t nout = r.family == kFamBinaryPackedBank ? 2 : 4;
+            const size_t y0 = view ? 4 : 3, r0 = y0 + nout, ci = r0 + nout;
+            const size_t cols = U(ci);
+            size_t rows = 0;
+            for (size_t m = 0; m < nout; ++m) rows += U(r0 + m);
+            if (int e = check_signed_shape(rows, cols)) return e;
+            if (gy != 1) return bad_geom("projection-bank kernels take one token");
+            signed_w(0, 1, rows, cols);
+            if (view) {
+                const size_t nplanes = U(ci + 1);
+                if (nplanes < 2 || nplanes > 6) return bad_geom("activation views hold 2 to 6 planes");
+                need[2] = (cols / 128) * nplanes * 16; align[2] = 16;
+                need[3] = (cols / 128) * 2;
+            } else {
+                need[2] = cols * 2; align[2] = 16;
+            }
+            for (size_t m = 0; m < nout; ++m) {
+                need[y0 + m] = U(r0 + m) * 2;
+                written[y0 + m] = true;
+            }
+            L.lds = view ? plane_lds(cols, 1) : signed_lds(cols, 1);
+            break;
+        }
+        case kFamBinaryTwoMatrix: {
+            // C1 S1 C2 S2 x y1 y2 rows1 rows2 cols
+            const size_t rows1 = U(7), rows2 = U(8), cols = U(9);
+            if (int e = check_signed_shape(rows1 + rows2, cols)) return e;
+            if (gy != 1) return bad_geom("projection-bank kernels take one token");
+            signed_w(0, 1, rows1, cols);
+            signed_w(2, 3, rows2, cols);
+            need[4] = cols * 2; align[4] = 16;
+            need[5] = rows1 * 2; written[5] = true;
+            need[6] = rows2 * 2; written[6] = true;
+            L.lds = signed_lds(cols, 1);
+            break;
+        }
         case kFamPlaneMatvec:
         case kFamPlaneAdd:
         case kFamPlaneGateUp: {
@@ -514,7 +571,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[pi + 1] = gy * groups * 2;
             need[pi + 2] = gy * rows * 2; written[pi + 2] = true;
             if (r.family == kFamPlaneAdd) need[pi + 3] = gy * rows * 2;
-            L.lds = signed_lds(cols, 1);
+            L.lds = plane_lds(cols, 1);
             break;
         }
         case kFamActivationPlanes:

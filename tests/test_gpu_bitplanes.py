@@ -242,3 +242,94 @@ def test_view_emitters_replay_a_signed_layer():
         gh.check_outputs(ctx.read(OUT, np.uint16, hidden), so.widen(ref_out, so.F16), fx.F16, "down + residual from the view")
     finally:
         ctx.close()
+
+
+def run_bank(ctx, name, mats, inputs, member_rows, cols, dtype):
+    """mats: [(packed, scales)] (one slab, or two matrices); inputs: list of arrays bound after them;
+    outputs follow, then one row count per output, then cols."""
+    wf = gh.WeightFile()
+    bufs, i = [], 0
+    for p, s in mats:
+        bufs += [(W, i, wf.add(p)), (W, i + 1, wf.add(s))]
+        i += 2
+    ctx.upload_weights(W, wf.image())
+    for k, arr in enumerate(inputs):
+        ctx.put(10 + k, arr)
+        bufs.append((10 + k, i, 0))
+        i += 1
+    for k, r in enumerate(member_rows):
+        ctx.alloc(20 + k, max(r, 1) * 2)
+        bufs.append((20 + k, i, 0))
+        i += 1
+    consts = [(i + k, r) for k, r in enumerate(member_rows)] + [(i + len(member_rows), cols)]
+    rec = rt.make_record(ctx.pipeline(name), bufs, consts, ((sum(member_rows) + 15) // 16, 1, 1), (256, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    return [ctx.read(20 + k, np.uint16, r) for k, r in enumerate(member_rows) if r]
+
+
+@pytest.mark.parametrize("fmt,planes", [(so.BINARY1, 2), (so.BINARY1, 3), (so.TERNARY2, 4), (so.TERNARY2, 6)])
+def test_view_bank4(env, fmt, planes):
+    ctx, dtype, odt = env
+    stem = "binary" if fmt == so.BINARY1 else "ternary"
+    member_rows, cols = [130, 37, 37, 64], 1280
+    rows = sum(member_rows)
+    packed, ws = signed_weights(60 + planes, rows, cols, fmt)
+    x = bits(fx.rng_for(127, planes).normal(0, 1, cols).astype(np.float32), dtype)
+    pl, asc, _ = so.activation_bitplanes(x, planes, odt)
+    outs = run_bank(ctx, f"signed_{stem}_bitplane_i{planes}_bank4_matvec_g128_rows8", [(packed, ws)], [pl, asc], member_rows, cols, dtype)
+    ref = so.signed_bitplane_matvec(fmt, packed, ws, pl, asc, rows, cols, odt)
+    at = 0
+    for got, r in zip(outs, member_rows):
+        gh.check_outputs(got, ref[at:at + r], dtype, f"{stem} view bank member at row {at}")
+        at += r
+
+
+def test_binary_packed_banks_and_two_matrix_banks(env):
+    ctx, dtype, odt = env
+    cols = 2560
+    x = bits(fx.rng_for(128, 0).normal(0, 1, cols).astype(np.float32), dtype)
+    xf = so.widen(x, odt)
+    for name, member_rows in (("signed_binary_packed_bank_matvec_g128_rows8", [200, 77]),
+                              ("signed_binary_packed_bank4_matvec_g128_rows8", [64, 3, 129, 40])):
+        rows = sum(member_rows)
+        packed, ws = signed_weights(70 + rows, rows, cols, so.BINARY1)
+        outs = run_bank(ctx, name, [(packed, ws)], [x], member_rows, cols, dtype)
+        ref = so.signed_matvec(so.BINARY1, packed, ws, xf, rows, cols, cols, 128)[0]
+        at = 0
+        for got, r in zip(outs, member_rows):
+            gh.check_outputs(got, ref[at:at + r], dtype, f"{name} member at row {at}")
+            at += r
+    # two physical matrices, one row space: the boundary falls inside a row tile
+    for name in ("signed_binary_dual_matvec_g128_rows8", "signed_binary_virtual_bank_matvec_g128_rows8"):
+        for rows1, rows2 in ((37, 91), (128, 5), (1, 300)):
+            a, b = signed_weights(80 + rows1, rows1, cols, so.BINARY1), signed_weights(81 + rows2, rows2, cols, so.BINARY1)
+            outs = run_bank(ctx, name, [a, b], [x], [rows1, rows2], cols, dtype)
+            gh.check_outputs(outs[0], so.signed_matvec(so.BINARY1, a[0], a[1], xf, rows1, cols, cols, 128)[0], dtype, f"{name} first")
+            gh.check_outputs(outs[1], so.signed_matvec(so.BINARY1, b[0], b[1], xf, rows2, cols, cols, 128)[0], dtype, f"{name} second")
+
+
+@pytest.mark.parametrize("tile,planes,batch", [(4, 5, 3), (4, 2, 9), (8, 4, 13), (16, 6, 16)])
+def test_view_matvec_over_prompt_rows(env, tile, planes, batch):
+    """signed_binary_bitplane_i{N}_matvec_g128_rows8_batched_b{4,8,16}: bit-exact with independent rows
+    (SignedQuantKernelTests.swift:664-860 checks the same property)."""
+    ctx, dtype, odt = env
+    rows, cols = 123, 1536
+    packed, ws = signed_weights(90 + tile, rows, cols, so.BINARY1)
+    x = bits(fx.rng_for(129, batch).normal(0, 1, (batch, cols)).astype(np.float32), dtype)
+    views = [so.activation_bitplanes(x[t], planes, odt) for t in range(batch)]
+    pl = np.stack([v[0] for v in views]); asc = np.stack([v[1] for v in views])
+    wf = gh.WeightFile()
+    a, b = wf.add(packed), wf.add(ws)
+    ctx.upload_weights(W, wf.image())
+    ctx.put(PL, pl); ctx.put(AS, asc); ctx.alloc(Y, batch * rows * 2); ctx.alloc(RES, batch * rows * 2)
+    rec = rt.make_record(ctx.pipeline(f"signed_binary_bitplane_i{planes}_matvec_g128_rows8_batched_b{tile}"),
+                         [(W, 0, a), (W, 1, b), (PL, 2, 0), (AS, 3, 0), (Y, 4, 0)], [(5, rows), (6, cols), (7, batch)],
+                         ((rows + 7) // 8, (batch + tile - 1) // tile, 1), (256, 1, 1))
+    single = rt.make_record(ctx.pipeline(f"signed_binary_bitplane_i{planes}_matvec_g128_rows8"),
+                            [(W, 0, a), (W, 1, b), (PL, 2, 0), (AS, 3, 0), (RES, 4, 0)], [(5, rows), (6, cols)],
+                            ((rows + 7) // 8, batch, 1), (256, 1, 1))
+    ctx.interpret_decode(ctx.table([rec, single])); ctx.wait()
+    got = ctx.read(Y, np.uint16, batch * rows).reshape(batch, rows)
+    assert np.array_equal(got, ctx.read(RES, np.uint16, batch * rows).reshape(batch, rows))
+    for t in (0, batch - 1):
+        gh.check_outputs(got[t], so.signed_bitplane_matvec(so.BINARY1, packed, ws, views[t][0], views[t][1], rows, cols, odt), dtype, "batched view matvec")
