@@ -72,7 +72,7 @@ __device__ __forceinline__ void lut_tiles(const LutMat (&mats)[NMAT], int rows, 
             for (int m = 0; m < NMAT; ++m)
 #pragma unroll
                 for (int r = 0; r < R; ++r)
-                    c[m][r] = *reinterpret_cast<const uint4_t*>(mats[m].indices + (size_t)row[r] * row_bytes + (size_t)u * 16);
+                    c[m][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(mats[m].indices + (size_t)row[r] * row_bytes + (size_t)u * 16));
             uint32_t xp[16];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {

@@ -339,11 +339,13 @@ __device__ __forceinline__ void load_item(const MatPtrs (&mats)[NMAT], const int
                 scales = mats[m].scales_hi;
                 rr -= mats[m].split;
             }
-            it.c[m][r] = *reinterpret_cast<const uint4_t*>(codes + (size_t)rr * row_stride + (size_t)u * 16);
+            // weights are read once per launch: the streaming hint keeps them from displacing the
+            // activations and the residual in the caches
+            it.c[m][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(codes + (size_t)rr * row_stride + (size_t)u * 16));
             const size_t si = (size_t)rr * groups_per_row + g;
-            it.s[m][r] = scales[si];
-            if (F::kHasBias) it.b[m][r] = mats[m].biases[si];
-            else if (F::kPerDwordScale) it.b[m][r] = scales[g + 1 < groups_per_row ? si + 1 : si];
+            it.s[m][r] = __builtin_nontemporal_load(scales + si);
+            if (F::kHasBias) it.b[m][r] = __builtin_nontemporal_load(mats[m].biases + si);
+            else if (F::kPerDwordScale) it.b[m][r] = __builtin_nontemporal_load(scales + (g + 1 < groups_per_row ? si + 1 : si));
             else it.b[m][r] = 0;
         }
 }

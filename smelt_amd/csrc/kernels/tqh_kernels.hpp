@@ -70,7 +70,7 @@ constexpr float kTqhInvSqrtG = 0.0883883476483184405f;
                 const float cb2 = F16::widen(codebook[g * 4u + 2u]), cb3 = F16::widen(codebook[g * 4u + 3u]); \
                 uint4_t c[4];                                                                      \
                 _Pragma("unroll") for (int r = 0; r < 4; ++r)                                      \
-                    c[r] = *reinterpret_cast<const uint4_t*>(codes + (size_t)row[r] * codes_per_row + (size_t)u * 16u); \
+                    c[r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(codes + (size_t)row[r] * codes_per_row + (size_t)u * 16u)); \
                 const float4_t* xv4 = reinterpret_cast<const float4_t*>(lds_x + (size_t)u * 64u);  \
                 _Pragma("unroll") for (int q = 0; q < 16; ++q) {                                   \
                     const float4_t xv = xv4[q];                                                    \
