@@ -374,11 +374,11 @@ int smelt_layout_make_dense_entry(int rows, int cols, int dtype, uint64_t* offse
 int smelt_route_decode_affine(int rows, int cols, int group, int fusion, int compute_units, SmeltRoute* out) {
     if (!out || rows <= 0 || cols <= 0 || cols % 32 != 0 || group < 32 || (group & (group - 1))) return SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY;
     const char* stem;
-    int rows_per_wave = 4;
+    const int rows_per_wave = 2;  // the R of the single-token affine kernels
     switch (fusion) {
         case SMELT_FUSION_NONE: stem = "affine_matvec"; break;
-        case SMELT_FUSION_GATE_UP_SWIGLU: stem = "fused_affine_gate_up_swiglu"; rows_per_wave = 2; break;
-        case SMELT_FUSION_DUAL_MATVEC: stem = "fused_dual_affine_matvec"; rows_per_wave = 2; break;
+        case SMELT_FUSION_GATE_UP_SWIGLU: stem = "fused_affine_gate_up_swiglu"; break;
+        case SMELT_FUSION_DUAL_MATVEC: stem = "fused_dual_affine_matvec"; break;
         default: return SMELT_SELECT_MISSING;
     }
     const bool spec = is_specialized_shape(rows, cols, group);

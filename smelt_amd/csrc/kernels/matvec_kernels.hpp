@@ -254,7 +254,7 @@ using u32 = uint32_t;
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         EpiStore<ACT> epi{{}, y, (int)rows};                                                          \
-        matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x, rows, cols,                                 \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 1>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
     }                                                                                             \
@@ -264,7 +264,7 @@ using u32 = uint32_t;
         using namespace smelt;                                                                    \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         EpiAdd<ACT> epi{{}, y, res, (int)rows};                                                       \
-        matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, x, rows, cols,                                 \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 1>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
     }                                                                                             \
@@ -587,7 +587,7 @@ struct EpiBank4 : EpiBase {
         float best_raw = __builtin_nanf("");                                                      \
         EpiArgmax<ACT> epi{keys, logit_cap, &best, &best_raw, wave_keys};                         \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
-        matvec_body<FmtU4, ACT, SC, 4, 1, 1>(mats, X, rows, cols,                                 \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 1>(mats, X, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group, 0, 1,  \
                                              epi);                                                \
     }

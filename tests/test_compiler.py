@@ -90,7 +90,7 @@ def test_shape_routes():
     assert r.pipeline == b"affine_matvec_c1024_r3584_g64" and r.specialized == 1 and r.threads == 256
     assert r.rows_per_group == 8 and r.grid_w == 448           # small matrix: one row per wave slot, two slots per wave
     r = cc.route_decode_affine(3584, 1024, 64, compute_units=32)
-    assert r.rows_per_group == 32 and r.grid_w == 112          # enough workgroups per CU: four rows per slot
+    assert r.rows_per_group == 16 and r.grid_w == 128          # enough workgroups per CU: two rows per slot
     r = cc.route_decode_affine(151936, 1024, 64)
     assert r.grid_w == 1024                                     # capped at four workgroups per compute unit
     r = cc.route_decode_affine(777, 1056, 32)
