@@ -322,35 +322,164 @@ struct ItemRegs {
     uint16_t res[R];       // epilogue operand fetched ahead with a row's last item (when the epilogue asks)
 };
 
-template <class F, int R, int NMAT>
-__device__ __forceinline__ void load_item(const MatPtrs (&mats)[NMAT], const int (&row)[R], int u,
-                                          int row_stride, int groups_per_row, int gshift,
-                                          ItemRegs<R, NMAT>& it) {
-    const int g = (u * FmtGeom<F>::kColsPerUnit) >> gshift;
-#pragma unroll
-    for (int m = 0; m < NMAT; ++m)
+// Byte offsets of the R rows a lane owns inside a tile: codes and 16-bit scales.  They do not
+// change from tile to tile, so the row * stride products are formed once per launch.
+template <int R>
+struct LaneRows {
+    int rin0;               // first of the lane's rows within a tile
+    uint32_t code[R];       // (rin0 + r) * row_stride
+    uint32_t scale[R];      // (rin0 + r) * groups_per_row * 2
+    __device__ __forceinline__ LaneRows(int first_row, int row_stride, int groups_per_row) : rin0(first_row) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint8_t* codes = mats[m].codes;
-            const uint16_t* scales = mats[m].scales;
-            int rr = row[r];
-            if (mats[m].split > 0 && rr >= mats[m].split) {
-                codes = mats[m].codes_hi;
-                scales = mats[m].scales_hi;
-                rr -= mats[m].split;
+            code[r] = (uint32_t)(first_row + r) * (uint32_t)row_stride;
+            scale[r] = (uint32_t)(first_row + r) * (uint32_t)groups_per_row * 2u;
+        }
+    }
+};
+
+// Loads unit `u` of the R rows this lane owns in the tile that starts at row `row0`, clamped to
+// the matrix in the last (partial) tile (clamped rows are computed, never stored).  row0 is
+// uniform over the wave, so every address is a scalar tile base plus a 32-bit lane offset and the
+// per-item address arithmetic stays off the vector ALU.
+template <class F, int R, int NMAT>
+__device__ __forceinline__ void load_item(const MatPtrs (&mats)[NMAT], int row0, int tile_rows, int rows,
+                                          const LaneRows<R>& lr, int u, int row_stride,
+                                          int groups_per_row, int gshift, ItemRegs<R, NMAT>& it) {
+    const int g = (u * FmtGeom<F>::kColsPerUnit) >> gshift;
+    const int g_next = g + 1 < groups_per_row ? g + 1 : g;
+    const int last = rows - 1 - row0;
+    const int max_rin = last < tile_rows - 1 ? last : tile_rows - 1;   // uniform
+    const uint32_t max_code = (uint32_t)max_rin * (uint32_t)row_stride;
+    const uint32_t max_scale = (uint32_t)max_rin * (uint32_t)groups_per_row * 2u;
+    auto at = [](const uint16_t* base, uint32_t byte_off) {
+        return reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(base) + byte_off);
+    };
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) {
+        const uint8_t* codes = mats[m].codes;
+        const uint16_t* scales = mats[m].scales;
+        int base_row = row0;
+        const int split = mats[m].split;
+        if (split > 0 && row0 < split && row0 + tile_rows > split) {
+            // the tile straddles the seam of a two-segment matrix: per-lane segment choice
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                int rr = row0 + (lr.rin0 + r < max_rin ? lr.rin0 + r : max_rin);
+                const bool hi = rr >= split;
+                const uint8_t* cb = hi ? mats[m].codes_hi : codes;
+                const uint16_t* sb = hi ? mats[m].scales_hi : scales;
+                if (hi) rr -= split;
+                it.c[m][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(cb + (size_t)rr * row_stride + (size_t)u * 16));
+                const size_t si = (size_t)rr * groups_per_row;
+                it.s[m][r] = __builtin_nontemporal_load(sb + si + g);
+                if (F::kHasBias) it.b[m][r] = __builtin_nontemporal_load(mats[m].biases + si + g);
+                else if (F::kPerDwordScale) it.b[m][r] = __builtin_nontemporal_load(sb + si + g_next);
+                else it.b[m][r] = 0;
             }
-            // weights are read once per launch: the streaming hint keeps them from displacing the
-            // activations and the residual in the caches
-            it.c[m][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(codes + (size_t)rr * row_stride + (size_t)u * 16));
-            const size_t si = (size_t)rr * groups_per_row + g;
-            it.s[m][r] = __builtin_nontemporal_load(scales + si);
-            if (F::kHasBias) it.b[m][r] = __builtin_nontemporal_load(mats[m].biases + si);
-            else if (F::kPerDwordScale) it.b[m][r] = __builtin_nontemporal_load(scales + (g + 1 < groups_per_row ? si + 1 : si));
+            continue;
+        }
+        if (split > 0 && row0 >= split) {
+            codes = mats[m].codes_hi;
+            scales = mats[m].scales_hi;
+            base_row = row0 - split;
+        }
+        // weights are read once per launch: the streaming hint keeps them from displacing the
+        // activations and the residual in the caches
+        const uint8_t* tile_codes = codes + (size_t)base_row * row_stride;
+        const uint16_t* tile_scales = scales + (size_t)base_row * groups_per_row;
+        const uint16_t* tile_biases = F::kHasBias ? mats[m].biases + (size_t)base_row * groups_per_row : nullptr;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t code_off = (lr.code[r] < max_code ? lr.code[r] : max_code) + (uint32_t)u * 16u;
+            const uint32_t scale_off = (lr.scale[r] < max_scale ? lr.scale[r] : max_scale) + (uint32_t)g * 2u;
+            it.c[m][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(tile_codes + code_off));
+            it.s[m][r] = __builtin_nontemporal_load(at(tile_scales, scale_off));
+            if (F::kHasBias) it.b[m][r] = __builtin_nontemporal_load(at(tile_biases, scale_off));
+            else if (F::kPerDwordScale) it.b[m][r] = __builtin_nontemporal_load(at(tile_scales, scale_off + (uint32_t)(g_next - g) * 2u));
             else it.b[m][r] = 0;
         }
+    }
+}
+
+// The activation side of one unit for one token: the fp16 pairs, the folded-out constant and the
+// plain sum of x (what a bias multiplies).  For a matrix whose rows fit one pass of the wave the
+// unit of a lane never changes, so these registers are filled once per launch.
+template <class F>
+struct XUnit {
+    using G = FmtGeom<F>;
+    uint32_t xp[G::kChunksPerUnit * 4];
+    float cr[G::kDPU];   // per dword (formats whose scale can change inside a unit)
+    float corr;          // whole unit
+    float xsum;
+};
+
+template <class F>
+__device__ __forceinline__ void load_xunit(XUnit<F>& xu, int b, int u, int U, const uint4_t* lds_pairs,
+                                           const float* lds_corr, const float* lds_xsum) {
+    using G = FmtGeom<F>;
+    constexpr int NCH = G::kChunksPerUnit;
+    constexpr int DPU = G::kDPU;
+#pragma unroll
+    for (int q = 0; q < NCH; ++q) {
+        const uint4_t t = lds_pairs[((size_t)b * NCH + q) * U + u];
+        xu.xp[4 * q + 0] = t.x; xu.xp[4 * q + 1] = t.y; xu.xp[4 * q + 2] = t.z; xu.xp[4 * q + 3] = t.w;
+    }
+    const float4_t* c4 = reinterpret_cast<const float4_t*>(lds_corr + ((size_t)b * U + u) * G::kCorrStride);
+    const float4_t lo = c4[0];
+    xu.cr[0] = lo.x; xu.cr[1] = lo.y; xu.cr[2] = lo.z; xu.cr[3] = lo.w;
+    if constexpr (DPU > 4) xu.cr[DPU - 1] = c4[1].x;
+    xu.corr = (xu.cr[0] + xu.cr[1]) + (xu.cr[2] + xu.cr[3]);
+    xu.xsum = 0.0f;
+    if (F::kHasBias) {
+        const float4_t xs = *reinterpret_cast<const float4_t*>(lds_xsum + ((size_t)b * U + u) * G::kCorrStride);
+        xu.xsum = (xs.x + xs.y) + (xs.z + xs.w);
+    }
 }
 
 // acc[m][r][b] += scale * (sum (base + code) * x  -  sum base * x) + bias * sum x   for unit u
+template <class F, class ScaleT, int R, int MB, int NMAT>
+__device__ __forceinline__ void compute_unit(const ItemRegs<R, NMAT>& it, const XUnit<F>& xu, int b, int u,
+                                             int gshift, const uint16_t* lut, float (&acc)[NMAT][R][MB]) {
+    using G = FmtGeom<F>;
+    constexpr int DPU = G::kDPU;
+    if constexpr (F::kPerDwordScale) {
+        const int g0 = (u * G::kColsPerUnit) >> gshift;
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                uint32_t dw[DPU];
+                F::decode(it.c[m][r], lut, dw);
+                const float s0 = F::kSemMul * ScaleT::widen(it.s[m][r]);
+                const float s1 = F::kSemMul * ScaleT::widen(it.b[m][r]);
+                float a = acc[m][r][b];
+#pragma unroll
+                for (int j = 0; j < DPU; ++j) {
+                    const float d = F::dot(dw[j], xu.xp + j * G::kPPD, -xu.cr[j]);
+                    const int gj = (u * G::kColsPerUnit + j * G::kColsPerDword) >> gshift;
+                    a = __builtin_fmaf(gj == g0 ? s0 : s1, d, a);
+                }
+                acc[m][r][b] = a;
+            }
+    } else {
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float d = -xu.corr;
+                d = F::dot(it.c[m][r].x, xu.xp + 0 * G::kPPD, d);
+                d = F::dot(it.c[m][r].y, xu.xp + 1 * G::kPPD, d);
+                d = F::dot(it.c[m][r].z, xu.xp + 2 * G::kPPD, d);
+                d = F::dot(it.c[m][r].w, xu.xp + 3 * G::kPPD, d);
+                float a = acc[m][r][b];
+                if (F::kHasBias) a = __builtin_fmaf(ScaleT::widen(it.b[m][r]), xu.xsum, a);
+                acc[m][r][b] = __builtin_fmaf(F::kSemMul * ScaleT::widen(it.s[m][r]), d, a);
+            }
+    }
+}
+
+// One work item against every token of the chunk.
 template <class F, class ScaleT, int R, int MB, int NMAT>
 __device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u, int U, int gshift,
                                              const uint4_t* lds_pairs, const float* lds_corr,
@@ -406,64 +535,11 @@ __device__ __forceinline__ void compute_item(const ItemRegs<R, NMAT>& it, int u,
         }
         return;
     }
-    using G = FmtGeom<F>;
-    constexpr int NCH = G::kChunksPerUnit;
-    constexpr int DPU = G::kDPU;
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
-        uint32_t xp[NCH * 4];
-#pragma unroll
-        for (int q = 0; q < NCH; ++q) {
-            const uint4_t t = lds_pairs[((size_t)b * NCH + q) * U + u];
-            xp[4 * q + 0] = t.x; xp[4 * q + 1] = t.y; xp[4 * q + 2] = t.z; xp[4 * q + 3] = t.w;
-        }
-        float cr[DPU];
-        {
-            const float4_t* c4 = reinterpret_cast<const float4_t*>(lds_corr + ((size_t)b * U + u) * G::kCorrStride);
-            const float4_t lo = c4[0];
-            cr[0] = lo.x; cr[1] = lo.y; cr[2] = lo.z; cr[3] = lo.w;
-            if constexpr (DPU > 4) cr[DPU - 1] = c4[1].x;
-        }
-        if constexpr (F::kPerDwordScale) {
-            const int g0 = (u * G::kColsPerUnit) >> gshift;
-#pragma unroll
-            for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    uint32_t dw[DPU];
-                    F::decode(it.c[m][r], lut, dw);
-                    const float s0 = F::kSemMul * ScaleT::widen(it.s[m][r]);
-                    const float s1 = F::kSemMul * ScaleT::widen(it.b[m][r]);
-                    float a = acc[m][r][b];
-#pragma unroll
-                    for (int j = 0; j < DPU; ++j) {
-                        const float d = F::dot(dw[j], xp + j * G::kPPD, -cr[j]);
-                        const int gj = (u * G::kColsPerUnit + j * G::kColsPerDword) >> gshift;
-                        a = __builtin_fmaf(gj == g0 ? s0 : s1, d, a);
-                    }
-                    acc[m][r][b] = a;
-                }
-        } else {
-            const float corr = (cr[0] + cr[1]) + (cr[2] + cr[3]);
-            float xsum = 0.0f;
-            if (F::kHasBias) {
-                const float4_t xs = *reinterpret_cast<const float4_t*>(lds_xsum + ((size_t)b * U + u) * G::kCorrStride);
-                xsum = (xs.x + xs.y) + (xs.z + xs.w);
-            }
-#pragma unroll
-            for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    float d = -corr;
-                    d = F::dot(it.c[m][r].x, xp + 0 * G::kPPD, d);
-                    d = F::dot(it.c[m][r].y, xp + 1 * G::kPPD, d);
-                    d = F::dot(it.c[m][r].z, xp + 2 * G::kPPD, d);
-                    d = F::dot(it.c[m][r].w, xp + 3 * G::kPPD, d);
-                    float a = acc[m][r][b];
-                    if (F::kHasBias) a = __builtin_fmaf(ScaleT::widen(it.b[m][r]), xsum, a);
-                    acc[m][r][b] = __builtin_fmaf(F::kSemMul * ScaleT::widen(it.s[m][r]), d, a);
-                }
-        }
+        XUnit<F> xu;
+        load_xunit<F>(xu, b, u, U, lds_pairs, lds_corr, lds_xsum);
+        compute_unit<F, ScaleT, R, MB, NMAT>(it, xu, b, u, gshift, lut, acc);
     }
 }
 

@@ -102,7 +102,8 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
     constexpr int S = kWave / L;
     constexpr int TILE = S * R;
     const int waves = blockDim.x / kWave;
-    const int wave = threadIdx.x / kWave;
+    // the wave index is uniform over the wave; saying so keeps the tile walk on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x & (kWave - 1);
     const int sub = lane & (L - 1);
     const int side = lane / L;
@@ -112,6 +113,7 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
     const int stride = gridDim.x * waves;
     const int my_tiles = first < tiles ? (tiles - first + stride - 1) / stride : 0;
     const int nq = my_tiles * nit;
+    const LaneRows<R> lane_rows(side * R, row_stride, gpr);
 
     for (int b0 = batch_lo; b0 < batch_hi; b0 += MB) {
         const int nb = batch_hi - b0 < MB ? batch_hi - b0 : MB;
@@ -120,17 +122,15 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
         int tile_c = first, it_c = 0, tile_n = first, it_n = 0;
         auto load = [&](ItemRegs<R, NMAT>& dst) {
             const int u = sub + L * it_n;
-            int row[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int rr = tile_n * TILE + side * R + r;
-                row[r] = rr < rows ? rr : rows - 1;  // clamped rows are computed, never stored
-            }
-            if (u < U) load_item<F, R, NMAT>(mats, row, u, row_stride, gpr, gshift, dst);
+            const int row0 = tile_n * TILE;
+            if (u < U) load_item<F, R, NMAT>(mats, row0, TILE, rows, lane_rows, u, row_stride, gpr, gshift, dst);
             if constexpr (Epi::kPrefetch && MB == 1) {
                 if (it_n == nit - 1 && sub == L - 1) {
 #pragma unroll
-                    for (int r = 0; r < R; ++r) dst.res[r] = epi.prefetch(b0, row[r]);
+                    for (int r = 0; r < R; ++r) {
+                        const int rr = row0 + side * R + r;
+                        dst.res[r] = epi.prefetch(b0, rr < rows ? rr : rows - 1);
+                    }
                 }
             }
             if (++it_n == nit) { it_n = 0; tile_n += stride; }
@@ -140,6 +140,13 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
         if (b0 != batch_lo) __syncthreads();
         stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum, x2, nplanes);
         __syncthreads();
+
+        // activation registers held across the walk when the lane's unit never changes
+        constexpr bool kHoldX = MB == 1 && !F::kBitplanes && FmtGeom<F>::kChunksPerUnit * 4 <= 16;
+        XUnit<F> xu;
+        if constexpr (kHoldX) {
+            if (nit == 1 && sub < U) load_xunit<F>(xu, 0, sub, U, lds_pairs, lds_corr, lds_xsum);
+        }
 
         float acc[NMAT][R][MB];
         auto step = [&](ItemRegs<R, NMAT>& cur, int q) {
@@ -152,7 +159,14 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
                         for (int b = 0; b < MB; ++b) acc[m][r][b] = 0.0f;
             }
             const int u = sub + L * it_c;
-            if (u < U) compute_item<F, ScaleT, R, MB, NMAT>(cur, u, U, gshift, lds_pairs, lds_corr, lds_xsum, lut, acc);
+            if (u < U) {
+                if constexpr (kHoldX) {
+                    if (nit > 1) load_xunit<F>(xu, 0, u, U, lds_pairs, lds_corr, lds_xsum);
+                    compute_unit<F, ScaleT, R, MB, NMAT>(cur, xu, 0, u, gshift, lut, acc);
+                } else {
+                    compute_item<F, ScaleT, R, MB, NMAT>(cur, u, U, gshift, lds_pairs, lds_corr, lds_xsum, lut, acc);
+                }
+            }
             if (it_c == nit - 1) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
