@@ -875,7 +875,7 @@ int smelt_emit_lm_head_argmax(smelt_emitter* e, int weights_slot, const SmeltWei
     if (!e || !w || batch_size <= 0) return efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "null emitter or weight");
     if (!affine_entry_ok(w)) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "fused lm_head argmax exists for affine_u4 weights");
     if (w->rows > (1 << 18)) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "argmax keys hold 18 index bits");
-    const MatvecGeometry g = matvec_geometry((uint32_t)w->cols / 2, w->rows, 4, e->compute_units);
+    const MatvecGeometry g = matvec_geometry((uint32_t)w->cols / 2, w->rows, 2, e->compute_units);
     const int bt = 8;
     RecordBuilder r1;
     bind_affine(r1, 0, weights_slot, w);
