@@ -137,6 +137,21 @@ int smelt_emit_matvec_add(smelt_emitter *e, int weights_slot, const SmeltWeightE
 int smelt_emit_gate_up_swiglu(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *gate,
                               const SmeltWeightEntryC *up, SmeltBinding input, SmeltBinding output,
                               int batch_size, int dynamic);
+/* rms_norm_scale_only (norms.metal:944-1008): writes one fp32 scale per row; the first dispatch of the
+ * scale-only + norm-scale pair (emitNormScaleAffineMatvecIfPossible, SmeltCodeEmitter.swift:2680-2754). */
+int smelt_emit_rms_norm_scale_only(smelt_emitter *e, SmeltBinding input, SmeltBinding scale_output,
+                                   int dim, float eps, int batch_size);
+/* norm_scale_affine_matvec (lut_matvec.metal:1294-1469; fixed shapes :2743-3170): the kernel reads a
+ * precomputed RMS scale and multiplies x_norm = half((x * scale) * (1 + norm_weight)); the normalised
+ * row is also stored to norm_output.  affine_u4 weights, one token. */
+int smelt_emit_norm_scale_matvec(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w,
+                                 SmeltBinding norm_scale, SmeltBinding input, SmeltBinding norm_weight,
+                                 SmeltBinding norm_output, SmeltBinding output);
+/* norm_scale_affine_gate_up_swiglu / _geglu (lut_matvec.metal:1471-1700): same prologue in front of
+ * the fused gate+up projection; geglu != 0 selects the GeGLU product (:2235-2243). */
+int smelt_emit_norm_scale_gate_up(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *gate,
+                                  const SmeltWeightEntryC *up, int geglu, SmeltBinding norm_scale,
+                                  SmeltBinding input, SmeltBinding norm_weight, SmeltBinding output);
 /* fused_dual_affine_matvec: two weights, one input, two outputs */
 int smelt_emit_dual_matvec(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w1,
                            const SmeltWeightEntryC *w2, SmeltBinding input, SmeltBinding output1,

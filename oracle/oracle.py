@@ -87,6 +87,8 @@ def _declare(l: C.CDLL) -> None:
         "so_ternary_affine_qmv": (None, [vp, vp, vp, vp, i32, i32, i32, vp]),
         "so_epilogue_residual_add": (u16, [f32, u16, i32]),
         "so_epilogue_affine_swiglu": (u16, [f32, f32, i32]),
+        "so_epilogue_geglu": (u16, [f32, f32, i32]),
+        "so_norm_scale_input": (None, [vp, f32, vp, i32, i32, vp]),
         "so_epilogue_signed_swiglu": (u16, [u16, u16, i32]),
         "so_rms_scale": (f32, [vp, i32, f32, i32]),
         "so_rms_norm_1pw": (None, [vp, vp, vp, i32, f32, i32, i32, vp]),
@@ -336,6 +338,22 @@ def epilogue_affine_swiglu(gate: np.ndarray, up: np.ndarray, dtype: int) -> np.n
     return np.array([l.so_epilogue_affine_swiglu(float(g), float(u), dtype)
                      for g, u in zip(np.ravel(gate), np.ravel(up))],
                     dtype=np.uint16).reshape(np.shape(gate))
+
+
+def epilogue_geglu(gate: np.ndarray, up: np.ndarray, dtype: int) -> np.ndarray:
+    l = lib()
+    return np.array([l.so_epilogue_geglu(float(g), float(u), dtype)
+                     for g, u in zip(np.ravel(gate), np.ravel(up))],
+                    dtype=np.uint16).reshape(np.shape(gate))
+
+
+def norm_scale_input(x_bits: np.ndarray, rs: float, w_bits: np.ndarray, dtype: int) -> np.ndarray:
+    """The activation row a norm-scale matvec consumes (and stores): narrow((x * rs) * (1 + w))."""
+    x = np.ascontiguousarray(x_bits, np.uint16).ravel()
+    out = np.zeros(x.size, np.uint16)
+    lib().so_norm_scale_input(_p(x, np.uint16), float(rs), _p(np.ascontiguousarray(w_bits, np.uint16).ravel(), np.uint16),
+                              dtype, x.size, _p(out, np.uint16))
+    return out.reshape(np.shape(x_bits))
 
 
 def epilogue_signed_swiglu(gate_bits: np.ndarray, up_bits: np.ndarray, dtype: int) -> np.ndarray:

@@ -610,6 +610,31 @@ SO_EXPORT uint16_t so_epilogue_affine_swiglu(float gate, float up, int dtype) {
     return narrow(gate / (1.0f + expf(-gate)) * up, dtype);
 }
 
+/* lut_matvec.metal:2235-2243 (agent_geglu_product): gate and up rounded to the 16-bit type, tanh
+ * form of GELU with its argument clamped to +-20, product clamped to the fp16 range. */
+SO_EXPORT uint16_t so_epilogue_geglu(float gate, float up, int dtype) {
+    gate = so_round_through(gate, dtype);
+    up = so_round_through(up, dtype);
+    float gate3 = gate * gate * gate;
+    float inner = 0.7978845608f * (gate + 0.044715f * gate3);
+    inner = inner < -20.0f ? -20.0f : (inner > 20.0f ? 20.0f : inner);
+    float gelu = 0.5f * gate * (1.0f + tanhf(inner));
+    float prod = gelu * up;
+    prod = prod < -65504.0f ? -65504.0f : (prod > 65504.0f ? 65504.0f : prod);
+    return narrow(prod, dtype);
+}
+
+/* lut_matvec.metal:1347-1379 (norm_scale_affine_matvec and its gate/up forms): the activation a
+ * norm-scale kernel multiplies is half((x * rs) * (1 + w)), products taken left to right. */
+SO_EXPORT void so_norm_scale_input(const uint16_t *x, float rs, const uint16_t *weight, int dtype,
+                                   int count, uint16_t *out) {
+    for (int i = 0; i < count; ++i) {
+        float scaled = widen(x[i], dtype) * rs;
+        float direct = 1.0f + widen(weight[i], dtype);
+        out[i] = narrow(scaled * direct, dtype);
+    }
+}
+
 /* signed_quant.metal:15-20 / signed_quant_precise.metal:31-36: every intermediate is
  * materialised in the activation type. gate/up arrive already rounded to that type. */
 SO_EXPORT uint16_t so_epilogue_signed_swiglu(uint16_t gate_bits, uint16_t up_bits, int dtype) {

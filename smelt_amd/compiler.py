@@ -75,6 +75,9 @@ def lib() -> C.CDLL:
         "smelt_emit_matvec": (i32, [vp, i32, we, Binding, Binding, i32, i32]),
         "smelt_emit_matvec_add": (i32, [vp, i32, we, Binding, Binding, Binding]),
         "smelt_emit_gate_up_swiglu": (i32, [vp, i32, we, we, Binding, Binding, i32, i32]),
+        "smelt_emit_rms_norm_scale_only": (i32, [vp, Binding, Binding, i32, C.c_float, i32]),
+        "smelt_emit_norm_scale_matvec": (i32, [vp, i32, we, Binding, Binding, Binding, Binding, Binding]),
+        "smelt_emit_norm_scale_gate_up": (i32, [vp, i32, we, we, i32, Binding, Binding, Binding, Binding]),
         "smelt_emit_dual_matvec": (i32, [vp, i32, we, we, Binding, Binding, Binding]),
         "smelt_emit_lm_head_argmax": (i32, [vp, i32, we, Binding, Binding, Binding, i32, C.c_float]),
         "smelt_emit_swap": (i32, [vp]),
@@ -237,6 +240,18 @@ class Emitter:
     def gate_up_swiglu(self, weights_slot, gate, up, x, y, batch=1, dynamic=False):
         self._check(self.l.smelt_emit_gate_up_swiglu(self.h, weights_slot, C.byref(gate), C.byref(up), x, y,
                                                      batch, int(dynamic)))
+
+    def rms_norm_scale_only(self, x, scale, dim, eps=1e-6, batch=1):
+        self._check(self.l.smelt_emit_rms_norm_scale_only(self.h, x, scale, dim, eps, batch))
+
+    def norm_scale_matvec(self, weights_slot, w, scale, x, norm_weight, norm_output, y):
+        """The affine matvec that normalises its input inline from a precomputed RMS scale."""
+        self._check(self.l.smelt_emit_norm_scale_matvec(self.h, weights_slot, C.byref(w), scale, x, norm_weight,
+                                                        norm_output, y))
+
+    def norm_scale_gate_up(self, weights_slot, gate, up, scale, x, norm_weight, y, geglu=False):
+        self._check(self.l.smelt_emit_norm_scale_gate_up(self.h, weights_slot, C.byref(gate), C.byref(up), int(geglu),
+                                                         scale, x, norm_weight, y))
 
     def dual_matvec(self, weights_slot, w1, w2, x, y1, y2):
         self._check(self.l.smelt_emit_dual_matvec(self.h, weights_slot, C.byref(w1), C.byref(w2), x, y1, y2))

@@ -67,6 +67,7 @@ const std::vector<SmeltMatvecCell>& meaningful_cells() {
                 add(SMELT_ACT_BF16, w, shape, SMELT_FUSION_NONE, SMELT_OUT_BF16, SMELT_SLOT_FIXED);
             add(SMELT_ACT_BF16, w, SMELT_SHAPE_GEMV, SMELT_FUSION_GATE_UP_SWIGLU, SMELT_OUT_BF16, SMELT_SLOT_FIXED);
         }
+        add(SMELT_ACT_BF16, SMELT_DTYPE_AFFINE_U4, SMELT_SHAPE_GEMV, SMELT_FUSION_GATE_UP_GEGLU, SMELT_OUT_BF16, SMELT_SLOT_FIXED);
         return c;
     }();
     return cells;
@@ -97,7 +98,8 @@ bool hip_has_kernel(const SmeltMatvecCell& c, int family) {
     if (family == SMELT_FAMILY_TQH) return c.activation != SMELT_ACT_FP32 && c.fusion == SMELT_FUSION_NONE;
     if (!quant) return false;
     if (c.activation == SMELT_ACT_FP32) return false;
-    if (c.fusion == SMELT_FUSION_GATE_UP_GEGLU) return false;
+    // GeGLU: the single-token affine kernel only (no prompt-tile form yet)
+    if (c.fusion == SMELT_FUSION_GATE_UP_GEGLU) return family == SMELT_FAMILY_AFFINE_U4 && c.shape == SMELT_SHAPE_GEMV;
     if (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_DUAL_MATVEC) return false;
     if (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_GATE_UP_SWIGLU && family == SMELT_FAMILY_TERNARY2) return false;
     return true;
@@ -379,6 +381,7 @@ int smelt_route_decode_affine(int rows, int cols, int group, int fusion, int com
         case SMELT_FUSION_NONE: stem = "affine_matvec"; break;
         case SMELT_FUSION_GATE_UP_SWIGLU: stem = "fused_affine_gate_up_swiglu"; break;
         case SMELT_FUSION_DUAL_MATVEC: stem = "fused_dual_affine_matvec"; break;
+        case SMELT_FUSION_GATE_UP_GEGLU: stem = "fused_affine_gate_up_geglu"; break;
         default: return SMELT_SELECT_MISSING;
     }
     const bool spec = is_specialized_shape(rows, cols, group);
@@ -468,6 +471,24 @@ int smelt_emit_rms_norm_1pw(smelt_emitter* e, SmeltBinding input, SmeltBinding w
     const int threads = std::min(1024, std::max(64, ((dim + 7) / 8 + 63) / 64 * 64));
     rb.grid((uint32_t)batch_size, 1, 1, (uint32_t)threads);
     rb.r.pipeline = e->pipeline_index(name);
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+// rms_norm_scale_only (norms.metal:944-1008): one fp32 scale 1 / sqrt(mean(x^2) + eps) per row, the
+// first half of the scale-only + norm-scale pair (emitNormScaleAffineMatvecIfPossible,
+// SmeltCodeEmitter.swift:2680-2754).
+int smelt_emit_rms_norm_scale_only(smelt_emitter* e, SmeltBinding input, SmeltBinding scale_output, int dim, float eps, int batch_size) {
+    if (!e) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (dim <= 0 || batch_size <= 0) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "rms norm needs positive dim and batch");
+    RecordBuilder rb;
+    rb.buffer(0, input);
+    rb.buffer(1, scale_output);
+    rb.constant(2, (uint32_t)dim);
+    rb.constant_f32(3, eps);
+    const int threads = std::min(1024, std::max(64, ((dim + 7) / 8 + 63) / 64 * 64));
+    rb.grid((uint32_t)batch_size, 1, 1, (uint32_t)threads);
+    rb.r.pipeline = e->pipeline_index(batch_size > 1 ? "rms_norm_scale_only_batched" : "rms_norm_scale_only");
     e->records.push_back(rb.r);
     return SMELT_HIP_OK;
 }
@@ -796,6 +817,60 @@ int smelt_emit_gate_up_swiglu(smelt_emitter* e, int weights_slot, const SmeltWei
         }
         rb.r.pipeline = e->pipeline_index(name);
     }
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+// norm_scale_affine_matvec (lut_matvec.metal:1294-1469): bindings 0 scale, 1 input, 2 norm weight,
+// 3 normalised row out, 4..6 W S B, 7 output, constant 8 rows (generic name only).
+int smelt_emit_norm_scale_matvec(smelt_emitter* e, int weights_slot, const SmeltWeightEntryC* w, SmeltBinding norm_scale,
+                                 SmeltBinding input, SmeltBinding norm_weight, SmeltBinding norm_output, SmeltBinding output) {
+    if (!e || !w) return efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "null emitter or weight");
+    int family = 0;
+    if (int rc = gateway(e, w, SMELT_SHAPE_GEMV, SMELT_FUSION_NONE, &family)) return rc;
+    if (family != SMELT_FAMILY_AFFINE_U4) return efail(e, SMELT_SELECT_MISSING, "the norm-scale prologue exists for affine_u4 weights only");
+    if (!affine_entry_ok(w)) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "unsupported affine geometry");
+    SmeltRoute route;
+    if (int rc = smelt_route_decode_affine(w->rows, w->cols, w->group_size, SMELT_FUSION_NONE, e->compute_units, &route)) return efail(e, rc, "no decode route");
+    RecordBuilder rb;
+    rb.buffer(0, norm_scale);
+    rb.buffer(1, input);
+    rb.buffer(2, norm_weight);
+    rb.buffer(3, norm_output);
+    bind_affine(rb, 4, weights_slot, w);
+    rb.buffer(7, output);
+    if (!route.specialized) rb.constant(8, (uint32_t)w->rows);
+    rb.grid((uint32_t)route.grid_w, 1, 1, (uint32_t)route.threads);
+    rb.r.pipeline = e->pipeline_index(std::string("norm_scale_") + route.pipeline);
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
+// norm_scale_affine_gate_up_swiglu / _geglu (lut_matvec.metal:1471-1700): bindings 0 scale, 1 input,
+// 2 norm weight, 3..5 gate W S B, 6..8 up W S B, 9 output, constant 10 rows (generic name only).
+int smelt_emit_norm_scale_gate_up(smelt_emitter* e, int weights_slot, const SmeltWeightEntryC* gate, const SmeltWeightEntryC* up,
+                                  int geglu, SmeltBinding norm_scale, SmeltBinding input, SmeltBinding norm_weight, SmeltBinding output) {
+    if (!e || !gate || !up) return efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "null emitter or weight");
+    if (gate->dtype != up->dtype || gate->rows != up->rows || gate->cols != up->cols || gate->group_size != up->group_size)
+        return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "gate and up projections must share dtype, shape and group size");
+    const int fusion = geglu ? SMELT_FUSION_GATE_UP_GEGLU : SMELT_FUSION_GATE_UP_SWIGLU;
+    int family = 0;
+    if (int rc = gateway(e, gate, SMELT_SHAPE_GEMV, fusion, &family)) return rc;
+    if (family != SMELT_FAMILY_AFFINE_U4) return efail(e, SMELT_SELECT_MISSING, "the norm-scale prologue exists for affine_u4 weights only");
+    if (!affine_entry_ok(gate) || !affine_entry_ok(up)) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "unsupported affine geometry");
+    SmeltRoute route;
+    if (int rc = smelt_route_decode_affine(gate->rows, gate->cols, gate->group_size, fusion, e->compute_units, &route)) return efail(e, rc, "no decode route");
+    RecordBuilder rb;
+    rb.buffer(0, norm_scale);
+    rb.buffer(1, input);
+    rb.buffer(2, norm_weight);
+    bind_affine(rb, 3, weights_slot, gate);
+    bind_affine(rb, 6, weights_slot, up);
+    rb.buffer(9, output);
+    if (!route.specialized) rb.constant(10, (uint32_t)gate->rows);
+    rb.grid((uint32_t)route.grid_w, 1, 1, 256);
+    // "fused_affine_gate_up_*" -> "norm_scale_affine_gate_up_*"
+    rb.r.pipeline = e->pipeline_index(std::string("norm_scale_") + (route.pipeline + 6));
     e->records.push_back(rb.r);
     return SMELT_HIP_OK;
 }

@@ -21,8 +21,12 @@ struct F16 {
     static __device__ __forceinline__ float widen(uint16_t b) {
         return (float)__builtin_bit_cast(_Float16, b);
     }
-    // round-to-nearest-even narrowing
+    // Round-to-nearest-even narrowing of a value that has already been rounded to fp32, which is
+    // what half(float) means in the reference.  The empty asm keeps the conversion apart from the
+    // arithmetic that produced v: folded into a mixed-precision multiply-add (v_fma_mixlo_f16) the
+    // exact product would be rounded once, and results on fp16 ties would differ by an ulp.
     static __device__ __forceinline__ uint16_t narrow(float v) {
+        asm("" : "+v"(v));
         return __builtin_bit_cast(uint16_t, (_Float16)v);
     }
     // bits of the same value as fp16 (identity)

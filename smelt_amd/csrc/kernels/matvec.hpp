@@ -240,11 +240,31 @@ __device__ __forceinline__ void stage_planes(const uint32_t* __restrict__ planes
     }
 }
 
+// Prologue of the norm-scale kernels (lut_matvec.metal:1288-1292): with rs != nullptr the staged
+// activation is narrow((x * rs[token]) * (1 + weight)), rounded to the 16-bit type exactly as a
+// staged norm would store it; the launch's first workgroup also writes that row to `out`.
+struct NormScale {
+    const float* rs = nullptr;
+    const uint16_t* weight = nullptr;
+    uint16_t* out = nullptr;
+};
+
+// (x * rs) * (1 + w) with each product and the sum rounded on its own: without the pragma the
+// compiler folds t * (1 + w) into fma(w, t, t), one rounding fewer than the staged norm performs.
+template <class ActT>
+__device__ __forceinline__ uint16_t norm_scale_value(uint16_t x, float rs, uint16_t w) {
+#pragma clang fp contract(off)
+    const float scaled = ActT::widen(x) * rs;
+    const float direct = 1.0f + ActT::widen(w);
+    return ActT::narrow(scaled * direct);
+}
+
 template <class F, class ActT, int MB>
 __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x, int cols, int U,
                                                   int b0, int nb, uint4_t* lds_pairs,
                                                   float* lds_corr, float* lds_xsum,
-                                                  const uint16_t* x2 = nullptr, int nplanes = 0) {
+                                                  const uint16_t* x2 = nullptr, int nplanes = 0,
+                                                  const NormScale& ns = NormScale{}) {
     if constexpr (F::kBitplanes) {
         stage_planes<F, ActT, MB>(reinterpret_cast<const uint32_t*>(x), x2, nplanes, U, b0, nb, lds_pairs, lds_corr);
         return;
@@ -275,6 +295,17 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
             for (int i = 0; i < CPD; ++i) {
                 const int c = col0 + i;
                 v[i] = (b < nb && c < cols) ? x[(size_t)(b0 + b) * cols + c] : (uint16_t)0;
+            }
+        }
+        if (ns.rs != nullptr && b < nb) {
+            const float rs = ns.rs[b0 + b];
+#pragma unroll
+            for (int i = 0; i < CPD; ++i) {
+                const int c = col0 + i;
+                if (c < cols) {
+                    v[i] = norm_scale_value<ActT>(v[i], rs, ns.weight[c]);
+                    if (ns.out != nullptr && blockIdx.x == 0) ns.out[(size_t)(b0 + b) * cols + c] = v[i];
+                }
             }
         }
         float corr = 0.0f, xsum = 0.0f;

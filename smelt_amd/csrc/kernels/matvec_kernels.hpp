@@ -57,6 +57,21 @@ struct EpiAffineSwiglu : EpiBase {
     }
 };
 
+// GeGLU (lut_matvec.metal:2235-2243): gate and up rounded to the 16-bit type, tanh-form GELU of the
+// gate with its argument clamped to +-20, product clamped to the fp16 range
+template <class ActT>
+struct EpiGeglu : EpiBase {
+    uint16_t* y;
+    int rows;
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        const float g = ActT::widen(ActT::narrow(v[0])), u = ActT::widen(ActT::narrow(v[1]));
+        float inner = 0.7978845608f * (g + 0.044715f * (g * g * g));
+        inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+        const float gelu = 0.5f * g * (1.0f + tanhf(inner));
+        y[(size_t)b * rows + row] = ActT::narrow(fminf(fmaxf(gelu * u, -65504.0f), 65504.0f));
+    }
+};
+
 // signed SwiGLU: gate and up are first rounded to the activation type and every intermediate
 // (exp, 1+e, reciprocal, 1-tail, gate*sigmoid, *up) is materialised in that type
 template <class ActT>
@@ -98,7 +113,8 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
                                           int cols, int U, int row_stride, int gpr, int gshift,
                                           int batch_lo, int batch_hi, uint4_t* lds_pairs,
                                           float* lds_corr, float* lds_xsum, const uint16_t* lut,
-                                          const Epi& epi, const uint16_t* x2 = nullptr, int nplanes = 0) {
+                                          const Epi& epi, const uint16_t* x2 = nullptr, int nplanes = 0,
+                                          const NormScale& ns = NormScale{}) {
     constexpr int S = kWave / L;
     constexpr int TILE = S * R;
     const int waves = blockDim.x / kWave;
@@ -138,7 +154,7 @@ __device__ __forceinline__ void run_tiles(const MatPtrs (&mats)[NMAT], const uin
         if (nq > 0) load(regs_a);
         if (nq > 1) load(regs_b);
         if (b0 != batch_lo) __syncthreads();
-        stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum, x2, nplanes);
+        stage_activations<F, ActT, MB>(x, cols, U, b0, nb, lds_pairs, lds_corr, lds_xsum, x2, nplanes, ns);
         __syncthreads();
 
         // activation registers held across the walk when the lane's unit never changes
@@ -213,7 +229,8 @@ template <class F, class ActT, class ScaleT, int R, int MB, int NMAT, class Epi>
 __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const uint16_t* x,
                                             int rows, int cols, int row_stride, int group,
                                             int batch_lo, int batch_hi, const Epi& epi,
-                                            const uint16_t* x2 = nullptr, int nplanes = 0) {
+                                            const uint16_t* x2 = nullptr, int nplanes = 0,
+                                            const NormScale& ns = NormScale{}) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int U = row_stride / 16;
     const int gshift = ilog2((uint32_t)group);
@@ -233,11 +250,11 @@ __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const u
         if constexpr (R > 1 && MB == 1) {
             const int tiles = (rows + (kWave / L) * R - 1) / ((kWave / L) * R);
             if (tiles < total_waves) {
-                run_tiles<F, ActT, ScaleT, 1, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi, x2, nplanes);
+                run_tiles<F, ActT, ScaleT, 1, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi, x2, nplanes, ns);
                 return;
             }
         }
-        run_tiles<F, ActT, ScaleT, R, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi, x2, nplanes);
+        run_tiles<F, ActT, ScaleT, R, MB, NMAT, L>(mats, x, rows, cols, U, row_stride, gpr, gshift, batch_lo, batch_hi, lds_pairs, lds_corr, lds_xsum, lut, epi, x2, nplanes, ns);
     };
     if (U > 32) go(std::integral_constant<int, 64>{});
     else if (U > 16) go(std::integral_constant<int, 32>{});
@@ -301,6 +318,50 @@ using u32 = uint32_t;
         matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
+    }                                                                                             \
+    SMELT_KERNEL_W5 void smelt_affine_gate_up_geglu_##T(                                          \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* x, u16* y, u32 rows, u32 cols, u32 group) {                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiGeglu<ACT> epi{{}, y, (int)rows};                                                      \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi);                    \
+    }                                                                                             \
+    /* norm-scale prologue: rs holds one fp32 scale per token (grid.y) */                         \
+    SMELT_KERNEL_W5 void smelt_norm_scale_affine_matvec_##T(                                      \
+        const float* rs, const u16* x, const u16* nw, u16* xn, const u8* W, const u16* S,         \
+        const u16* B, u16* y, u32 rows, u32 cols, u32 group) {                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, y, (int)rows};                                                      \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 1>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi, nullptr, 0,         \
+                                             NormScale{rs, nw, xn});                              \
+    }                                                                                             \
+    SMELT_KERNEL_W5 void smelt_norm_scale_affine_gate_up_swiglu_##T(                              \
+        const float* rs, const u16* x, const u16* nw, const u8* gW, const u16* gS, const u16* gB, \
+        const u8* uW, const u16* uS, const u16* uB, u16* y, u32 rows, u32 cols, u32 group) {      \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiAffineSwiglu<ACT> epi{{}, y, (int)rows};                                               \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi, nullptr, 0,         \
+                                             NormScale{rs, nw, nullptr});                         \
+    }                                                                                             \
+    SMELT_KERNEL_W5 void smelt_norm_scale_affine_gate_up_geglu_##T(                               \
+        const float* rs, const u16* x, const u16* nw, const u8* gW, const u16* gS, const u16* gB, \
+        const u8* uW, const u16* uS, const u16* uB, u16* y, u32 rows, u32 cols, u32 group) {      \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiGeglu<ACT> epi{{}, y, (int)rows};                                                      \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi, nullptr, 0,         \
+                                             NormScale{rs, nw, nullptr});                         \
     }
 
 #define SMELT_AFFINE_BATCHED(T, ACT, SC, MBV)                                                     \
@@ -316,6 +377,19 @@ using u32 = uint32_t;
         matvec_body<FmtU4, ACT, SC, 4, MBV, 1>(mats, X, rows, cols,                               \
                                                packed_row_stride<FmtU4>(cols, group), group, lo,  \
                                                hi, epi);                                          \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_norm_scale_affine_matvec_batched_mb##MBV##_##T(                       \
+        const float* rs, const u16* X, const u16* nw, u16* XN, const u8* W, const u16* S,         \
+        const u16* B, u16* Y, u32 batch, u32 rows, u32 cols, u32 group, u32 batch_tile) {         \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        matvec_body<FmtU4, ACT, SC, 4, MBV, 1>(mats, X, rows, cols,                               \
+                                               packed_row_stride<FmtU4>(cols, group), group, lo,  \
+                                               hi, epi, nullptr, 0, NormScale{rs, nw, XN});       \
     }                                                                                             \
     SMELT_KERNEL void smelt_affine_matvec_add_batched_mb##MBV##_##T(                              \
         const u8* W, const u16* S, const u16* B, const u16* X, u16* Y, const u16* res, u32 batch, \

@@ -213,6 +213,10 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         else if (name == "fused_affine_matvec_add") { out->family = kFamAffineAdd; out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; }
         else if (name == "fused_affine_gate_up_swiglu") { out->family = kFamAffineGateUp; out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; }
         else if (name == "fused_dual_affine_matvec") { out->family = kFamAffineDual; out->symbol = "smelt_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; }
+        else if (name == "fused_affine_gate_up_geglu") { out->family = kFamAffineGateUp; out->symbol = "smelt_affine_gate_up_geglu_" + t; out->kinds = "PPPPPPPPUUU"; }
+        else if (name == "norm_scale_affine_matvec") { out->family = kFamNormScaleAffineMatvec; out->symbol = "smelt_norm_scale_affine_matvec_" + t; out->kinds = "PPPPPPPPUUU"; }
+        else if (name == "norm_scale_affine_gate_up_swiglu") { out->family = kFamNormScaleAffineGateUp; out->symbol = "smelt_norm_scale_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPPPUUU"; }
+        else if (name == "norm_scale_affine_gate_up_geglu") { out->family = kFamNormScaleAffineGateUp; out->symbol = "smelt_norm_scale_affine_gate_up_geglu_" + t; out->kinds = "PPPPPPPPPPUUU"; }
         else if (name == "affine_bank4_matvec") { out->family = kFamAffineBank4; out->symbol = "smelt_affine_bank4_matvec_" + t; out->kinds = "PPPPPPPPUUUUUU"; }
         else { *why = "no HIP kernel for function-constant pipeline '" + name + "'"; return kResolveUnknown; }
         if (!is_pow2(group) || group < 32 || cols % 32 != 0 || cols == 0) {
@@ -231,6 +235,10 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         {"fused_affine_matvec_add", kFamAffineAdd},
         {"fused_affine_gate_up_swiglu", kFamAffineGateUp},
         {"fused_dual_affine_matvec", kFamAffineDual},
+        {"fused_affine_gate_up_geglu", kFamAffineGateUp},
+        {"norm_scale_affine_matvec", kFamNormScaleAffineMatvec},
+        {"norm_scale_affine_gate_up_swiglu", kFamNormScaleAffineGateUp},
+        {"norm_scale_affine_gate_up_geglu", kFamNormScaleAffineGateUp},
     };
     for (const AffineName& a : kAffine) {
         const size_t n = strlen(a.prefix);
@@ -290,11 +298,16 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                 case kFamAffineAdd: out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; break;
                 case kFamAffineGateUp: out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; break;
                 case kFamAffineDual: out->symbol = "smelt_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; break;
+                case kFamNormScaleAffineMatvec: out->symbol = "smelt_norm_scale_affine_matvec_" + t; out->kinds = "PPPPPPPPUUU"; break;
+                case kFamNormScaleAffineGateUp: out->symbol = std::string("smelt_") + a.prefix + "_" + t; out->kinds = "PPPPPPPPPPUUU"; break;
                 default: break;
             }
+            if (a.m1 == kFamAffineGateUp && strstr(a.prefix, "geglu")) out->symbol = "smelt_affine_gate_up_geglu_" + t;
+            const bool prologue = a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp;
+            if (prologue && want_mfma) { *why = "no matrix-core form of '" + entry + "'"; return kResolveUnknown; }
             out->appended = {rows, cols, group};
             const uint32_t nmat = a.m1 == kFamAffineGateUp ? 2 : 1;
-            if (a.m1 != kFamAffineDual)
+            if (a.m1 != kFamAffineDual && !prologue && !strstr(a.prefix, "geglu"))
                 if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, 1, nmat, lds_limit) : 0) {
                     out->mfma_kw = kw;
                     out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_" : (a.m1 == kFamAffineAdd ? "smelt_affine_mm_matvec_add_" : "smelt_affine_mm_gate_up_swiglu_")) + (kw == 1 ? "stream_" : "split_") + t;
@@ -302,6 +315,10 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                     out->appended.push_back(kw);
                 }
             return kResolveOk;
+        }
+        if (a.m1 == kFamNormScaleAffineGateUp || strstr(a.prefix, "geglu") || (a.m1 == kFamNormScaleAffineMatvec && (full || want_mfma))) {
+            *why = "no batched HIP kernel for '" + entry + "'";
+            return kResolveUnknown;
         }
         if (full && skinny) {
             if (group != 64 || cols % 512 != 0) { *why = "skinny qmm needs group 64 and cols % 512 == 0: '" + entry + "'"; return kResolveMalformed; }
@@ -329,6 +346,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         out->lds_variant = mb;
         const std::string mbs = "mb" + std::to_string(mb) + "_" + t;
         if (a.m1 == kFamAffineMatvec) { out->family = kFamAffineBatched; out->symbol = "smelt_affine_matvec_batched_" + mbs; out->kinds = "PPPPPUUUUU"; }
+        else if (a.m1 == kFamNormScaleAffineMatvec) { out->family = kFamNormScaleAffineBatched; out->symbol = "smelt_norm_scale_affine_matvec_batched_" + mbs; out->kinds = "PPPPPPPPUUUUU"; }
         else if (a.m1 == kFamAffineGateUp) { out->family = kFamAffineGateUpBatched; out->symbol = "smelt_affine_gate_up_swiglu_batched_" + mbs; out->kinds = "PPPPPPPPUUUUU"; }
         else { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
         out->appended = {rows, cols, group, bt};

@@ -68,6 +68,9 @@ enum FamilyId {
     kFamBinaryPackedBank4,    // C S x y0 y1 y2 y3 rows0 rows1 rows2 rows3 cols
     kFamBinaryTwoMatrix,      // C1 S1 C2 S2 x y1 y2 rows1 rows2 cols
     kFamCopy16,               // src dst count
+    kFamNormScaleAffineMatvec,   // rs x nw xn W S B y | rows cols group           (grid.y = token)
+    kFamNormScaleAffineGateUp,   // rs x nw gW gS gB uW uS uB y | rows cols group
+    kFamNormScaleAffineBatched,  // rs X nw XN W S B Y batch | rows cols group batch_tile
     kFamCount
 };
 

@@ -128,7 +128,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
     const bool plane_matvec = r.family == kFamPlaneMatvec || r.family == kFamPlaneAdd || r.family == kFamPlaneGateUp ||
                               r.family == kFamPlaneBank4 || r.family == kFamPlaneBatched || r.family == kFamBinaryPackedBank || r.family == kFamBinaryPackedBank4 ||
                               r.family == kFamBinaryTwoMatrix;
-    const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec;
+    const bool norm_scale_matvec = r.family == kFamNormScaleAffineMatvec || r.family == kFamNormScaleAffineGateUp || r.family == kFamNormScaleAffineBatched;
+    const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec || norm_scale_matvec;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
     if (matvec_like) {
@@ -192,6 +193,43 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             if (r.family == kFamAffineDual) { need[8] = gy * rows * 2; written[8] = true; }
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
             mm_cols = cols; mm_nmat = 2;
+            break;
+        }
+        case kFamNormScaleAffineMatvec: {
+            const size_t rows = U(8), cols = U(9), group = U(10);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            affine(4, 5, 6, rows, cols, group);
+            need[0] = gy * 4; align[0] = 4;
+            need[1] = gy * cols * 2; align[1] = 16;
+            need[2] = cols * 2;
+            need[3] = gy * cols * 2; written[3] = true;
+            need[7] = gy * rows * 2; written[7] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamNormScaleAffineGateUp: {
+            const size_t rows = U(10), cols = U(11), group = U(12);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            affine(3, 4, 5, rows, cols, group);
+            affine(6, 7, 8, rows, cols, group);
+            need[0] = gy * 4; align[0] = 4;
+            need[1] = gy * cols * 2; align[1] = 16;
+            need[2] = cols * 2;
+            need[9] = gy * rows * 2; written[9] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamNormScaleAffineBatched: {
+            const size_t batch = U(8), rows = U(9), cols = U(10), group = U(11), bt = U(12);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (bt == 0 || gy * bt < batch) return bad_geom("grid height * batch tile does not cover the batch");
+            affine(4, 5, 6, rows, cols, group);
+            need[0] = batch * 4; align[0] = 4;
+            need[1] = batch * cols * 2; align[1] = 16;
+            need[2] = cols * 2;
+            need[3] = batch * cols * 2; written[3] = true;
+            need[7] = batch * rows * 2; written[7] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), r.lds_variant);
             break;
         }
         case kFamAffineBatched:

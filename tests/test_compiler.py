@@ -45,7 +45,8 @@ def test_gateway_has_no_holes_and_never_defaults():
     assert cc.select(cc.ACT_FP16, cc.U4_LUT, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.U4_LUT, cc.GEMM, hip_backend=True)[0] == cc.SELECT_MISSING      # no batched u4_lut kernel
     assert cc.select(cc.ACT_FP16, cc.TURBO_QUANT_H, hip_backend=True)[0] == cc.SELECT_OK
-    assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_MISSING
+    assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_OK
+    assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, cc.GEMM, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_MISSING   # no prompt-tile GeGLU kernel
 
 
 def test_weight_layout_alignment_sizes_and_no_overlap():
@@ -97,6 +98,8 @@ def test_shape_routes():
     assert r.pipeline == b"affine_matvec:1056:32" and r.specialized == 0
     r = cc.route_decode_affine(3584, 1024, 64, fusion=cc.FUSION_GATE_UP_SWIGLU)
     assert r.pipeline == b"fused_affine_gate_up_swiglu_c1024_r3584_g64"
+    r = cc.route_decode_affine(6144, 1536, 128, fusion=cc.FUSION_GATE_UP_GEGLU)
+    assert r.pipeline == b"fused_affine_gate_up_geglu:1536:128"
     with pytest.raises(ValueError):
         cc.route_decode_affine(64, 1000, 64)                    # cols not a multiple of 32
     r = cc.route_prefill_affine(9216, 2560, 64, max_batch=8)     # 5..32 tokens, g64: split-K skinny MFMA kernel

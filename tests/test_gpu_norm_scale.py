@@ -1,0 +1,217 @@
+"""Norm-scale affine kernels and the GeGLU epilogue on the GPU.
+
+The norm-scale kernels (lut_matvec.metal:1288-1575, fixed forms :2743-3170, batched :4268-4440) read
+a precomputed RMS scale and normalise their input inline, x_norm = half((x * rs) * (1 + w)); the
+invariant the reference leans on is that the fused kernel equals the staged pair (a norm that
+stores x_norm, then the plain matvec) bit for bit.  GeGLU: lut_matvec.metal:2235-2243.
+"""
+import numpy as np
+import pytest
+
+import fixtures as fx
+import gpu_harness as gh
+import oracle.oracle as so
+from smelt_amd import runtime as rt
+from test_gpu_matvec import run_affine
+
+pytestmark = pytest.mark.gpu
+
+RS_SLOT, NW_SLOT, XN_SLOT = 6, 7, 8
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = rt.Context()
+    yield c
+    c.close()
+
+
+def norm_inputs(batch, cols, dtype, seed):
+    rng = np.random.default_rng(seed)
+    x = fx.to_bits(rng.normal(0, 2.0, (batch, cols)).astype(np.float32), dtype)
+    w = fx.to_bits(rng.normal(0, 0.3, cols).astype(np.float32), dtype)
+    rs = np.array([so.rms_scale(x[b], 1e-6, dtype) for b in range(batch)], np.float32)
+    return x, w, rs
+
+
+def run_norm_scale_matvec(ctx, weights, x, w, rs, dtype, entry, consts, batch_tile=None):
+    packed, scales, biases = weights
+    rows, cols = packed.shape[0], packed.shape[1] * 2
+    batch = x.shape[0]
+    wf = gh.WeightFile()
+    ow, os_, ob = wf.add(packed), wf.add(scales), wf.add(biases)
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(RS_SLOT, rs)
+    ctx.put(gh.X_SLOT, x)
+    ctx.put(NW_SLOT, w)
+    ctx.alloc(XN_SLOT, batch * cols * 2)
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+    bufs = [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0), (XN_SLOT, 3, 0), (0, 4, ow), (0, 5, os_), (0, 6, ob),
+            (gh.Y_SLOT, 7, 0)]
+    gy = batch if batch_tile is None else (batch + batch_tile - 1) // batch_tile
+    pipe = ctx.pipeline(entry + gh.t_suffix(dtype))
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, consts, (min(1024, (rows + 7) // 8), gy, 1), (256, 1, 1))) == 1
+    ctx.wait()
+    return (ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows),
+            ctx.read(XN_SLOT, np.uint16, batch * cols).reshape(batch, cols))
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("rows,cols,group", [(2048, 1536, 128), (777, 1056, 32), (6144, 1024, 64)])
+def test_norm_scale_matvec_equals_staged_pair(ctx, dtype, rows, cols, group):
+    weights = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=3)
+    x, w, rs = norm_inputs(1, cols, dtype, seed=rows)
+    xn_ref = so.norm_scale_input(x[0], rs[0], w, dtype)
+    y, xn = run_norm_scale_matvec(ctx, weights, x, w, rs, dtype, f"norm_scale_affine_matvec:{cols}:{group}", [(8, rows)])
+    assert np.array_equal(xn[0], xn_ref)                     # the stored normalised row, bit for bit
+    staged = run_affine(ctx, *weights, xn, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    assert np.array_equal(y, staged)                          # fused == staged
+    ref = so.affine_matvec(*weights, fx.from_bits(xn_ref, dtype).reshape(1, cols), rows, cols, group, dtype)
+    gh.check_outputs(y, ref, dtype, "norm_scale_affine_matvec")
+    if cols % 32 == 0 and (group & (group - 1)) == 0:
+        for suffix in ("_rows4", "_rows8", ""):
+            y2, _ = run_norm_scale_matvec(ctx, weights, x, w, rs, dtype,
+                                          f"norm_scale_affine_matvec_c{cols}_r{rows}_g{group}{suffix}", [])
+            assert np.array_equal(y, y2)
+
+
+@pytest.mark.parametrize("batch,tile", [(3, 8), (8, 8), (11, 8)])
+def test_norm_scale_matvec_batched_rows_use_their_own_scale(ctx, batch, tile):
+    """Per-token scale scalePtr[token] (lut_matvec.metal:4318-4322); every row equals the batch-1 kernel."""
+    rows, cols, group, dtype = 2048, 2560, 128, fx.F16
+    weights = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=1)
+    x, w, rs = norm_inputs(batch, cols, dtype, seed=batch)
+    y, xn = run_norm_scale_matvec(ctx, weights, x, w, rs, dtype,
+                                  f"norm_scale_affine_matvec_c{cols}_r{rows}_g{group}_batched", [(8, batch)], batch_tile=tile)
+    for b in range(batch):
+        assert np.array_equal(xn[b], so.norm_scale_input(x[b], rs[b], w, dtype))
+        y1, _ = run_norm_scale_matvec(ctx, weights, x[b:b + 1], w, rs[b:b + 1], dtype,
+                                      f"norm_scale_affine_matvec:{cols}:{group}", [(8, rows)])
+        assert np.array_equal(y[b], y1[0])
+    # grid.y of the single-token kernel is the token index as well
+    yg, xg = run_norm_scale_matvec(ctx, weights, x, w, rs, dtype, f"norm_scale_affine_matvec:{cols}:{group}", [(8, rows)])
+    assert np.array_equal(yg, y) and np.array_equal(xg, xn)
+
+
+def run_gate_up(ctx, gw, uw, dtype, entry, consts, x, norm=None):
+    rows, cols = gw[0].shape[0], gw[0].shape[1] * 2
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*gw, *uw)]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(gh.X_SLOT, x)
+    ctx.alloc(gh.Y_SLOT, rows * 2)
+    if norm is None:
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
+    else:
+        w, rs = norm
+        ctx.put(RS_SLOT, rs)
+        ctx.put(NW_SLOT, w)
+        bufs = [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0)] + [(0, 3 + i, o) for i, o in enumerate(offs)] + \
+               [(gh.Y_SLOT, 9, 0)]
+    pipe = ctx.pipeline(entry + gh.t_suffix(dtype))
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, consts, (512, 1, 1), (256, 1, 1))) == 1
+    ctx.wait()
+    return ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("act", ["swiglu", "geglu"])
+def test_norm_scale_gate_up_equals_staged_pair(ctx, dtype, act):
+    rows, cols, group = 3584, 1024, 64
+    gw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=4)
+    uw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=5)
+    x, w, rs = norm_inputs(1, cols, dtype, seed=17)
+    xn = so.norm_scale_input(x[0], rs[0], w, dtype).reshape(1, cols)
+    fused = run_gate_up(ctx, gw, uw, dtype, f"norm_scale_affine_gate_up_{act}:{cols}:{group}", [(10, rows)], x, norm=(w, rs))
+    staged = run_gate_up(ctx, gw, uw, dtype, f"fused_affine_gate_up_{act}:{cols}:{group}", [(8, rows)], xn)
+    assert np.array_equal(fused, staged)
+    fixed = run_gate_up(ctx, gw, uw, dtype, f"norm_scale_affine_gate_up_{act}_c{cols}_r{rows}_g{group}_rows4", [], x, norm=(w, rs))
+    assert np.array_equal(fused, fixed)
+    xf = fx.from_bits(xn, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
+    u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
+    epi = so.epilogue_affine_swiglu if act == "swiglu" else so.epilogue_geglu
+    ref = fx.from_bits(epi(g, u, dtype), dtype)
+    gh.check_outputs(fused, ref, dtype, f"norm_scale gate_up {act}", rel_tol=4e-3 if dtype == fx.F16 else 1.6e-2)
+
+
+def test_geglu_fixed_name_and_clamps(ctx):
+    """Large gates saturate tanh (argument clamped to +-20) and the product is clamped to +-65504."""
+    rows, cols, group, dtype = 512, 1024, 64, fx.F16
+    gw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=6)
+    uw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=7)
+    x = fx.to_bits(np.full((1, cols), 30.0, np.float32) * np.where(np.arange(cols) % 2, 1.0, 0.75), dtype)
+    y = run_gate_up(ctx, gw, uw, dtype, f"fused_affine_gate_up_geglu_c{cols}_r{rows}_g{group}_rows4", [], x)
+    xf = fx.from_bits(x, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
+    u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
+    assert np.abs(g).max() > 30                                  # the clamp region is exercised
+    ref_bits = so.epilogue_geglu(g, u, dtype)
+    got = fx.from_bits(y, dtype).ravel().astype(np.float64)
+    ref = fx.from_bits(ref_bits, dtype).ravel().astype(np.float64)
+    assert np.isfinite(got).all() and np.abs(got).max() <= 65504
+    tol = 4e-3 * np.maximum(np.abs(ref), np.abs(ref).max() * 2.0 ** -6) + gh.ulp_of(ref, dtype)
+    assert (np.abs(got - ref) <= tol).all()
+
+
+def test_norm_scale_launches_are_validated(ctx):
+    rows, cols, group, dtype = 256, 1024, 64, fx.F16
+    weights = fx.synth_affine(rows, cols, group, dtype, config=0, tensor=0)
+    x, w, rs = norm_inputs(1, cols, dtype, seed=5)
+    wf = gh.WeightFile()
+    ow, os_, ob = wf.add(weights[0]), wf.add(weights[1]), wf.add(weights[2])
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
+    ctx.alloc(XN_SLOT, cols * 2 - 64)                             # too small for the normalised row
+    ctx.alloc(gh.Y_SLOT, rows * 2)
+    bufs = [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0), (XN_SLOT, 3, 0), (0, 4, ow), (0, 5, os_), (0, 6, ob),
+            (gh.Y_SLOT, 7, 0)]
+    pipe = ctx.pipeline(f"norm_scale_affine_matvec:{cols}:{group}")
+    with pytest.raises(rt.SmeltHipError):
+        ctx.encode_decode(rt.make_record(pipe, bufs, [(8, rows)], (32, 1, 1), (256, 1, 1)))
+    # the qmm forms of the prologue are not built: the name fails to resolve instead of running something else
+    with pytest.raises(rt.SmeltHipError):
+        ctx.pipeline(f"norm_scale_affine_matvec_c{cols}_r{rows}_g{group}_batched_full")
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
+    """The pair the reference emits (rms_norm_scale_only, then the norm-scale kernel;
+    SmeltCodeEmitter.swift:2680-2754) against the unfused records: same projection bits, and the
+    stored normalised row is the oracle's."""
+    from smelt_amd import compiler as cc
+    hidden, rows, ffn, group = 1536, 2048, 6144, 128
+    lay = cc.Layout()
+    wq, wg, wu = lay.affine(rows, hidden, group), lay.affine(ffn, hidden, group), lay.affine(ffn, hidden, group)
+    image = np.zeros(lay.total_bytes, np.uint8)
+    for i, e in enumerate((wq, wg, wu)):
+        cc.write_affine(image, e, *fx.synth_affine(e.rows, e.cols, group, dtype, config=1, tensor=40 + i))
+    X, NW, SCALE, XN, Q, F1, F2, Q2, F3 = range(1, 10)
+    act = rt.ACT_BF16 if dtype == fx.BF16 else rt.ACT_F16
+    em = cc.Emitter(act)
+    em.rms_norm_scale_only(cc.bind(X), cc.bind(SCALE), hidden)
+    em.norm_scale_matvec(0, wq, cc.bind(SCALE), cc.bind(X), cc.bind(NW), cc.bind(XN), cc.bind(Q))
+    em.norm_scale_gate_up(0, wg, wu, cc.bind(SCALE), cc.bind(X), cc.bind(NW), cc.bind(F1))
+    em.norm_scale_gate_up(0, wg, wu, cc.bind(SCALE), cc.bind(X), cc.bind(NW), cc.bind(F2), geglu=True)
+    # unfused: plain matvec / gate+up on the stored normalised row
+    em.matvec(0, wq, cc.bind(XN), cc.bind(Q2))
+    em.gate_up_swiglu(0, wg, wu, cc.bind(XN), cc.bind(F3))
+    ctx = rt.Context(act_dtype=act)
+    try:
+        em.install(ctx)
+        ctx.upload_weights(0, image)
+        x, w, _ = norm_inputs(1, hidden, dtype, seed=3)
+        ctx.put(X, x); ctx.put(NW, w)
+        ctx.alloc(SCALE, 4); ctx.alloc(XN, hidden * 2)
+        for slot, n in ((Q, rows), (Q2, rows), (F1, ffn), (F2, ffn), (F3, ffn)):
+            ctx.alloc(slot, n * 2)
+        assert ctx.interpret_decode(em.records()) == 6
+        ctx.wait()
+        rs = float(ctx.read(SCALE, np.float32, 1)[0])
+        assert abs(rs - so.rms_scale(x[0], 1e-6, dtype)) <= 5e-6 * rs
+        assert np.array_equal(ctx.read(XN, np.uint16, hidden), so.norm_scale_input(x[0], rs, w, dtype))
+        assert np.array_equal(ctx.read(Q, np.uint16, rows), ctx.read(Q2, np.uint16, rows))
+        assert np.array_equal(ctx.read(F1, np.uint16, ffn), ctx.read(F3, np.uint16, ffn))
+        assert np.abs(fx.from_bits(ctx.read(F2, np.uint16, ffn), dtype)).max() > 0
+    finally:
+        ctx.close()

@@ -87,3 +87,59 @@ def test_elementwise_matches_numpy_float16():
     a, b = f16(rng.normal(0, 100, 5000)), f16(rng.normal(0, 0.01, 5000))
     assert np.array_equal(so.elementwise(a, b, so.F16).view(np.float16), a.view(np.float16) + b.view(np.float16))
     assert np.array_equal(so.elementwise(a, b, so.F16, True).view(np.float16), a.view(np.float16) * b.view(np.float16))
+
+
+def test_norm_scale_input_closed_forms_and_rounding_order():
+    """x_norm = half((x * rs) * (1 + w)): products left to right, each rounded to fp32, one final
+    narrowing (lut_matvec.metal:1347-1379)."""
+    x = f16([1.0, -2.0, 0.5, 3.0])
+    zero = f16(np.zeros(4))
+    assert np.array_equal(so.norm_scale_input(x, 1.0, zero, so.F16), x)                          # rs = 1, w = 0: identity
+    assert np.array_equal(so.norm_scale_input(x, 0.25, zero, so.F16), f16([0.25, -0.5, 0.125, 0.75]))
+    assert np.array_equal(so.norm_scale_input(x, 0.5, f16([1.0, 3.0, -1.0, -0.5]), so.F16), f16([1.0, -4.0, 0.0, 0.75]))
+    # a product that lands exactly on an fp16 tie after its fp32 rounding, while the exact product lies
+    # below the tie: narrowing the fp32 value gives 0x2670, a single rounding of the exact product 0x266F
+    xt = np.array([np.float16(0.043273926)], np.float16).view(np.uint16)
+    wt = np.array([np.float16(0.15661621)], np.float16).view(np.uint16)
+    rs = float(np.float32(0.5022615))
+    exact = float(xt.view(np.float16)[0]) * rs * (1.0 + float(wt.view(np.float16)[0]))
+    assert np.float16(exact).view(np.uint16) == 0x266F
+    assert so.norm_scale_input(xt, rs, wt, so.F16)[0] == 0x2670
+    # against float64 on random data: never more than one 16-bit ulp away, almost always identical
+    rng = fx.rng_for(97, 0)
+    for dt, npdt in ((so.F16, np.float16),):
+        xb, wb = f16(rng.normal(0, 2, 8192)), f16(rng.normal(0, 0.3, 8192))
+        got = so.widen(so.norm_scale_input(xb, 0.7371, wb, dt), dt).astype(np.float64)
+        ref = so.widen(xb, dt).astype(np.float64) * float(np.float32(0.7371)) * (1.0 + so.widen(wb, dt).astype(np.float64))
+        ulp = np.spacing(np.abs(ref).astype(npdt)).astype(np.float64)
+        assert np.all(np.abs(got - ref) <= ulp)
+        assert np.mean(got == ref.astype(npdt).astype(np.float64)) > 0.995
+    # bf16: same formula in the wider-exponent type; the staged norm of the same row agrees within an ulp
+    xb, wb = so.narrow(rng.normal(0, 2, 2048).astype(np.float32), so.BF16), so.narrow(rng.normal(0, 0.3, 2048).astype(np.float32), so.BF16)
+    rs = so.rms_scale(xb, 1e-6, so.BF16)
+    a = so.widen(so.norm_scale_input(xb, rs, wb, so.BF16), so.BF16).astype(np.float64)
+    b = so.widen(so.rms_norm_1pw(xb, wb, 1e-6, so.BF16, False), so.BF16).astype(np.float64)
+    assert np.all(np.abs(a - b) <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(b), 1e-30))) - 7))
+
+
+def test_geglu_closed_forms_clamps_and_float64():
+    """lut_matvec.metal:2235-2243."""
+    def geglu(g, u, dt=so.F16):
+        return so.widen(so.epilogue_geglu(np.float32(g), np.float32(u), dt), dt)
+    assert geglu([0.0], [5.0])[0] == 0.0                                   # gelu(0) = 0
+    assert geglu([10.0], [0.5])[0] == 5.0                                  # tanh saturates: gelu(g) = g
+    assert geglu([-10.0], [3.0])[0] == 0.0                                 # ... and gelu(-g) = 0
+    assert geglu([100.0], [1000.0])[0] == 65504.0 and geglu([100.0], [-1000.0])[0] == -65504.0   # product clamp
+    assert geglu([1.0 + 2.0 ** -12], [1.0])[0] == geglu([1.0], [1.0])[0]   # inputs are rounded to the 16-bit type first
+    assert abs(float(geglu([1.0], [1.0])[0]) - 0.8411919906) < 1e-3        # 0.5 * (1 + tanh(0.79788 * 1.044715))
+    rng = fx.rng_for(98, 0)
+    g = rng.normal(0, 3, 4096).astype(np.float32)
+    u = rng.normal(0, 2, 4096).astype(np.float32)
+    gh_, uh = g.astype(np.float16).astype(np.float64), u.astype(np.float16).astype(np.float64)
+    inner = np.clip(float(np.float32(0.7978845608)) * (gh_ + float(np.float32(0.044715)) * gh_ ** 3), -20, 20)
+    ref = np.clip(0.5 * gh_ * (1 + np.tanh(inner)) * uh, -65504, 65504)
+    got = geglu(g, u).astype(np.float64)
+    # 1 + tanh(inner) is formed in fp32: for negative gates its rounding error (2^-24 of 1) is scaled by g * u / 2
+    tol = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + np.abs(gh_ * uh) * 2.0 ** -22
+    assert np.all(np.abs(got - ref) <= tol)
+    assert np.mean(got == ref.astype(np.float16).astype(np.float64)) > 0.94
