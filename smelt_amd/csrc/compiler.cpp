@@ -98,8 +98,8 @@ bool hip_has_kernel(const SmeltMatvecCell& c, int family) {
     if (family == SMELT_FAMILY_TQH) return c.activation != SMELT_ACT_FP32 && c.fusion == SMELT_FUSION_NONE;
     if (!quant) return false;
     if (c.activation == SMELT_ACT_FP32) return false;
-    // GeGLU: the single-token affine kernel only (no prompt-tile form yet)
-    if (c.fusion == SMELT_FUSION_GATE_UP_GEGLU) return family == SMELT_FAMILY_AFFINE_U4 && c.shape == SMELT_SHAPE_GEMV;
+    // GeGLU: affine only (single-token kernel and the MFMA slab kernel)
+    if (c.fusion == SMELT_FUSION_GATE_UP_GEGLU) return family == SMELT_FAMILY_AFFINE_U4;
     if (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_DUAL_MATVEC) return false;
     if (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_GATE_UP_SWIGLU && family == SMELT_FAMILY_TERNARY2) return false;
     return true;
@@ -398,9 +398,16 @@ int smelt_route_prefill_affine(int rows, int cols, int group, int fusion, int ma
     switch (fusion) {
         case SMELT_FUSION_NONE: stem = "affine_matvec"; break;
         case SMELT_FUSION_GATE_UP_SWIGLU: stem = "fused_affine_gate_up_swiglu"; break;
+        case SMELT_FUSION_GATE_UP_GEGLU: stem = "fused_affine_gate_up_geglu"; break;
         default: return SMELT_SELECT_MISSING;
     }
     const std::string base = std::string(stem) + shape_tag(rows, cols, group);
+    if (fusion == SMELT_FUSION_GATE_UP_GEGLU) {
+        // GeGLU has the MFMA slab kernel only
+        const int bt = max_batch > 32 ? 64 : 16;
+        set_route(out, base + (bt == 16 ? "_batched_full" : "_batched_full_b64"), true, 64, bt, 256, (rows + 63) / 64);
+        return SMELT_HIP_OK;
+    }
     if (max_batch <= 4) {
         // weights stream once per four tokens through the matvec kernel
         const int rpw = fusion == SMELT_FUSION_NONE ? 4 : 2;

@@ -52,6 +52,25 @@ struct BF16 {
     }
 };
 
+// Prologue of the norm-scale kernels (lut_matvec.metal:1288-1292): with rs != nullptr the staged
+// activation is narrow((x * rs[token]) * (1 + weight)), rounded to the 16-bit type exactly as a
+// staged norm would store it; the launch's first workgroup also writes that row to `out`.
+struct NormScale {
+    const float* rs = nullptr;
+    const uint16_t* weight = nullptr;
+    uint16_t* out = nullptr;
+};
+
+// (x * rs) * (1 + w) with each product and the sum rounded on its own: without the pragma the
+// compiler folds t * (1 + w) into fma(w, t, t), one rounding fewer than the staged norm performs.
+template <class ActT>
+__device__ __forceinline__ uint16_t norm_scale_value(uint16_t x, float rs, uint16_t w) {
+#pragma clang fp contract(off)
+    const float scaled = ActT::widen(x) * rs;
+    const float direct = 1.0f + ActT::widen(w);
+    return ActT::narrow(scaled * direct);
+}
+
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 
 // D = a.x*b.x + a.y*b.y + acc with fp32 accumulation (v_dot2c_f32_f16).

@@ -211,6 +211,23 @@ struct QEpiAdd {
     }
 };
 
+// agent_geglu_product (lut_matvec.metal:2235-2243)
+template <class ActT>
+struct QEpiGeglu {
+    uint16_t* y;
+    __device__ __forceinline__ void operator()(int tok, int n, int rows, const float (&v)[2][4]) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n + i < rows) {
+                const float g = ActT::widen(ActT::narrow(v[0][i])), u = ActT::widen(ActT::narrow(v[1][i]));
+                float inner = 0.7978845608f * (g + 0.044715f * (g * g * g));
+                inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+                const float gelu = 0.5f * g * (1.0f + tanhf(inner));
+                y[(size_t)tok * rows + n + i] = ActT::narrow(fminf(fmaxf(gelu * u, -65504.0f), 65504.0f));
+            }
+    }
+};
+
 template <class ActT>
 struct QEpiSwiglu {
     uint16_t* y;
@@ -242,7 +259,7 @@ __device__ __forceinline__ void qmm_affine_tile(const uint8_t* const (&W)[NMAT],
                                                 const uint16_t* const (&B)[NMAT], const uint16_t* X,
                                                 int rows, int cols, int gpr, int gshift, int batch,
                                                 int n0, int m0, unsigned char* smem,
-                                                float4_t (&acc)[NMAT][MT]) {
+                                                float4_t (&acc)[NMAT][MT], const NormScale& ns = NormScale{}) {
     // LDS: codes [NMAT][64][kQxLdW] bytes | x [16*MT][kQmmLd] fp16 (k permuted per 8) |
     //      xsum [16*MT][4] float (per 32-column quarter) | scale, bias [NMAT][4][64] float
     uint8_t* lds_c = smem;
@@ -300,7 +317,22 @@ __device__ __forceinline__ void qmm_affine_tile(const uint8_t* const (&W)[NMAT],
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 uint4_t v = {0, 0, 0, 0};
-                if (tok < batch && k + e * 8 < cols) v = *reinterpret_cast<const uint4_t*>(X + (size_t)tok * cols + k + e * 8);
+                if (tok < batch && k + e * 8 < cols) {
+                    v = *reinterpret_cast<const uint4_t*>(X + (size_t)tok * cols + k + e * 8);
+                    // norm-scale prologue: the tile multiplies the normalised row; the first row slab stores it
+                    if (ns.rs != nullptr) {
+                        uint32_t* p = reinterpret_cast<uint32_t*>(&v);
+                        const float rs = ns.rs[tok];
+                        const uint16_t* nw = ns.weight + k + e * 8;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint16_t lo = norm_scale_value<ActT>((uint16_t)(p[i] & 0xFFFF), rs, nw[2 * i]);
+                            const uint16_t hi = norm_scale_value<ActT>((uint16_t)(p[i] >> 16), rs, nw[2 * i + 1]);
+                            p[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+                        }
+                        if (ns.out != nullptr && n0 == 0) *reinterpret_cast<uint4_t*>(ns.out + (size_t)tok * cols + k + e * 8) = v;
+                    }
+                }
                 uint16_t h[8];
                 const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -385,7 +417,7 @@ template <class ActT, class ScaleT, int MT, int NMAT, class Epi>
 __device__ __forceinline__ void qmm_affine_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
                                                 const uint16_t* const (&B)[NMAT], const uint16_t* X,
                                                 int rows, int cols, int group, int batch, int batch_tile,
-                                                const Epi& epi) {
+                                                const Epi& epi, const NormScale& ns = NormScale{}) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int gshift = ilog2((uint32_t)group);
     const int gpr = (cols + group - 1) / group;
@@ -398,7 +430,7 @@ __device__ __forceinline__ void qmm_affine_body(const uint8_t* const (&W)[NMAT],
         const int n0 = slab * kQmmBN;
         for (int m0 = m_lo; m0 < m_hi; m0 += 16 * MT) {
             float4_t acc[NMAT][MT];
-            qmm_affine_tile<ActT, ScaleT, MT, NMAT>(W, S, B, X, rows, cols, gpr, gshift, batch, n0, m0, smem, acc);
+            qmm_affine_tile<ActT, ScaleT, MT, NMAT>(W, S, B, X, rows, cols, gpr, gshift, batch, n0, m0, smem, acc, ns);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const int tok = m0 + t * 16 + li;
@@ -450,6 +482,56 @@ __device__ __forceinline__ void qmm_affine_body(const uint8_t* const (&W)[NMAT],
         const uint16_t* const b[2] = {gB, uB};                                                     \
         QEpiSwiglu<ACT> epi{Y};                                                                    \
         qmm_affine_body<ACT, SC, MTV, 2>(w, s, b, X, rows, cols, group, batch, batch_tile, epi);   \
+    }                                                                                              \
+    SMELT_QMM_KERNEL void smelt_affine_qmm_gate_up_geglu_mt##MTV##_##T(                            \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t group, uint32_t batch_tile) {                       \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        QEpiGeglu<ACT> epi{Y};                                                                     \
+        qmm_affine_body<ACT, SC, MTV, 2>(w, s, b, X, rows, cols, group, batch, batch_tile, epi);   \
+    }                                                                                              \
+    /* norm-scale prologue (agent_affine_qmm.h:790-...): rs[token], normalised rows stored by slab 0 */ \
+    SMELT_QMM_KERNEL void smelt_norm_scale_affine_qmm_mt##MTV##_##T(                               \
+        const float* rs, const uint16_t* X, const uint16_t* nw, uint16_t* XN, const uint8_t* W,    \
+        const uint16_t* S, const uint16_t* B, uint16_t* Y, uint32_t batch, uint32_t rows,          \
+        uint32_t cols, uint32_t group, uint32_t batch_tile) {                                      \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        QEpiStore<ACT> epi{Y};                                                                     \
+        qmm_affine_body<ACT, SC, MTV, 1>(w, s, b, X, rows, cols, group, batch, batch_tile, epi,    \
+                                         NormScale{rs, nw, XN});                                   \
+    }                                                                                              \
+    SMELT_QMM_KERNEL void smelt_norm_scale_affine_qmm_gate_up_swiglu_mt##MTV##_##T(                \
+        const float* rs, const uint16_t* X, const uint16_t* nw, const uint8_t* gW,                 \
+        const uint16_t* gS, const uint16_t* gB, const uint8_t* uW, const uint16_t* uS,             \
+        const uint16_t* uB, uint16_t* Y, uint32_t batch, uint32_t rows, uint32_t cols,             \
+        uint32_t group, uint32_t batch_tile) {                                                     \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        QEpiSwiglu<ACT> epi{Y};                                                                    \
+        qmm_affine_body<ACT, SC, MTV, 2>(w, s, b, X, rows, cols, group, batch, batch_tile, epi,    \
+                                         NormScale{rs, nw, nullptr});                              \
+    }                                                                                              \
+    SMELT_QMM_KERNEL void smelt_norm_scale_affine_qmm_gate_up_geglu_mt##MTV##_##T(                 \
+        const float* rs, const uint16_t* X, const uint16_t* nw, const uint8_t* gW,                 \
+        const uint16_t* gS, const uint16_t* gB, const uint8_t* uW, const uint16_t* uS,             \
+        const uint16_t* uB, uint16_t* Y, uint32_t batch, uint32_t rows, uint32_t cols,             \
+        uint32_t group, uint32_t batch_tile) {                                                     \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        QEpiGeglu<ACT> epi{Y};                                                                     \
+        qmm_affine_body<ACT, SC, MTV, 2>(w, s, b, X, rows, cols, group, batch, batch_tile, epi,    \
+                                         NormScale{rs, nw, nullptr});                              \
     }
 
 #define SMELT_TERNARY_QMM(T, ACT, MTV)                                                             \

@@ -316,9 +316,30 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                 }
             return kResolveOk;
         }
-        if (a.m1 == kFamNormScaleAffineGateUp || strstr(a.prefix, "geglu") || (a.m1 == kFamNormScaleAffineMatvec && (full || want_mfma))) {
-            *why = "no batched HIP kernel for '" + entry + "'";
-            return kResolveUnknown;
+        const bool geglu = strstr(a.prefix, "geglu") != nullptr;
+        if (a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp || geglu) {
+            // prologue and GeGLU forms: the MFMA slab kernel for "_batched_full", the vector-ALU
+            // token tile for the plain "_batched" matvec, nothing else
+            if (want_mfma || skinny || (!full && a.m1 != kFamNormScaleAffineMatvec)) {
+                *why = "no batched HIP kernel for '" + entry + "'";
+                return kResolveUnknown;
+            }
+            if (full) {
+                const uint32_t mt = bt >= 64 ? 4 : 1;
+                out->lds_variant = mt;
+                const std::string mts = "mt" + std::to_string(mt) + "_" + t;
+                if (a.m1 == kFamNormScaleAffineMatvec) {
+                    out->family = kFamNormScaleAffineQmm; out->symbol = "smelt_norm_scale_affine_qmm_" + mts; out->kinds = "PPPPPPPPUUUUU";
+                } else if (a.m1 == kFamNormScaleAffineGateUp) {
+                    out->family = kFamNormScaleAffineQmmGateUp;
+                    out->symbol = std::string("smelt_norm_scale_affine_qmm_gate_up_") + (geglu ? "geglu_" : "swiglu_") + mts;
+                    out->kinds = "PPPPPPPPPPUUUUU";
+                } else {
+                    out->family = kFamAffineQmmGateUp; out->symbol = "smelt_affine_qmm_gate_up_geglu_" + mts; out->kinds = "PPPPPPPPUUUUU";
+                }
+                out->appended = {rows, cols, group, bt};
+                return kResolveOk;
+            }
         }
         if (full && skinny) {
             if (group != 64 || cols % 512 != 0) { *why = "skinny qmm needs group 64 and cols % 512 == 0: '" + entry + "'"; return kResolveMalformed; }

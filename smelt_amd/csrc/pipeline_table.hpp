@@ -71,6 +71,8 @@ enum FamilyId {
     kFamNormScaleAffineMatvec,   // rs x nw xn W S B y | rows cols group           (grid.y = token)
     kFamNormScaleAffineGateUp,   // rs x nw gW gS gB uW uS uB y | rows cols group
     kFamNormScaleAffineBatched,  // rs X nw XN W S B Y batch | rows cols group batch_tile
+    kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
+    kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile
     kFamCount
 };
 

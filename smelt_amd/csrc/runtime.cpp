@@ -128,7 +128,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
     const bool plane_matvec = r.family == kFamPlaneMatvec || r.family == kFamPlaneAdd || r.family == kFamPlaneGateUp ||
                               r.family == kFamPlaneBank4 || r.family == kFamPlaneBatched || r.family == kFamBinaryPackedBank || r.family == kFamBinaryPackedBank4 ||
                               r.family == kFamBinaryTwoMatrix;
-    const bool norm_scale_matvec = r.family == kFamNormScaleAffineMatvec || r.family == kFamNormScaleAffineGateUp || r.family == kFamNormScaleAffineBatched;
+    const bool norm_scale_matvec = r.family == kFamNormScaleAffineMatvec || r.family == kFamNormScaleAffineGateUp || r.family == kFamNormScaleAffineBatched ||
+                                   r.family == kFamNormScaleAffineQmm || r.family == kFamNormScaleAffineQmmGateUp;
     const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec || norm_scale_matvec;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
@@ -230,6 +231,29 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[3] = batch * cols * 2; written[3] = true;
             need[7] = batch * rows * 2; written[7] = true;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), r.lds_variant);
+            break;
+        }
+        case kFamNormScaleAffineQmm:
+        case kFamNormScaleAffineQmmGateUp: {
+            if (int e = need_256()) return e;
+            const bool gate_up = r.family == kFamNormScaleAffineQmmGateUp;
+            const size_t o = gate_up ? 10 : 8;
+            const size_t batch = U(o), rows = U(o + 1), cols = U(o + 2), group = U(o + 3), bt = U(o + 4);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (bt == 0 || gy * bt < batch) return bad_geom("grid height * batch tile does not cover the batch");
+            need[0] = batch * 4; align[0] = 4;
+            need[1] = batch * cols * 2; align[1] = 16;
+            need[2] = cols * 2; align[2] = 16;
+            if (gate_up) {
+                affine(3, 4, 5, rows, cols, group);
+                affine(6, 7, 8, rows, cols, group);
+                need[9] = batch * rows * 2; written[9] = true;
+            } else {
+                need[3] = batch * cols * 2; align[3] = 16; written[3] = true;
+                affine(4, 5, 6, rows, cols, group);
+                need[7] = batch * rows * 2; written[7] = true;
+            }
+            L.lds = qmm_affine_lds_bytes(gate_up ? 2 : 1, r.lds_variant);
             break;
         }
         case kFamAffineBatched:

@@ -46,7 +46,8 @@ def test_gateway_has_no_holes_and_never_defaults():
     assert cc.select(cc.ACT_FP16, cc.U4_LUT, cc.GEMM, hip_backend=True)[0] == cc.SELECT_MISSING      # no batched u4_lut kernel
     assert cc.select(cc.ACT_FP16, cc.TURBO_QUANT_H, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_OK
-    assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, cc.GEMM, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_MISSING   # no prompt-tile GeGLU kernel
+    assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, cc.GEMM, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_OK
+    assert cc.select(cc.ACT_FP16, cc.BINARY1, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_NOT_MEANINGFUL
 
 
 def test_weight_layout_alignment_sizes_and_no_overlap():

@@ -169,9 +169,12 @@ def test_norm_scale_launches_are_validated(ctx):
     pipe = ctx.pipeline(f"norm_scale_affine_matvec:{cols}:{group}")
     with pytest.raises(rt.SmeltHipError):
         ctx.encode_decode(rt.make_record(pipe, bufs, [(8, rows)], (32, 1, 1), (256, 1, 1)))
-    # the qmm forms of the prologue are not built: the name fails to resolve instead of running something else
-    with pytest.raises(rt.SmeltHipError):
-        ctx.pipeline(f"norm_scale_affine_matvec_c{cols}_r{rows}_g{group}_batched_full")
+    # forms that are not built fail to resolve instead of running something else
+    for name in (f"norm_scale_affine_matvec_c{cols}_r{rows}_g{group}_batched_skinny",
+                 f"norm_scale_affine_gate_up_swiglu_c{cols}_r{rows}_g{group}_batched",
+                 f"fused_affine_gate_up_geglu_c{cols}_r{rows}_g{group}_batched_tile4"):
+        with pytest.raises(rt.SmeltHipError):
+            ctx.pipeline(name)
 
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
@@ -215,3 +218,68 @@ def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
         assert np.abs(fx.from_bits(ctx.read(F2, np.uint16, ffn), dtype)).max() > 0
     finally:
         ctx.close()
+
+
+def run_qmm(ctx, entry, dtype, batch, bufs_fn, rows, grid_w, bt, batch_index):
+    pipe = ctx.pipeline(entry + gh.t_suffix(dtype))
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+    rec = rt.make_record(pipe, bufs_fn(), [(batch_index, batch)], (grid_w, (batch + bt - 1) // bt, 1), (256, 1, 1))
+    assert ctx.encode_decode(rec) == 1
+    ctx.wait()
+    return ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("batch,suffix,bt", [(14, "_batched_full", 16), (37, "_batched_full", 16), (70, "_batched_full_b64", 64)])
+def test_norm_scale_qmm_equals_plain_qmm_on_the_stored_rows(ctx, dtype, batch, suffix, bt):
+    """agent_norm_scale_affine_qmm_fixed_batched_full (lut_matvec.metal:8496-8530): per-token scales,
+    normalised rows stored, and the product equal to the plain qmm run on those rows bit for bit."""
+    rows, cols, group = 1000, 1024, 64
+    weights = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=2)
+    x, w, rs = norm_inputs(batch, cols, dtype, seed=batch)
+    wf = gh.WeightFile()
+    ow, os_, ob = (wf.add(a) for a in weights)
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
+    ctx.alloc(XN_SLOT, batch * cols * 2)
+    shape = f"_c{cols}_r{rows}_g{group}"
+    fused = run_qmm(ctx, "norm_scale_affine_matvec" + shape + suffix, dtype, batch,
+                    lambda: [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0), (XN_SLOT, 3, 0), (0, 4, ow), (0, 5, os_),
+                             (0, 6, ob), (gh.Y_SLOT, 7, 0)], rows, (rows + 63) // 64, bt, 8)
+    xn = ctx.read(XN_SLOT, np.uint16, batch * cols).reshape(batch, cols)
+    for b in range(batch):
+        assert np.array_equal(xn[b], so.norm_scale_input(x[b], rs[b], w, dtype)), b
+    ctx.put(gh.X_SLOT, xn)
+    staged = run_qmm(ctx, "affine_matvec" + shape + suffix, dtype, batch,
+                     lambda: [(0, 0, ow), (0, 1, os_), (0, 2, ob), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)],
+                     rows, (rows + 63) // 64, bt, 5)
+    assert np.array_equal(fused, staged)
+    ref = so.affine_matvec(*weights, fx.from_bits(xn, dtype), rows, cols, group, dtype)
+    gh.check_outputs(fused, ref, dtype, "norm_scale qmm")
+
+
+@pytest.mark.parametrize("act", ["swiglu", "geglu"])
+def test_norm_scale_gate_up_qmm_and_geglu_qmm(ctx, act):
+    rows, cols, group, dtype, batch, bt = 640, 1024, 64, fx.F16, 21, 16
+    gw = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=3)
+    uw = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=4)
+    x, w, rs = norm_inputs(batch, cols, dtype, seed=77)
+    xn = np.stack([so.norm_scale_input(x[b], rs[b], w, dtype) for b in range(batch)])
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*gw, *uw)]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
+    shape = f"_c{cols}_r{rows}_g{group}_batched_full"
+    fused = run_qmm(ctx, f"norm_scale_affine_gate_up_{act}" + shape, dtype, batch,
+                    lambda: [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0)] + [(0, 3 + i, o) for i, o in enumerate(offs)] +
+                            [(gh.Y_SLOT, 9, 0)], rows, (rows + 63) // 64, bt, 10)
+    ctx.put(gh.X_SLOT, xn)
+    staged = run_qmm(ctx, f"fused_affine_gate_up_{act}" + shape, dtype, batch,
+                     lambda: [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)],
+                     rows, (rows + 63) // 64, bt, 8)
+    assert np.array_equal(fused, staged)
+    xf = fx.from_bits(xn, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
+    u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
+    epi = so.epilogue_affine_swiglu if act == "swiglu" else so.epilogue_geglu
+    gh.check_outputs(fused, fx.from_bits(epi(g, u, dtype), dtype), dtype, f"gate_up {act} qmm", rel_tol=4e-3)
