@@ -59,6 +59,9 @@ struct NormScale {
     const float* rs = nullptr;
     const uint16_t* weight = nullptr;
     uint16_t* out = nullptr;
+    // norm_add_scale form (lut_matvec.metal:2896-2990): the rounded norm plus this row, added and
+    // rounded in the 16-bit type, is what the kernel multiplies and stores
+    const uint16_t* residual = nullptr;
 };
 
 // (x * rs) * (1 + w) with each product and the sum rounded on its own: without the pragma the
@@ -69,6 +72,14 @@ __device__ __forceinline__ uint16_t norm_scale_value(uint16_t x, float rs, uint1
     const float scaled = ActT::widen(x) * rs;
     const float direct = 1.0f + ActT::widen(w);
     return ActT::narrow(scaled * direct);
+}
+
+// one element of the prologue: norm, then the optional residual add
+template <class ActT>
+__device__ __forceinline__ uint16_t norm_scale_element(const NormScale& ns, uint16_t x, float rs, size_t token_offset, int c) {
+    uint16_t v = norm_scale_value<ActT>(x, rs, ns.weight[c]);
+    if (ns.residual != nullptr) v = ActT::narrow(ActT::widen(v) + ActT::widen(ns.residual[token_offset + c]));
+    return v;
 }
 
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }

@@ -284,7 +284,7 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
             for (int i = 0; i < CPD; ++i) {
                 const int c = col0 + i;
                 if (c < cols) {
-                    v[i] = norm_scale_value<ActT>(v[i], rs, ns.weight[c]);
+                    v[i] = norm_scale_element<ActT>(ns, v[i], rs, (size_t)(b0 + b) * cols, c);
                     if (ns.out != nullptr && blockIdx.x == 0) ns.out[(size_t)(b0 + b) * cols + c] = v[i];
                 }
             }

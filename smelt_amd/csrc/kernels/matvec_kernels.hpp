@@ -341,6 +341,29 @@ using u32 = uint32_t;
                                              blockIdx.y, blockIdx.y + 1, epi, nullptr, 0,         \
                                              NormScale{rs, nw, xn});                              \
     }                                                                                             \
+    SMELT_KERNEL_W5 void smelt_norm_add_scale_affine_matvec_##T(                                  \
+        const float* rs, const u16* x, const u16* nw, const u16* res, u16* xn, const u8* W,       \
+        const u16* S, const u16* B, u16* y, u32 rows, u32 cols, u32 group) {                      \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, y, (int)rows};                                                      \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 1>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi, nullptr, 0,         \
+                                             NormScale{rs, nw, xn, res});                         \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_norm_scale_affine_dual_matvec_##T(                                    \
+        const float* rs, const u16* x, const u16* nw, const u8* W1, const u16* S1, const u16* B1, \
+        const u8* W2, const u16* S2, const u16* B2, u16* y1, u16* y2, u32 rows, u32 cols,         \
+        u32 group) {                                                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
+        EpiDual<ACT> epi{{}, y1, y2, (int)rows};                                                  \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi, nullptr, 0,         \
+                                             NormScale{rs, nw, nullptr});                         \
+    }                                                                                             \
     SMELT_KERNEL_W5 void smelt_norm_scale_affine_gate_up_swiglu_##T(                              \
         const float* rs, const u16* x, const u16* nw, const u8* gW, const u16* gS, const u16* gB, \
         const u8* uW, const u16* uS, const u16* uB, u16* y, u32 rows, u32 cols, u32 group) {      \

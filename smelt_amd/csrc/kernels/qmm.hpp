@@ -323,11 +323,10 @@ __device__ __forceinline__ void qmm_affine_tile(const uint8_t* const (&W)[NMAT],
                     if (ns.rs != nullptr) {
                         uint32_t* p = reinterpret_cast<uint32_t*>(&v);
                         const float rs = ns.rs[tok];
-                        const uint16_t* nw = ns.weight + k + e * 8;
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            const uint16_t lo = norm_scale_value<ActT>((uint16_t)(p[i] & 0xFFFF), rs, nw[2 * i]);
-                            const uint16_t hi = norm_scale_value<ActT>((uint16_t)(p[i] >> 16), rs, nw[2 * i + 1]);
+                            const uint16_t lo = norm_scale_element<ActT>(ns, (uint16_t)(p[i] & 0xFFFF), rs, (size_t)tok * cols, k + e * 8 + 2 * i);
+                            const uint16_t hi = norm_scale_element<ActT>(ns, (uint16_t)(p[i] >> 16), rs, (size_t)tok * cols, k + e * 8 + 2 * i + 1);
                             p[i] = (uint32_t)lo | ((uint32_t)hi << 16);
                         }
                         if (ns.out != nullptr && n0 == 0) *reinterpret_cast<uint4_t*>(ns.out + (size_t)tok * cols + k + e * 8) = v;

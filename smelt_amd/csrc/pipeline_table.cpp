@@ -237,6 +237,8 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         {"fused_dual_affine_matvec", kFamAffineDual},
         {"fused_affine_gate_up_geglu", kFamAffineGateUp},
         {"norm_scale_affine_matvec", kFamNormScaleAffineMatvec},
+        {"norm_add_scale_affine_matvec", kFamNormAddScaleAffineMatvec},
+        {"norm_scale_fused_dual_affine_matvec", kFamNormScaleAffineDual},
         {"norm_scale_affine_gate_up_swiglu", kFamNormScaleAffineGateUp},
         {"norm_scale_affine_gate_up_geglu", kFamNormScaleAffineGateUp},
     };
@@ -257,7 +259,9 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             want_mfma = true;
             suffix.resize(suffix.size() - 5);
         }
-        const bool m1 = suffix.empty() || suffix == "_rows4" || suffix == "_rows8" || suffix == "_rows4_sg1";
+        // the norm-scale dual kernel's "_batched" form takes its token from grid.y, like the single-token kernels
+        const bool m1 = suffix.empty() || suffix == "_rows4" || suffix == "_rows8" || suffix == "_rows4_sg1" ||
+                        (a.m1 == kFamNormScaleAffineDual && suffix == "_batched");
         if (want_mfma && mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 2, lds_limit) == 0) {
             *why = "matrix-core matvec needs group 64, cols % 256 == 0 and at least 8M weights: '" + entry + "'";
             return kResolveMalformed;
@@ -300,10 +304,13 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                 case kFamAffineDual: out->symbol = "smelt_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; break;
                 case kFamNormScaleAffineMatvec: out->symbol = "smelt_norm_scale_affine_matvec_" + t; out->kinds = "PPPPPPPPUUU"; break;
                 case kFamNormScaleAffineGateUp: out->symbol = std::string("smelt_") + a.prefix + "_" + t; out->kinds = "PPPPPPPPPPUUU"; break;
+                case kFamNormAddScaleAffineMatvec: out->symbol = "smelt_norm_add_scale_affine_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; break;
+                case kFamNormScaleAffineDual: out->symbol = "smelt_norm_scale_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPPPUUU"; break;
                 default: break;
             }
             if (a.m1 == kFamAffineGateUp && strstr(a.prefix, "geglu")) out->symbol = "smelt_affine_gate_up_geglu_" + t;
-            const bool prologue = a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp;
+            const bool prologue = a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp ||
+                                  a.m1 == kFamNormAddScaleAffineMatvec || a.m1 == kFamNormScaleAffineDual;
             if (prologue && want_mfma) { *why = "no matrix-core form of '" + entry + "'"; return kResolveUnknown; }
             out->appended = {rows, cols, group};
             const uint32_t nmat = a.m1 == kFamAffineGateUp ? 2 : 1;
@@ -317,6 +324,10 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             return kResolveOk;
         }
         const bool geglu = strstr(a.prefix, "geglu") != nullptr;
+        if (a.m1 == kFamNormAddScaleAffineMatvec || a.m1 == kFamNormScaleAffineDual) {
+            *why = "no batched HIP kernel for '" + entry + "'";
+            return kResolveUnknown;
+        }
         if (a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp || geglu) {
             // prologue and GeGLU forms: the MFMA slab kernel for "_batched_full", the vector-ALU
             // token tile for the plain "_batched" matvec, nothing else

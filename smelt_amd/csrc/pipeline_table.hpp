@@ -71,6 +71,8 @@ enum FamilyId {
     kFamNormScaleAffineMatvec,   // rs x nw xn W S B y | rows cols group           (grid.y = token)
     kFamNormScaleAffineGateUp,   // rs x nw gW gS gB uW uS uB y | rows cols group
     kFamNormScaleAffineBatched,  // rs X nw XN W S B Y batch | rows cols group batch_tile
+    kFamNormAddScaleAffineMatvec,// rs x nw res xn W S B y | rows cols group           (grid.y = token)
+    kFamNormScaleAffineDual,     // rs x nw W1 S1 B1 W2 S2 B2 y1 y2 | rows cols group (grid.y = token)
     kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
     kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile
     kFamCount

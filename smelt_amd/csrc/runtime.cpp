@@ -129,7 +129,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
                               r.family == kFamPlaneBank4 || r.family == kFamPlaneBatched || r.family == kFamBinaryPackedBank || r.family == kFamBinaryPackedBank4 ||
                               r.family == kFamBinaryTwoMatrix;
     const bool norm_scale_matvec = r.family == kFamNormScaleAffineMatvec || r.family == kFamNormScaleAffineGateUp || r.family == kFamNormScaleAffineBatched ||
-                                   r.family == kFamNormScaleAffineQmm || r.family == kFamNormScaleAffineQmmGateUp;
+                                   r.family == kFamNormScaleAffineQmm || r.family == kFamNormScaleAffineQmmGateUp ||
+                                   r.family == kFamNormAddScaleAffineMatvec || r.family == kFamNormScaleAffineDual;
     const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec || norm_scale_matvec;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
@@ -205,6 +206,32 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[2] = cols * 2;
             need[3] = gy * cols * 2; written[3] = true;
             need[7] = gy * rows * 2; written[7] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamNormAddScaleAffineMatvec: {
+            const size_t rows = U(9), cols = U(10), group = U(11);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            affine(5, 6, 7, rows, cols, group);
+            need[0] = gy * 4; align[0] = 4;
+            need[1] = gy * cols * 2; align[1] = 16;
+            need[2] = cols * 2;
+            need[3] = gy * cols * 2;
+            need[4] = gy * cols * 2; written[4] = true;
+            need[8] = gy * rows * 2; written[8] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamNormScaleAffineDual: {
+            const size_t rows = U(11), cols = U(12), group = U(13);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            affine(3, 4, 5, rows, cols, group);
+            affine(6, 7, 8, rows, cols, group);
+            need[0] = gy * 4; align[0] = 4;
+            need[1] = gy * cols * 2; align[1] = 16;
+            need[2] = cols * 2;
+            need[9] = gy * rows * 2; written[9] = true;
+            need[10] = gy * rows * 2; written[10] = true;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
             break;
         }

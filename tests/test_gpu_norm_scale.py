@@ -283,3 +283,57 @@ def test_norm_scale_gate_up_qmm_and_geglu_qmm(ctx, act):
     u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
     epi = so.epilogue_affine_swiglu if act == "swiglu" else so.epilogue_geglu
     gh.check_outputs(fused, fx.from_bits(epi(g, u, dtype), dtype), dtype, f"gate_up {act} qmm", rel_tol=4e-3)
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_norm_add_scale_matvec(ctx, dtype):
+    """norm_add_scale_affine_matvec_c2560_r256_g128_rows4 (lut_matvec.metal:2896-3040): the row the
+    matvec multiplies, and stores, is half(half(norm) + residual)."""
+    rows, cols, group = 256, 2560, 128
+    weights = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=5)
+    x, w, rs = norm_inputs(1, cols, dtype, seed=41)
+    res = fx.to_bits(np.random.default_rng(42).normal(0, 1, (1, cols)).astype(np.float32), dtype)
+    normed = so.norm_scale_input(x[0], rs[0], w, dtype)
+    row_ref = so.elementwise(normed, res[0], dtype)
+    wf = gh.WeightFile()
+    ow, os_, ob = (wf.add(a) for a in weights)
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w); ctx.put(gh.RES_SLOT, res)
+    ctx.alloc(XN_SLOT, cols * 2); ctx.alloc(gh.Y_SLOT, rows * 2)
+    bufs = [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0), (gh.RES_SLOT, 3, 0), (XN_SLOT, 4, 0), (0, 5, ow), (0, 6, os_),
+            (0, 7, ob), (gh.Y_SLOT, 8, 0)]
+    pipe = ctx.pipeline(f"norm_add_scale_affine_matvec_c{cols}_r{rows}_g{group}_rows4" + gh.t_suffix(dtype))
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, [], (rows // 4, 1, 1), (64, 1, 1))) == 1
+    ctx.wait()
+    row = ctx.read(XN_SLOT, np.uint16, cols)
+    y = ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+    assert np.array_equal(row, row_ref)
+    staged = run_affine(ctx, *weights, row.reshape(1, cols), dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    assert np.array_equal(y, staged)
+    ref = so.affine_matvec(*weights, fx.from_bits(row_ref, dtype).reshape(1, cols), rows, cols, group, dtype)
+    gh.check_outputs(y, ref, dtype, "norm_add_scale_affine_matvec")
+
+
+@pytest.mark.parametrize("rows", [512, 1024])
+def test_norm_scale_dual_matvec_per_token(ctx, rows):
+    """norm_scale_fused_dual_affine_matvec_c2560_r{512,1024}_g128_batched (lut_matvec.metal:2030-2150):
+    grid.y is the token, scalePtr[token] its scale; both outputs equal single norm-scale matvecs."""
+    cols, group, dtype, batch = 2560, 128, fx.F16, 3
+    w1 = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=6)
+    w2 = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=7)
+    x, w, rs = norm_inputs(batch, cols, dtype, seed=rows)
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*w1, *w2)]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2); ctx.alloc(gh.AUX_SLOT, batch * rows * 2)
+    bufs = [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0)] + [(0, 3 + i, o) for i, o in enumerate(offs)] + \
+           [(gh.Y_SLOT, 9, 0), (gh.AUX_SLOT, 10, 0)]
+    pipe = ctx.pipeline(f"norm_scale_fused_dual_affine_matvec_c{cols}_r{rows}_g{group}_batched")
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, [], (rows // 8, batch, 1), (64, 1, 1))) == 1
+    ctx.wait()
+    y1 = ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    y2 = ctx.read(gh.AUX_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    s1, _ = run_norm_scale_matvec(ctx, w1, x, w, rs, dtype, f"norm_scale_affine_matvec:{cols}:{group}", [(8, rows)])
+    s2, _ = run_norm_scale_matvec(ctx, w2, x, w, rs, dtype, f"norm_scale_affine_matvec:{cols}:{group}", [(8, rows)])
+    assert np.array_equal(y1, s1) and np.array_equal(y2, s2)
