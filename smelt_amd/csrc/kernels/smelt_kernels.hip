@@ -13,6 +13,8 @@
 
 SMELT_AFFINE_KERNELS(f16, smelt::F16, smelt::F16)
 SMELT_AFFINE_KERNELS(bf16, smelt::BF16, smelt::BF16)
+SMELT_AFFINE_FUSED_NORM(f16, smelt::F16, smelt::F16)
+SMELT_AFFINE_FUSED_NORM(bf16, smelt::BF16, smelt::BF16)
 SMELT_AFFINE_BATCHED(f16, smelt::F16, smelt::F16, 1)
 SMELT_AFFINE_BATCHED(f16, smelt::F16, smelt::F16, 2)
 SMELT_AFFINE_BATCHED(f16, smelt::F16, smelt::F16, 4)

@@ -217,6 +217,8 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         else if (name == "norm_scale_affine_matvec") { out->family = kFamNormScaleAffineMatvec; out->symbol = "smelt_norm_scale_affine_matvec_" + t; out->kinds = "PPPPPPPPUUU"; }
         else if (name == "norm_scale_affine_gate_up_swiglu") { out->family = kFamNormScaleAffineGateUp; out->symbol = "smelt_norm_scale_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPPPUUU"; }
         else if (name == "norm_scale_affine_gate_up_geglu") { out->family = kFamNormScaleAffineGateUp; out->symbol = "smelt_norm_scale_affine_gate_up_geglu_" + t; out->kinds = "PPPPPPPPPPUUU"; }
+        else if (name == "atomic_norm_affine_matvec") { out->family = kFamFusedNormAffineMatvec; out->symbol = "smelt_atomic_norm_affine_matvec_" + t; out->kinds = "PPPPPPPPUFUU"; }
+        else if (name == "atomic_norm_affine_gate_up_swiglu") { out->family = kFamFusedNormAffineGateUp; out->symbol = "smelt_atomic_norm_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPPPUFUU"; }
         else if (name == "affine_bank4_matvec") { out->family = kFamAffineBank4; out->symbol = "smelt_affine_bank4_matvec_" + t; out->kinds = "PPPPPPPPUUUUUU"; }
         else { *why = "no HIP kernel for function-constant pipeline '" + name + "'"; return kResolveUnknown; }
         if (!is_pow2(group) || group < 32 || cols % 32 != 0 || cols == 0) {

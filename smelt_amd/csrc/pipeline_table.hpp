@@ -73,6 +73,8 @@ enum FamilyId {
     kFamNormScaleAffineBatched,  // rs X nw XN W S B Y batch | rows cols group batch_tile
     kFamNormAddScaleAffineMatvec,// rs x nw res xn W S B y | rows cols group           (grid.y = token)
     kFamNormScaleAffineDual,     // rs x nw W1 S1 B1 W2 S2 B2 y1 y2 | rows cols group (grid.y = token)
+    kFamFusedNormAffineMatvec,   // x nw xn W S B y scratch rows eps | cols group
+    kFamFusedNormAffineGateUp,   // x nw gW gS gB uW uS uB y scratch rows eps | cols group
     kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
     kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile
     kFamCount

@@ -130,7 +130,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
                               r.family == kFamBinaryTwoMatrix;
     const bool norm_scale_matvec = r.family == kFamNormScaleAffineMatvec || r.family == kFamNormScaleAffineGateUp || r.family == kFamNormScaleAffineBatched ||
                                    r.family == kFamNormScaleAffineQmm || r.family == kFamNormScaleAffineQmmGateUp ||
-                                   r.family == kFamNormAddScaleAffineMatvec || r.family == kFamNormScaleAffineDual;
+                                   r.family == kFamNormAddScaleAffineMatvec || r.family == kFamNormScaleAffineDual ||
+                                   r.family == kFamFusedNormAffineMatvec || r.family == kFamFusedNormAffineGateUp;
     const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec || norm_scale_matvec;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
@@ -206,6 +207,32 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[2] = cols * 2;
             need[3] = gy * cols * 2; written[3] = true;
             need[7] = gy * rows * 2; written[7] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamFusedNormAffineMatvec: {
+            const size_t rows = U(8), cols = U(10), group = U(11);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (gy != 1) return bad_geom("the fused-norm kernels take one token");
+            affine(3, 4, 5, rows, cols, group);
+            need[0] = cols * 2; align[0] = 16;
+            need[1] = cols * 2;
+            need[2] = cols * 2; written[2] = true;
+            need[6] = rows * 2; written[6] = true;
+            need[7] = 8; align[7] = 4; written[7] = true;
+            L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
+            break;
+        }
+        case kFamFusedNormAffineGateUp: {
+            const size_t rows = U(10), cols = U(12), group = U(13);
+            if (int e = check_affine_shape(rows, cols, group)) return e;
+            if (gy != 1) return bad_geom("the fused-norm kernels take one token");
+            affine(2, 3, 4, rows, cols, group);
+            affine(5, 6, 7, rows, cols, group);
+            need[0] = cols * 2; align[0] = 16;
+            need[1] = cols * 2;
+            need[8] = rows * 2; written[8] = true;
+            need[9] = 8; align[9] = 4; written[9] = true;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
             break;
         }

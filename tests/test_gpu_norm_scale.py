@@ -337,3 +337,47 @@ def test_norm_scale_dual_matvec_per_token(ctx, rows):
     s1, _ = run_norm_scale_matvec(ctx, w1, x, w, rs, dtype, f"norm_scale_affine_matvec:{cols}:{group}", [(8, rows)])
     s2, _ = run_norm_scale_matvec(ctx, w2, x, w, rs, dtype, f"norm_scale_affine_matvec:{cols}:{group}", [(8, rows)])
     assert np.array_equal(y1, s1) and np.array_equal(y2, s2)
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("threads", [64, 256])
+def test_norm_fused_into_matvec_and_gate_up(ctx, dtype, threads):
+    """atomic_norm_affine_matvec / _gate_up_swiglu (fused_norm_matvec.metal:19-297): the norm's scale is
+    computed inside the consumer.  The scale lands in scratch[0] with the ready flag in scratch[1]; the
+    stored row and the products equal the scale-only + norm-scale pair run with that scale."""
+    rows, cols, group = 1024, 2048, 64
+    weights = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=8)
+    uw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=9)
+    x, w, _ = norm_inputs(1, cols, dtype, seed=threads)
+    SCR = 9
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*weights, *uw)]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
+    ctx.alloc(XN_SLOT, cols * 2); ctx.alloc(gh.Y_SLOT, rows * 2); ctx.alloc(SCR, 8)
+    bufs = [(gh.X_SLOT, 0, 0), (NW_SLOT, 1, 0), (XN_SLOT, 2, 0), (0, 3, offs[0]), (0, 4, offs[1]), (0, 5, offs[2]),
+            (gh.Y_SLOT, 6, 0), (SCR, 7, 0)]
+    pipe = ctx.pipeline(f"atomic_norm_affine_matvec:{cols}:{group}" + gh.t_suffix(dtype))
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, [(8, rows), (9, 1e-6)], (rows // 8, 1, 1), (threads, 1, 1))) == 1
+    ctx.wait()
+    scratch = ctx.read(SCR, np.uint32, 2)
+    rs = float(scratch[:1].view(np.float32)[0])
+    assert scratch[1] == 1
+    ref_rs = so.rms_scale(x[0], 1e-6, dtype)
+    assert abs(rs - ref_rs) <= 5e-6 * ref_rs
+    xn = ctx.read(XN_SLOT, np.uint16, cols)
+    assert np.array_equal(xn, so.norm_scale_input(x[0], rs, w, dtype))
+    y = ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+    staged = run_affine(ctx, *weights, xn.reshape(1, cols), dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    assert np.array_equal(y, staged)
+    # gate + up + SwiGLU with the norm inside
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())      # run_affine replaced the image
+    ctx.put(gh.X_SLOT, x); ctx.alloc(gh.Y_SLOT, rows * 2); ctx.alloc(SCR, 8)
+    bufs = [(gh.X_SLOT, 0, 0), (NW_SLOT, 1, 0)] + [(0, 2 + i, o) for i, o in enumerate(offs)] + [(gh.Y_SLOT, 8, 0), (SCR, 9, 0)]
+    pipe = ctx.pipeline(f"atomic_norm_affine_gate_up_swiglu:{cols}:{group}" + gh.t_suffix(dtype))
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, [(10, rows), (11, 1e-6)], (rows // 8, 1, 1), (threads, 1, 1))) == 1
+    ctx.wait()
+    fused = ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+    assert ctx.read(SCR, np.uint32, 2)[1] == 1
+    staged = run_gate_up(ctx, weights, uw, dtype, f"fused_affine_gate_up_swiglu:{cols}:{group}", [(8, rows)], xn.reshape(1, cols))
+    assert np.array_equal(fused, staged)
