@@ -97,6 +97,8 @@ def _declare(l: C.CDLL) -> None:
         "so_bitplane_max_q": (i32, [i32]),
         "so_signed_activation_bitplanes": (None, [vp, i32, i32, i32, vp, vp, vp]),
         "so_swiglu_signed_activation_bitplanes": (None, [vp, vp, i32, i32, i32, vp, vp]),
+        "so_sigmoid_mul_signed_activation_bitplanes": (None, [vp, vp, i32, i32, i32, vp, vp]),
+        "so_sigmoid_mul": (u16, [u16, u16, i32]),
         "so_norm_scale_signed_activation_bitplanes": (None, [f32, vp, vp, i32, i32, i32, vp, vp]),
         "so_signed_bitplane_matvec": (None, [i32, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
         "so_lut_matvec": (None, [vp, vp, vp, i32, i32, i32, vp]),
@@ -412,6 +414,22 @@ def activation_bitplanes(x_bits, planes: int, dtype: int):
     lib().so_signed_activation_bitplanes(_p(x, np.uint16), x.size, planes, dtype, _p(out, np.uint32),
                                          _p(scales, np.uint16), _p(q, np.int32))
     return out, scales, q
+
+
+def sigmoid_mul(a_bits, b_bits, dtype: int) -> np.ndarray:
+    l = lib()
+    return np.array([l.so_sigmoid_mul(int(a), int(b), dtype) for a, b in zip(np.ravel(a_bits), np.ravel(b_bits))],
+                    dtype=np.uint16).reshape(np.shape(a_bits))
+
+
+def sigmoid_mul_activation_bitplanes(a_bits, b_bits, planes: int, dtype: int):
+    a = np.ascontiguousarray(a_bits, np.uint16)
+    b = np.ascontiguousarray(b_bits, np.uint16)
+    out = np.zeros((a.size // 128, planes, 4), np.uint32)
+    scales = np.zeros(a.size // 128, np.uint16)
+    lib().so_sigmoid_mul_signed_activation_bitplanes(_p(a, np.uint16), _p(b, np.uint16), a.size, planes, dtype,
+                                                     _p(out, np.uint32), _p(scales, np.uint16))
+    return out, scales
 
 
 def swiglu_activation_bitplanes(gate_bits, up_bits, planes: int, dtype: int):

@@ -767,6 +767,30 @@ SO_EXPORT void so_swiglu_signed_activation_bitplanes(const uint16_t *gate, const
     }
 }
 
+/* sigmoid_mul_signed_activation_bitplanes_i6_g128 (signed_quant.metal:985-1027): a * sigmoid(b) with
+ * exp, 1 + e, the reciprocal, 1 - tail and the product each materialised in the 16-bit type, then the view. */
+SO_EXPORT uint16_t so_sigmoid_mul(uint16_t a_bits, uint16_t b_bits, int dtype) {
+    float a = widen(a_bits, dtype), b = widen(b_bits, dtype);
+    float e = so_round_through(expf(fabsf(b)), dtype);
+    float denom = so_round_through(1.0f + e, dtype);
+    float tail = so_round_through(1.0f / denom, dtype);
+    float sig = b < 0.0f ? tail : so_round_through(1.0f - tail, dtype);
+    return narrow(a * sig, dtype);
+}
+
+SO_EXPORT void so_sigmoid_mul_signed_activation_bitplanes(const uint16_t *a, const uint16_t *b, int cols,
+                                                          int planes, int dtype, uint32_t *out_planes,
+                                                          uint16_t *out_scales) {
+    int groups = cols / 128;
+    for (int g = 0; g < groups; ++g) {
+        float v[128];
+        int q[128];
+        for (int i = 0; i < 128; ++i) v[i] = widen(so_sigmoid_mul(a[g * 128 + i], b[g * 128 + i], dtype), dtype);
+        out_scales[g] = bitplane_quantize_group(v, planes, dtype, q);
+        bitplane_pack_group(q, planes, out_planes + (size_t)g * planes * 4);
+    }
+}
+
 /* norm_scale_signed_activation_bitplanes_i{2..6}_g128 (:1175-1223): rms_norm_1pw's two-step value
  * half(x * rs) * half(1 + w) from a precomputed scale, then the view. */
 SO_EXPORT void so_norm_scale_signed_activation_bitplanes(float rs, const uint16_t *x, const uint16_t *w,

@@ -1,7 +1,7 @@
 // Producers of signed activation views (signed_quant.metal:746-1298): every group of 128
 // activations becomes a 16-bit scale (largest magnitude / largest integer) and sign-magnitude
 // integers stored as bit planes, [group][plane][4 words], word w bit l = value 32 w + l.
-//   values   plain input, the staged SwiGLU of (gate, up), or rms_norm_1pw's two-step value
+//   values   plain input, the staged SwiGLU of (gate, up), a * sigmoid(b), or rms_norm_1pw's two-step value
 //            half(x * rs) * half(1 + w) from a precomputed scale
 //   scale    i2 and i3 views quantise with the unrounded fp32 scale, i4..i6 with the stored one
 //   integer  round-half-away(clamp(value / scale, -max, +max)), max = 1 (i2) or 2^(planes-1) - 1
@@ -11,7 +11,7 @@
 
 namespace smelt {
 
-enum BitplaneSource : int { kPlaneSrcPlain = 0, kPlaneSrcSwiglu = 1, kPlaneSrcNormScale = 2 };
+enum BitplaneSource : int { kPlaneSrcPlain = 0, kPlaneSrcSwiglu = 1, kPlaneSrcNormScale = 2, kPlaneSrcSigmoidMul = 3 };
 
 template <class ActT, int SRC>
 __device__ __forceinline__ float bitplane_value(const float* norm_scale, const uint16_t* a, const uint16_t* b, size_t i) {
@@ -24,6 +24,13 @@ __device__ __forceinline__ float bitplane_value(const float* norm_scale, const u
         const float tail = rt(1.0f / rt(1.0f + e));
         const float sig = g < 0.0f ? tail : rt(1.0f - tail);
         return rt(rt(g * sig) * u);
+    } else if constexpr (SRC == kPlaneSrcSigmoidMul) {
+        // a * sigmoid(b) with the sigmoid's every step in the 16-bit type (signed_quant.metal:1000-1006)
+        auto rt = [](float v) { return ActT::widen(ActT::narrow(v)); };
+        const float x = ActT::widen(a[i]), gate = ActT::widen(b[i]);
+        const float tail = rt(1.0f / rt(1.0f + rt(expf(fabsf(gate)))));
+        const float sig = gate < 0.0f ? tail : rt(1.0f - tail);
+        return rt(x * sig);
     } else {
         const float normalized = ActT::widen(ActT::narrow(ActT::widen(a[i]) * norm_scale[0]));
         const float direct = ActT::widen(ActT::narrow(1.0f + ActT::widen(b[i])));
@@ -41,7 +48,7 @@ __device__ __forceinline__ void activation_bitplanes_body(const float* norm_scal
     const uint32_t waves = (blockDim.x + 63u) / 64u;
     const uint32_t batch = blockIdx.y;
     a += (size_t)batch * cols;
-    if (SRC == kPlaneSrcSwiglu) b += (size_t)batch * cols;           // the norm weight is shared by every token
+    if (SRC == kPlaneSrcSwiglu || SRC == kPlaneSrcSigmoidMul) b += (size_t)batch * cols;           // the norm weight is shared by every token
     planes += (size_t)batch * groups * nplanes * 4;
     scales += (size_t)batch * groups;
     const int max_q = nplanes == 2 ? 1 : (1 << (nplanes - 1)) - 1;
@@ -95,6 +102,12 @@ __device__ __forceinline__ void activation_bitplanes_body(const float* norm_scal
         uint32_t cols, uint32_t nplanes) {                                                         \
         smelt::activation_bitplanes_body<ACT, smelt::kPlaneSrcSwiglu>(nullptr, gate, up, planes,   \
                                                                       scales, cols, nplanes);      \
+    }                                                                                              \
+    SMELT_PLANE_KERNEL void smelt_sigmoid_mul_signed_activation_bitplanes_##T(                     \
+        const uint16_t* a, const uint16_t* b, uint32_t* planes, uint16_t* scales, uint32_t cols,   \
+        uint32_t nplanes) {                                                                        \
+        smelt::activation_bitplanes_body<ACT, smelt::kPlaneSrcSigmoidMul>(nullptr, a, b, planes,   \
+                                                                          scales, cols, nplanes);  \
     }                                                                                              \
     SMELT_PLANE_KERNEL void smelt_norm_scale_signed_activation_bitplanes_##T(                      \
         const float* norm_scale, const uint16_t* x, const uint16_t* w, uint32_t* planes,           \

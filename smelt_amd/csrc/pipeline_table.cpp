@@ -517,6 +517,12 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->kinds = "PPPUU"; out->appended = {n};
             return kResolveOk;
         }
+        if (entry == "sigmoid_mul_signed_activation_bitplanes_i6_g128") {
+            // same bindings as the SwiGLU producer: a b planes scales cols
+            out->family = kFamSwigluPlanes; out->symbol = "smelt_sigmoid_mul_signed_activation_bitplanes_" + t;
+            out->kinds = "PPPPUU"; out->appended = {6u};
+            return kResolveOk;
+        }
         if (entry == "swiglu_signed_activation_bitplanes_i5_g128") {
             out->family = kFamSwigluPlanes; out->symbol = "smelt_swiglu_signed_activation_bitplanes_" + t;
             out->kinds = "PPPPUU"; out->appended = {5u};

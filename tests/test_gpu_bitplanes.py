@@ -75,6 +75,18 @@ def test_fused_producers(env):
     assert np.array_equal(ctx.read(PL, np.uint32, groups * 20), fused_pl) and np.array_equal(ctx.read(AS, np.uint16, groups), fused_sc)
     ref_pl, ref_sc = so.swiglu_activation_bitplanes(g, u, 5, odt)     # exp may differ in its last bit
     assert np.mean(fused_pl == ref_pl.reshape(-1)) > 0.98 and np.mean(fused_sc == ref_sc) > 0.9
+    # sigmoid-mul producer (i6): against the plain producer run on the oracle's staged values
+    ctx.alloc(PL, groups * 6 * 16)
+    rec = rt.make_record(ctx.pipeline("sigmoid_mul_signed_activation_bitplanes_i6_g128"), [(X, 0, 0), (X2, 1, 0), (PL, 2, 0), (AS, 3, 0)],
+                         [(4, cols)], (groups, 1, 1), (32, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    sm_pl, sm_sc = ctx.read(PL, np.uint32, groups * 24), ctx.read(AS, np.uint16, groups)
+    ref_pl, ref_sc = so.sigmoid_mul_activation_bitplanes(g, u, 6, odt)
+    assert np.mean(sm_pl == ref_pl.reshape(-1)) > 0.98 and np.mean(sm_sc == ref_sc) > 0.9
+    ctx.put(Y, so.sigmoid_mul(g, u, odt))
+    rec = rt.make_record(ctx.pipeline("signed_activation_bitplanes_i6_g128"), [(Y, 0, 0), (PL, 1, 0), (AS, 2, 0)], [(3, cols)], (groups, 1, 1), (32, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    assert np.mean(ctx.read(PL, np.uint32, groups * 24) == sm_pl) > 0.98
     # norm-scale producer: the scale is an input, everything after it is exact
     x, w = bits(rng.normal(0, 1, cols).astype(np.float32), dtype), bits(rng.normal(0, 0.2, cols).astype(np.float32), dtype)
     rs = so.rms_scale(x, 1e-6, odt)

@@ -104,3 +104,28 @@ def test_fused_producers_equal_their_staged_forms():
         staged = so.activation_bitplanes(so.rms_norm_1pw(x, w, 1e-6, so.F16, True), planes, so.F16)
         fused = so.norm_scale_activation_bitplanes(rs, x, w, planes, so.F16)
         assert np.array_equal(staged[0], fused[0]) and np.array_equal(staged[1], fused[1])
+
+
+def test_sigmoid_mul_producer_closed_forms_and_numpy_float16():
+    """sigmoid_mul_signed_activation_bitplanes_i6_g128 (signed_quant.metal:985-1027): a * sigmoid(b)
+    with the sigmoid staged in the 16-bit type, then the i6 view of those values."""
+    h = lambda v: so.narrow(np.asarray(v, np.float32), so.F16)
+    val = lambda a, b: so.widen(so.sigmoid_mul(h(a), h(b), so.F16), so.F16)
+    assert val([3.0], [0.0])[0] == 1.5                                     # sigmoid(0) = 1/2
+    assert val([3.0], [12.0])[0] == 3.0 and abs(val([3.0], [-12.0])[0]) < 1e-4   # saturates to 1 and ~0
+    assert val([-2.0], [1.0])[0] == -val([2.0], [1.0])[0]                  # odd in a
+    rng = fx.rng_for(113, 0)
+    a, b = h(rng.normal(0, 2, 4096)), h(rng.normal(0, 3, 4096))
+    af, bf = a.view(np.float16), b.view(np.float16)
+    one = np.float16(1.0)
+    tail = one / (one + np.exp(np.abs(bf)))                                 # float16 at every step
+    sig = np.where(bf < 0, tail, one - tail).astype(np.float16)
+    ref = (af * sig).astype(np.float16)
+    got = so.sigmoid_mul(a, b, so.F16).view(np.float16)
+    ulp = np.spacing(np.abs(ref)).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - ref.astype(np.float64)) <= ulp)   # exp may differ in its last bit
+    assert np.mean(got.view(np.uint16) == ref.view(np.uint16)) > 0.995
+    # the fused producer is the plain i6 producer applied to those values
+    staged = so.activation_bitplanes(so.sigmoid_mul(a, b, so.F16), 6, so.F16)
+    fused = so.sigmoid_mul_activation_bitplanes(a, b, 6, so.F16)
+    assert np.array_equal(staged[0], fused[0]) and np.array_equal(staged[1], fused[1])
