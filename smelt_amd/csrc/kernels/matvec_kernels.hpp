@@ -488,6 +488,19 @@ using u32 = uint32_t;
                                                packed_row_stride<FmtU4>(cols, group), group, lo,  \
                                                hi, epi);                                          \
     }                                                                                             \
+    SMELT_KERNEL void smelt_affine_gate_up_geglu_batched_mb##MBV##_##T(                           \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* X, u16* Y, u32 batch, u32 rows, u32 cols, u32 group, u32 batch_tile) {         \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiGeglu<ACT> epi{{}, Y, (int)rows};                                                      \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        matvec_body<FmtU4, ACT, SC, 2, MBV, 2>(mats, X, rows, cols,                               \
+                                               packed_row_stride<FmtU4>(cols, group), group, lo,  \
+                                               hi, epi);                                          \
+    }                                                                                             \
     SMELT_KERNEL void smelt_affine_gate_up_swiglu_batched_mb##MBV##_##T(                          \
         const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
         const u16* X, u16* Y, u32 batch, u32 rows, u32 cols, u32 group, u32 batch_tile) {         \

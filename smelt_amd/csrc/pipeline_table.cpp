@@ -263,7 +263,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         }
         // the norm-scale dual kernel's "_batched" form takes its token from grid.y, like the single-token kernels
         const bool m1 = suffix.empty() || suffix == "_rows4" || suffix == "_rows8" || suffix == "_rows4_sg1" ||
-                        (a.m1 == kFamNormScaleAffineDual && suffix == "_batched");
+                        ((a.m1 == kFamNormScaleAffineDual || a.m1 == kFamAffineDual) && suffix == "_batched");
         if (want_mfma && mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 2, lds_limit) == 0) {
             *why = "matrix-core matvec needs group 64, cols % 256 == 0 and at least 8M weights: '" + entry + "'";
             return kResolveMalformed;
@@ -277,6 +277,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         else if (suffix == "_batched_ext_b5" || suffix == "_batched_sg4_bt5") bt = 5;
         else if (suffix == "_batched_full") { bt = 16; full = true; }
         else if (starts_with(suffix, "_batched_full_b") && parse_uint(suffix.substr(15), &bt) && bt >= 1 && bt <= 4096) { full = true; }
+        else if (suffix == "_batched_bt4_sg4" && strstr(a.prefix, "geglu")) bt = 4;
         else if (!m1) { *why = "unknown kernel variant '" + suffix + "' in '" + entry + "'"; return kResolveUnknown; }
 
         if (a.m1 == kFamAffineArgmax) {
@@ -329,6 +330,17 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         if (a.m1 == kFamNormAddScaleAffineMatvec || a.m1 == kFamNormScaleAffineDual) {
             *why = "no batched HIP kernel for '" + entry + "'";
             return kResolveUnknown;
+        }
+        if (a.m1 == kFamAffineGateUp && geglu && !want_mfma && (suffix == "_batched" || suffix == "_batched_bt4_sg4")) {
+            // small-batch GeGLU (lut_matvec.metal:8342-8364, 8752-8753): token tiles of 3 and 4
+            bt = suffix == "_batched" ? 3 : 4;
+            const uint32_t mbv = pick_mb(kCodesU4, row_stride, 4, lds_limit);
+            out->lds_variant = mbv;
+            out->family = kFamAffineGateUpBatched;
+            out->symbol = "smelt_affine_gate_up_geglu_batched_mb" + std::to_string(mbv) + "_" + t;
+            out->kinds = "PPPPPPPPUUUUU";
+            out->appended = {rows, cols, group, bt};
+            return kResolveOk;
         }
         if (a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp || geglu) {
             // prologue and GeGLU forms: the MFMA slab kernel for "_batched_full", the vector-ALU

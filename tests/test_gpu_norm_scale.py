@@ -381,3 +381,37 @@ def test_norm_fused_into_matvec_and_gate_up(ctx, dtype, threads):
     assert ctx.read(SCR, np.uint32, 2)[1] == 1
     staged = run_gate_up(ctx, weights, uw, dtype, f"fused_affine_gate_up_swiglu:{cols}:{group}", [(8, rows)], xn.reshape(1, cols))
     assert np.array_equal(fused, staged)
+
+
+def test_dual_matvec_per_token_and_small_batch_geglu(ctx):
+    """fused_dual_affine_matvec_*_batched (lut_matvec.metal:7570-7591: grid.y = token) and the
+    small-batch GeGLU kernels (:8342-8364, token tiles of 3 and 4): per-token results are the
+    single-token kernels' bits."""
+    rows, cols, group, dtype, batch = 512, 1024, 64, fx.F16, 5
+    w1 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=10)
+    w2 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=11)
+    x = fx.synth_activation(batch, cols, dtype, config=1, tensor=72)
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*w1, *w2)]
+    image = wf.image()
+    ctx.upload_weights(gh.WEIGHTS_SLOT, image)
+    ctx.put(gh.X_SLOT, x); ctx.alloc(gh.Y_SLOT, batch * rows * 2); ctx.alloc(gh.AUX_SLOT, batch * rows * 2)
+    bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0), (gh.AUX_SLOT, 8, 0)]
+    pipe = ctx.pipeline(f"fused_dual_affine_matvec_c{cols}_r{rows}_g{group}_batched")
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, [], (rows // 8, batch, 1), (64, 1, 1))) == 1
+    ctx.wait()
+    y1 = ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    y2 = ctx.read(gh.AUX_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    s1 = run_affine(ctx, *w1, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    s2 = run_affine(ctx, *w2, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    assert np.array_equal(y1, s1) and np.array_equal(y2, s2)
+    single = np.stack([run_gate_up(ctx, w1, w2, dtype, f"fused_affine_gate_up_geglu:{cols}:{group}", [(8, rows)], x[b:b + 1])[0]
+                       for b in range(batch)])
+    for suffix, bt in (("_batched", 3), ("_batched_bt4_sg4", 4)):
+        ctx.upload_weights(gh.WEIGHTS_SLOT, image)
+        ctx.put(gh.X_SLOT, x); ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
+        pipe = ctx.pipeline(f"fused_affine_gate_up_geglu_c{cols}_r{rows}_g{group}{suffix}")
+        assert ctx.encode_decode(rt.make_record(pipe, bufs, [(8, batch)], (rows // 8, (batch + bt - 1) // bt, 1), (256, 1, 1))) == 1
+        ctx.wait()
+        assert np.array_equal(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), single), suffix
