@@ -88,6 +88,9 @@ def _declare(l: C.CDLL) -> None:
         "so_epilogue_residual_add": (u16, [f32, u16, i32]),
         "so_epilogue_affine_swiglu": (u16, [f32, f32, i32]),
         "so_epilogue_geglu": (u16, [f32, f32, i32]),
+        "so_rms_norm_1pw_add_scalar": (None, [vp, vp, vp, u16, i32, f32, i32, vp]),
+        "so_rms_norm_1pw_from_fp32": (None, [vp, vp, i32, f32, i32, vp]),
+        "so_rms_norm_gated": (None, [vp, vp, vp, i32, i32, f32, i32, vp]),
         "so_norm_scale_input": (None, [vp, f32, vp, i32, i32, vp]),
         "so_epilogue_signed_swiglu": (u16, [u16, u16, i32]),
         "so_rms_scale": (f32, [vp, i32, f32, i32]),
@@ -374,13 +377,40 @@ def rms_scale(x_bits: np.ndarray, eps: float, dtype: int) -> float:
     return float(lib().so_rms_scale(_p(x, np.uint16), x.size, eps, dtype))
 
 
-def rms_norm_1pw(x_bits, w_bits, eps: float, dtype: int, two_step: bool, residual_bits=None) -> np.ndarray:
+def rms_norm_1pw(x_bits, w_bits, eps: float, dtype: int, two_step, residual_bits=None) -> np.ndarray:
+    """two_step: False/0 = x * (rs * (1 + w)), True/1 = half(1 + w) * half(x * rs), 2 = (x * rs) * (1 + w)."""
     x = np.ascontiguousarray(x_bits, np.uint16)
     w = np.ascontiguousarray(w_bits, np.uint16)
     out = np.zeros(x.size, np.uint16)
     res = None if residual_bits is None else np.ascontiguousarray(residual_bits, np.uint16)
     lib().so_rms_norm_1pw(_p(x, np.uint16), _p(w, np.uint16), None if res is None else _p(res, np.uint16),
                           x.size, eps, dtype, int(two_step), _p(out, np.uint16))
+    return out
+
+
+def rms_norm_1pw_add_scalar(x_bits, w_bits, residual_bits, scalar_bits: int, eps: float, dtype: int) -> np.ndarray:
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    out = np.zeros(x.size, np.uint16)
+    lib().so_rms_norm_1pw_add_scalar(_p(x, np.uint16), _p(np.ascontiguousarray(w_bits, np.uint16), np.uint16),
+                                     _p(np.ascontiguousarray(residual_bits, np.uint16), np.uint16), int(scalar_bits),
+                                     x.size, eps, dtype, _p(out, np.uint16))
+    return out
+
+
+def rms_norm_1pw_from_fp32(x_f32, w_bits, eps: float, dtype: int) -> np.ndarray:
+    x = np.ascontiguousarray(x_f32, np.float32)
+    out = np.zeros(x.size, np.uint16)
+    lib().so_rms_norm_1pw_from_fp32(_p(x, np.float32), _p(np.ascontiguousarray(w_bits, np.uint16), np.uint16), x.size,
+                                    eps, dtype, _p(out, np.uint16))
+    return out
+
+
+def rms_norm_gated(x_bits, gate_bits, w_bits, heads: int, head_dim: int, eps: float, dtype: int) -> np.ndarray:
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    out = np.zeros(x.size, np.uint16)
+    lib().so_rms_norm_gated(_p(x, np.uint16), _p(np.ascontiguousarray(gate_bits, np.uint16), np.uint16),
+                            _p(np.ascontiguousarray(w_bits, np.uint16), np.uint16), heads, head_dim, eps, dtype,
+                            _p(out, np.uint16))
     return out
 
 

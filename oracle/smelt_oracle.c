@@ -673,16 +673,58 @@ SO_EXPORT void so_rms_norm_1pw(const uint16_t *x, const uint16_t *w, const uint1
     for (int i = 0; i < n; ++i) {
         float v = widen(x[i], dtype), wt = widen(w[i], dtype);
         uint16_t y;
-        if (two_step) {
+        if (two_step == 1) {
             float normalized = so_round_through(v * rs, dtype);
             float direct = so_round_through(1.0f + wt, dtype);
             y = narrow(direct * normalized, dtype);
+        } else if (two_step == 2) {   /* the d256 kernels: x * rs * (1 + w), left to right (norms.metal:213) */
+            float scaled = v * rs;
+            y = narrow(scaled * (1.0f + wt), dtype);
         } else {
             float scale = rs * (1.0f + wt);
             y = narrow(v * scale, dtype);
         }
         if (residual) y = narrow(widen(y, dtype) + widen(residual[i], dtype), dtype);
         out[i] = y;
+    }
+}
+
+/* rms_norm_1pw_d256_add_scalar_weight (norms.metal:218-260): the d256 norm, + residual, * scalar[0],
+ * each step rounded to the 16-bit type. */
+SO_EXPORT void so_rms_norm_1pw_add_scalar(const uint16_t *x, const uint16_t *w, const uint16_t *residual,
+                                          uint16_t scalar, int n, float eps, int dtype, uint16_t *out) {
+    so_rms_norm_1pw(x, w, residual, n, eps, dtype, 2, out);
+    for (int i = 0; i < n; ++i) out[i] = narrow(widen(out[i], dtype) * widen(scalar, dtype), dtype);
+}
+
+/* rms_norm_1pw_from_fp32 (norms_fp32.metal:50-88): fp32 input, running fp32 sum of squares,
+ * half(clamp(x * rs * (1 + w), +-65504)). */
+SO_EXPORT void so_rms_norm_1pw_from_fp32(const float *x, const uint16_t *w, int n, float eps, int dtype,
+                                         uint16_t *out) {
+    float sum = 0.0f;
+    for (int i = 0; i < n; ++i) sum += x[i] * x[i];
+    float rs = 1.0f / sqrtf(sum / (float)n + eps);
+    for (int i = 0; i < n; ++i) {
+        float scaled = x[i] * rs;
+        float v = scaled * (1.0f + widen(w[i], dtype));
+        v = v < -65504.0f ? -65504.0f : (v > 65504.0f ? 65504.0f : v);
+        out[i] = narrow(v, dtype);
+    }
+}
+
+/* rms_norm_gated (norms.metal:1093-1153): per head half(w * (x * rs) * silu(gate)), SiLU in fp32. */
+SO_EXPORT void so_rms_norm_gated(const uint16_t *x, const uint16_t *gate, const uint16_t *w, int heads,
+                                 int head_dim, float eps, int dtype, uint16_t *out) {
+    for (int h = 0; h < heads; ++h) {
+        const uint16_t *xr = x + (size_t)h * head_dim, *gr = gate + (size_t)h * head_dim;
+        float rs = so_rms_scale(xr, head_dim, eps, dtype);
+        for (int i = 0; i < head_dim; ++i) {
+            float g = widen(gr[i], dtype);
+            float silu = g / (1.0f + expf(-g));
+            float normalized = widen(xr[i], dtype) * rs;
+            float weighted = widen(w[i], dtype) * normalized;
+            out[(size_t)h * head_dim + i] = narrow(weighted * silu, dtype);
+        }
     }
 }
 

@@ -53,12 +53,17 @@ __device__ __forceinline__ float inv_rms(float sum_squares, uint32_t dim, float 
     return 1.0f / __builtin_sqrtf(sum_squares / (float)dim + eps);
 }
 
-// two_step: half(1 + w) * half(x * rs), both factors materialised in the 16-bit type first (the
-// generic rms_norm_1pw, norms.metal:54-62); otherwise half(x * (rs * (1 + w))) (the fixed-dimension
-// kernels, norms.metal:164-170).  residual != nullptr adds it to the rounded norm in the 16-bit type.
+// mode 1 (two-step): half(1 + w) * half(x * rs), both factors materialised in the 16-bit type first (the
+// generic rms_norm_1pw, norms.metal:54-62); mode 0: half(x * (rs * (1 + w))) (the vectorised
+// fixed-dimension kernels, norms.metal:164-170); mode 2: half((x * rs) * (1 + w)), products left to
+// right (the d256 kernels, norms.metal:213, 256).  residual != nullptr adds it to the rounded norm
+// in the 16-bit type; scalar != nullptr then multiplies the rounded sum by scalar[0] (norms.metal:257-259).
+enum NormMode : uint32_t { kNormScaleFirst = 0, kNormTwoStep = 1, kNormLeftToRight = 2 };
+
 template <class ActT>
 __device__ __forceinline__ void rms_norm_1pw_row(const uint16_t* x, const uint16_t* weight, const uint16_t* residual,
-                                                 uint16_t* out, uint32_t dim, float eps, bool two_step) {
+                                                 uint16_t* out, uint32_t dim, float eps, uint32_t mode,
+                                                 const uint16_t* scalar = nullptr) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float* scratch = reinterpret_cast<float*>(smem);
     uint16_t* row = reinterpret_cast<uint16_t*>(smem + 64);
@@ -67,15 +72,64 @@ __device__ __forceinline__ void rms_norm_1pw_row(const uint16_t* x, const uint16
         const float v = ActT::widen(row[i]);
         const float w = ActT::widen(weight[i]);
         uint16_t y;
-        if (two_step) {
+        if (mode == kNormTwoStep) {
             const float normalized = ActT::widen(ActT::narrow(v * rs));
             const float direct = ActT::widen(ActT::narrow(1.0f + w));
             y = ActT::narrow(direct * normalized);
+        } else if (mode == kNormLeftToRight) {
+            y = norm_scale_value<ActT>(row[i], rs, weight[i]);
         } else {
             y = ActT::narrow(v * (rs * (1.0f + w)));
         }
         if (residual) y = ActT::narrow(ActT::widen(y) + ActT::widen(residual[i]));
+        if (scalar) y = ActT::narrow(ActT::widen(y) * ActT::widen(scalar[0]));
         out[i] = y;
+    }
+}
+
+// rms_norm_1pw_from_fp32 (norms_fp32.metal:50-88): fp32 row in, 16-bit row out, the product clamped
+// to the fp16 range before it is narrowed.
+template <class ActT>
+__device__ __forceinline__ void rms_norm_from_fp32_row(const float* x, const uint16_t* weight, uint16_t* out,
+                                                       uint32_t dim, float eps) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float* scratch = reinterpret_cast<float*>(smem);
+    float sum = 0.0f;
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) sum = __builtin_fmaf(x[i], x[i], sum);
+    const float rs = inv_rms(block_sum(sum, scratch), dim, eps);
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
+        float v;
+        {
+#pragma clang fp contract(off)
+            const float scaled = x[i] * rs;
+            v = scaled * (1.0f + ActT::widen(weight[i]));
+        }
+        out[i] = ActT::narrow(__builtin_fminf(__builtin_fmaxf(v, -65504.0f), 65504.0f));
+    }
+}
+
+// rms_norm_gated (norms.metal:1093-1153): per head, half(w * (x * rs) * silu(gate)) with the SiLU in fp32.
+template <class ActT>
+__device__ __forceinline__ void rms_norm_gated_row(const uint16_t* x, const uint16_t* gate, const uint16_t* weight,
+                                                   uint16_t* out, uint32_t dim, float eps) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float* scratch = reinterpret_cast<float*>(smem);
+    float sum = 0.0f;
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
+        const float v = ActT::widen(x[i]);
+        sum = __builtin_fmaf(v, v, sum);
+    }
+    const float rs = inv_rms(block_sum(sum, scratch), dim, eps);
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
+        const float g = ActT::widen(gate[i]);
+        const float silu = g / (1.0f + expf(-g));
+        float v;
+        {
+#pragma clang fp contract(off)
+            const float normalized = ActT::widen(x[i]) * rs;
+            v = (ActT::widen(weight[i]) * normalized) * silu;
+        }
+        out[i] = ActT::narrow(v);
     }
 }
 
@@ -89,14 +143,31 @@ __device__ __forceinline__ void rms_norm_1pw_row(const uint16_t* x, const uint16
                                                    uint16_t* y, uint32_t dim, float eps,          \
                                                    uint32_t two_step) {                           \
         const size_t at = (size_t)blockIdx.x * dim;                                               \
-        smelt::rms_norm_1pw_row<ACT>(x + at, w, nullptr, y + at, dim, eps, two_step != 0);        \
+        smelt::rms_norm_1pw_row<ACT>(x + at, w, nullptr, y + at, dim, eps, two_step);        \
     }                                                                                             \
     SMELT_LAYER_KERNEL void smelt_rms_norm_1pw_add_##T(const uint16_t* x, const uint16_t* w,      \
                                                        const uint16_t* res, uint16_t* y,          \
                                                        uint32_t dim, float eps,                   \
                                                        uint32_t two_step) {                       \
         const size_t at = (size_t)blockIdx.x * dim;                                               \
-        smelt::rms_norm_1pw_row<ACT>(x + at, w, res + at, y + at, dim, eps, two_step != 0);       \
+        smelt::rms_norm_1pw_row<ACT>(x + at, w, res + at, y + at, dim, eps, two_step);       \
+    }                                                                                             \
+    SMELT_LAYER_KERNEL void smelt_rms_norm_1pw_add_scalar_##T(                                    \
+        const uint16_t* x, const uint16_t* w, const uint16_t* res, const uint16_t* scalar,        \
+        uint16_t* y, uint32_t dim, float eps, uint32_t mode) {                                    \
+        const size_t at = (size_t)blockIdx.x * dim;                                               \
+        smelt::rms_norm_1pw_row<ACT>(x + at, w, res + at, y + at, dim, eps, mode, scalar);        \
+    }                                                                                             \
+    SMELT_LAYER_KERNEL void smelt_rms_norm_1pw_from_fp32_##T(const float* x, const uint16_t* w,   \
+                                                             uint16_t* y, uint32_t dim, float eps) { \
+        const size_t at = (size_t)blockIdx.x * dim;                                               \
+        smelt::rms_norm_from_fp32_row<ACT>(x + at, w, y + at, dim, eps);                          \
+    }                                                                                             \
+    SMELT_LAYER_KERNEL void smelt_rms_norm_gated_##T(const uint16_t* x, const uint16_t* gate,     \
+                                                     const uint16_t* w, uint16_t* y,              \
+                                                     uint32_t head_dim, float eps) {              \
+        const size_t at = (size_t)blockIdx.x * head_dim;                                          \
+        smelt::rms_norm_gated_row<ACT>(x + at, gate + at, w, y + at, head_dim, eps);              \
     }                                                                                             \
     SMELT_LAYER_KERNEL void smelt_rms_norm_scale_only_##T(const uint16_t* x, float* scale,        \
                                                           uint32_t dim, float eps) {              \

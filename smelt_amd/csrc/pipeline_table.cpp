@@ -472,6 +472,19 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             if (s.size() >= n && s.compare(s.size() - n, n, suffix) == 0) { s.resize(s.size() - n); return true; }
             return false;
         };
+        if (entry == "rms_norm_1pw_d256_add_scalar_weight") {
+            out->family = kFamRmsNormAddScalar; out->symbol = "smelt_rms_norm_1pw_add_scalar_" + t;
+            out->kinds = "PPPPPUUU"; out->appended = {256u, eps_bits(1e-6f), 2u};
+            return kResolveOk;
+        }
+        if (entry == "rms_norm_1pw_from_fp32" || entry == "rms_norm_1pw_from_fp32_batched") {
+            out->family = kFamRmsNormFromFp32; out->symbol = "smelt_rms_norm_1pw_from_fp32_" + t; out->kinds = "PPPUF";
+            return kResolveOk;
+        }
+        if (entry == "rms_norm_gated") {
+            out->family = kFamRmsNormGated; out->symbol = "smelt_rms_norm_gated_" + t; out->kinds = "PPPPUF";
+            return kResolveOk;
+        }
         if (starts_with(entry, "rms_norm_1pw")) {
             std::string rest = entry.substr(12);
             strip(rest, "_batched");            // batch rows are the grid width either way
@@ -483,7 +496,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
                 out->family = add ? kFamRmsNormAdd : kFamRmsNorm;
                 out->symbol = std::string(add ? "smelt_rms_norm_1pw_add_" : "smelt_rms_norm_1pw_") + t;
                 if (dim == 0) { out->kinds = "PPPUFU"; out->appended = {1u}; }                  // dim, eps from the record
-                else { out->kinds = add ? "PPPPUUU" : "PPPUUU"; out->appended = {dim, eps_bits(1e-6f), 0u}; }
+                else { out->kinds = add ? "PPPPUUU" : "PPPUUU"; out->appended = {dim, eps_bits(1e-6f), dim == 256 ? 2u : 0u}; }   // d256: products left to right
                 return kResolveOk;
             }
         }

@@ -75,6 +75,9 @@ enum FamilyId {
     kFamNormScaleAffineDual,     // rs x nw W1 S1 B1 W2 S2 B2 y1 y2 | rows cols group (grid.y = token)
     kFamFusedNormAffineMatvec,   // x nw xn W S B y scratch rows eps | cols group
     kFamFusedNormAffineGateUp,   // x nw gW gS gB uW uS uB y scratch rows eps | cols group
+    kFamRmsNormAddScalar,        // x w res scalar y | dim eps mode             (grid.x = token row)
+    kFamRmsNormFromFp32,         // x(fp32) w y dim eps
+    kFamRmsNormGated,            // x gate w y head_dim eps                      (grid.x = head)
     kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
     kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile
     kFamCount

@@ -538,6 +538,25 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             L.lds = 64 + dim * 2;
             break;
         }
+        case kFamRmsNormAddScalar:
+        case kFamRmsNormFromFp32:
+        case kFamRmsNormGated: {
+            const size_t first_u = r.family == kFamRmsNormAddScalar ? 5 : (r.family == kFamRmsNormFromFp32 ? 3 : 4);
+            const size_t dim = U(first_u), tokens = L.grid[0];
+            if (dim == 0) return bad_geom("dim must be positive");
+            if (L.block[0] % 64 != 0 || L.block[1] != 1 || L.block[2] != 1 || L.grid[1] != 1 || L.grid[2] != 1)
+                return bad_geom("norm kernels run whole waves in a 1-D launch, one workgroup per row");
+            const size_t row = tokens * dim * 2;
+            if (r.family == kFamRmsNormAddScalar) {
+                need[0] = row; need[1] = dim * 2; need[2] = row; need[3] = 2; need[4] = row; written[4] = true;
+            } else if (r.family == kFamRmsNormFromFp32) {
+                need[0] = tokens * dim * 4; align[0] = 4; need[1] = dim * 2; need[2] = row; written[2] = true;
+            } else {
+                need[0] = row; need[1] = row; need[2] = dim * 2; need[3] = row; written[3] = true;
+            }
+            L.lds = 64 + dim * 2;
+            break;
+        }
         case kFamElementwise:
         case kFamCopy16: {
             const size_t ci = r.family == kFamCopy16 ? 2 : 3;

@@ -264,3 +264,55 @@ def test_whole_layer_record_list_eager_and_graph():
         ctx.graph_destroy(graph)
     finally:
         ctx.close()
+
+
+def test_norm_variants(env):
+    """rms_norm_1pw_d256_add_scalar_weight (norms.metal:218-260), rms_norm_1pw_from_fp32[_batched]
+    (norms_fp32.metal:50-130) and rms_norm_gated (norms.metal:1093-1153) against the oracle: last-place
+    agreement (the sum of squares is formed in another order), at least 97 % of the elements identical."""
+    ctx, dtype, odt = env
+    rng = fx.rng_for(97, 3)
+    x = bits(rng.normal(0, 1.5, 256).astype(np.float32), dtype)
+    w = bits(rng.normal(0, 0.2, 256).astype(np.float32), dtype)
+    res = bits(rng.normal(0, 1.0, 256).astype(np.float32), dtype)
+    scalar = bits(np.float32([0.75]), dtype)
+    ctx.put(1, x); ctx.put(2, w); ctx.put(3, res); ctx.put(4, scalar); ctx.alloc(5, 512)
+    rec = rt.make_record(ctx.pipeline("rms_norm_1pw_d256_add_scalar_weight"), [(1, 0, 0), (2, 1, 0), (3, 2, 0), (4, 3, 0), (5, 4, 0)],
+                         [], (1, 1, 1), (256, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    got = ctx.read(5, np.uint16, 256)
+    ref = so.rms_norm_1pw_add_scalar(x, w, res, int(scalar[0]), 1e-6, odt)
+    normed = so.widen(so.rms_norm_1pw(x, w, 1e-6, odt, 2), odt).astype(np.float64)
+    g, r = fx.from_bits(got, dtype).astype(np.float64), so.widen(ref, odt).astype(np.float64)
+    bound = gh.ulp_of(np.where(normed == 0, 1e-30, normed), dtype) + 2 * gh.ulp_of(np.where(r == 0, 1e-30, r), dtype)
+    assert np.all(np.abs(g - r) <= bound) and np.mean(got == ref) >= 0.97
+    # the plain d256 add kernel now multiplies left to right as the reference's does
+    ctx.alloc(5, 512)
+    rec = rt.make_record(ctx.pipeline("rms_norm_1pw_d256_add"), [(1, 0, 0), (2, 1, 0), (3, 2, 0), (5, 3, 0)], [], (1, 1, 1), (256, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    assert np.mean(ctx.read(5, np.uint16, 256) == so.rms_norm_1pw(x, w, 1e-6, odt, 2, res)) >= 0.97
+
+    tokens, dim = 3, 1536
+    x32 = rng.normal(0, 3, (tokens, dim)).astype(np.float32)
+    x32[1, 7] = 3.0e5                                  # one row whose product clamps at the fp16 limit
+    w = bits(rng.normal(0, 0.2, dim).astype(np.float32), dtype)
+    ctx.put(1, x32); ctx.put(2, w); ctx.alloc(3, tokens * dim * 2)
+    rec = rt.make_record(ctx.pipeline("rms_norm_1pw_from_fp32_batched"), [(1, 0, 0), (2, 1, 0), (3, 2, 0)], [(3, dim), (4, 1e-6)],
+                         (tokens, 1, 1), (256, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    got = ctx.read(3, np.uint16, tokens * dim).reshape(tokens, dim)
+    for t in range(tokens):
+        assert_last_place(got[t], so.rms_norm_1pw_from_fp32(x32[t], w, 1e-6, odt), dtype, f"from_fp32 token {t}", exact_fraction=0.97)
+    assert fx.from_bits(got[1], dtype).max() <= 65504.0
+
+    heads, d = 16, 128
+    xh = bits((rng.normal(0, 1, (heads, d)) * rng.uniform(0.1, 8, (heads, 1))).astype(np.float32), dtype)
+    gate = bits(rng.normal(0, 2, (heads, d)).astype(np.float32), dtype)
+    wg = bits((1.0 + rng.normal(0, 0.1, d)).astype(np.float32), dtype)
+    ctx.put(1, xh); ctx.put(2, gate); ctx.put(3, wg); ctx.alloc(4, heads * d * 2)
+    rec = rt.make_record(ctx.pipeline("rms_norm_gated"), [(1, 0, 0), (2, 1, 0), (3, 2, 0), (4, 3, 0)], [(4, d), (5, 1e-6)],
+                         (heads, 1, 1), (64, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    got = ctx.read(4, np.uint16, heads * d)
+    ref = so.rms_norm_gated(xh.ravel(), gate.ravel(), wg, heads, d, 1e-6, odt)
+    assert_last_place(got, ref, dtype, "rms_norm_gated", exact_fraction=0.97)

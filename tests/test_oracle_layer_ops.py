@@ -143,3 +143,47 @@ def test_geglu_closed_forms_clamps_and_float64():
     tol = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + np.abs(gh_ * uh) * 2.0 ** -22
     assert np.all(np.abs(got - ref) <= tol)
     assert np.mean(got == ref.astype(np.float16).astype(np.float64)) > 0.94
+
+
+def test_norm_variants_closed_forms():
+    """d256 left-to-right norm + residual + scalar (norms.metal:218-260), the fp32-input norm
+    (norms_fp32.metal:50-88) and the gated norm (norms.metal:1093-1153)."""
+    rng = fx.rng_for(99, 0)
+    # from_fp32: unit weight (w = 0) on a constant row is +-1; large rows clamp at the fp16 limit
+    assert np.array_equal(so.widen(so.rms_norm_1pw_from_fp32(np.full(64, -3.0, np.float32), f16(np.zeros(64)), 0.0, so.F16), so.F16),
+                          np.full(64, -1.0, np.float32))
+    big = np.zeros(16, np.float32); big[0] = 1.0
+    out = so.widen(so.rms_norm_1pw_from_fp32(big, f16(np.full(16, 60000.0)), 0.0, so.F16), so.F16)
+    assert out[0] == 65504.0 and np.all(out[1:] == 0)                                  # 4 * (1 + 60000) clamps
+    x32 = rng.normal(0, 3, 1536).astype(np.float32)
+    w = f16(rng.normal(0, 0.2, 1536))
+    got = so.widen(so.rms_norm_1pw_from_fp32(x32, w, 1e-6, so.F16), so.F16).astype(np.float64)
+    rs = 1.0 / np.sqrt(np.mean(x32.astype(np.float64) ** 2) + 1e-6)
+    ref = x32.astype(np.float64) * rs * (1.0 + so.widen(w, so.F16).astype(np.float64))
+    assert np.all(np.abs(got - ref) <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64))
+    # fp16 input given as fp32 equals the left-to-right 16-bit norm when nothing clamps
+    x = f16(rng.normal(0, 1.5, 256))
+    assert np.mean(so.rms_norm_1pw_from_fp32(so.widen(x, so.F16), w[:256], 1e-6, so.F16) == so.rms_norm_1pw(x, w[:256], 1e-6, so.F16, 2)) > 0.99
+    # left-to-right against scale-first: same value up to the last place
+    a = so.widen(so.rms_norm_1pw(x, w[:256], 1e-6, so.F16, 2), so.F16).astype(np.float64)
+    b = so.widen(so.rms_norm_1pw(x, w[:256], 1e-6, so.F16, 0), so.F16).astype(np.float64)
+    assert np.all(np.abs(a - b) <= np.spacing(np.abs(b).astype(np.float16)).astype(np.float64)) and np.mean(a == b) > 0.9
+    # + residual, * scalar: scalar 1 is the add form, scalar 0.5 halves it exactly, scalar 0 gives zeros
+    res = f16(rng.normal(0, 1, 256))
+    added = so.rms_norm_1pw(x, w[:256], 1e-6, so.F16, 2, res)
+    assert np.array_equal(so.rms_norm_1pw_add_scalar(x, w[:256], res, int(f16([1.0])[0]), 1e-6, so.F16), added)
+    half = so.widen(so.rms_norm_1pw_add_scalar(x, w[:256], res, int(f16([0.5])[0]), 1e-6, so.F16), so.F16)
+    assert np.array_equal(half[np.abs(half) > 1e-3], (so.widen(added, so.F16) * 0.5)[np.abs(half) > 1e-3])
+    assert not so.widen(so.rms_norm_1pw_add_scalar(x, w[:256], res, 0, 1e-6, so.F16), so.F16).any()
+    # gated: gate 0 -> 0; large gate -> w * x * rs * gate; heads are normalised separately
+    heads, d = 3, 128
+    xh = f16(rng.normal(0, 1, heads * d) * np.repeat([1.0, 10.0, 0.1], d))
+    wg = f16(1.0 + rng.normal(0, 0.1, d))
+    assert not so.widen(so.rms_norm_gated(xh, f16(np.zeros(heads * d)), wg, heads, d, 1e-6, so.F16), so.F16).any()
+    gate = f16(rng.normal(0, 2, heads * d))
+    got = so.widen(so.rms_norm_gated(xh, gate, wg, heads, d, 1e-6, so.F16), so.F16).astype(np.float64)
+    xf, gf = so.widen(xh, so.F16).astype(np.float64).reshape(heads, d), so.widen(gate, so.F16).astype(np.float64).reshape(heads, d)
+    rs = 1.0 / np.sqrt((xf ** 2).mean(axis=1, keepdims=True) + 1e-6)
+    ref = (so.widen(wg, so.F16).astype(np.float64)[None, :] * xf * rs * gf / (1.0 + np.exp(-gf))).ravel()
+    assert np.all(np.abs(got - ref) <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + 1e-7)
+    assert np.mean(got == ref.astype(np.float16).astype(np.float64)) > 0.98
