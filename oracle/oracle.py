@@ -90,7 +90,8 @@ def _declare(l: C.CDLL) -> None:
         "so_epilogue_geglu": (u16, [f32, f32, i32]),
         "so_rms_norm_1pw_add_scalar": (None, [vp, vp, vp, u16, i32, f32, i32, vp]),
         "so_rms_norm_1pw_from_fp32": (None, [vp, vp, i32, f32, i32, vp]),
-        "so_rms_norm_gated": (None, [vp, vp, vp, i32, i32, f32, i32, vp]),
+        "so_rms_norm_gated": (None, [vp, vp, vp, i32, i32, f32, i32, i32, vp]),
+        "so_rms_norm_gated_signed_activation_bitplanes": (None, [vp, vp, vp, i32, f32, i32, i32, vp, vp]),
         "so_norm_scale_input": (None, [vp, f32, vp, i32, i32, vp]),
         "so_epilogue_signed_swiglu": (u16, [u16, u16, i32]),
         "so_rms_scale": (f32, [vp, i32, f32, i32]),
@@ -405,13 +406,25 @@ def rms_norm_1pw_from_fp32(x_f32, w_bits, eps: float, dtype: int) -> np.ndarray:
     return out
 
 
-def rms_norm_gated(x_bits, gate_bits, w_bits, heads: int, head_dim: int, eps: float, dtype: int) -> np.ndarray:
+def rms_norm_gated(x_bits, gate_bits, w_bits, heads: int, head_dim: int, eps: float, dtype: int, precise: bool = False) -> np.ndarray:
     x = np.ascontiguousarray(x_bits, np.uint16)
     out = np.zeros(x.size, np.uint16)
     lib().so_rms_norm_gated(_p(x, np.uint16), _p(np.ascontiguousarray(gate_bits, np.uint16), np.uint16),
                             _p(np.ascontiguousarray(w_bits, np.uint16), np.uint16), heads, head_dim, eps, dtype,
-                            _p(out, np.uint16))
+                            int(precise), _p(out, np.uint16))
     return out
+
+
+def rms_norm_gated_activation_bitplanes(x_bits, gate_bits, w_bits, heads: int, eps: float, dtype: int, precise: bool):
+    """(planes [heads, 6, 4] u32, scales [heads] u16) of the gated norm of `heads` heads of 128 values."""
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    out = np.zeros((heads, 6, 4), np.uint32)
+    scales = np.zeros(heads, np.uint16)
+    lib().so_rms_norm_gated_signed_activation_bitplanes(
+        _p(x, np.uint16), _p(np.ascontiguousarray(gate_bits, np.uint16), np.uint16),
+        _p(np.ascontiguousarray(w_bits, np.uint16), np.uint16), heads, eps, dtype, int(precise), _p(out, np.uint32),
+        _p(scales, np.uint16))
+    return out, scales
 
 
 def swiglu_fused(gate_bits, up_bits, dtype: int) -> np.ndarray:

@@ -712,19 +712,30 @@ SO_EXPORT void so_rms_norm_1pw_from_fp32(const float *x, const uint16_t *w, int 
     }
 }
 
-/* rms_norm_gated (norms.metal:1093-1153): per head half(w * (x * rs) * silu(gate)), SiLU in fp32. */
+/* rms_norm_gated (norms.metal:1093-1153): per head half(w * (x * rs) * silu(gate)), SiLU in fp32.
+ * precise != 0: the d128 kernels (norms_gated_precise.metal:7-18): half(w) * half(x * rs) as a 16-bit
+ * product, SiLU from the stable sigmoid in fp32, one final narrowing. */
+static uint16_t rms_norm_gated_value(uint16_t x, uint16_t gate, uint16_t w, float rs, int precise, int dtype) {
+    float g = widen(gate, dtype);
+    if (precise) {
+        float normalized = so_round_through(widen(w, dtype) * so_round_through(widen(x, dtype) * rs, dtype), dtype);
+        float tail = 1.0f / (1.0f + expf(fabsf(g)));
+        float sigmoid = g < 0.0f ? tail : 1.0f - tail;
+        return narrow(normalized * (g * sigmoid), dtype);
+    }
+    float silu = g / (1.0f + expf(-g));
+    float normalized = widen(x, dtype) * rs;
+    float weighted = widen(w, dtype) * normalized;
+    return narrow(weighted * silu, dtype);
+}
+
 SO_EXPORT void so_rms_norm_gated(const uint16_t *x, const uint16_t *gate, const uint16_t *w, int heads,
-                                 int head_dim, float eps, int dtype, uint16_t *out) {
+                                 int head_dim, float eps, int dtype, int precise, uint16_t *out) {
     for (int h = 0; h < heads; ++h) {
         const uint16_t *xr = x + (size_t)h * head_dim, *gr = gate + (size_t)h * head_dim;
         float rs = so_rms_scale(xr, head_dim, eps, dtype);
-        for (int i = 0; i < head_dim; ++i) {
-            float g = widen(gr[i], dtype);
-            float silu = g / (1.0f + expf(-g));
-            float normalized = widen(xr[i], dtype) * rs;
-            float weighted = widen(w[i], dtype) * normalized;
-            out[(size_t)h * head_dim + i] = narrow(weighted * silu, dtype);
-        }
+        for (int i = 0; i < head_dim; ++i)
+            out[(size_t)h * head_dim + i] = rms_norm_gated_value(xr[i], gr[i], w[i], rs, precise, dtype);
     }
 }
 
@@ -830,6 +841,22 @@ SO_EXPORT void so_sigmoid_mul_signed_activation_bitplanes(const uint16_t *a, con
         for (int i = 0; i < 128; ++i) v[i] = widen(so_sigmoid_mul(a[g * 128 + i], b[g * 128 + i], dtype), dtype);
         out_scales[g] = bitplane_quantize_group(v, planes, dtype, q);
         bitplane_pack_group(q, planes, out_planes + (size_t)g * planes * 4);
+    }
+}
+
+/* rms_norm_gated_d128_signed_activation_bitplanes_i6_g128 (signed_quant.metal:1029-1173): the gated norm of
+ * one 128-value head (precise or generic arithmetic, as the launch selects), then its i6 view. */
+SO_EXPORT void so_rms_norm_gated_signed_activation_bitplanes(const uint16_t *x, const uint16_t *gate, const uint16_t *w,
+                                                             int heads, float eps, int dtype, int precise,
+                                                             uint32_t *out_planes, uint16_t *out_scales) {
+    for (int h = 0; h < heads; ++h) {
+        uint16_t row[128];
+        float v[128];
+        int q[128];
+        so_rms_norm_gated(x + (size_t)h * 128, gate + (size_t)h * 128, w, 1, 128, eps, dtype, precise, row);
+        for (int i = 0; i < 128; ++i) v[i] = widen(row[i], dtype);
+        out_scales[h] = bitplane_quantize_group(v, 6, dtype, q);
+        bitplane_pack_group(q, 6, out_planes + (size_t)h * 24);
     }
 }
 

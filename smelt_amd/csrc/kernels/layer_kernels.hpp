@@ -108,31 +108,6 @@ __device__ __forceinline__ void rms_norm_from_fp32_row(const float* x, const uin
     }
 }
 
-// rms_norm_gated (norms.metal:1093-1153): per head, half(w * (x * rs) * silu(gate)) with the SiLU in fp32.
-template <class ActT>
-__device__ __forceinline__ void rms_norm_gated_row(const uint16_t* x, const uint16_t* gate, const uint16_t* weight,
-                                                   uint16_t* out, uint32_t dim, float eps) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    float* scratch = reinterpret_cast<float*>(smem);
-    float sum = 0.0f;
-    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
-        const float v = ActT::widen(x[i]);
-        sum = __builtin_fmaf(v, v, sum);
-    }
-    const float rs = inv_rms(block_sum(sum, scratch), dim, eps);
-    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
-        const float g = ActT::widen(gate[i]);
-        const float silu = g / (1.0f + expf(-g));
-        float v;
-        {
-#pragma clang fp contract(off)
-            const float normalized = ActT::widen(x[i]) * rs;
-            v = (ActT::widen(weight[i]) * normalized) * silu;
-        }
-        out[i] = ActT::narrow(v);
-    }
-}
-
 }  // namespace smelt
 
 #define SMELT_LAYER_KERNEL extern "C" __global__ __launch_bounds__(1024)
@@ -162,12 +137,6 @@ __device__ __forceinline__ void rms_norm_gated_row(const uint16_t* x, const uint
                                                              uint16_t* y, uint32_t dim, float eps) { \
         const size_t at = (size_t)blockIdx.x * dim;                                               \
         smelt::rms_norm_from_fp32_row<ACT>(x + at, w, y + at, dim, eps);                          \
-    }                                                                                             \
-    SMELT_LAYER_KERNEL void smelt_rms_norm_gated_##T(const uint16_t* x, const uint16_t* gate,     \
-                                                     const uint16_t* w, uint16_t* y,              \
-                                                     uint32_t head_dim, float eps) {              \
-        const size_t at = (size_t)blockIdx.x * head_dim;                                          \
-        smelt::rms_norm_gated_row<ACT>(x + at, gate + at, w, y + at, head_dim, eps);              \
     }                                                                                             \
     SMELT_LAYER_KERNEL void smelt_rms_norm_scale_only_##T(const uint16_t* x, float* scale,        \
                                                           uint32_t dim, float eps) {              \

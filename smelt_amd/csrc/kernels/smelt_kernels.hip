@@ -54,6 +54,8 @@ SMELT_BITPLANE_KERNELS(ternary, smelt::FmtTerPlanes, f16, smelt::F16)
 SMELT_BITPLANE_KERNELS(ternary, smelt::FmtTerPlanes, bf16, smelt::BF16)
 SMELT_ACTIVATION_BITPLANE_KERNELS(f16, smelt::F16)
 SMELT_ACTIVATION_BITPLANE_KERNELS(bf16, smelt::BF16)
+SMELT_GATED_NORM_KERNELS(f16, smelt::F16)
+SMELT_GATED_NORM_KERNELS(bf16, smelt::BF16)
 SMELT_LUT_KERNELS(f16, smelt::F16)
 SMELT_LUT_KERNELS(bf16, smelt::BF16)
 SMELT_TQH_KERNELS(f16, smelt::F16)

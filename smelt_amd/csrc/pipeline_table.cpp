@@ -481,8 +481,23 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->family = kFamRmsNormFromFp32; out->symbol = "smelt_rms_norm_1pw_from_fp32_" + t; out->kinds = "PPPUF";
             return kResolveOk;
         }
-        if (entry == "rms_norm_gated") {
-            out->family = kFamRmsNormGated; out->symbol = "smelt_rms_norm_gated_" + t; out->kinds = "PPPPUF";
+        if (entry == "rms_norm_gated") {                      // head_dim, eps from the record
+            out->family = kFamRmsNormGated; out->symbol = "smelt_rms_norm_gated_" + t; out->kinds = "PPPPUFU"; out->appended = {0u};
+            return kResolveOk;
+        }
+        if (entry == "rms_norm_gated_d128") {                 // norms_gated_precise.metal:20-52
+            out->family = kFamRmsNormGated; out->symbol = "smelt_rms_norm_gated_" + t; out->kinds = "PPPPUUU";
+            out->appended = {128u, eps_bits(1e-6f), 1u};
+            return kResolveOk;
+        }
+        if (entry == "rms_norm_gated_d128_batched") {         // heads per token from the record (:54-88)
+            out->family = kFamRmsNormGatedBatched; out->symbol = "smelt_rms_norm_gated_batched_" + t; out->kinds = "PPPPUUUU";
+            out->appended = {128u, eps_bits(1e-6f), 1u};
+            return kResolveOk;
+        }
+        if (entry == "rms_norm_gated_d128_signed_activation_bitplanes_i6_g128") {   // signed_quant.metal:1149-1173
+            out->family = kFamRmsNormGatedPlanes; out->symbol = "smelt_rms_norm_gated_signed_activation_bitplanes_" + t;
+            out->kinds = "PPPPPUF";
             return kResolveOk;
         }
         if (starts_with(entry, "rms_norm_1pw")) {

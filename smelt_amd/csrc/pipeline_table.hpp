@@ -77,7 +77,9 @@ enum FamilyId {
     kFamFusedNormAffineGateUp,   // x nw gW gS gB uW uS uB y scratch rows eps | cols group
     kFamRmsNormAddScalar,        // x w res scalar y | dim eps mode             (grid.x = token row)
     kFamRmsNormFromFp32,         // x(fp32) w y dim eps
-    kFamRmsNormGated,            // x gate w y head_dim eps                      (grid.x = head)
+    kFamRmsNormGated,            // x gate w y head_dim eps | precise            (grid.x = head)
+    kFamRmsNormGatedBatched,     // x gate w y heads_per_token | head_dim eps precise (grid = heads x tokens)
+    kFamRmsNormGatedPlanes,      // x gate w planes scales head_dim eps          (grid.x = head = 128-value group)
     kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
     kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile
     kFamCount

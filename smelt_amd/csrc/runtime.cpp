@@ -538,10 +538,31 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             L.lds = 64 + dim * 2;
             break;
         }
+        case kFamRmsNormGated:
+        case kFamRmsNormGatedBatched:
+        case kFamRmsNormGatedPlanes: {
+            // one workgroup (32 threads or whole waves) per head
+            const bool batched = r.family == kFamRmsNormGatedBatched, view = r.family == kFamRmsNormGatedPlanes;
+            const size_t dim = U(batched ? 5 : (view ? 5 : 4));
+            if (dim == 0) return bad_geom("head_dim must be positive");
+            if ((L.block[0] != 32 && L.block[0] % 64 != 0) || L.block[1] != 1 || L.block[2] != 1 || L.grid[2] != 1)
+                return bad_geom("gated norm kernels run 32 threads or whole waves per workgroup");
+            if (!batched && L.grid[1] != 1) return bad_geom("one token per launch");
+            if (batched && U(4) != L.grid[0]) return bad_geom("grid width must equal the heads per token");
+            const size_t heads = (size_t)L.grid[0] * L.grid[1];
+            need[0] = heads * dim * 2; need[1] = heads * dim * 2; need[2] = dim * 2;
+            if (view) {
+                if (dim != 128) return bad_geom("the gated-norm view producer takes heads of 128 values");
+                need[3] = heads * 6 * 16; align[3] = 16; written[3] = true;
+                need[4] = heads * 2; written[4] = true;
+            } else {
+                need[3] = heads * dim * 2; written[3] = true;
+            }
+            break;
+        }
         case kFamRmsNormAddScalar:
-        case kFamRmsNormFromFp32:
-        case kFamRmsNormGated: {
-            const size_t first_u = r.family == kFamRmsNormAddScalar ? 5 : (r.family == kFamRmsNormFromFp32 ? 3 : 4);
+        case kFamRmsNormFromFp32: {
+            const size_t first_u = r.family == kFamRmsNormAddScalar ? 5 : 3;
             const size_t dim = U(first_u), tokens = L.grid[0];
             if (dim == 0) return bad_geom("dim must be positive");
             if (L.block[0] % 64 != 0 || L.block[1] != 1 || L.block[2] != 1 || L.grid[1] != 1 || L.grid[2] != 1)
@@ -549,10 +570,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             const size_t row = tokens * dim * 2;
             if (r.family == kFamRmsNormAddScalar) {
                 need[0] = row; need[1] = dim * 2; need[2] = row; need[3] = 2; need[4] = row; written[4] = true;
-            } else if (r.family == kFamRmsNormFromFp32) {
-                need[0] = tokens * dim * 4; align[0] = 4; need[1] = dim * 2; need[2] = row; written[2] = true;
             } else {
-                need[0] = row; need[1] = row; need[2] = dim * 2; need[3] = row; written[3] = true;
+                need[0] = tokens * dim * 4; align[0] = 4; need[1] = dim * 2; need[2] = row; written[2] = true;
             }
             L.lds = 64 + dim * 2;
             break;

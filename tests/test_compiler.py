@@ -163,7 +163,8 @@ def test_pipeline_names_resolve_to_kernels_with_the_reference_binding_counts():
     assert cc.resolve_pipeline_name("tqh_matvec_batched")[1:] == ("smelt_tqh_matvec_f16", "PPPPUUU")
     assert cc.resolve_pipeline_name("u4_lut_qmm")[0] == -4
     assert cc.resolve_pipeline_name("rms_norm_1pw_from_fp32")[1:] == ("smelt_rms_norm_1pw_from_fp32_f16", "PPPUF")
-    assert cc.resolve_pipeline_name("rms_norm_gated_d128")[0] == -4        # the d128 gated form is not built
+    assert cc.resolve_pipeline_name("rms_norm_gated_d128")[1] == "smelt_rms_norm_gated_f16"
+    assert cc.resolve_pipeline_name("rms_norm_head_f32")[0] == -4          # fp32 trunk kernels are out of scope
     assert cc.resolve_pipeline_name("rope_apply")[0] == -4
 
 

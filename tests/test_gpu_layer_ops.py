@@ -316,3 +316,42 @@ def test_norm_variants(env):
     got = ctx.read(4, np.uint16, heads * d)
     ref = so.rms_norm_gated(xh.ravel(), gate.ravel(), wg, heads, d, 1e-6, odt)
     assert_last_place(got, ref, dtype, "rms_norm_gated", exact_fraction=0.97)
+
+
+@pytest.mark.parametrize("threads", [32, 128])
+def test_gated_norm_precise_batched_and_view(env, threads):
+    """rms_norm_gated_d128[_batched] (norms_gated_precise.metal:20-88) and the fused gated-norm -> i6 view
+    (signed_quant.metal:1149-1173), which takes the precise arithmetic exactly when launched with 32
+    threads per 128-value head, as the reference's does."""
+    ctx, dtype, odt = env
+    rng = fx.rng_for(98, threads)
+    tokens, heads, d = 2, 8, 128
+    x = bits((rng.normal(0, 1, (tokens * heads, d)) * rng.uniform(0.2, 5, (tokens * heads, 1))).astype(np.float32), dtype)
+    gate = bits(rng.normal(0, 2, (tokens * heads, d)).astype(np.float32), dtype)
+    w = bits((1.0 + rng.normal(0, 0.1, d)).astype(np.float32), dtype)
+    ctx.put(1, x); ctx.put(2, gate); ctx.put(3, w); ctx.alloc(4, x.size * 2)
+    rec = rt.make_record(ctx.pipeline("rms_norm_gated_d128_batched"), [(1, 0, 0), (2, 1, 0), (3, 2, 0), (4, 3, 0)], [(4, heads)],
+                         (heads, tokens, 1), (threads, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    got = ctx.read(4, np.uint16, x.size)
+    ref = so.rms_norm_gated(x.ravel(), gate.ravel(), w, tokens * heads, d, 1e-6, odt, precise=True)
+    assert_last_place(got, ref, dtype, "rms_norm_gated_d128_batched", exact_fraction=0.97, max_ulps=2.0)
+    ctx.alloc(4, heads * d * 2)
+    rec = rt.make_record(ctx.pipeline("rms_norm_gated_d128"), [(1, 0, 0), (2, 1, 0), (3, 2, 0), (4, 3, 0)], [], (heads, 1, 1), (threads, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    assert np.array_equal(ctx.read(4, np.uint16, heads * d), got[:heads * d])          # token 0 of the batched run
+    # fused view: equal to the plain i6 producer run on this backend's own norm output of the same arithmetic
+    n = tokens * heads
+    ctx.alloc(5, n * 6 * 16); ctx.alloc(6, n * 2); ctx.alloc(7, x.size * 2)
+    rec = rt.make_record(ctx.pipeline("rms_norm_gated_d128_signed_activation_bitplanes_i6_g128"),
+                         [(1, 0, 0), (2, 1, 0), (3, 2, 0), (5, 3, 0), (6, 4, 0)], [(5, d), (6, 1e-6)], (n, 1, 1), (threads, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    fused_pl, fused_sc = ctx.read(5, np.uint32, n * 24), ctx.read(6, np.uint16, n)
+    norm_name, consts = ("rms_norm_gated_d128", []) if threads == 32 else ("rms_norm_gated", [(4, d), (5, 1e-6)])
+    staged = [rt.make_record(ctx.pipeline(norm_name), [(1, 0, 0), (2, 1, 0), (3, 2, 0), (7, 3, 0)], consts, (n, 1, 1), (threads, 1, 1)),
+              rt.make_record(ctx.pipeline("signed_activation_bitplanes_i6_g128"), [(7, 0, 0), (5, 1, 0), (6, 2, 0)], [(3, n * d)], (n, 1, 1), (32, 1, 1))]
+    ctx.alloc(5, n * 6 * 16); ctx.alloc(6, n * 2)
+    ctx.interpret_decode(ctx.table(staged)); ctx.wait()
+    assert np.array_equal(ctx.read(5, np.uint32, n * 24), fused_pl) and np.array_equal(ctx.read(6, np.uint16, n), fused_sc)
+    ref_pl, ref_sc = so.rms_norm_gated_activation_bitplanes(x.ravel(), gate.ravel(), w, n, 1e-6, odt, threads == 32)
+    assert np.mean(fused_pl == ref_pl.reshape(-1)) > 0.97 and np.mean(fused_sc == ref_sc) > 0.85

@@ -187,3 +187,32 @@ def test_norm_variants_closed_forms():
     ref = (so.widen(wg, so.F16).astype(np.float64)[None, :] * xf * rs * gf / (1.0 + np.exp(-gf))).ravel()
     assert np.all(np.abs(got - ref) <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + 1e-7)
     assert np.mean(got == ref.astype(np.float16).astype(np.float64)) > 0.98
+
+
+def test_gated_norm_precise_form_and_its_view():
+    """rms_norm_gated_d128 (norms_gated_precise.metal:7-52): half(w) * half(x * rs) is a 16-bit product
+    before the fp32 SiLU; restated in numpy float16, and the fused view is the plain i6 view of it."""
+    rng = fx.rng_for(100, 0)
+    heads, d = 4, 128
+    x = f16(rng.normal(0, 1, heads * d) * np.repeat([1.0, 6.0, 0.2, 1.0], d))
+    gate = f16(rng.normal(0, 2, heads * d))
+    w = f16(1.0 + rng.normal(0, 0.1, d))
+    got = so.rms_norm_gated(x, gate, w, heads, d, 1e-6, so.F16, precise=True).view(np.float16)
+    xf = so.widen(x, so.F16).reshape(heads, d)
+    rs = np.array([so.rms_scale(x[h * d:(h + 1) * d], 1e-6, so.F16) for h in range(heads)], np.float32)[:, None]
+    normalized = (w.view(np.float16)[None, :] * (xf * rs).astype(np.float16)).astype(np.float16)      # float16 x float16
+    g = so.widen(gate, so.F16).reshape(heads, d)
+    tail = np.float32(1) / (np.float32(1) + np.exp(np.abs(g), dtype=np.float32))
+    sig = np.where(g < 0, tail, np.float32(1) - tail).astype(np.float32)
+    ref = (normalized.astype(np.float32) * (g * sig)).astype(np.float16).ravel()
+    ulp = np.spacing(np.abs(ref)).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - ref.astype(np.float64)) <= ulp)          # exp may differ in its last bit
+    assert np.mean(got.view(np.uint16) == ref.view(np.uint16)) > 0.99
+    # the two arithmetic forms agree to a couple of 16-bit ulps and are not the same function
+    generic = so.rms_norm_gated(x, gate, w, heads, d, 1e-6, so.F16).view(np.float16)
+    assert np.all(np.abs(generic.astype(np.float64) - got.astype(np.float64)) <= 3 * np.spacing(np.abs(got)).astype(np.float64) + 1e-7)
+    assert np.any(generic.view(np.uint16) != got.view(np.uint16))
+    for precise in (False, True):
+        staged = so.activation_bitplanes(so.rms_norm_gated(x, gate, w, heads, d, 1e-6, so.F16, precise), 6, so.F16)
+        fused = so.rms_norm_gated_activation_bitplanes(x, gate, w, heads, 1e-6, so.F16, precise)
+        assert np.array_equal(staged[0], fused[0]) and np.array_equal(staged[1], fused[1])
