@@ -91,9 +91,10 @@ bool family_for(int weight, int* family) {
 bool hip_has_kernel(const SmeltMatvecCell& c, int family) {
     const bool quant = family == SMELT_FAMILY_AFFINE_U4 || family == SMELT_FAMILY_BINARY1 ||
                        family == SMELT_FAMILY_TERNARY2 || family == SMELT_FAMILY_TRIT5;
-    // u4_lut: single-token matvec, dual and gate+up+SwiGLU kernels (no batched / qmm form)
+    // u4_lut: single-token matvec, dual and gate+up+SwiGLU kernels; prompt rows run the per-token matmul
     if (family == SMELT_FAMILY_LUT_U4)
-        return c.activation != SMELT_ACT_FP32 && c.shape == SMELT_SHAPE_GEMV && c.fusion != SMELT_FUSION_GATE_UP_GEGLU;
+        return c.activation != SMELT_ACT_FP32 && c.fusion != SMELT_FUSION_GATE_UP_GEGLU &&
+               (c.shape == SMELT_SHAPE_GEMV || (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_NONE));
     // turbo_quant_h: prepare + matvec pair (the batched names cover prefill rows), no fused forms
     if (family == SMELT_FAMILY_TQH) return c.activation != SMELT_ACT_FP32 && c.fusion == SMELT_FUSION_NONE;
     if (!quant) return false;

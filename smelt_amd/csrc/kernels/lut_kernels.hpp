@@ -141,6 +141,15 @@ __device__ __forceinline__ void lut_matvec_body(const LutMat (&mats)[NMAT], cons
         auto epi = [=](int r, const float* v) { y[r] = ACT::narrow(v[0]); };                      \
         smelt::lut_matvec_body<ACT, 1>(mats, x, rows, cols, group, epi);                          \
     }                                                                                             \
+    /* fused_lut_matmul (prefill_matmul.metal:13-62): grid.y = token, rows of X and Y per token */  \
+    SMELT_LUT_KERNEL void smelt_lut_matmul_##T(const uint8_t* W, const uint16_t* lut,             \
+                                               const uint16_t* X, uint16_t* Y, uint32_t cols,     \
+                                               uint32_t group, uint32_t rows) {                   \
+        const smelt::LutMat mats[1] = {{W, lut}};                                                 \
+        uint16_t* y = Y + (size_t)blockIdx.y * rows;                                              \
+        auto epi = [=](int r, const float* v) { y[r] = ACT::narrow(v[0]); };                      \
+        smelt::lut_matvec_body<ACT, 1>(mats, X + (size_t)blockIdx.y * cols, rows, cols, group, epi); \
+    }                                                                                             \
     /* half(float(residual) + acc): the sum is not rounded before the add (lut_matvec.metal:334-340) */ \
     SMELT_LUT_KERNEL void smelt_lut_matvec_add_##T(const uint8_t* W, const uint16_t* lut,         \
                                                    const uint16_t* x, uint16_t* y,                \

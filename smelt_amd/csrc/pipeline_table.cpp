@@ -615,6 +615,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
         out->family = kFamTqhMatvec; out->symbol = "smelt_tqh_matvec_" + t; out->kinds = "PPPPUUU"; return kResolveOk;
     }
     if (entry == "tqh_embedding_gather") { out->family = kFamTqhGather; out->symbol = "smelt_tqh_embedding_gather_" + t; out->kinds = "PPPPUU"; return kResolveOk; }
+    if (entry == "fused_lut_matmul") { out->family = kFamLutMatmul; out->symbol = "smelt_lut_matmul_" + t; out->kinds = "PPPPUUU"; return kResolveOk; }
     if (entry == "lut_embedding_gather") { out->family = kFamLutGather; out->symbol = "smelt_lut_embedding_gather"; out->kinds = "PPPPUU"; return kResolveOk; }
     // binary projection banks on the direct path (signed_quant.metal:2638-2935)
     if (entry == "signed_binary_packed_bank_matvec_g128_rows8") {

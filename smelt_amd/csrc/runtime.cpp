@@ -124,7 +124,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
     auto bad_geom = [&](const std::string& m) {
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
     };
-    const bool lut_matvec = r.family == kFamLutMatvec || r.family == kFamLutAdd || r.family == kFamLutDual || r.family == kFamLutGateUp;
+    const bool lut_matvec = r.family == kFamLutMatvec || r.family == kFamLutAdd || r.family == kFamLutDual || r.family == kFamLutGateUp ||
+                            r.family == kFamLutMatmul;
     const bool plane_matvec = r.family == kFamPlaneMatvec || r.family == kFamPlaneAdd || r.family == kFamPlaneGateUp ||
                               r.family == kFamPlaneBank4 || r.family == kFamPlaneBatched || r.family == kFamBinaryPackedBank || r.family == kFamBinaryPackedBank4 ||
                               r.family == kFamBinaryTwoMatrix;
@@ -606,6 +607,16 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             if (r.family == kFamLutDual) { need[xi + 2] = rows * 2; written[xi + 2] = true; }
             if (r.family == kFamLutAdd) need[xi + 2] = rows * 2;
             L.lds = cols * 2 + (L.block[0] / 64) * nmat * 4 * 1024;
+            break;
+        }
+        case kFamLutMatmul: {
+            const size_t cols = U(4), group = U(5), rows = U(6);
+            if (rows == 0 || cols == 0 || cols % 32 != 0 || group < 8) return bad_geom("u4_lut kernels need rows > 0, cols % 32 == 0 and at least 8 rows per table");
+            need[0] = rows * (cols / 2); align[0] = 16;
+            need[1] = cdiv(rows, group) * 32;
+            need[2] = gy * cols * 2; align[2] = 16;
+            need[3] = gy * rows * 2; written[3] = true;
+            L.lds = cols * 2 + (L.block[0] / 64) * 4 * 1024;
             break;
         }
         case kFamLutGather: {

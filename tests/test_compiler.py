@@ -43,7 +43,7 @@ def test_gateway_has_no_holes_and_never_defaults():
     assert cc.select(cc.ACT_FP16, cc.BINARY1, cc.GEMM, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.FP16, hip_backend=True)[0] == cc.SELECT_MISSING
     assert cc.select(cc.ACT_FP16, cc.U4_LUT, hip_backend=True)[0] == cc.SELECT_OK
-    assert cc.select(cc.ACT_FP16, cc.U4_LUT, cc.GEMM, hip_backend=True)[0] == cc.SELECT_MISSING      # no batched u4_lut kernel
+    assert cc.select(cc.ACT_FP16, cc.U4_LUT, cc.GEMM, hip_backend=True)[0] == cc.SELECT_OK            # fused_lut_matmul, one token per grid row
     assert cc.select(cc.ACT_FP16, cc.TURBO_QUANT_H, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, cc.GEMM, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_OK

@@ -95,6 +95,31 @@ def test_lut_matvec_family(env, rows, cols, group, grid):
 
 
 @pytest.mark.gpu
+def test_lut_matmul_rows_equal_the_single_token_kernel(env):
+    """fused_lut_matmul (prefill_matmul.metal:13-62): one token per grid row, constants cols, group, rows;
+    every row of the output is the single-token kernel's."""
+    ctx, dtype, odt = env
+    rows, cols, group, tokens = 300, 1024, 16, 5
+    idx, lut = lut_case(77, rows, cols, group)
+    x = bits(fx.rng_for(134, 0).normal(0, 1, (tokens, cols)).astype(np.float32), dtype)
+    wf = gh.WeightFile()
+    a, b = wf.add(idx), wf.add(lut)
+    ctx.upload_weights(W, wf.image())
+    ctx.put(X, x); ctx.alloc(Y, tokens * rows * 2)
+    rec = rt.make_record(ctx.pipeline("fused_lut_matmul"), [(W, 0, a), (W, 1, b), (X, 2, 0), (Y, 3, 0)],
+                         [(4, cols), (5, group), (6, rows)], (rows, tokens, 1), (256, 1, 1))
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    got = ctx.read(Y, np.uint16, tokens * rows).reshape(tokens, rows)
+    for t in range(tokens):
+        ctx.put(X, x[t]); ctx.alloc(Y2, rows * 2)
+        one = rt.make_record(ctx.pipeline(f"fused_lut_matvec:{cols}:{group}"), [(W, 0, a), (W, 1, b), (X, 2, 0), (Y2, 3, 0)],
+                             [(4, rows)], ((rows + 7) // 8, 1, 1), (256, 1, 1))
+        ctx.interpret_decode(ctx.table([one])); ctx.wait()
+        assert np.array_equal(got[t], ctx.read(Y2, np.uint16, rows))
+        gh.check_outputs(got[t], so.lut_matvec(idx, lut, so.widen(x[t], odt), rows, cols, group), dtype, "fused_lut_matmul")
+
+
+@pytest.mark.gpu
 def test_lut_embedding_gather_and_bad_records(env):
     ctx, dtype, odt = env
     rows, cols, group = 100, 1024, 16
