@@ -255,6 +255,11 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             return kResolveMalformed;
         }
         const uint32_t row_stride = cols / 2;
+        // A/B variants the reference keeps beside its tuned kernels compute the same thing
+        for (const char* alias : {"_padded_reference", "_nocache_reference"}) {
+            const size_t n_alias = strlen(alias);
+            if (suffix.size() >= n_alias && suffix.compare(suffix.size() - n_alias, n_alias, alias) == 0) suffix.resize(suffix.size() - n_alias);
+        }
         // "_mfma" after the variant suffix asks for the matrix-core matvec of the same pipeline
         bool want_mfma = false;
         if (suffix.size() >= 5 && suffix.compare(suffix.size() - 5, 5, "_mfma") == 0) {
