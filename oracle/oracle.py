@@ -88,6 +88,7 @@ def _declare(l: C.CDLL) -> None:
         "so_epilogue_residual_add": (u16, [f32, u16, i32]),
         "so_epilogue_affine_swiglu": (u16, [f32, f32, i32]),
         "so_epilogue_geglu": (u16, [f32, f32, i32]),
+        "so_unary": (u16, [i32, u16, f32, i32]),
         "so_rms_norm_1pw_add_scalar": (None, [vp, vp, vp, u16, i32, f32, i32, vp]),
         "so_rms_norm_1pw_from_fp32": (None, [vp, vp, i32, f32, i32, vp]),
         "so_rms_norm_gated": (None, [vp, vp, vp, i32, i32, f32, i32, i32, vp]),
@@ -425,6 +426,14 @@ def rms_norm_gated_activation_bitplanes(x_bits, gate_bits, w_bits, heads: int, e
         _p(np.ascontiguousarray(w_bits, np.uint16), np.uint16), heads, eps, dtype, int(precise), _p(out, np.uint32),
         _p(scales, np.uint16))
     return out, scales
+
+
+UNARY_OPS = {"silu": 0, "sigmoid_kernel": 1, "softplus": 2, "scalar_mul": 3, "logit_cap": 4}
+
+
+def unary(name: str, x_bits, dtype: int, param: float = 0.0) -> np.ndarray:
+    l, op = lib(), UNARY_OPS[name]
+    return np.array([l.so_unary(op, int(b), float(param), dtype) for b in np.ravel(x_bits)], np.uint16).reshape(np.shape(x_bits))
 
 
 def swiglu_fused(gate_bits, up_bits, dtype: int) -> np.ndarray:

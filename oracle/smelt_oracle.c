@@ -739,6 +739,20 @@ SO_EXPORT void so_rms_norm_gated(const uint16_t *x, const uint16_t *gate, const 
     }
 }
 
+/* Pointwise activations (activations.metal:5-40, 98-108, 166-177), fp32 arithmetic, one narrowing:
+ * op 0 silu, 1 sigmoid, 2 softplus (x itself above 20), 3 x * param, 4 param * tanh(x / param). */
+SO_EXPORT uint16_t so_unary(int op, uint16_t x_bits, float param, int dtype) {
+    float x = widen(x_bits, dtype), v;
+    switch (op) {
+        case 0: v = x / (1.0f + expf(-x)); break;
+        case 1: v = 1.0f / (1.0f + expf(-x)); break;
+        case 2: v = x > 20.0f ? x : logf(1.0f + expf(x)); break;
+        case 3: v = x * param; break;
+        default: v = param * tanhf(x / param); break;
+    }
+    return narrow(v, dtype);
+}
+
 /* swiglu_fused (activations_precise.metal:9-22), elementwise_add / _mul (activations.metal:56-66, 85-95) */
 SO_EXPORT void so_swiglu_fused(const uint16_t *gate, const uint16_t *up, int n, int dtype, uint16_t *out) {
     for (int i = 0; i < n; ++i) out[i] = so_epilogue_signed_swiglu(gate[i], up[i], dtype);

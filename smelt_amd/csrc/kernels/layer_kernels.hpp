@@ -174,6 +174,55 @@ __device__ __forceinline__ void rms_norm_from_fp32_row(const float* x, const uin
         const float sig = g < 0.0f ? tail : rt(1.0f - tail);                                      \
         out[i] = ACT::narrow(rt(g * sig) * u);                                                    \
     }                                                                                             \
+    /* pointwise activations of activations.metal:5-40, 98-177 and activations_precise.metal:26-38;     \
+       op: 0 silu, 1 sigmoid, 2 softplus, 3 x * param, 4 param * tanh(x / param) */                  \
+    SMELT_LAYER_KERNEL void smelt_unary_##T(const uint16_t* in, uint16_t* out, uint32_t count,    \
+                                            float param, uint32_t op) {                           \
+        const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \
+        if (i >= count) return;                                                                   \
+        const float x = ACT::widen(in[i]);                                                        \
+        float v;                                                                                  \
+        switch (op) {                                                                             \
+            case 0: v = x / (1.0f + expf(-x)); break;                                             \
+            case 1: v = 1.0f / (1.0f + expf(-x)); break;                                          \
+            case 2: v = x > 20.0f ? x : logf(1.0f + expf(x)); break;                              \
+            case 3: v = x * param; break;                                                         \
+            default: v = param * tanhf(x / param); break;                                         \
+        }                                                                                         \
+        out[i] = ACT::narrow(v);                                                                  \
+    }                                                                                             \
+    SMELT_LAYER_KERNEL void smelt_scalar_mul_param_first_##T(const uint16_t* in, uint16_t* out,   \
+                                                             float scalar, uint32_t count) {      \
+        const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \
+        if (i < count) out[i] = ACT::narrow(ACT::widen(in[i]) * scalar);                          \
+    }                                                                                             \
+    SMELT_LAYER_KERNEL void smelt_scalar_mul_weight_##T(const uint16_t* in, const uint16_t* s,    \
+                                                        uint16_t* out, uint32_t count) {          \
+        const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \
+        if (i < count) out[i] = ACT::narrow(ACT::widen(in[i]) * ACT::widen(s[0]));                \
+    }                                                                                             \
+    /* attention * sigmoid(gate), the sigmoid staged in the 16-bit type (activations_precise.metal:26-38) */ \
+    SMELT_LAYER_KERNEL void smelt_sigmoid_mul_##T(const uint16_t* a, const uint16_t* gate,        \
+                                                  uint16_t* out, uint32_t count) {                \
+        const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \
+        if (i >= count) return;                                                                   \
+        auto rt = [](float v) { return ACT::widen(ACT::narrow(v)); };                             \
+        const float g = ACT::widen(gate[i]);                                                      \
+        const float tail = rt(1.0f / rt(1.0f + rt(expf(fabsf(g)))));                              \
+        const float sig = g < 0.0f ? tail : rt(1.0f - tail);                                      \
+        out[i] = ACT::narrow(ACT::widen(a[i]) * sig);                                             \
+    }                                                                                             \
+    /* gelu(gate) * up, tanh form, clamped (activations.metal:124-140) */                         \
+    SMELT_LAYER_KERNEL void smelt_geglu_fused_##T(const uint16_t* gate, const uint16_t* up,       \
+                                                  uint16_t* out, uint32_t count) {                \
+        const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \
+        if (i >= count) return;                                                                   \
+        const float g = ACT::widen(gate[i]), u = ACT::widen(up[i]);                               \
+        float inner = 0.7978845608f * (g + 0.044715f * (g * g * g));                              \
+        inner = fminf(fmaxf(inner, -20.0f), 20.0f);                                               \
+        const float gelu = 0.5f * g * (1.0f + tanhf(inner));                                      \
+        out[i] = ACT::narrow(fminf(fmaxf(gelu * u, -65504.0f), 65504.0f));                        \
+    }                                                                                             \
     SMELT_LAYER_KERNEL void smelt_elementwise_add_##T(const uint16_t* a, const uint16_t* b,       \
                                                       uint16_t* out, uint32_t count) {            \
         const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \

@@ -543,6 +543,18 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->family = kFamElementwise; out->symbol = "smelt_" + entry + "_" + t; out->kinds = "PPPU";
             return kResolveOk;
         }
+        if (entry == "sigmoid_mul" || entry == "geglu_fused") {
+            out->family = kFamElementwise; out->symbol = "smelt_" + entry + "_" + t; out->kinds = "PPPU";
+            return kResolveOk;
+        }
+        if (entry == "silu" || entry == "sigmoid_kernel" || entry == "softplus") {
+            out->family = kFamUnary; out->symbol = "smelt_unary_" + t; out->kinds = "PPUUU";
+            out->appended = {0u, entry == "silu" ? 0u : (entry == "sigmoid_kernel" ? 1u : 2u)};
+            return kResolveOk;
+        }
+        if (entry == "logit_cap") { out->family = kFamUnary; out->symbol = "smelt_unary_" + t; out->kinds = "PPUFU"; out->appended = {4u}; return kResolveOk; }
+        if (entry == "scalar_mul") { out->family = kFamScalarMul; out->symbol = "smelt_scalar_mul_param_first_" + t; out->kinds = "PPFU"; return kResolveOk; }
+        if (entry == "scalar_mul_weight") { out->family = kFamScalarMulWeight; out->symbol = "smelt_scalar_mul_weight_" + t; out->kinds = "PPPU"; return kResolveOk; }
         if (entry == "buffer_copy") { out->family = kFamCopy16; out->symbol = "smelt_buffer_copy16"; out->kinds = "PPU"; return kResolveOk; }
     }
     // ---- signed activation views (bit planes): signed_quant.metal:746-2260 ----------------------

@@ -80,6 +80,9 @@ enum FamilyId {
     kFamRmsNormGated,            // x gate w y head_dim eps | precise            (grid.x = head)
     kFamRmsNormGatedBatched,     // x gate w y heads_per_token | head_dim eps precise (grid = heads x tokens)
     kFamRmsNormGatedPlanes,      // x gate w planes scales head_dim eps          (grid.x = head = 128-value group)
+    kFamUnary,                   // in out count [param] | ... op                 (threads grid)
+    kFamScalarMul,               // in out scalar count
+    kFamScalarMulWeight,         // in scalar out count
     kFamLutMatmul,               // W lut X Y cols group rows                    (grid.y = token)
     kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
     kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile

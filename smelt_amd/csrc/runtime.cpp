@@ -577,6 +577,17 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             L.lds = 64 + dim * 2;
             break;
         }
+        case kFamUnary:
+        case kFamScalarMul:
+        case kFamScalarMulWeight: {
+            const size_t count = U(r.family == kFamUnary ? 2 : 3);
+            if (L.block[1] != 1 || L.block[2] != 1 || L.grid[1] != 1 || L.grid[2] != 1) return bad_geom("1-D launch expected");
+            if ((size_t)L.grid[0] * L.block[0] < count) return bad_geom("grid covers " + std::to_string((size_t)L.grid[0] * L.block[0]) + " of " + std::to_string(count) + " elements");
+            need[0] = count * 2;
+            if (r.family == kFamScalarMulWeight) { need[1] = 2; need[2] = count * 2; written[2] = true; }
+            else { need[1] = count * 2; written[1] = true; }
+            break;
+        }
         case kFamElementwise:
         case kFamCopy16: {
             const size_t ci = r.family == kFamCopy16 ? 2 : 3;

@@ -355,3 +355,52 @@ def test_gated_norm_precise_batched_and_view(env, threads):
     assert np.array_equal(ctx.read(5, np.uint32, n * 24), fused_pl) and np.array_equal(ctx.read(6, np.uint16, n), fused_sc)
     ref_pl, ref_sc = so.rms_norm_gated_activation_bitplanes(x.ravel(), gate.ravel(), w, n, 1e-6, odt, threads == 32)
     assert np.mean(fused_pl == ref_pl.reshape(-1)) > 0.97 and np.mean(fused_sc == ref_sc) > 0.85
+
+
+def test_pointwise_activations(env):
+    """silu / sigmoid_kernel / softplus / scalar_mul / scalar_mul_weight / logit_cap / sigmoid_mul /
+    geglu_fused (activations.metal, activations_precise.metal:26-38) against the oracle: identical up to the
+    last bit of exp / tanh / log; scalar multiplies bit for bit."""
+    ctx, dtype, odt = env
+    rng = fx.rng_for(99, 1)
+    n = 5000
+    x = bits(rng.normal(0, 4, n).astype(np.float32), dtype)
+    y = bits(rng.normal(0, 2, n).astype(np.float32), dtype)
+    ctx.put(1, x); ctx.put(2, y); ctx.alloc(3, n * 2)
+    grid, tg = ((n + 255) // 256 * 256, 1, 1), (256, 1, 1)
+
+    def run(name, bufs, consts):
+        ctx.alloc(3, n * 2)
+        ctx.interpret_decode(ctx.table([rt.make_record(ctx.pipeline(name), bufs, consts, grid, tg, style=rt.STYLE_THREADS)])); ctx.wait()
+        return ctx.read(3, np.uint16, n)
+
+    for name in ("silu", "sigmoid_kernel", "softplus"):
+        assert_last_place(run(name, [(1, 0, 0), (3, 1, 0)], [(2, n)]), so.unary(name, x, odt), dtype, name, exact_fraction=0.97)
+    assert_last_place(run("logit_cap", [(1, 0, 0), (3, 1, 0)], [(2, n), (3, 30.0)]), so.unary("logit_cap", x, odt, 30.0), dtype,
+                      "logit_cap", exact_fraction=0.97)
+    assert np.array_equal(run("scalar_mul", [(1, 0, 0), (3, 1, 0)], [(2, 0.37), (3, n)]), so.unary("scalar_mul", x, odt, 0.37))
+    scalar = bits(np.float32([0.75]), dtype)
+    ctx.put(4, scalar)
+    assert np.array_equal(run("scalar_mul_weight", [(1, 0, 0), (4, 1, 0), (3, 2, 0)], [(3, n)]),
+                          so.unary("scalar_mul", x, odt, float(fx.from_bits(scalar, dtype)[0])))
+    assert_last_place(run("sigmoid_mul", [(1, 0, 0), (2, 1, 0), (3, 2, 0)], [(3, n)]), so.sigmoid_mul(x, y, odt), dtype, "sigmoid_mul",
+                      exact_fraction=0.97)
+    got = run("geglu_fused", [(1, 0, 0), (2, 1, 0), (3, 2, 0)], [(3, n)])
+    ref = so.epilogue_geglu(so.widen(x, odt), so.widen(y, odt), odt)
+    # 1 + tanh cancels for negative gates: absolute slack of 2^-22 |g u| beside the last place
+    g, r = fx.from_bits(got, dtype).astype(np.float64), so.widen(ref, odt).astype(np.float64)
+    slack = np.abs(so.widen(x, odt).astype(np.float64) * so.widen(y, odt).astype(np.float64)) * 2.0 ** -21
+    assert np.all(np.abs(g - r) <= gh.ulp_of(np.where(r == 0, 1e-30, r), dtype) + slack) and np.mean(got == ref) > 0.95
+    # fused sigmoid-mul view == sigmoid_mul then the plain i6 view, bit for bit on the device
+    cols = 4096
+    groups = cols // 128
+    ctx.alloc(5, groups * 6 * 16); ctx.alloc(6, groups * 2)
+    fused = rt.make_record(ctx.pipeline("sigmoid_mul_signed_activation_bitplanes_i6_g128"), [(1, 0, 0), (2, 1, 0), (5, 2, 0), (6, 3, 0)],
+                           [(4, cols)], (groups, 1, 1), (32, 1, 1))
+    ctx.interpret_decode(ctx.table([fused])); ctx.wait()
+    f_pl, f_sc = ctx.read(5, np.uint32, groups * 24), ctx.read(6, np.uint16, groups)
+    staged = [rt.make_record(ctx.pipeline("sigmoid_mul"), [(1, 0, 0), (2, 1, 0), (3, 2, 0)], [(3, cols)], (cols, 1, 1), (256, 1, 1), style=rt.STYLE_THREADS),
+              rt.make_record(ctx.pipeline("signed_activation_bitplanes_i6_g128"), [(3, 0, 0), (5, 1, 0), (6, 2, 0)], [(3, cols)], (groups, 1, 1), (32, 1, 1))]
+    ctx.alloc(5, groups * 6 * 16); ctx.alloc(6, groups * 2)
+    ctx.interpret_decode(ctx.table(staged)); ctx.wait()
+    assert np.array_equal(ctx.read(5, np.uint32, groups * 24), f_pl) and np.array_equal(ctx.read(6, np.uint16, groups), f_sc)

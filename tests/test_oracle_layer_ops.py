@@ -216,3 +216,23 @@ def test_gated_norm_precise_form_and_its_view():
         staged = so.activation_bitplanes(so.rms_norm_gated(x, gate, w, heads, d, 1e-6, so.F16, precise), 6, so.F16)
         fused = so.rms_norm_gated_activation_bitplanes(x, gate, w, heads, 1e-6, so.F16, precise)
         assert np.array_equal(staged[0], fused[0]) and np.array_equal(staged[1], fused[1])
+
+
+def test_pointwise_activations_closed_forms_and_float64():
+    """activations.metal:5-40, 98-108, 166-177."""
+    one = lambda name, v, p=0.0: float(so.widen(so.unary(name, f16([v]), so.F16, p), so.F16)[0])
+    assert one("silu", 0.0) == 0.0 and one("sigmoid_kernel", 0.0) == 0.5
+    assert one("softplus", 25.0) == 25.0 and abs(one("softplus", 0.0) - np.log(2)) < 1e-3      # x itself above 20
+    assert one("scalar_mul", 3.0, 0.25) == 0.75
+    assert abs(one("logit_cap", 0.01, 30.0) - 0.01) < 1e-5 and abs(one("logit_cap", 1000.0, 30.0) - 30.0) < 1e-2
+    rng = fx.rng_for(101, 0)
+    x = f16(rng.normal(0, 4, 4096))
+    xf = so.widen(x, so.F16).astype(np.float64)
+    refs = {"silu": xf / (1 + np.exp(-xf)), "sigmoid_kernel": 1 / (1 + np.exp(-xf)),
+            "softplus": np.where(xf > 20, xf, np.log1p(np.exp(xf))), "scalar_mul": xf * float(np.float32(0.37)),
+            "logit_cap": 30.0 * np.tanh(xf / 30.0)}
+    for name, ref in refs.items():
+        got = so.widen(so.unary(name, x, so.F16, 0.37 if name == "scalar_mul" else 30.0), so.F16).astype(np.float64)
+        ulp = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64)
+        assert np.all(np.abs(got - ref) <= ulp + 1e-7 * np.abs(xf)), name
+        assert np.mean(got == ref.astype(np.float16).astype(np.float64)) > 0.97, name
