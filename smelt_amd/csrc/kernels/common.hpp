@@ -62,7 +62,14 @@ struct NormScale {
     // norm_add_scale form (lut_matvec.metal:2896-2990): the rounded norm plus this row, added and
     // rounded in the 16-bit type, is what the kernel multiplies and stores
     const uint16_t* residual = nullptr;
+    // self_eps >= 0: there is no precomputed scale; the workgroup forms 1 / sqrt(mean(x^2) + self_eps)
+    // itself when it stages the row, and the launch's first workgroup publishes {scale, 1u} to `publish`
+    float self_eps = -1.0f;
+    float* publish = nullptr;
 };
+
+
+
 
 // (x * rs) * (1 + w) with each product and the sum rounded on its own: without the pragma the
 // compiler folds t * (1 + w) into fma(w, t, t), one rounding fewer than the staged norm performs.
@@ -146,5 +153,23 @@ __device__ __forceinline__ uint2_t wave_argmax_key(uint2_t k) {
 }
 
 __device__ __forceinline__ int ilog2(uint32_t v) { return 31 - __builtin_clz(v); }
+
+// 1 / sqrt(mean(x^2) + eps) of one row, every thread of the workgroup returning the same value:
+// threads stride over the row, waves reduce with DPP adds, wave totals meet in `wave_sums`.
+template <class ActT>
+__device__ __forceinline__ float row_inv_rms(const uint16_t* x, uint32_t cols, float eps, float* wave_sums) {
+    float sum = 0.0f;
+    for (uint32_t i = threadIdx.x; i < cols; i += blockDim.x) {
+        const float v = ActT::widen(x[i]);
+        sum = __builtin_fmaf(v, v, sum);
+    }
+    sum = group_sum_last<64>(sum);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == kWave - 1) wave_sums[wave] = sum;
+    __syncthreads();
+    float total = 0.0f;
+    for (int w = 0; w < (int)(blockDim.x / kWave); ++w) total += wave_sums[w];
+    return 1.0f / __builtin_sqrtf(total / (float)cols + eps);
+}
 
 }  // namespace smelt

@@ -255,6 +255,15 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
     constexpr int CPD = G::kColsPerDword;
     constexpr int DPU = G::kDPU;
     const int dwords = U * DPU;
+    float self_rs = 0.0f;
+    if (ns.self_eps >= 0.0f) {   // uniform over the workgroup; one token (b0) per launch
+        __shared__ float wave_sums[4];
+        self_rs = row_inv_rms<ActT>(x + (size_t)b0 * cols, (uint32_t)cols, ns.self_eps, wave_sums);
+        if (ns.publish != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+            ns.publish[0] = self_rs;
+            reinterpret_cast<uint32_t*>(ns.publish)[1] = 1u;
+        }
+    }
     for (int item = threadIdx.x; item < MB * dwords; item += blockDim.x) {
         const int b = item / dwords;
         const int D = item - b * dwords;
@@ -278,8 +287,8 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
                 v[i] = (b < nb && c < cols) ? x[(size_t)(b0 + b) * cols + c] : (uint16_t)0;
             }
         }
-        if (ns.rs != nullptr && b < nb) {
-            const float rs = ns.rs[b0 + b];
+        if ((ns.rs != nullptr || ns.self_eps >= 0.0f) && b < nb) {
+            const float rs = ns.self_eps >= 0.0f ? self_rs : ns.rs[b0 + b];
 #pragma unroll
             for (int i = 0; i < CPD; ++i) {
                 const int c = col0 + i;

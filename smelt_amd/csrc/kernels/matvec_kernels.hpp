@@ -261,24 +261,6 @@ __device__ __forceinline__ void matvec_body(const MatPtrs (&mats)[NMAT], const u
     else go(std::integral_constant<int, 16>{});
 }
 
-// 1 / sqrt(mean(x^2) + eps) of one row, every thread of the workgroup returning the same value:
-// threads stride over the row, waves reduce with DPP adds, wave totals meet in `wave_sums`.
-template <class ActT>
-__device__ __forceinline__ float row_inv_rms(const uint16_t* x, uint32_t cols, float eps, float* wave_sums) {
-    float sum = 0.0f;
-    for (uint32_t i = threadIdx.x; i < cols; i += blockDim.x) {
-        const float v = ActT::widen(x[i]);
-        sum = __builtin_fmaf(v, v, sum);
-    }
-    sum = group_sum_last<64>(sum);
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    if (lane == kWave - 1) wave_sums[wave] = sum;
-    __syncthreads();
-    float total = 0.0f;
-    for (int w = 0; w < (int)(blockDim.x / kWave); ++w) total += wave_sums[w];
-    return 1.0f / __builtin_sqrtf(total / (float)cols + eps);
-}
-
 template <class F>
 __device__ __forceinline__ int packed_row_stride(int cols, int group) {
     if (F::kPerDwordScale) return (((cols + 4) / 5) + 15) & ~15;  // trit5: 5 digits per byte, 16-byte rows
@@ -407,45 +389,33 @@ using u32 = uint32_t;
 
 // Norm fused into its consumer (fused_norm_matvec.metal:19-297).  The reference lets workgroup 0
 // compute the RMS scale and makes every other workgroup spin on a flag; here each workgroup sums the
-// squares of the (cache-resident, few-KB) row itself, so no workgroup waits on another.  Workgroup 0
+// squares of the (cache-resident, few-KB) row itself while its first weight loads are in flight, so no
+// workgroup waits on another.  Workgroup 0
 // still publishes the scale and the ready flag in the scratch pair the record binds.
 #define SMELT_AFFINE_FUSED_NORM(T, ACT, SC)                                                       \
     SMELT_KERNEL void smelt_atomic_norm_affine_matvec_##T(                                        \
         const u16* x, const u16* nw, u16* xn, const u8* W, const u16* S, const u16* B, u16* y,    \
         float* scratch, u32 rows, float eps, u32 cols, u32 group) {                               \
         using namespace smelt;                                                                    \
-        __shared__ float wave_sums[4];                                                            \
-        __shared__ float rs_lds[1];                                                               \
-        const float rs = row_inv_rms<ACT>(x, cols, eps, wave_sums);                               \
-        if (threadIdx.x == 0) {                                                                   \
-            rs_lds[0] = rs;                                                                       \
-            if (blockIdx.x == 0) { scratch[0] = rs; reinterpret_cast<u32*>(scratch)[1] = 1u; }    \
-        }                                                                                         \
-        __syncthreads();                                                                          \
         const MatPtrs mats[1] = {{W, S, B}};                                                      \
         EpiStore<ACT> epi{{}, y, (int)rows};                                                      \
         matvec_body<FmtU4, ACT, SC, 2, 1, 1>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group, 0, 1,  \
-                                             epi, nullptr, 0, NormScale{rs_lds, nw, xn});         \
+                                             epi, nullptr, 0,                                     \
+                                             NormScale{nullptr, nw, xn, nullptr, eps, scratch});  \
     }                                                                                             \
     SMELT_KERNEL void smelt_atomic_norm_affine_gate_up_swiglu_##T(                                \
         const u16* x, const u16* nw, const u8* gW, const u16* gS, const u16* gB, const u8* uW,    \
         const u16* uS, const u16* uB, u16* y, float* scratch, u32 rows, float eps, u32 cols,      \
         u32 group) {                                                                              \
         using namespace smelt;                                                                    \
-        __shared__ float wave_sums[4];                                                            \
-        __shared__ float rs_lds[1];                                                               \
-        const float rs = row_inv_rms<ACT>(x, cols, eps, wave_sums);                               \
-        if (threadIdx.x == 0) {                                                                   \
-            rs_lds[0] = rs;                                                                       \
-            if (blockIdx.x == 0) { scratch[0] = rs; reinterpret_cast<u32*>(scratch)[1] = 1u; }    \
-        }                                                                                         \
-        __syncthreads();                                                                          \
         const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
         EpiAffineSwiglu<ACT> epi{{}, y, (int)rows};                                               \
         matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
                                              packed_row_stride<FmtU4>(cols, group), group, 0, 1,  \
-                                             epi, nullptr, 0, NormScale{rs_lds, nw, nullptr});    \
+                                             epi, nullptr, 0,                                     \
+                                             NormScale{nullptr, nw, nullptr, nullptr, eps,        \
+                                                       scratch});                                 \
     }
 
 #define SMELT_AFFINE_BATCHED(T, ACT, SC, MBV)                                                     \
