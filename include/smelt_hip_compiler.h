@@ -152,6 +152,14 @@ int smelt_emit_norm_scale_matvec(smelt_emitter *e, int weights_slot, const Smelt
 int smelt_emit_norm_scale_gate_up(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *gate,
                                   const SmeltWeightEntryC *up, int geglu, SmeltBinding norm_scale,
                                   SmeltBinding input, SmeltBinding norm_weight, SmeltBinding output);
+/* AtomicNormFusionPass (SmeltDispatchOptimizer.swift:918-1046; kernels fused_norm_matvec.metal:19-297):
+ * rms_norm_1pw and its affine consumer in one dispatch.  up == NULL: matvec, the normalised row is also
+ * stored (norm_output required).  up != NULL: gate+up+SwiGLU, norm_output ignored.  scratch holds two
+ * 32-bit words {scale, ready flag}. */
+int smelt_emit_fused_norm_matvec(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w,
+                                 const SmeltWeightEntryC *up, SmeltBinding input, SmeltBinding norm_weight,
+                                 const SmeltBinding *norm_output, SmeltBinding output, SmeltBinding scratch,
+                                 float eps);
 /* fused_dual_affine_matvec: two weights, one input, two outputs */
 int smelt_emit_dual_matvec(smelt_emitter *e, int weights_slot, const SmeltWeightEntryC *w1,
                            const SmeltWeightEntryC *w2, SmeltBinding input, SmeltBinding output1,

@@ -76,6 +76,7 @@ def lib() -> C.CDLL:
         "smelt_emit_matvec_add": (i32, [vp, i32, we, Binding, Binding, Binding]),
         "smelt_emit_gate_up_swiglu": (i32, [vp, i32, we, we, Binding, Binding, i32, i32]),
         "smelt_emit_rms_norm_scale_only": (i32, [vp, Binding, Binding, i32, C.c_float, i32]),
+        "smelt_emit_fused_norm_matvec": (i32, [vp, i32, we, we, Binding, Binding, C.POINTER(Binding), Binding, Binding, C.c_float]),
         "smelt_emit_norm_scale_matvec": (i32, [vp, i32, we, Binding, Binding, Binding, Binding, Binding]),
         "smelt_emit_norm_scale_gate_up": (i32, [vp, i32, we, we, i32, Binding, Binding, Binding, Binding]),
         "smelt_emit_dual_matvec": (i32, [vp, i32, we, we, Binding, Binding, Binding]),
@@ -252,6 +253,12 @@ class Emitter:
     def norm_scale_gate_up(self, weights_slot, gate, up, scale, x, norm_weight, y, geglu=False):
         self._check(self.l.smelt_emit_norm_scale_gate_up(self.h, weights_slot, C.byref(gate), C.byref(up), int(geglu),
                                                          scale, x, norm_weight, y))
+
+    def fused_norm_matvec(self, weights_slot, w, x, norm_weight, y, scratch, norm_output=None, up=None, eps=1e-6):
+        """rms_norm_1pw + affine matvec (or gate+up+SwiGLU when `up` is given) in one dispatch."""
+        self._check(self.l.smelt_emit_fused_norm_matvec(self.h, weights_slot, C.byref(w), C.byref(up) if up is not None else None,
+                                                        x, norm_weight, C.byref(norm_output) if norm_output is not None else None,
+                                                        y, scratch, eps))
 
     def dual_matvec(self, weights_slot, w1, w2, x, y1, y2):
         self._check(self.l.smelt_emit_dual_matvec(self.h, weights_slot, C.byref(w1), C.byref(w2), x, y1, y2))

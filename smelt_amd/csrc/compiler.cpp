@@ -883,6 +883,41 @@ int smelt_emit_norm_scale_gate_up(smelt_emitter* e, int weights_slot, const Smel
     return SMELT_HIP_OK;
 }
 
+// AtomicNormFusionPass (SmeltDispatchOptimizer.swift:918-1046): rms_norm_1pw followed by its consumer
+// becomes one dispatch.  Matvec: 0 input, 1 norm weight, 2 normalised row out, 3..5 W S B, 6 output,
+// 7 scratch {scale, flag}, constants 8 rows, 9 eps.  up != NULL emits the gate+up+SwiGLU form: 0 input,
+// 1 norm weight, 2..7 weights, 8 output, 9 scratch, constants 10 rows, 11 eps (no normalised row out).
+int smelt_emit_fused_norm_matvec(smelt_emitter* e, int weights_slot, const SmeltWeightEntryC* w, const SmeltWeightEntryC* up,
+                                 SmeltBinding input, SmeltBinding norm_weight, const SmeltBinding* norm_output,
+                                 SmeltBinding output, SmeltBinding scratch, float eps) {
+    if (!e || !w) return efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "null emitter or weight");
+    if (!up && !norm_output) return efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "the matvec form stores the normalised row: bind it");
+    if (up && (w->dtype != up->dtype || w->rows != up->rows || w->cols != up->cols || w->group_size != up->group_size))
+        return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "gate and up projections must share dtype, shape and group size");
+    int family = 0;
+    if (int rc = gateway(e, w, SMELT_SHAPE_GEMV, up ? SMELT_FUSION_GATE_UP_SWIGLU : SMELT_FUSION_NONE, &family)) return rc;
+    if (family != SMELT_FAMILY_AFFINE_U4) return efail(e, SMELT_SELECT_MISSING, "the fused norm exists for affine_u4 weights only");
+    if (!affine_entry_ok(w) || (up && !affine_entry_ok(up))) return efail(e, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "unsupported affine geometry");
+    const MatvecGeometry g = matvec_geometry((uint32_t)w->cols / 2, w->rows, 2, e->compute_units);
+    RecordBuilder rb;
+    rb.buffer(0, input);
+    rb.buffer(1, norm_weight);
+    uint8_t next = 2;
+    if (!up) rb.buffer(next++, *norm_output);
+    bind_affine(rb, next, weights_slot, w);
+    next += 3;
+    if (up) { bind_affine(rb, next, weights_slot, up); next += 3; }
+    rb.buffer(next++, output);
+    rb.buffer(next++, scratch);
+    rb.constant(next++, (uint32_t)w->rows);
+    rb.constant_f32(next, eps);
+    rb.grid((uint32_t)g.grid_w, 1, 1, 256);
+    rb.r.pipeline = e->pipeline_index(std::string(up ? "atomic_norm_affine_gate_up_swiglu:" : "atomic_norm_affine_matvec:") +
+                                      std::to_string(w->cols) + ":" + std::to_string(w->group_size));
+    e->records.push_back(rb.r);
+    return SMELT_HIP_OK;
+}
+
 int smelt_emit_dual_matvec(smelt_emitter* e, int weights_slot, const SmeltWeightEntryC* w1, const SmeltWeightEntryC* w2,
                            SmeltBinding input, SmeltBinding output1, SmeltBinding output2) {
     if (!e || !w1 || !w2) return efail(e, SMELT_HIP_ERR_INVALID_ARGUMENT, "null emitter or weight");

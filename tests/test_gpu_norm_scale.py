@@ -199,6 +199,10 @@ def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
     # unfused: plain matvec / gate+up on the stored normalised row
     em.matvec(0, wq, cc.bind(XN), cc.bind(Q2))
     em.gate_up_swiglu(0, wg, wu, cc.bind(XN), cc.bind(F3))
+    # norm inside the consumer (one dispatch each)
+    XN2, Q3, F4, SCR = 10, 11, 12, 13
+    em.fused_norm_matvec(0, wq, cc.bind(X), cc.bind(NW), cc.bind(Q3), cc.bind(SCR), norm_output=cc.bind(XN2))
+    em.fused_norm_matvec(0, wg, cc.bind(X), cc.bind(NW), cc.bind(F4), cc.bind(SCR), up=wu)
     ctx = rt.Context(act_dtype=act)
     try:
         em.install(ctx)
@@ -206,9 +210,10 @@ def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
         x, w, _ = norm_inputs(1, hidden, dtype, seed=3)
         ctx.put(X, x); ctx.put(NW, w)
         ctx.alloc(SCALE, 4); ctx.alloc(XN, hidden * 2)
-        for slot, n in ((Q, rows), (Q2, rows), (F1, ffn), (F2, ffn), (F3, ffn)):
+        for slot, n in ((Q, rows), (Q2, rows), (F1, ffn), (F2, ffn), (F3, ffn), (XN2, hidden), (Q3, rows), (F4, ffn)):
             ctx.alloc(slot, n * 2)
-        assert ctx.interpret_decode(em.records()) == 6
+        ctx.alloc(SCR, 8)
+        assert ctx.interpret_decode(em.records()) == 8
         ctx.wait()
         rs = float(ctx.read(SCALE, np.float32, 1)[0])
         assert abs(rs - so.rms_scale(x[0], 1e-6, dtype)) <= 5e-6 * rs
@@ -216,6 +221,14 @@ def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
         assert np.array_equal(ctx.read(Q, np.uint16, rows), ctx.read(Q2, np.uint16, rows))
         assert np.array_equal(ctx.read(F1, np.uint16, ffn), ctx.read(F3, np.uint16, ffn))
         assert np.abs(fx.from_bits(ctx.read(F2, np.uint16, ffn), dtype)).max() > 0
+        # the in-kernel scale is summed in another order than rms_norm_scale_only's: last-place agreement
+        rs2 = float(ctx.read(SCR, np.float32, 1)[0])
+        assert abs(rs2 - rs) <= 2e-6 * rs and ctx.read(SCR, np.uint32, 2)[1] == 1
+        assert np.array_equal(ctx.read(XN2, np.uint16, hidden), so.norm_scale_input(x[0], rs2, w, dtype))
+        gh.check_outputs(ctx.read(Q3, np.uint16, rows).reshape(1, rows), fx.from_bits(ctx.read(Q, np.uint16, rows), dtype).reshape(1, rows),
+                         dtype, "fused norm matvec against the pair", rel_tol=4e-3 if dtype == fx.F16 else 1.6e-2)
+        gh.check_outputs(ctx.read(F4, np.uint16, ffn).reshape(1, ffn), fx.from_bits(ctx.read(F1, np.uint16, ffn), dtype).reshape(1, ffn),
+                         dtype, "fused norm gate+up against the pair", rel_tol=4e-3 if dtype == fx.F16 else 1.6e-2)
     finally:
         ctx.close()
 
