@@ -384,3 +384,43 @@ def test_bad_records_are_rejected_before_launch(ctx):
     # everything still works afterwards
     assert ctx.encode_decode(rt.make_record(pipe, good, [(5, rows)], (8, 1, 1), (256, 1, 1))) == 1
     ctx.wait()
+
+
+def test_fused_argmax_at_the_largest_vocabulary(ctx):
+    """The key holds 18 index bits (lut_matvec.metal:4048-4074): 262 144 rows is the largest table.
+    The winning row is planted first at the very last index, then duplicated at an earlier one
+    (identical rows give identical logits): the tie must go to the lower index."""
+    rows, cols, group, dtype = 1 << 18, 256, 64, fx.F16
+    rng = np.random.default_rng(7)
+    packed = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)
+    scales = fx.f16_bits(np.full((rows, cols // group), 0.01, np.float32))
+    biases = fx.f16_bits(np.full((rows, cols // group), -0.075, np.float32))
+    x = fx.f16_bits(np.abs(rng.normal(0, 1, (1, cols))).astype(np.float32))      # positive activations
+    packed[rows - 1] = 0xFF                                                       # largest code everywhere: the unique maximum
+    p1 = ctx.pipeline(f"affine_matvec_argmax_c{cols}_r{rows}_g{group}_batched")
+    p2 = ctx.pipeline(f"lm_head_argmax_reduce_r{rows}")
+    grid_w = 1024
+    for dup in (None, 123457):
+        if dup is not None:
+            packed[dup] = 0xFF
+        wf = gh.WeightFile()
+        offs = [wf.add(a) for a in (packed, scales, biases)]
+        ctx.upload_weights(0, wf.image())
+        ctx.put(gh.X_SLOT, x)
+        ctx.alloc(gh.AUX_SLOT, grid_w * 8)
+        ctx.alloc(gh.Y_SLOT, 4)
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.AUX_SLOT, 4, 0)]
+        r1 = rt.make_record(p1, bufs, [(5, 1), (6, 0.0)], (grid_w, 1, 1), (256, 1, 1))
+        r2 = rt.make_record(p2, [(gh.AUX_SLOT, 0, 0), (gh.Y_SLOT, 1, 0)], [(2, 1), (3, grid_w)], (1, 1, 1), (256, 1, 1))
+        assert ctx.interpret_decode(ctx.table([r1, r2])) == 2
+        ctx.wait()
+        assert int(ctx.read(gh.Y_SLOT, np.int32, 1)[0]) == (rows - 1 if dup is None else dup)
+    # one row more does not fit the key: the launch is refused, nothing runs
+    with pytest.raises(rt.SmeltHipError):
+        ctx.pipeline(f"affine_matvec_argmax_c{cols}_r{rows + 8}_g{group}_batched")
+        wf = gh.WeightFile()
+        offs = [wf.add(np.zeros((rows + 8, cols // 2), np.uint8)), wf.add(np.zeros((rows + 8, 4), np.uint16)), wf.add(np.zeros((rows + 8, 4), np.uint16))]
+        ctx.upload_weights(0, wf.image())
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.AUX_SLOT, 4, 0)]
+        ctx.encode_decode(rt.make_record(ctx.pipeline(f"affine_matvec_argmax_c{cols}_r{rows + 8}_g{group}_batched"), bufs,
+                                         [(5, 1), (6, 0.0)], (grid_w, 1, 1), (256, 1, 1)))
