@@ -85,6 +85,8 @@ def _declare(l: C.CDLL) -> None:
         "so_signed_matvec_mt": (i32, [i32, vp, i64, vp, vp, i32, i32, i32, i32, vp]),
         "so_signed_matvec_f64": (i32, [i32, vp, i64, vp, vp, i32, i32, i32, i32, i32, vp]),
         "so_ternary_affine_qmv": (None, [vp, vp, vp, vp, i32, i32, i32, vp]),
+        "so_ternary_affine_qmm_weights": (None, [vp, vp, vp, i32, i32, vp]),
+        "so_ternary_affine_qmm": (None, [vp, vp, vp, vp, i32, i32, i32, vp]),
         "so_epilogue_residual_add": (u16, [f32, u16, i32]),
         "so_epilogue_affine_swiglu": (u16, [f32, f32, i32]),
         "so_epilogue_geglu": (u16, [f32, f32, i32]),
@@ -319,6 +321,28 @@ def ternary_affine_qmv(packed, scales, x_bits, rows, cols):
     scales = np.ascontiguousarray(scales)
     lib().so_ternary_affine_qmv(_p(packed, np.uint8), _p(scales, np.uint16), _p(scales, np.uint16),
                                 _p(x, np.uint16), rows, cols, x.shape[0], _p(out, np.uint16))
+    return out
+
+
+def ternary_affine_qmm_weights(packed, scales, rows, cols, bias_scales=None):
+    """fp16 bits [rows, cols] of the QMM weight tile with per-byte-lane rounded subscales."""
+    packed = np.ascontiguousarray(packed)
+    scales = np.ascontiguousarray(scales)
+    bias_scales = scales if bias_scales is None else np.ascontiguousarray(bias_scales)
+    out = np.zeros((rows, cols), np.uint16)
+    lib().so_ternary_affine_qmm_weights(_p(packed, np.uint8), _p(scales, np.uint16),
+                                        _p(bias_scales, np.uint16), rows, cols, _p(out, np.uint16))
+    return out
+
+
+def ternary_affine_qmm(packed, scales, x_bits, rows, cols, bias_scales=None):
+    x = np.ascontiguousarray(np.atleast_2d(x_bits), dtype=np.uint16)
+    packed = np.ascontiguousarray(packed)
+    scales = np.ascontiguousarray(scales)
+    bias_scales = scales if bias_scales is None else np.ascontiguousarray(bias_scales)
+    out = np.zeros((x.shape[0], rows), np.float32)
+    lib().so_ternary_affine_qmm(_p(packed, np.uint8), _p(scales, np.uint16), _p(bias_scales, np.uint16),
+                                _p(x, np.uint16), rows, cols, x.shape[0], _p(out, np.float32))
     return out
 
 

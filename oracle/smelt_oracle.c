@@ -15,6 +15,8 @@
  *   - binary1/ternary2 codec ...... SmeltSignedQuantCodecTests.swift:16-107
  *   - MLX scale normalisation ..... SmeltSignedQuantCodecTests.swift:109-204
  *   - ternary affine QMV .......... MLX golden bits, SignedQuantKernelTests.swift:87-199
+ *   - ternary affine QMM .......... MLX golden bits, SignedQuantKernelTests.swift:527-601, and
+ *                                   an independent numpy float16 evaluation of the weight tile
  *   - affine / signed matvec ...... exact-rational recomputation on dyadic fixtures,
  *                                   brute-force dequant-then-dot cross-check
  *   - argmax key .................. special cases (ties, signed zero) + brute force
@@ -28,6 +30,7 @@
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #define SO_EXPORT __attribute__((visibility("default")))
@@ -592,6 +595,67 @@ SO_EXPORT void so_ternary_affine_qmv(const uint8_t *codes, const uint16_t *scale
             out[(size_t)b * rows + r] = so_f32_to_f16(lane_result[0]);
         }
     }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Ternary "affine" QMM weight tile, the arithmetic of MLX affine_qmm_t<half,128,2> */
+/* signed_quant_precise.metal:407-439. Each two-bit field stays at its position */
+/* inside the byte; byte lane k multiplies it by a separately rounded fp16      */
+/* subscale fp16(scale / 4^k) and adds -bias_scale, all in half arithmetic.     */
+/* (The product of a subscale and a shifted ternary field is exact in fp16, so   */
+/* a fused and an unfused half multiply-add round identically.)                */
+/* out_bits: fp16 [rows, cols].                                               */
+/* ------------------------------------------------------------------------- */
+static float f64_to_f32_round_odd(double v) {
+    float f = (float)v;
+    if ((double)f == v || v != v) return f;
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if (fabs((double)f) > fabs(v)) u -= 1; /* back to the truncated magnitude */
+    u |= 1u;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+SO_EXPORT void so_ternary_affine_qmm_weights(const uint8_t *codes, const uint16_t *scales,
+                                             const uint16_t *bias_scales, int rows, int cols,
+                                             uint16_t *out_bits) {
+    const int G = 128;
+    int groups = cols / G;
+    int row_bytes = cols / 4;
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < cols; ++c) {
+            size_t si = (size_t)r * groups + c / G;
+            float scale = h2f(scales[si]);
+            float bias = -h2f(bias_scales[si]);
+            int lane = c & 3;
+            float sub = lane == 0 ? scale : hround(scale / (float)(1 << (2 * lane)));
+            uint32_t field = (codes[(size_t)r * row_bytes + c / 4] >> (2 * lane)) & 3u;
+            /* widened product and sum are exact in double; one rounding to half
+             * (through a round-to-odd float so that the two-step narrowing cannot
+             * double-round when scale and bias_scale differ widely in magnitude) */
+            double v = (double)sub * (double)(field << (2 * lane)) + (double)bias;
+            out_bits[(size_t)r * cols + c] = so_f32_to_f16(f64_to_f32_round_odd(v));
+        }
+}
+
+/* QMM result over that tile (signed_quant_precise.metal:441-489): fp16 weights  */
+/* times fp16 activations accumulated in fp32 by the 8x8 matrix unit, whose       */
+/* internal order is not specified; restated as a double-precision dot rounded    */
+/* once to float. x fp16 bits [batch, cols]; out float [batch, rows].            */
+SO_EXPORT void so_ternary_affine_qmm(const uint8_t *codes, const uint16_t *scales,
+                                     const uint16_t *bias_scales, const uint16_t *x, int rows,
+                                     int cols, int batch, float *out) {
+    uint16_t *w = (uint16_t *)malloc((size_t)rows * cols * sizeof(uint16_t));
+    so_ternary_affine_qmm_weights(codes, scales, bias_scales, rows, cols, w);
+    for (int b = 0; b < batch; ++b)
+        for (int r = 0; r < rows; ++r) {
+            double acc = 0;
+            for (int c = 0; c < cols; ++c)
+                acc += (double)h2f(w[(size_t)r * cols + c]) * (double)h2f(x[(size_t)b * cols + c]);
+            out[(size_t)b * rows + r] = (float)acc;
+        }
+    free(w);
 }
 
 /* ------------------------------------------------------------------------- */

@@ -44,20 +44,29 @@ struct QmmU4 {
 };
 
 struct QmmTer2 {
-    static constexpr bool kHasBias = false;
+    static constexpr bool kHasBias = true;
     static __device__ __forceinline__ int row_stride(int cols) { return cols / 4; }
+    // signed_quant_precise.metal:407-439: the two-bit field keeps its position inside the byte;
+    // byte lane k multiplies it by its own fp16-rounded subscale fp16(scale / 4^k) and adds
+    // -bias_scale. For scales whose quarter/sixteenth/sixty-fourth is not an fp16 value (small
+    // scales reaching the subnormal range) this differs from (code - 1) * scale in the last bits.
+    // The half-precision fused multiply-add rounds the exact value once; the unfused half form
+    // gives the same bits because a subscale times a shifted ternary field is exact in fp16.
     template <class ScaleT>
     static __device__ __forceinline__ void dequant32(const uint8_t* row, int k, const uint16_t* srow,
-                                                     const uint16_t*, int gshift, uint16_t* out) {
+                                                     const uint16_t* brow, int gshift, uint16_t* out) {
         const uint2_t c = *reinterpret_cast<const uint2_t*>(row + k / 4);
         const uint32_t w[2] = {c.x, c.y};
-        const float s = F16::widen(srow[k >> gshift]);
+        const _Float16 s = __builtin_bit_cast(_Float16, srow[k >> gshift]);
+        const _Float16 nb = -__builtin_bit_cast(_Float16, brow[k >> gshift]);
+        const _Float16 sub[4] = {s, s * (_Float16)0.25f, s * (_Float16)0.0625f, s * (_Float16)0.015625f};
 #pragma unroll
         for (int d = 0; d < 2; ++d)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const float v = (float)((int)((w[d] >> (2 * i)) & 3u) - 1);
-                out[16 * d + i] = F16::narrow(__fmul_rn(v, s));
+                const int lane = i & 3;
+                const _Float16 field = (_Float16)(int)(((w[d] >> (2 * i)) & 3u) << (2 * lane));
+                out[16 * d + i] = __builtin_bit_cast(uint16_t, __builtin_fmaf16(sub[lane], field, nb));
             }
     }
 };

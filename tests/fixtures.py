@@ -60,6 +60,16 @@ def mlx_ternary_fixture(rows: int, cols: int, batch: int, scale_unit: float):
     return codes, scales, x
 
 
+def mlx_ternary_qmm_fixture(rows: int, cols: int, batch: int, scale_bits):
+    """SignedQuantKernelTests.swift:527-546 — same codes and activations as above, scales
+    cycling through a list of fp16 bit patterns."""
+    codes, _, x = mlx_ternary_fixture(rows, cols, batch, 1.0)
+    groups = cols // 128
+    pool = np.array([int(b, 16) if isinstance(b, str) else int(b) for b in scale_bits], np.uint16)
+    scales = pool[np.arange(rows * groups) % pool.size].reshape(rows, groups)
+    return codes, scales, x
+
+
 def signed_synthetic_fixture(fmt: int, rows=5, cols=256, batch=5):
     """SignedQuantKernelTests.swift:989-1016 — binary (13r+7c)&1, ternary (13r+7c)%3,
     scales 0.03125*(i%5+1), x[i] = sin(17i+3)*0.75 (fp32 sin, rounded to fp16)."""

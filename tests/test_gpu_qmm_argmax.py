@@ -154,6 +154,42 @@ def test_ternary_qmm_matches_per_row_matvec_and_oracle(ctx):
     gh.check_outputs(y_mv, ref[:5], fx.F16, "ternary qmv")
 
 
+def test_ternary_qmm_reproduces_mlx_golden_bits_and_byte_lane_subscales(ctx):
+    """SignedQuantKernelTests.swift:527-601: the 112 bit patterns MLX's affine_qmm_t gives for
+    M=14, and the same shape with scales small enough that scale/16 and scale/64 round in the
+    fp16 subnormal range (signed_quant_precise.metal:407-439). Every fp32 partial sum of both
+    fixtures is exact, so summation order cannot matter and the bits must be equal; on the
+    second fixture (code - 1) * scale would miss by up to 6 % on the small outputs."""
+    case = fx.golden_vectors()["ternary_qmm_mlx_m14"]
+    rows, cols, batch = case["rows"], case["cols"], case["batch"]
+    golden = np.array([int(b, 16) for b in case["expected_bits"]], np.uint16)
+    small = ["1b95", "1797", "1b93", "17ff", "1a01"]
+    for scale_bits, want, separate_bias in ((case["scale_bits"], golden, False), (small, None, False),
+                                            (small, None, True)):
+        codes, scales, x = fx.mlx_ternary_qmm_fixture(rows, cols, batch, scale_bits)
+        bias_scales = np.roll(scales, 1, axis=0) if separate_bias else scales
+        packed = fx.pack_signed_np(codes, fx.TERNARY2)
+        ref = so.ternary_affine_qmm(packed, scales, x, rows, cols, bias_scales=bias_scales)
+        ref_bits = ref.astype(np.float16).view(np.uint16).ravel()
+        if want is None:
+            want = ref_bits
+            naive = so.signed_matvec(so.TERNARY2, packed, scales, fx.from_bits(x, fx.F16), rows, cols, cols, 128)
+            assert (naive.astype(np.float16).view(np.uint16).ravel() != want).sum() > 40
+        else:
+            assert np.array_equal(ref_bits, want)
+        wf = gh.WeightFile()
+        oc, os_, ob = wf.add(packed), wf.add(scales), wf.add(bias_scales)
+        ctx.upload_weights(0, wf.image())
+        ctx.put(gh.X_SLOT, x)
+        ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+        ctx.encode_decode(rt.make_record(
+            ctx.pipeline("signed_ternary_affine_qmm_g128_bm32_bn32_bk32"),
+            [(0, 0, oc), (0, 1, os_), (0, 2, ob), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)],
+            [(5, rows), (6, cols), (7, batch)], (1, 1, 1), (256, 1, 1)))
+        ctx.wait()
+        assert np.array_equal(ctx.read(gh.Y_SLOT, np.uint16, want.size), want), (scale_bits, separate_bias)
+
+
 def test_lm_head_argmax_fused_and_staged(ctx):
     """Identical argmax over the lm_head row block: fused matvec+argmax, and argmax over the
     materialised logits, both equal the oracle's argmax of its rounded logits."""

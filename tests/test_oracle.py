@@ -299,6 +299,67 @@ def test_ternary_affine_qmv_reproduces_mlx_golden_bits():
                 assert np.float16(float(acc)).view(np.uint16) == want[b * case["rows"] + r]
 
 
+def _exact_qmm_bits(w_bits, x_bits):
+    """fp16 outputs [batch, rows] of fp16 weights times fp16 activations with an exact
+    rational sum and one rounding to half."""
+    w = w_bits.view(np.float16)
+    x = x_bits.view(np.float16)
+    out = np.zeros((x.shape[0], w.shape[0]), np.uint16)
+    for b in range(x.shape[0]):
+        for r in range(w.shape[0]):
+            acc = sum((Fraction(float(a)) * Fraction(float(v)) for a, v in zip(x[b], w[r])), Fraction(0))
+            # float(acc) is exact here: every product is a multiple of 2^-28 and |acc| < 2
+            assert Fraction(float(acc)) == acc
+            out[b, r] = np.float16(float(acc)).view(np.uint16)
+    return out
+
+
+def test_ternary_affine_qmm_reproduces_mlx_golden_bits():
+    """The 112 bit patterns MLX's affine_qmm_t produced (SignedQuantKernelTests.swift:549-568).
+    Every fp32 partial sum of this fixture is exact, so the unspecified order inside the matrix
+    unit does not matter and one rounding of the exact sum must give the same bits."""
+    case = fx.golden_vectors()["ternary_qmm_mlx_m14"]
+    rows, cols, batch = case["rows"], case["cols"], case["batch"]
+    codes, scales, x = fx.mlx_ternary_qmm_fixture(rows, cols, batch, case["scale_bits"])
+    packed = so.signed_pack(codes, so.TERNARY2)
+    want = np.array([int(b, 16) for b in case["expected_bits"]], np.uint16).reshape(batch, rows)
+    w = so.ternary_affine_qmm_weights(packed, scales, rows, cols)
+    assert np.array_equal(_exact_qmm_bits(w, x), want)
+    out = so.ternary_affine_qmm(packed, scales, x, rows, cols)
+    assert np.array_equal(out.astype(np.float16).view(np.uint16), want)
+
+
+def test_ternary_affine_qmm_weight_tile_uses_rounded_byte_lane_subscales():
+    """signed_quant_precise.metal:407-439 against an independent numpy float16 evaluation, on
+    scales whose /16 and /64 fall into the fp16 subnormal range with bits to lose: there the
+    tile is not (code - 1) * scale, and a zero code does not dequantise to exactly zero."""
+    rows, cols = 8, 256
+    scale_bits = ["1b95", "1797", "0c01", "13ff", "2057", "0801"]
+    codes, scales, _ = fx.mlx_ternary_qmm_fixture(rows, cols, 1, scale_bits)
+    packed = so.signed_pack(codes, so.TERNARY2)
+    got = so.ternary_affine_qmm_weights(packed, scales, rows, cols)
+    s = np.repeat(scales.view(np.float16), 128, axis=1)
+    lane = (np.arange(cols) & 3)[None, :]
+    sub = s.copy()
+    for k in (1, 2, 3):
+        sub = np.where(lane == k, s / np.float16(4 ** k), sub)       # float16 division: rounds once
+    assert sub.dtype == np.float16
+    shifted = (codes.astype(np.int32) << (2 * lane)).astype(np.float16)
+    prod = sub * shifted                                             # exact for fields 0, 1, 2
+    assert np.array_equal(prod.astype(np.float64), sub.astype(np.float64) * shifted.astype(np.float64))
+    want = (prod.astype(np.float64) - s.astype(np.float64)).astype(np.float16)  # exact sum, one rounding
+    assert np.array_equal(got, want.view(np.uint16))
+    naive = ((codes.astype(np.float32) - 1) * s.astype(np.float32)).astype(np.float16)
+    differs = got != naive.view(np.uint16)
+    assert differs.any() and not differs[:, lane[0] == 0].any()
+    assert (got.view(np.float16)[codes == 1] != 0).any()
+    # a separate bias buffer is honoured (binding 2 of the reference kernel)
+    other = np.roll(scales, 1, axis=1)
+    got2 = so.ternary_affine_qmm_weights(packed, scales, rows, cols, bias_scales=other)
+    want2 = (prod.astype(np.float64) - np.repeat(other.view(np.float16), 128, axis=1).astype(np.float64))
+    assert np.array_equal(got2, want2.astype(np.float16).view(np.uint16))
+
+
 @pytest.mark.parametrize("fmt", [so.BINARY1, so.TERNARY2, so.TRIT5])
 def test_signed_matvec_against_numpy_dequant_dot(fmt):
     base = fx.TERNARY2 if fmt == so.TRIT5 else fmt
