@@ -66,22 +66,37 @@ constexpr float kTqhInvSqrtG = 0.0883883476483184405f;
             }                                                                                      \
             for (uint32_t u = lane; u < units; u += kWave) {                                       \
                 const uint32_t g = u >> 1;                                                         \
-                const float cb0 = F16::widen(codebook[g * 4u]), cb1 = F16::widen(codebook[g * 4u + 1u]);      \
-                const float cb2 = F16::widen(codebook[g * 4u + 2u]), cb3 = F16::widen(codebook[g * 4u + 3u]); \
+                /* the group's four fp16 entries as a byte table: low bytes in one dword, high */  \
+                /* bytes in another, so that one byte permute looks up four codes at once */       \
+                const uint2_t cbw = *reinterpret_cast<const uint2_t*>(codebook + g * 4u);          \
+                const uint32_t cb_lo = __builtin_amdgcn_perm(cbw.y, cbw.x, 0x06040200u);           \
+                const uint32_t cb_hi = __builtin_amdgcn_perm(cbw.y, cbw.x, 0x07050301u);           \
                 uint4_t c[4];                                                                      \
                 _Pragma("unroll") for (int r = 0; r < 4; ++r)                                      \
                     c[r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(codes + (size_t)row[r] * codes_per_row + (size_t)u * 16u)); \
                 const float4_t* xv4 = reinterpret_cast<const float4_t*>(lds_x + (size_t)u * 64u);  \
-                _Pragma("unroll") for (int q = 0; q < 16; ++q) {                                   \
-                    const float4_t xv = xv4[q];                                                    \
-                    const float xs[4] = {xv.x, xv.y, xv.z, xv.w};                                  \
+                _Pragma("unroll") for (int d = 0; d < 4; ++d) {                                    \
+                    /* xs[i][k] = xhat of column 16 d + 4 i + k of this unit */                    \
+                    float xs[4][4];                                                                \
+                    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                \
+                        const float4_t xv = xv4[4 * d + i];                                        \
+                        xs[i][0] = xv.x; xs[i][1] = xv.y; xs[i][2] = xv.z; xs[i][3] = xv.w;        \
+                    }                                                                              \
                     _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                \
                         const uint32_t words[4] = {c[r].x, c[r].y, c[r].z, c[r].w};                \
-                        const uint32_t byte = (words[q >> 2] >> (8 * (q & 3))) & 0xFFu;            \
                         _Pragma("unroll") for (int k = 0; k < 4; ++k) {                            \
-                            const uint32_t code = (byte >> (2 * k)) & 3u;                          \
-                            const float w = (code & 2u) ? ((code & 1u) ? cb3 : cb2) : ((code & 1u) ? cb1 : cb0); \
-                            acc[r] = __builtin_fmaf(w, xs[k], acc[r]);                             \
+                            /* byte i of sel = code of column 4 i + k (byte i of the dword) */     \
+                            const uint32_t sel = (words[d] >> (2 * k)) & 0x03030303u;              \
+                            const uint32_t lo = __builtin_amdgcn_perm(0u, cb_lo, sel);             \
+                            const uint32_t hi = __builtin_amdgcn_perm(0u, cb_hi, sel);             \
+                            const uint32_t w01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);       \
+                            const uint32_t w23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);       \
+                            const half2_t p01 = __builtin_bit_cast(half2_t, w01);                  \
+                            const half2_t p23 = __builtin_bit_cast(half2_t, w23);                  \
+                            acc[r] = __builtin_fmaf((float)p01.x, xs[0][k], acc[r]);               \
+                            acc[r] = __builtin_fmaf((float)p01.y, xs[1][k], acc[r]);               \
+                            acc[r] = __builtin_fmaf((float)p23.x, xs[2][k], acc[r]);               \
+                            acc[r] = __builtin_fmaf((float)p23.y, xs[3][k], acc[r]);               \
                         }                                                                          \
                     }                                                                              \
                 }                                                                                  \

@@ -660,7 +660,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             if (L.block[0] % 64 != 0 || L.block[0] > 256 || L.block[1] != 1 || L.block[2] != 1 || L.grid[2] != 1)
                 return bad_geom("tqh_matvec runs 64..256 threads in whole waves");
             need[0] = rows * cpr; align[0] = 16;
-            need[1] = groups * 8;
+            need[1] = groups * 8; align[1] = 8;
             need[2] = gy * groups * 128 * 4; align[2] = 16;
             need[3] = gy * rows * 2; written[3] = true;
             L.lds = groups * 128 * 4;
