@@ -209,8 +209,8 @@ def committed_traffic():
 
 
 def side_measurements(ctx, fx, cc, rt, cus) -> dict:
-    """27B-layer binary / ternary / trit5 matvec sets, the 4B FFN qmm at M in {7,8,9,32,512} and the
-    affine 4-bit quantiser.  Reported beside the headline; not part of `value`."""
+    """27B-layer binary / ternary / trit5 matvec sets, the 4B FFN qmm at M in {7,8,9,32,512}, the
+    affine 4-bit quantiser and a turbo_quant_h matvec.  Reported beside the headline; not part of `value`."""
     out = {}
     W, X, Y, ACT = 20, 21, 22, 23
     shapes = [(17408, 5120), (17408, 5120), (5120, 17408), (5120, 5120), (5120, 5120), (1024, 5120), (1024, 5120)]
@@ -351,6 +351,39 @@ def side_measurements(ctx, fx, cc, rt, cus) -> dict:
             quant[f"{src_name}_{clip_name}"] = {"us": round(us, 1), "GBps": round(moved / us / 1e3, 1),
                                                "Gweights_per_s": round(rows * cols / us / 1e3, 2)}
     out["affine_quantize_u4_9216x2560_g64"] = quant
+    c.close()
+    # turbo_quant_h matvec (2-bit codes, four-entry codebook per 128 columns) over a 65536 x 2560 matrix
+    c = rt.Context(act_dtype=rt.ACT_F16)
+    rows, cols = 65536, 2560
+    groups = cols // 128
+    rng = fx.rng_for(6, 0)
+    copies = 4
+    image = bytearray()
+    offs = []
+    for _ in range(copies):
+        codes = rng.integers(0, 256, (rows, groups * 32), dtype=np.uint8)
+        book = fx.f16_bits(np.sort(rng.normal(0, 0.1, (groups, 4)).astype(np.float32), axis=1))
+        offs.append((len(image), len(image) + codes.nbytes))
+        image += codes.tobytes() + book.tobytes() + bytes(-(codes.nbytes + book.nbytes) % 256)
+    c.upload_weights(W, np.frombuffer(bytes(image), np.uint8))
+    del image
+    c.put(X, fx.f16_bits(rng.normal(0, 1, cols).astype(np.float32)))
+    c.alloc(ACT, groups * 128 * 4)
+    c.alloc(Y, rows * 2)
+    prep = rt.make_record(c.pipeline("tqh_matvec_prepare_input"), [(X, 0, 0), (ACT, 1, 0)], [(2, cols)],
+                          (groups * 128, 1, 1), (128, 1, 1), style=rt.STYLE_THREADS)
+    c.interpret_decode(c.table([prep]))
+    c.wait()
+    mv = c.pipeline("tqh_matvec")
+    recs = [rt.make_record(mv, [(W, 0, a), (W, 1, b), (ACT, 2, 0), (Y, 3, 0)],
+                           [(4, rows), (5, cols), (6, groups * 32)], (cus * 8, 1, 1), (256, 1, 1)) for a, b in offs]
+    g, n = c.capture_decode(c.table(recs * 4))
+    c.graph_time(g, 2)
+    us = c.graph_time(g, 5) / (5 * n)
+    c.graph_destroy(g)
+    code_bytes = rows * groups * 32
+    out["tqh_matvec_65536x2560"] = {"us": round(us, 2), "code_GBps": round(code_bytes / us / 1e3, 1),
+                                    "pct_of_hbm_peak": round(100 * code_bytes / us / 1e3 / HBM_PEAK_GBS, 2)}
     c.close()
     return out
 
