@@ -223,6 +223,28 @@ __device__ __forceinline__ void rms_norm_from_fp32_row(const float* x, const uin
         const float gelu = 0.5f * g * (1.0f + tanhf(inner));                                      \
         out[i] = ACT::narrow(fminf(fmaxf(gelu * u, -65504.0f), 65504.0f));                        \
     }                                                                                             \
+    /* the same over [batch, count] with the up operand at its own row stride; grid.y = token       \
+       (activations.metal:142-163) */                                                             \
+    SMELT_LAYER_KERNEL void smelt_geglu_fused_strided_batched_##T(                                \
+        const uint16_t* gate, const uint16_t* up, uint16_t* out, uint32_t count,                  \
+        uint32_t up_stride) {                                                                     \
+        const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \
+        if (i >= count) return;                                                                   \
+        const size_t at = (size_t)blockIdx.y * count + i;                                         \
+        const float g = ACT::widen(gate[at]), u = ACT::widen(up[(size_t)blockIdx.y * up_stride + i]); \
+        float inner = 0.7978845608f * (g + 0.044715f * (g * g * g));                              \
+        inner = fminf(fmaxf(inner, -20.0f), 20.0f);                                               \
+        const float gelu = 0.5f * g * (1.0f + tanhf(inner));                                      \
+        out[at] = ACT::narrow(fminf(fmaxf(gelu * u, -65504.0f), 65504.0f));                       \
+    }                                                                                             \
+    /* out[token, row] = in[token, row] + bias[row]; grid.y = token (activations.metal:69-82) */  \
+    SMELT_LAYER_KERNEL void smelt_projection_bias_add_batched_##T(                                \
+        const uint16_t* in, const uint16_t* bias, uint16_t* out, uint32_t rows) {                 \
+        const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \
+        if (i >= rows) return;                                                                    \
+        const size_t at = (size_t)blockIdx.y * rows + i;                                          \
+        out[at] = ACT::narrow(ACT::widen(in[at]) + ACT::widen(bias[i]));                          \
+    }                                                                                             \
     SMELT_LAYER_KERNEL void smelt_elementwise_add_##T(const uint16_t* a, const uint16_t* b,       \
                                                       uint16_t* out, uint32_t count) {            \
         const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;                                 \

@@ -547,6 +547,14 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
             out->family = kFamElementwise; out->symbol = "smelt_" + entry + "_" + t; out->kinds = "PPPU";
             return kResolveOk;
         }
+        if (entry == "geglu_fused_strided_batched") {
+            out->family = kFamGegluStridedBatched; out->symbol = "smelt_geglu_fused_strided_batched_" + t; out->kinds = "PPPUU";
+            return kResolveOk;
+        }
+        if (entry == "projection_bias_add_batched") {
+            out->family = kFamBiasAddBatched; out->symbol = "smelt_projection_bias_add_batched_" + t; out->kinds = "PPPU";
+            return kResolveOk;
+        }
         if (entry == "silu" || entry == "sigmoid_kernel" || entry == "softplus") {
             out->family = kFamUnary; out->symbol = "smelt_unary_" + t; out->kinds = "PPUUU";
             out->appended = {0u, entry == "silu" ? 0u : (entry == "sigmoid_kernel" ? 1u : 2u)};

@@ -84,6 +84,8 @@ enum FamilyId {
     kFamScalarMul,               // in out scalar count
     kFamScalarMulWeight,         // in scalar out count
     kFamLutMatmul,               // W lut X Y cols group rows                    (grid.y = token)
+    kFamGegluStridedBatched,     // gate up out count up_stride                  (threads grid, grid.y = token)
+    kFamBiasAddBatched,          // in bias out rows                             (threads grid, grid.y = token)
     kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
     kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile
     kFamCount

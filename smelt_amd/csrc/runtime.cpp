@@ -588,6 +588,18 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             else { need[1] = count * 2; written[1] = true; }
             break;
         }
+        case kFamGegluStridedBatched:
+        case kFamBiasAddBatched: {
+            const bool geglu = r.family == kFamGegluStridedBatched;
+            const size_t count = U(3), stride = geglu ? U(4) : 0;
+            if (L.block[1] != 1 || L.block[2] != 1 || L.grid[2] != 1) return bad_geom("threads x tokens launch expected");
+            if (count == 0 || gy == 0) return bad_geom("count and token rows must be positive");
+            if ((size_t)L.grid[0] * L.block[0] < count) return bad_geom("grid covers " + std::to_string((size_t)L.grid[0] * L.block[0]) + " of " + std::to_string(count) + " elements");
+            need[0] = gy * count * 2;
+            need[1] = geglu ? ((gy - 1) * stride + count) * 2 : count * 2;
+            need[2] = gy * count * 2; written[2] = true;
+            break;
+        }
         case kFamElementwise:
         case kFamCopy16: {
             const size_t ci = r.family == kFamCopy16 ? 2 : 3;

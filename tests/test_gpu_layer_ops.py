@@ -404,3 +404,49 @@ def test_pointwise_activations(env):
     ctx.alloc(5, groups * 6 * 16); ctx.alloc(6, groups * 2)
     ctx.interpret_decode(ctx.table(staged)); ctx.wait()
     assert np.array_equal(ctx.read(5, np.uint32, groups * 24), f_pl) and np.array_equal(ctx.read(6, np.uint16, groups), f_sc)
+
+
+def test_batched_geglu_with_strided_up_and_batched_bias_add(env):
+    """geglu_fused_strided_batched (activations.metal:142-163): token b reads gate[b, :count] and
+    up[b * upStride : b * upStride + count]; it must equal the single-row geglu_fused applied to those
+    slices bit for bit on the device and stay within the last place of the oracle.
+    projection_bias_add_batched (activations.metal:69-82): bit-exact row-broadcast add."""
+    ctx, dtype, odt = env
+    rng = fx.rng_for(99, 7)
+    count, stride, batch = 1000, 1536, 5
+    gate = bits(rng.normal(0, 3, (batch, count)).astype(np.float32), dtype)
+    up = bits(rng.normal(0, 2, (batch, stride)).astype(np.float32), dtype)
+    ctx.put(1, gate); ctx.put(2, up); ctx.alloc(3, batch * count * 2)
+    grid, tg = ((count + 255) // 256 * 256, batch, 1), (256, 1, 1)
+    rec = rt.make_record(ctx.pipeline("geglu_fused_strided_batched"), [(1, 0, 0), (2, 1, 0), (3, 2, 0)],
+                         [(3, count), (4, stride)], grid, tg, style=rt.STYLE_THREADS)
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    got = ctx.read(3, np.uint16, batch * count).reshape(batch, count)
+    ref = so.epilogue_geglu(so.widen(gate, odt).ravel(), so.widen(up[:, :count], odt).ravel(), odt).reshape(batch, count)
+    g, r = fx.from_bits(got, dtype).astype(np.float64), so.widen(ref, odt).astype(np.float64)
+    slack = np.abs(so.widen(gate, odt).astype(np.float64) * so.widen(up[:, :count], odt).astype(np.float64)) * 2.0 ** -21
+    assert np.all(np.abs(g - r) <= gh.ulp_of(np.where(r == 0, 1e-30, r), dtype) + slack) and np.mean(got == ref) > 0.95
+    one = ctx.pipeline("geglu_fused")
+    for b in (0, batch - 1):
+        ctx.alloc(4, count * 2)
+        ctx.interpret_decode(ctx.table([rt.make_record(one, [(1, 0, b * count * 2), (2, 1, b * stride * 2), (4, 2, 0)], [(3, count)],
+                                                       ((count + 255) // 256 * 256, 1, 1), tg, style=rt.STYLE_THREADS)]))
+        ctx.wait()
+        assert np.array_equal(ctx.read(4, np.uint16, count), got[b])
+    # a stride shorter than the last row needs is caught before launch
+    ctx.alloc(5, ((batch - 1) * stride + count) * 2 - 2)
+    bad = rt.make_record(ctx.pipeline("geglu_fused_strided_batched"), [(1, 0, 0), (5, 1, 0), (3, 2, 0)],
+                         [(3, count), (4, stride)], grid, tg, style=rt.STYLE_THREADS)
+    with pytest.raises(rt.SmeltHipError):
+        ctx.interpret_decode(ctx.table([bad]))
+
+    rows = 777
+    x = bits(rng.normal(0, 4, (batch, rows)).astype(np.float32), dtype)
+    bias = bits(rng.normal(0, 1, rows).astype(np.float32), dtype)
+    ctx.put(1, x); ctx.put(2, bias); ctx.alloc(3, batch * rows * 2)
+    rec = rt.make_record(ctx.pipeline("projection_bias_add_batched"), [(1, 0, 0), (2, 1, 0), (3, 2, 0)], [(3, rows)],
+                         ((rows + 255) // 256 * 256, batch, 1), tg, style=rt.STYLE_THREADS)
+    ctx.interpret_decode(ctx.table([rec])); ctx.wait()
+    want = so.elementwise(x.ravel(), np.tile(bias, batch), odt)
+    assert np.array_equal(ctx.read(3, np.uint16, batch * rows), want)
+
