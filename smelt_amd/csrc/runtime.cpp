@@ -675,7 +675,18 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
             need[1] = groups * 8; align[1] = 8;
             need[2] = gy * groups * 128 * 4; align[2] = 16;
             need[3] = gy * rows * 2; written[3] = true;
-            L.lds = groups * 128 * 4;
+            {
+                // rotated activations at 272 bytes per 64-value unit (bank padding), then per wave one
+                // float4 of partial sums per (row quad, unit) item; the quad bound follows the kernel's
+                // own rule (tqh_max_quads_per_tile in tqh_kernels.hpp)
+                const size_t units = groups * 2, waves = L.block[0] / 64;
+                size_t low = units & (0 - units);
+                if (low > 64) low = 64;
+                size_t q = 64 / low;
+                if (q > 8) q = 8;
+                while (q > 1 && q * units * 16 * waves > 32768) q >>= 1;
+                L.lds = units * 17 * 16 + waves * q * units * 16;
+            }
             break;
         }
         case kFamTqhGather: {
