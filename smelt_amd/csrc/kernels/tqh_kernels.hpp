@@ -93,8 +93,9 @@ __device__ __forceinline__ void tqh_matvec_body(const uint8_t* codes, const uint
     const uint32_t units = groups * 2u;  // 16 bytes = 64 codes = half a group
     const uint32_t max_quads = tqh_max_quads_per_tile(units, waves);
     uint32_t quads = max_quads;
-    // keep at least one tile for every second wave of the grid
-    while (quads > 1u && (rows + quads * 4u - 1u) / (quads * 4u) < gridDim.x * waves / 2u) quads >>= 1;
+    // keep a tile for every launched wave, up to two waves per SIMD of the 256-CU part
+    const uint32_t want_tiles = gridDim.x * waves < 2048u ? gridDim.x * waves : 2048u;
+    while (quads > 1u && (rows + quads * 4u - 1u) / (quads * 4u) < want_tiles) quads >>= 1;
     if (quads == 1u) {
         // one quad per wave tile: lanes stride over the units, partial sums stay in registers
         const uint32_t tiles4 = (rows + 3u) / 4u;
