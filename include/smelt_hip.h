@@ -169,6 +169,20 @@ int smelt_hip_encode_decode_record(smelt_hip_context *ctx, const SmeltDispatchRe
  * grids :6186-6207, skip constants). */
 int smelt_hip_encode_prefill_record(smelt_hip_context *ctx, const SmeltDispatchRecord *rec,
                                     int cur, int alt, int32_t seq_len, int32_t start_pos);
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the same as
+ * smelt_hip_encode_prefill_record, except that kernels which split K across workgroups (the
+ * "_batched_skinny" qmm pipelines) keep their partial sums and arrival counters in a file-scope
+ * device array of the library instead of the workspace a context allocates, and the call itself
+ * allocates and frees nothing.  A record whose partials need more than
+ * SMELT_HIP_STATIC_SCRATCH_BYTES (4 KB per workgroup and matrix) or more than 16384 row tiles is
+ * rejected with SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY.  Each GPU holds one copy of the array for the
+ * life of the process, shared by every context on it: calls that overlap on one GPU (two streams)
+ * race; calls on one stream are ordered. */
+#define SMELT_HIP_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+int smelt_hip_encode_prefill_record_static_scratch(smelt_hip_context *ctx,
+                                                   const SmeltDispatchRecord *rec, int cur, int alt,
+                                                   int32_t seq_len, int32_t start_pos);
 /* interpretDispatchTable: SmeltRuntime.swift:3251-3275 / interpretPrefillDispatchTable
  * :6059-6084 — walks the records, flipping cur/alt (initially cur = cur0, alt = alt0) on
  * swap records.  Returns the number of kernels launched or a negative status. */

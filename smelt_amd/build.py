@@ -4,7 +4,8 @@
 
 Outputs (git-ignored, shipped to the GPU box as built files):
     smelt_amd/lib/smelt_kernels.hsaco   hipcc --genco, gfx950 only
-    smelt_amd/lib/libsmelt_hip.so       host runtime + record emitters (links libamdhip64)
+    smelt_amd/lib/libsmelt_hip.so       host runtime + record emitters (links libamdhip64); carries one
+                                        small gfx950 image of its own (static_scratch.hip)
 """
 from __future__ import annotations
 
@@ -43,8 +44,12 @@ def build_host() -> str:
     os.makedirs(LIB, exist_ok=True)
     srcs = [os.path.join(CSRC, s) for s in HOST_SOURCES if os.path.exists(os.path.join(CSRC, s))]
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    # the one host-library source with device code in it: the file-scope scratch array, its fill
+    # kernel and the entry point that uses them
+    scratch_obj = os.path.join(LIB, "static_scratch.o")
+    _run([HIPCC, *DEVICE_FLAGS, "-fPIC", "-c", "-o", scratch_obj, os.path.join(CSRC, "static_scratch.hip")])
     _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
-          "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", "-o", HOST_LIB, *srcs,
+          "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", "-o", HOST_LIB, *srcs, scratch_obj,
           f"-L{rocm}/lib", f"-Wl,-rpath,{rocm}/lib", "-lamdhip64", "-lpthread"])
     return HOST_LIB
 

@@ -13,6 +13,7 @@
 
 #include "../../include/smelt_hip.h"
 #include "pipeline_table.hpp"
+#include "runtime_internal.hpp"
 
 using namespace smelt_host;
 
@@ -103,8 +104,22 @@ struct Arg {
     bool writable = false;
 };
 
+// Argument list of one launch; fixed capacity, so encoding a record touches no heap.
+constexpr size_t kMaxLaunchArgs = 40;
+struct ArgList {
+    Arg items[kMaxLaunchArgs];
+    size_t count = 0;
+    size_t size() const { return count; }
+    void resize(size_t n) { count = n; }
+    void push_back(const Arg& a) { items[count++] = a; }
+    Arg& operator[](size_t i) { return items[i]; }
+    const Arg& operator[](size_t i) const { return items[i]; }
+    const Arg* begin() const { return items; }
+    const Arg* end() const { return items + count; }
+};
+
 struct Launch {
-    std::vector<Arg> args;
+    ArgList args;
     uint32_t grid[3];
     uint32_t block[3];
     size_t lds = 0;
@@ -114,12 +129,13 @@ size_t cdiv(size_t a, size_t b) { return (a + b - 1) / b; }
 
 // Checks operand extents against what the kernel will touch, and computes its LDS need.
 // Every hand-written kernel is only launched after this passes.
-int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
+int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const SplitKWorkspace& ws) {
     const ResolvedPipeline& r = p.res;
     auto U = [&](size_t i) -> size_t { return L.args[i].value; };
-    std::vector<size_t> need(L.args.size(), 0);
-    std::vector<bool> written(L.args.size(), false);
-    std::vector<size_t> align(L.args.size(), 2);
+    size_t need[kMaxLaunchArgs] = {};
+    bool written[kMaxLaunchArgs] = {};
+    size_t align[kMaxLaunchArgs];
+    for (size_t i = 0; i < kMaxLaunchArgs; ++i) align[i] = 2;
     const size_t gy = L.grid[1];
     auto bad_geom = [&](const std::string& m) {
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "pipeline '" + p.entry + "': " + m);
@@ -414,8 +430,10 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L) {
                 const uint32_t ksplit = (uint32_t)(L.grid[0] / tiles);
                 L.lds = qmm_skinny_lds_bytes((uint32_t)cols, ksplit, nmat, (uint32_t)std::min(batch, bt), L.block[0] / 64);
                 if (ksplit > 1) {
-                    if ((size_t)L.grid[0] * gy * nmat * 4096 > ctx->ws_partial_bytes || tiles * gy * 4 > ctx->ws_counter_bytes)
-                        return bad_geom("split-K partials exceed the context workspace");
+                    if ((size_t)L.grid[0] * gy * nmat * 4096 > ws.partial_bytes || tiles * gy * 4 > ws.counter_bytes)
+                        return bad_geom("split-K partials (" + std::to_string((size_t)L.grid[0] * gy * nmat * 4096) + " bytes, " +
+                                        std::to_string(tiles * gy) + " counters) exceed the workspace (" +
+                                        std::to_string(ws.partial_bytes) + " bytes, " + std::to_string(ws.counter_bytes / 4) + " counters)");
                 }
                 break;
             }
@@ -955,8 +973,12 @@ const Pipeline* pipeline_for(smelt_hip_context* ctx, uint32_t index) {
 }
 
 // Returns 1 launched, 0 skipped, <0 error.
-int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cur, int alt, const Dyn& d) {
+int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cur, int alt, const Dyn& d,
+                  const SplitKWorkspace* ws_override = nullptr) {
     if (!ctx || !rec) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or record");
+    SplitKWorkspace ws;
+    if (ws_override) ws = *ws_override;
+    else { ws.partial = ctx->ws_partial; ws.counters = ctx->ws_counters; ws.partial_bytes = ctx->ws_partial_bytes; ws.counter_bytes = ctx->ws_counter_bytes; }
     if (rec->op_kind != SMELT_OP_DISPATCH) return 0;
     if (d.prefill && rec->min_seq_len > 0 && (uint32_t)d.seq_len < (uint32_t)rec->min_seq_len) return 0;
     if (rec->buffer_count > SMELT_MAX_BUFFERS_PER_DISPATCH || rec->constant_count > SMELT_MAX_CONSTANTS_PER_DISPATCH)
@@ -965,6 +987,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     if (!p) return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "record names pipeline index " + std::to_string(rec->pipeline) + " which has no launchable kernel");
 
     const std::string& kinds = p->res.kinds;
+    if (kinds.size() + 1 > kMaxLaunchArgs)
+        return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "pipeline '" + p->entry + "' has too many arguments");
     Launch L;
     L.args.resize(kinds.size());
     const size_t own = kinds.size() - p->res.appended.size();
@@ -1030,7 +1054,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     }
     if ((size_t)L.block[0] * L.block[1] * L.block[2] > 1024)
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "threadgroup exceeds 1024 threads");
-    if (int e = validate_launch(ctx, *p, L)) return e;
+    if (int e = validate_launch(ctx, *p, L, ws)) return e;
     hipFunction_t fn = p->fn;
     if (p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
         // signed g128 matvec: large matrices run on the matrix cores (same bytes, same arguments + kw)
@@ -1062,8 +1086,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     }
     if (p->res.workspace) {
         pos = (pos + 7) & ~(size_t)7;
-        memcpy(kernarg + pos, &ctx->ws_partial, 8);
-        memcpy(kernarg + pos + 8, &ctx->ws_counters, 8);
+        memcpy(kernarg + pos, &ws.partial, 8);
+        memcpy(kernarg + pos + 8, &ws.counters, 8);
         pos += 16;
     }
     size_t kernarg_size = pos;
@@ -1096,6 +1120,20 @@ int interpret(smelt_hip_context* ctx, const SmeltDispatchRecord* table, size_t c
 
 }  // namespace
 
+namespace smelt_host {
+
+int encode_prefill_with_workspace(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cur, int alt,
+                                  int32_t seq_len, int32_t start_pos, const SplitKWorkspace& ws) {
+    Dyn d{true, 0, seq_len, start_pos};
+    return encode_record(ctx, rec, cur, alt, d, &ws);
+}
+
+int context_device(const smelt_hip_context* ctx) { return ctx->device; }
+hipStream_t context_stream(const smelt_hip_context* ctx) { return ctx->stream; }
+int context_fail(const smelt_hip_context* ctx, int code, const std::string& message) { return fail(ctx, code, message); }
+
+}  // namespace smelt_host
+
 extern "C" {
 
 int smelt_hip_context_create(int device_index, smelt_hip_context** out) {
@@ -1110,11 +1148,17 @@ int smelt_hip_context_create(int device_index, smelt_hip_context** out) {
     smelt_hip_context* ctx = new smelt_hip_context();
     ctx->device = device_index;
     ctx->slots.resize(64);
-    auto bail = [&](hipError_t err, const char* what) {
-        int rc = hip_fail(nullptr, err, what);
+    auto release = [&]() {
         if (ctx->ws_partial) (void)hipFree(ctx->ws_partial);
         if (ctx->ws_counters) (void)hipFree(ctx->ws_counters);
+        if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+        if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
+        if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
         delete ctx;
+    };
+    auto bail = [&](hipError_t err, const char* what) {
+        int rc = hip_fail(nullptr, err, what);
+        release();
         return rc;
     };
     if ((e = hipSetDevice(device_index)) != hipSuccess) return bail(e, "hipSetDevice");
@@ -1128,6 +1172,12 @@ int smelt_hip_context_create(int device_index, smelt_hip_context** out) {
     if ((e = hipMalloc(&ctx->ws_partial, ctx->ws_partial_bytes)) != hipSuccess) return bail(e, "hipMalloc(workspace)");
     if ((e = hipMalloc(&ctx->ws_counters, ctx->ws_counter_bytes)) != hipSuccess) return bail(e, "hipMalloc(workspace counters)");
     if ((e = hipMemset(ctx->ws_counters, 0, ctx->ws_counter_bytes)) != hipSuccess) return bail(e, "hipMemset(workspace counters)");
+    // the library's static scratch on this device (used by smelt_hip_encode_prefill_record_static_scratch)
+    std::string why;
+    if (int rc = static_scratch_prepare(device_index, ctx->stream, &why)) {
+        release();
+        return fail(nullptr, rc, why);
+    }
     *out = ctx;
     return SMELT_HIP_OK;
 }

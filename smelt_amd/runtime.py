@@ -118,6 +118,7 @@ def load_library() -> C.CDLL:
         "smelt_hip_dispatch_table_count": (i32, [sz, C.POINTER(sz)]),
         "smelt_hip_encode_decode_record": (i32, [vp, rp, i32, i32, C.c_int32]),
         "smelt_hip_encode_prefill_record": (i32, [vp, rp, i32, i32, C.c_int32, C.c_int32]),
+        "smelt_hip_encode_prefill_record_static_scratch": (i32, [vp, rp, i32, i32, C.c_int32, C.c_int32]),
         "smelt_hip_interpret_decode_table": (i32, [vp, rp, sz, i32, i32, C.c_int32]),
         "smelt_hip_interpret_prefill_table": (i32, [vp, rp, sz, i32, i32, C.c_int32, C.c_int32]),
         "smelt_hip_submit": (i32, [vp]),
@@ -229,6 +230,11 @@ class Context:
     def encode_prefill(self, rec: DispatchRecord, cur=0, alt=1, seq_len=1, start_pos=0) -> int:
         return self.check(self.lib.smelt_hip_encode_prefill_record(self.h, C.byref(rec), cur, alt,
                                                                    seq_len, start_pos))
+
+    def encode_prefill_static_scratch(self, rec: DispatchRecord, cur=0, alt=1, seq_len=1, start_pos=0) -> int:
+        """encode_prefill with the split-K scratch in the library's file-scope device array."""
+        return self.check(self.lib.smelt_hip_encode_prefill_record_static_scratch(
+            self.h, C.byref(rec), cur, alt, seq_len, start_pos))
 
     @staticmethod
     def table(records) -> C.Array:
