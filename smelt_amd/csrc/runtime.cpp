@@ -1401,8 +1401,15 @@ int smelt_hip_benchmark_record(smelt_hip_context* ctx, const SmeltDispatchRecord
         if (rc == 0) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "record does not dispatch for these arguments");
     }
     if (int e = smelt_hip_wait(ctx)) return e;
-    std::vector<hipEvent_t> ev((size_t)iters * 2);
-    for (hipEvent_t& e : ev) HIP_TRY(ctx, hipEventCreate(&e));
+    std::vector<hipEvent_t> ev((size_t)iters * 2, nullptr);
+    for (hipEvent_t& e : ev) {
+        const hipError_t err = hipEventCreate(&e);
+        if (err != hipSuccess) {
+            for (hipEvent_t& made : ev)
+                if (made) (void)hipEventDestroy(made);
+            return hip_fail(ctx, err, "hipEventCreate");
+        }
+    }
     int status = SMELT_HIP_OK;
     ctx->batch_open = true;  // keep encode_record from re-recording the batch start event
     for (int i = 0; i < iters && status == SMELT_HIP_OK; ++i) {
