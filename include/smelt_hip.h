@@ -122,9 +122,20 @@ const char *smelt_hip_last_error(const smelt_hip_context *ctx);
  * every quantized matvec (MatvecKernelTable.swift:158-181). */
 int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
 
-/* dev.makeLibrary(URL: model.metallib): SmeltRuntime.swift:833-835.  The code object is the
- * gfx950 image produced by hipcc --genco; loaded with hipModuleLoadData. */
+/* Which kernel a single-token quantized matvec record runs.  AUTO (the default): matrices of
+ * 8M weights and more take the single-pass matrix-core kernel of the same pipeline, smaller ones
+ * the vector-ALU kernel; MATRIX_CORE drops the size threshold (every shape the matrix-core kernel
+ * can express takes it); VECTOR keeps every record on the vector-ALU kernels.  Results of the two
+ * differ in summation order only.  No counterpart in the reference (one kernel per pipeline name
+ * there); meant for A/B measurement and for tests. */
+enum { SMELT_HIP_MATVEC_AUTO = 0, SMELT_HIP_MATVEC_MATRIX_CORE = 1, SMELT_HIP_MATVEC_VECTOR = 2 };
+int smelt_hip_set_matvec_engine(smelt_hip_context *ctx, int engine);
+
+/* dev.makeLibrary(URL: model.metallib): SmeltRuntime.swift:833-835.  A code object is a gfx950
+ * image produced by hipcc --genco, loaded with hipModuleLoadData.  The kernels ship as several
+ * code objects (smelt_kernels*.hsaco); load every one of them before creating pipelines. */
 int smelt_hip_module_load(smelt_hip_context *ctx, const void *code_object, size_t bytes);
+/* `path` names one code object, or a directory: then every smelt_kernels*.hsaco in it is loaded. */
 int smelt_hip_module_load_file(smelt_hip_context *ctx, const char *path);
 
 /* pipelineFunction(for:library:) + makePipelineState: SmeltRuntime.swift:6229-6306.

@@ -41,7 +41,8 @@ enum {
     SMELT_IMPORT_ERR_BUFFER_TOO_SMALL = -23 /* .bufferTooSmall */
 };
 
-/* Creates an importer on one GPU with the kernels of `code_object_path` (smelt_kernels.hsaco). */
+/* Creates an importer on one GPU with the kernels under `code_object_path` (the directory that
+ * holds the build's smelt_kernels*.hsaco files, or one code object). */
 int smelt_hip_importer_create(int device_index, const char *code_object_path, smelt_hip_importer **out);
 void smelt_hip_importer_destroy(smelt_hip_importer *imp);
 const char *smelt_hip_importer_last_error(const smelt_hip_importer *imp);

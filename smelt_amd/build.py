@@ -3,7 +3,7 @@
     python -m smelt_amd.build          # compile everything
 
 Outputs (git-ignored, shipped to the GPU box as built files):
-    smelt_amd/lib/smelt_kernels.hsaco   hipcc --genco, gfx950 only
+    smelt_amd/lib/smelt_kernels*.hsaco  hipcc --genco, gfx950 only, one per translation unit
     smelt_amd/lib/libsmelt_hip.so       host runtime + record emitters (links libamdhip64); carries one
                                         small gfx950 image of its own (static_scratch.hip)
 """
@@ -17,6 +17,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "lib")
 HSACO = os.path.join(LIB, "smelt_kernels.hsaco")
+# every translation unit under csrc/kernels becomes one code object; the runtime loads them all
+KERNEL_UNITS = ["smelt_kernels", "smelt_kernels_batched_f16", "smelt_kernels_batched_bf16",
+                "smelt_kernels_signed", "smelt_kernels_planes", "smelt_kernels_mfma", "smelt_kernels_qmm",
+                "smelt_kernels_layer", "smelt_kernels_mm1"]
 HOST_LIB = os.path.join(LIB, "libsmelt_hip.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -33,11 +37,22 @@ def _run(cmd: list[str]) -> None:
         raise RuntimeError("build step failed: " + " ".join(cmd))
 
 
-def build_kernels() -> str:
+def code_objects() -> list[str]:
+    return [os.path.join(LIB, unit + ".hsaco") for unit in KERNEL_UNITS]
+
+
+def build_kernels() -> list[str]:
+    """Compiles the translation units side by side (one hipcc process each)."""
+    from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIB, exist_ok=True)
-    src = os.path.join(CSRC, "kernels", "smelt_kernels.hip")
-    _run([HIPCC, *DEVICE_FLAGS, "--genco", "-o", HSACO, src])
-    return HSACO
+
+    def one(unit: str) -> str:
+        out = os.path.join(LIB, unit + ".hsaco")
+        _run([HIPCC, *DEVICE_FLAGS, "--genco", "-o", out, os.path.join(CSRC, "kernels", unit + ".hip")])
+        return out
+
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        return list(pool.map(one, KERNEL_UNITS))
 
 
 def build_host() -> str:
@@ -61,5 +76,6 @@ def build_all() -> None:
 
 if __name__ == "__main__":
     build_all()
-    print(HSACO)
+    for path in code_objects():
+        print(path)
     print(HOST_LIB)

@@ -103,9 +103,12 @@ __device__ __forceinline__ uint16_t trit5_lut_entry(uint32_t b) {
         smelt::signed_gather_body<2, ACT>(C, S, ids, out, hidden, lut);                           \
     }
 
+#ifndef SMELT_NO_INCLUDE_INSTANCES
 SMELT_GATHER_KERNELS(f16, smelt::F16)
 SMELT_GATHER_KERNELS(bf16, smelt::BF16)
+#endif
 
+#ifndef SMELT_NO_INCLUDE_INSTANCES
 // ---- argmax over materialised 16-bit logits ---------------------------------------------------
 // Largest value wins, ties go to the lowest index, -0 equals +0.  The ordering of the 16-bit
 // pattern is the same for fp16 and bf16 (sign + magnitude), so one kernel serves both.
@@ -128,6 +131,7 @@ SMELT_MISC_KERNEL void smelt_argmax16_partials(const uint16_t* logits, smelt::ui
         partials[blockIdx.x] = best;
     }
 }
+#endif
 
 // Best key of row[0 .. n) over the workgroup's threads, four independent loads in flight per
 // thread (a one-load-per-iteration loop pays a full memory round trip per iteration).
@@ -148,6 +152,7 @@ __device__ __forceinline__ uint2_t strided_key_max(const uint2_t* row, uint32_t 
 }
 }  // namespace smelt
 
+#ifndef SMELT_NO_INCLUDE_INSTANCES
 // one block per batch row (blockIdx.x); partials are [batch, num_partials]
 SMELT_MISC_KERNEL void smelt_argmax_key_reduce(const smelt::uint2_t* partials, int* output,
                                                uint32_t num_partials) {
@@ -193,3 +198,4 @@ extern "C" __global__ __launch_bounds__(256) void smelt_copy_u128(const smelt::u
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
+#endif

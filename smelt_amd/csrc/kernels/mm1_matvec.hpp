@@ -1,0 +1,474 @@
+// Single-pass matrix-core matvec for gfx950: y[r] = sum_c w(r, c) * x[c] for one activation row,
+// for matrices whose packed weights stream from HBM (batch-1 decode at large-model layer shapes).
+//
+// The kernel is built around the latency of one memory round trip.  Every wave owns one job, a
+// tile of 16 weight rows times a run of up to NL 64-byte row segments, and issues every weight
+// load of that job (one 16-byte load per lane and segment, plus the group scales) before it does
+// anything else; nothing in the kernel waits on memory twice.  While the loads are in flight the
+// wave stages the slice of the activation row its segments need, privately, in LDS.  K is split
+// over the `kc` waves of a workgroup that share a row tile; their partial sums meet in LDS.
+//
+// Arithmetic: v_mfma_f32_16x16x32_{f16,bf16} with the weights as the B operand.
+//   * MFMA lane (n = lane % 16, q = lane / 16) supplies eight weights of row n taken from the
+//     16-byte piece q of the current 64-byte segment.  Packed codes become (base + code) operands
+//     with one AND-OR per pair of weights: a code whose lowest bit sits at mantissa bit m of a
+//     16-bit float with exponent 2^(M - m) (M = mantissa width) counts in units of one.
+//   * The MFMA contracts over all four q, which would mix four 16-byte pieces (up to four scale
+//     groups).  The A operand (the activations) separates them: token slot 4 q carries x only in
+//     k-block q, every other slot is zero, so D[4 q][n] is the dot product of piece q of row n and
+//     lands in accumulator register 0 of lane (n, q).  Only lanes 0, 20, 40 and 60 of the A
+//     operand are ever non-zero; they alone read the staged activations.
+//   * sum((base + offset) * x) per 16-byte piece is formed at staging time and subtracted before
+//     the group scale is applied in fp32.
+// Activations enter the MFMA in their own type (fp16 or bf16), unconverted.
+#pragma once
+#include "matvec_kernels.hpp"
+
+namespace smelt {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+// 16-bit float geometry of the activation type
+template <class ActT>
+struct Elem16;
+template <>
+struct Elem16<F16> {
+    static constexpr int kMant = 10, kExpBias = 15;
+    static __device__ __forceinline__ float4_t mfma(const uint4_t& a, const uint4_t& b, const float4_t& c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+    }
+    // acc + lo(pair) * lo(k) + hi(pair) * hi(k), fp32 accumulate
+    static __device__ __forceinline__ float dot2k(uint32_t pair, uint32_t k, float acc) {
+        return __builtin_amdgcn_fdot2(as_half2(pair), as_half2(k), acc, false);
+    }
+};
+template <>
+struct Elem16<BF16> {
+    static constexpr int kMant = 7, kExpBias = 127;
+    static __device__ __forceinline__ float4_t mfma(const uint4_t& a, const uint4_t& b, const float4_t& c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float dot2k(uint32_t pair, uint32_t k, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), __builtin_bit_cast(bf16x2_t, k), acc, false);
+    }
+};
+
+// Where the codes of a dword go.  A dword holds 32 / WIDTH codes, LSB first.  Pair j is codes
+// (j, j + 16 / WIDTH): the two sit at the same bit of the low and the high half-word, so one
+// 32-bit AND-OR forms both operands.  kPerPass pairs share one shifted copy of the dword; the
+// code of pair j then sits at mantissa bit kMLo + WIDTH * (j % kPerPass).  A larger kMLo means
+// smaller bases (less cancellation in sum (base + code) x - sum base x) and more shifts.
+template <int WIDTH, class ActT>
+struct M1Plan;
+template <> struct M1Plan<1, BF16> { static constexpr int kPerPass = 7, kMLo = 0; };
+template <> struct M1Plan<1, F16> { static constexpr int kPerPass = 7, kMLo = 3; };
+template <> struct M1Plan<2, BF16> { static constexpr int kPerPass = 3, kMLo = 0; };
+template <> struct M1Plan<2, F16> { static constexpr int kPerPass = 4, kMLo = 2; };
+template <> struct M1Plan<4, BF16> { static constexpr int kPerPass = 1, kMLo = 0; };
+template <> struct M1Plan<4, F16> { static constexpr int kPerPass = 2, kMLo = 2; };
+
+template <int WIDTH, class ActT>
+struct M1Codes {
+    using E = Elem16<ActT>;
+    using P = M1Plan<WIDTH, ActT>;
+    static constexpr int kFields = 32 / WIDTH;          // columns per dword
+    static constexpr int kPairs = kFields / 2;
+    static constexpr int kFPD = kPairs / 4;             // MFMAs (operand fragments) per dword
+    static constexpr int kFPL = 4 * kFPD;               // per 16-byte piece
+    static constexpr int kPieceCols = 4 * kFields;      // columns of one lane's 16 bytes
+    static constexpr int kPasses = (kPairs + P::kPerPass - 1) / P::kPerPass;
+    static __device__ __forceinline__ constexpr int mant_pos(int j) { return P::kMLo + WIDTH * (j % P::kPerPass); }
+    // right shift (left when negative) that brings the codes of a pass to their mantissa positions
+    static __device__ __forceinline__ constexpr int pass_shift(int pass) { return WIDTH * P::kPerPass * pass - P::kMLo; }
+    static __device__ __forceinline__ constexpr uint32_t both(uint32_t h) { return h | (h << 16); }
+    static __device__ __forceinline__ constexpr uint32_t mask(int j) { return both(((1u << WIDTH) - 1u) << mant_pos(j)); }
+    static __device__ __forceinline__ constexpr uint32_t base_half(int j) { return (uint32_t)(E::kExpBias + E::kMant - mant_pos(j)) << E::kMant; }
+    // bits of (base, base) as a pair of 16-bit floats: what the AND-OR adds to the codes of pair j
+    static __device__ __forceinline__ constexpr uint32_t base_pair(int j) { return both(base_half(j)); }
+    // one packed dword -> the B operands of its kFPD MFMAs
+    static __device__ __forceinline__ void operands(uint32_t c, uint4_t (&out)[kFPD]) {
+        uint32_t src[kPasses];
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p) {
+            const int sh = pass_shift(p);
+            src[p] = sh == 0 ? c : (sh > 0 ? c >> sh : c << -sh);
+        }
+        uint32_t r[kPairs];
+#pragma unroll
+        for (int j = 0; j < kPairs; ++j) r[j] = and_or(src[j / P::kPerPass], mask(j), base_pair(j));
+#pragma unroll
+        for (int t = 0; t < kFPD; ++t) out[t] = uint4_t{r[4 * t], r[4 * t + 1], r[4 * t + 2], r[4 * t + 3]};
+    }
+};
+
+// semantic weight = kSemMul * (code - kOffset) * scale (+ bias for affine codes)
+template <class ActT>
+struct M1Bin : M1Codes<1, ActT> {
+    static constexpr bool kHasBias = false;
+    static constexpr float kSemMul = 2.0f, kOffset = 0.5f;
+};
+template <class ActT>
+struct M1Ter2 : M1Codes<2, ActT> {
+    static constexpr bool kHasBias = false;
+    static constexpr float kSemMul = 1.0f, kOffset = 1.0f;
+};
+template <class ActT>
+struct M1U4 : M1Codes<4, ActT> {
+    static constexpr bool kHasBias = true;
+    static constexpr float kSemMul = 1.0f, kOffset = 0.0f;
+};
+
+// LDS layout of a workgroup of `waves` waves with `nl` segments each:
+//   per wave: operand fragments [nl * 8 pieces][frags per piece] x 16 B, then per piece the
+//             folded-out constant and the plain sum of x (8 B), then one piece of zero fragments;
+//   then the scale rows (and bias rows) of the workgroup's eight rows, one block per matrix and
+//   plane; then the waves' partial sums [wave][matrix][8] (fp32).
+__host__ __device__ constexpr size_t mm1_wave_lds_bytes(int frags_per_piece, int nl) {
+    return (size_t)nl * 8 * frags_per_piece * 16 + (size_t)nl * 8 * 8 + (size_t)frags_per_piece * 16;
+}
+__host__ __device__ constexpr size_t mm1_lds_bytes(int frags_per_piece, int nl, int waves, int nmat, int gpr, bool has_bias) {
+    return (size_t)waves * mm1_wave_lds_bytes(frags_per_piece, nl) + (size_t)nmat * (has_bias ? 2 : 1) * 8 * gpr * 2 +
+           (size_t)waves * nmat * 32;
+}
+
+__device__ __forceinline__ float quad_sum(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    return dpp_add<0x4E>(v);  // quad_perm [2,3,0,1]
+}
+
+// One workgroup = one tile of eight rows; its kc waves split K: wave `chunk` owns the 128-byte
+// segments [chunk * NL, chunk * NL + NL) of every row of the tile.
+template <class F, class ActT, class ScaleT, int NMAT, int NL, class Epi>
+__device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint16_t* __restrict__ x_all, int rows,
+                                         int cols, int row_stride, int group, const Epi& epi) {
+    using E = Elem16<ActT>;
+    constexpr int FPD = F::kFPD, FPL = F::kFPL, FIELDS = F::kFields, PAIRS = F::kPairs;
+    constexpr int NITEMS = NL * 32;                        // staging items of a wave: 8 pieces x 4 dwords per segment
+    constexpr int ITEMS = (NITEMS + kWave - 1) / kWave;    // per lane
+    constexpr int PLANES = F::kHasBias ? 2 : 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int chunk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int kc = blockDim.x / kWave;
+    const int n = lane & 15, q = lane >> 4;
+    const int token = blockIdx.y;
+    const uint16_t* __restrict__ x = x_all + (size_t)token * cols;
+    const int pieces = row_stride >> 4;               // 16-byte pieces per packed row
+    const int gshift = ilog2((uint32_t)group);
+    const int gpr = (cols + group - 1) >> gshift;     // 16-byte pieces of one plane's scale block, too
+    const int row0 = blockIdx.x * 8;
+    const int piece0 = chunk * NL * 8;                // first piece of this wave's run
+    // Weight loads are issued in memory order, eight consecutive lanes on the 128 bytes of one row
+    // segment (lane = 8 * row-in-tile + piece); a cross-lane transpose then hands MFMA lane (n, q)
+    // the piece 4 * (n / 8) + q of row n % 8.
+    const int ld_q = lane & 7, ld_r = lane >> 3;
+    const int hh = n >> 3, rn = n & 7;                // which half of the segment, which row of the tile
+    const int xpose = (8 * rn + 4 * hh + q) * 4;      // byte address of the source lane for ds_bpermute
+
+    // Nothing below branches or predicates a load until every load of the job is issued (a load
+    // under a branch invites the compiler to move its consumer, and the wait, in there too).
+    // Loads return in issue order, so what is needed first is asked for first.  A row or piece
+    // past the end re-reads the last valid one and is discarded later (zero scale, no store).
+    //
+    // ---- 1. the scale (and bias) rows of the tile: one contiguous block per matrix and plane ----
+    const int plane_pieces = (rows * gpr * 2 + 15) >> 4;
+    uint4_t sp[NMAT][PLANES];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int pl = 0; pl < PLANES; ++pl) {
+            const uint4_t* base = reinterpret_cast<const uint4_t*>(pl == 0 ? mats[m].scales : mats[m].biases);
+            int idx = (int)threadIdx.x;
+            if (idx > gpr - 1) idx = gpr - 1;
+            int src = blockIdx.x * gpr + idx;         // row0 * gpr * 2 bytes = blockIdx.x * gpr pieces
+            if (src > plane_pieces - 1) src = plane_pieces - 1;
+            sp[m][pl] = base[src];
+        }
+    // ---- 2. this wave's slice of x ---------------------------------------------------------------
+    // One item = the columns of one packed dword; item it = 4 * (piece within the run) + dword.
+    uint32_t xe[ITEMS][FIELDS / 2];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        int it = lane + k * kWave;
+        if (it > NITEMS - 1) it = NITEMS - 1;
+        int col0 = (piece0 + (it >> 2)) * F::kPieceCols + (it & 3) * FIELDS;
+        if (col0 > cols - FIELDS) col0 = cols - FIELDS;   // cols is a multiple of kFields
+#pragma unroll
+        for (int v = 0; v < FIELDS / 8; ++v) {
+            const uint4_t t = *reinterpret_cast<const uint4_t*>(x + col0 + 8 * v);
+            xe[k][4 * v] = t.x; xe[k][4 * v + 1] = t.y; xe[k][4 * v + 2] = t.z; xe[k][4 * v + 3] = t.w;
+        }
+    }
+    // ---- 3. every weight load of the job -------------------------------------------------------------
+    uint4_t codes[NMAT][NL];
+    {
+        int ld_row = row0 + ld_r;
+        if (ld_row > rows - 1) ld_row = rows - 1;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            int piece = piece0 + i * 8 + ld_q;
+            if (piece > pieces - 1) piece = pieces - 1;
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+                codes[m][i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(mats[m].codes + (size_t)ld_row * row_stride + (size_t)piece * 16));
+        }
+    }
+    uint16_t res = 0;
+    if constexpr (Epi::kPrefetch) {
+        if (chunk == 0 && lane < 8 && row0 + lane < rows) res = epi.prefetch(token, row0 + lane);
+    }
+
+    // ---- 4. scales into LDS ----------------------------------------------------------------------------
+    const size_t wave_bytes = mm1_wave_lds_bytes(FPL, NL);
+    uint4_t* lds_scales = reinterpret_cast<uint4_t*>(smem + (size_t)kc * wave_bytes);
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int pl = 0; pl < PLANES; ++pl) {
+            // threads past the end of the block hold its last piece again and store it again
+            int idx = (int)threadIdx.x;
+            if (idx > gpr - 1) idx = gpr - 1;
+            lds_scales[(m * PLANES + pl) * gpr + idx] = sp[m][pl];
+        }
+
+    // ---- 5. x as operand fragments, wave-private in LDS --------------------------------------------
+    // kFields consecutive activations become the kFPD fragments that dword's MFMAs take (k-slots
+    // 2v, 2v+1 of fragment t = columns 4t+v, 4t+v+kPairs).  The four items of a 16-byte piece sit
+    // in the four lanes of a quad, which add up their sum(base * x) and sum(x).
+    uint4_t* wfrag = reinterpret_cast<uint4_t*>(smem + (size_t)chunk * wave_bytes);
+    float* wsum = reinterpret_cast<float*>(wfrag + (size_t)NL * 8 * FPL);   // [piece][2]: constant, sum x
+    uint4_t* wzero = reinterpret_cast<uint4_t*>(wsum + NL * 16);            // FPL zero fragments
+    if (lane < FPL) wzero[lane] = uint4_t{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        // lanes past the last item hold the last item again (whole quads of them: d == 3) and store
+        // the same fragments again
+        int it = lane + k * kWave;
+        if (it > NITEMS - 1) it = NITEMS - 1;
+        const int pl = it >> 2, d = it & 3;
+        float cb = 0.0f, xs = 0.0f;
+        constexpr uint32_t kOnes = F::both((uint32_t)E::kExpBias << E::kMant);   // (1.0, 1.0)
+        uint32_t fr[PAIRS];
+#pragma unroll
+        for (int j = 0; j < PAIRS; ++j) {
+            const uint32_t lo = xe[k][j >> 1], hi = xe[k][(PAIRS >> 1) + (j >> 1)];
+            fr[j] = __builtin_amdgcn_perm(hi, lo, (j & 1) ? 0x07060302u : 0x05040100u);   // (x[j], x[j + kPairs])
+            cb = E::dot2k(fr[j], F::base_pair(j), cb);
+            xs = E::dot2k(fr[j], kOnes, xs);
+        }
+        cb = quad_sum(cb);
+        xs = quad_sum(xs);
+#pragma unroll
+        for (int t = 0; t < FPD; ++t)
+            wfrag[(size_t)pl * FPL + d * FPD + t] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
+        if (d == 0) *reinterpret_cast<float2*>(wsum + 2 * pl) = float2{__builtin_fmaf(F::kOffset, xs, cb), xs};
+    }
+    __syncthreads();   // scales of every wave, fragments of this one
+
+    // ---- 6. the job --------------------------------------------------------------------------------
+    // A-operand lanes 20q and 20q + 1 (token slots 4q and 4q + 1 in k-block q: the two halves of
+    // the segment) read fragments; the other fifty-six read the zero fragments, so no lane is
+    // masked off.
+    const int a_half = n - 4 * q;
+    const bool a_live = a_half == 0 || a_half == 1;
+    const uint16_t* lds_s16 = reinterpret_cast<const uint16_t*>(lds_scales);
+    float y[NMAT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) y[m] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        float4_t acc[NMAT];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) acc[m] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        const uint4_t* pf = a_live ? wfrag + (size_t)(i * 8 + 4 * a_half + q) * FPL : wzero;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint4_t afr[FPD];
+#pragma unroll
+            for (int f = 0; f < FPD; ++f) afr[f] = pf[d * FPD + f];
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                const uint4_t lw = codes[m][i];
+                const uint32_t cw = (uint32_t)__builtin_amdgcn_ds_bpermute(xpose, (int)(d == 0 ? lw.x : (d == 1 ? lw.y : (d == 2 ? lw.z : lw.w))));
+                uint4_t ops[FPD];
+                F::operands(cw, ops);
+#pragma unroll
+                for (int f = 0; f < FPD; ++f) acc[m] = E::mfma(afr[f], ops[f], acc[m]);
+            }
+        }
+        const float2 cs = *reinterpret_cast<const float2*>(wsum + 2 * (i * 8 + 4 * hh + q));
+        const int piece = piece0 + i * 8 + 4 * hh + q;
+        const bool piece_ok = piece < pieces;
+        const int g = ((piece_ok ? piece : pieces - 1) * F::kPieceCols) >> gshift;
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            const int sidx = (m * PLANES) * (8 * gpr) + rn * gpr + g;
+            const float sv = F::kSemMul * ScaleT::widen(lds_s16[sidx]);
+            const float dotp = hh ? acc[m].y : acc[m].x;   // token slot 4q + hh
+            y[m] = __builtin_fmaf(piece_ok ? sv : 0.0f, dotp - cs.x, y[m]);
+            if (F::kHasBias) {
+                const float bv = ScaleT::widen(lds_s16[sidx + 8 * gpr]);
+                y[m] = __builtin_fmaf(piece_ok ? bv : 0.0f, cs.y, y[m]);
+            }
+        }
+    }
+    // the eight pieces of a segment: lanes rn + 8 * {0..7}
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) {
+        y[m] += __shfl_xor(y[m], 8);
+        y[m] += __shfl_xor(y[m], 16);
+        y[m] += __shfl_xor(y[m], 32);
+    }
+
+    // ---- 7. the kc waves of the workgroup -----------------------------------------------------------
+    if (kc > 1) {
+        float* red = reinterpret_cast<float*>(smem + (size_t)kc * wave_bytes + (size_t)NMAT * PLANES * 8 * gpr * 2);
+        if (lane < 8) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) red[(chunk * NMAT + m) * 8 + lane] = y[m];
+        }
+        __syncthreads();
+        if (chunk == 0 && lane < 8) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                float sum = y[m];
+                for (int k = 1; k < kc; ++k) sum += red[(k * NMAT + m) * 8 + lane];
+                y[m] = sum;
+            }
+        }
+    }
+    if (chunk == 0 && lane < 8 && row0 + lane < rows) {
+        if constexpr (Epi::kPrefetch) epi.finish(token, row0 + lane, y, res);
+        else epi(token, row0 + lane, y);
+    }
+}
+
+}  // namespace smelt
+
+#define SMELT_MM1_KERNEL extern "C" __global__ __launch_bounds__(1024)
+
+// Signed g128 formats: same argument lists as the vector-ALU kernels of the pipelines.  The launch
+// supplies the split: one workgroup per NT row tiles, one wave per NL segments of a row.
+#define SMELT_SIGNED_MM1_KERNELS(FN, FMT, T, ACT, NLV)                                       \
+    SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_matvec_##T(                  \
+        const u8* C, const u16* S, const u16* X, u16* Y, u32 rows, u32 cols) {                    \
+        using namespace smelt;                                                                    \
+        using F = FMT<ACT>;                                                                       \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<F, ACT, F16, 1, NLV>(mats, X, rows, cols,                                   \
+                                           (cols + 127) / 128 * 128 * 4 / F::kFields, 128, epi);  \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_matvec_add_##T(              \
+        const u8* C, const u16* S, const u16* X, u16* Y, const u16* res, u32 rows, u32 cols) {    \
+        using namespace smelt;                                                                    \
+        using F = FMT<ACT>;                                                                       \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        mm1_body<F, ACT, F16, 1, NLV>(mats, X, rows, cols,                                   \
+                                           (cols + 127) / 128 * 128 * 4 / F::kFields, 128, epi);  \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_gate_up_swiglu_##T(          \
+        const u8* gC, const u16* gS, const u8* uC, const u16* uS, const u16* X, u16* Y, u32 rows, \
+        u32 cols) {                                                                      \
+        using namespace smelt;                                                                    \
+        using F = FMT<ACT>;                                                                       \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        mm1_body<F, ACT, F16, 2, NLV>(mats, X, rows, cols,                                   \
+                                           (cols + 127) / 128 * 128 * 4 / F::kFields, 128, epi);  \
+    }
+
+// Affine 4-bit: argument lists of the vector-ALU kernels of the same pipelines.
+#define SMELT_AFFINE_MM1_KERNELS(T, ACT, SC, NLV)                                            \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_matvec_##T(                         \
+        const u8* W, const u16* S, const u16* B, const u16* X, u16* Y, u32 rows, u32 cols,        \
+        u32 group) {                                                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<M1U4<ACT>, ACT, SC, 1, NLV>(mats, X, rows, cols, cols / 2, group, epi);     \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_matvec_add_##T(                     \
+        const u8* W, const u16* S, const u16* B, const u16* X, u16* Y, const u16* res, u32 rows,  \
+        u32 cols, u32 group) {                                                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        mm1_body<M1U4<ACT>, ACT, SC, 1, NLV>(mats, X, rows, cols, cols / 2, group, epi);     \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_gate_up_swiglu_##T(                 \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* X, u16* Y, u32 rows, u32 cols, u32 group) {                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiAffineSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        mm1_body<M1U4<ACT>, ACT, SC, 2, NLV>(mats, X, rows, cols, cols / 2, group, epi);     \
+    }
+
+#define SMELT_AFFINE_MM1_BANK(T, ACT, SC, NLV)                                                    \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_bank4_matvec_##T(                            \
+        const u8* W, const u16* S, const u16* B, const u16* X, u16* y0, u16* y1, u16* y2,         \
+        u16* y3, u32 rows0, u32 rows1, u32 rows2, u32 rows3, u32 cols, u32 group) {               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        mm1_body<M1U4<ACT>, ACT, SC, 1, NLV>(mats, X, rows0 + rows1 + rows2 + rows3, cols,        \
+                                             cols / 2, group, epi);                               \
+    }
+
+// Ternary "affine" pipelines bind the scale plane a second time where MLX binds a bias plane; it
+// is ignored as in the vector-ALU kernels.
+#define SMELT_TERAFF_MM1_KERNELS(T, ACT, NLV)                                                     \
+    SMELT_MM1_KERNEL void smelt_teraff_mm1_nl##NLV##_matvec_##T(                                  \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* Y, u32 rows, u32 cols) {        \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<M1Ter2<ACT>, ACT, F16, 1, NLV>(mats, X, rows, cols, cols / 4, 128, epi);         \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_teraff_mm1_nl##NLV##_matvec_add_##T(                              \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* Y, const u16* res, u32 rows,    \
+        u32 cols) {                                                                               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        mm1_body<M1Ter2<ACT>, ACT, F16, 1, NLV>(mats, X, rows, cols, cols / 4, 128, epi);         \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_teraff_mm1_nl##NLV##_gate_up_swiglu_##T(                          \
+        const u8* gC, const u16* gS, const u16*, const u8* uC, const u16* uS, const u16*,         \
+        const u16* X, u16* Y, u32 rows, u32 cols) {                                               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        mm1_body<M1Ter2<ACT>, ACT, F16, 2, NLV>(mats, X, rows, cols, cols / 4, 128, epi);         \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_teraff_mm1_nl##NLV##_bank4_matvec_##T(                            \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* y0, u16* y1, u16* y2, u16* y3,  \
+        u32 rows0, u32 rows1, u32 rows2, u32 rows3, u32 cols) {                                   \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        mm1_body<M1Ter2<ACT>, ACT, F16, 1, NLV>(mats, X, rows0 + rows1 + rows2 + rows3, cols,     \
+                                                cols / 4, 128, epi);                              \
+    }
+
+#define SMELT_BINARY_MM1_BANKS(T, ACT, NLV)                                                       \
+    SMELT_MM1_KERNEL void smelt_signed_binary_mm1_nl##NLV##_packed_bank_matvec_##T(               \
+        const u8* C, const u16* S, const u16* X, u16* y0, u16* y1, u32 rows0, u32 rows1,          \
+        u32 cols) {                                                                               \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, nullptr, nullptr}, {rows0, rows1, 0u, 0u}};                \
+        mm1_body<M1Bin<ACT>, ACT, F16, 1, NLV>(mats, X, rows0 + rows1, cols, cols / 8, 128, epi); \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_signed_binary_mm1_nl##NLV##_packed_bank4_matvec_##T(              \
+        const u8* C, const u16* S, const u16* X, u16* y0, u16* y1, u16* y2, u16* y3, u32 rows0,   \
+        u32 rows1, u32 rows2, u32 rows3, u32 cols) {                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        mm1_body<M1Bin<ACT>, ACT, F16, 1, NLV>(mats, X, rows0 + rows1 + rows2 + rows3, cols,      \
+                                               cols / 8, 128, epi);                               \
+    }

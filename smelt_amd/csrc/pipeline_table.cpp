@@ -147,8 +147,93 @@ uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
     }
 }
 
+bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
+              bool force, Mm1Plan* out) {
+    uint32_t row_stride, frags, nl_max;
+    switch (layout) {
+        case kCodesU4: row_stride = cols / 2; frags = 4; nl_max = 6; break;
+        case kCodesTernary2: row_stride = (cols + 127u) / 128u * 32u; frags = 8; nl_max = 3; break;
+        case kCodesBinary1: row_stride = (cols + 127u) / 128u * 16u; frags = 16; nl_max = 3; break;
+        default: return false;
+    }
+    if (rows == 0 || cols == 0 || row_stride % 16 != 0 || group < 32 || (group & (group - 1))) return false;
+    if (layout != kCodesU4 && group != 128) return false;
+    // small matrices are launch-bound either way and stay where they are tuned
+    if (!force && (uint64_t)rows * cols < (8u << 20)) return false;
+    const uint32_t pieces = row_stride / 16, nseg = (pieces + 7) / 8, gpr = (cols + group - 1) / group;
+    const uint32_t planes = layout == kCodesU4 ? 2 : 1;
+    auto lds_of = [&](uint32_t kc, uint32_t nl) {
+        const size_t wave = (size_t)nl * 8 * frags * 16 + (size_t)nl * 8 * 8 + (size_t)frags * 16;
+        return kc * wave + (size_t)nmat * planes * 8 * gpr * 2 + (size_t)kc * nmat * 32;
+    };
+    Mm1Plan best;
+    uint32_t best_waste = ~0u;
+    const uint32_t tolerated = nseg / 10 > 1 ? nseg / 10 : 1;
+    for (uint32_t nl = nl_max; nl >= 1; --nl) {
+        const uint32_t kc = (nseg + nl - 1) / nl;
+        if (kc > 16 || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
+        const size_t lds = lds_of(kc, nl);
+        if (lds > lds_limit) continue;
+        const uint32_t waste = kc * nl - nseg;
+        if (waste <= tolerated) { best.kc = kc; best.nl = nl; best.lds = lds; best_waste = waste; break; }
+        if (waste < best_waste) { best.kc = kc; best.nl = nl; best.lds = lds; best_waste = waste; }
+    }
+    if (best.kc == 0) return false;
+    *out = best;
+    return true;
+}
+
+namespace {
+
+// The vector-ALU kernels that have a single-pass matrix-core form, by symbol stem.
+void attach_mm1(ResolvedPipeline* r) {
+    struct Form { const char* stem; const char* prefix; const char* tail; CodeLayout layout; uint32_t nmat; };
+    static const Form kForms[] = {
+        {"smelt_affine_matvec_", "smelt_affine_mm1_", "matvec_", kCodesU4, 1},
+        {"smelt_affine_matvec_add_", "smelt_affine_mm1_", "matvec_add_", kCodesU4, 1},
+        {"smelt_affine_gate_up_swiglu_", "smelt_affine_mm1_", "gate_up_swiglu_", kCodesU4, 2},
+        {"smelt_affine_bank4_matvec_", "smelt_affine_mm1_", "bank4_matvec_", kCodesU4, 1},
+        {"smelt_signed_binary_matvec_", "smelt_signed_binary_mm1_", "matvec_", kCodesBinary1, 1},
+        {"smelt_signed_binary_matvec_add_", "smelt_signed_binary_mm1_", "matvec_add_", kCodesBinary1, 1},
+        {"smelt_signed_binary_gate_up_swiglu_", "smelt_signed_binary_mm1_", "gate_up_swiglu_", kCodesBinary1, 2},
+        {"smelt_signed_binary_packed_bank_matvec_", "smelt_signed_binary_mm1_", "packed_bank_matvec_", kCodesBinary1, 1},
+        {"smelt_signed_binary_packed_bank4_matvec_", "smelt_signed_binary_mm1_", "packed_bank4_matvec_", kCodesBinary1, 1},
+        {"smelt_signed_ternary_matvec_", "smelt_signed_ternary_mm1_", "matvec_", kCodesTernary2, 1},
+        {"smelt_signed_ternary_matvec_add_", "smelt_signed_ternary_mm1_", "matvec_add_", kCodesTernary2, 1},
+        {"smelt_signed_ternary_gate_up_swiglu_", "smelt_signed_ternary_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},
+        {"smelt_teraff_matvec_", "smelt_teraff_mm1_", "matvec_", kCodesTernary2, 1},
+        {"smelt_teraff_matvec_add_", "smelt_teraff_mm1_", "matvec_add_", kCodesTernary2, 1},
+        {"smelt_teraff_gate_up_swiglu_", "smelt_teraff_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},
+        {"smelt_teraff_bank4_matvec_", "smelt_teraff_mm1_", "bank4_matvec_", kCodesTernary2, 1},
+    };
+    const std::string t = act_suffix(r->act);
+    for (const Form& f : kForms) {
+        if (r->symbol == std::string(f.stem) + t) {
+            r->mm1_prefix = f.prefix;
+            r->mm1_tail = std::string(f.tail) + t;
+            r->mm1_layout = (int)f.layout;
+            r->mm1_nmat = f.nmat;
+            return;
+        }
+    }
+}
+
+ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType default_act, size_t lds_limit,
+                                     ResolvedPipeline* out, std::string* why);
+
+}  // namespace
+
 ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act,
                                size_t lds_limit, ResolvedPipeline* out, std::string* why) {
+    const ResolveStatus st = resolve_pipeline_entry(entry_in, default_act, lds_limit, out, why);
+    if (st == kResolveOk) attach_mm1(out);
+    return st;
+}
+
+namespace {
+
+ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType default_act,
+                                     size_t lds_limit, ResolvedPipeline* out, std::string* why) {
     std::string entry = entry_in;
     ActDType act = default_act;
     size_t at = entry.find('@');
@@ -660,5 +745,7 @@ ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act
     *why = "no HIP kernel named '" + entry + "'";
     return kResolveUnknown;
 }
+
+}  // namespace
 
 }  // namespace smelt_host

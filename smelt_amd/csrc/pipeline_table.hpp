@@ -109,6 +109,11 @@ struct ResolvedPipeline {
     std::string symbol_mm_stream, symbol_mm_split;  // optional matrix-core kernels picked per launch by shape
     int rows_arg = -1, cols_arg = -1;               // where that launch finds rows and cols
     uint32_t mfma_kw = 0;            // > 0: matrix-core matvec variant, waves that share a row tile
+    // Single-pass matrix-core matvec of the same pipeline, picked per launch by shape: the kernel is
+    // mm1_prefix + "nl<N>_" + mm1_tail for N segments per wave (empty prefix: the pipeline has none).
+    std::string mm1_prefix, mm1_tail;
+    int mm1_layout = -1;             // CodeLayout of its weights
+    uint32_t mm1_nmat = 1;
     bool workspace = false;          // kernel takes the context's (partials, counters) pointers last
 };
 
@@ -141,5 +146,16 @@ size_t qmm_lds_bytes(uint32_t nmat, uint32_t mt);
 size_t qmm_affine_lds_bytes(uint32_t nmat, uint32_t mt);
 
 uint32_t signed_row_stride(SignedFormat f, uint32_t cols);
+
+// Launch plan of the single-pass matrix-core matvec: one workgroup of `kc` waves per eight rows,
+// `nl` 128-byte row segments per wave.  False when the shape stays on the vector-ALU kernels
+// (`force` drops the size threshold, not the geometry limits).
+constexpr uint32_t kMm1MaxSegments = 6;
+struct Mm1Plan {
+    uint32_t kc = 0, nl = 0;
+    size_t lds = 0;
+};
+bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
+              bool force, Mm1Plan* out);
 
 }  // namespace smelt_host

@@ -3,6 +3,8 @@
 // MTLBuffer / MTLComputeCommandEncoder (SmeltRuntime.swift:668-998, 3150-3275, 5990-6207).
 #include <hip/hip_runtime.h>
 
+#include <dirent.h>
+
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
@@ -42,6 +44,7 @@ struct Pipeline {
     hipFunction_t fn = nullptr;
     hipFunction_t fn_single = nullptr;  // used when the record's batch argument is 1
     hipFunction_t fn_mm_stream = nullptr, fn_mm_split = nullptr;  // matrix-core variants picked by shape
+    hipFunction_t fn_mm1[kMm1MaxSegments + 1] = {};               // single-pass matrix-core matvec, by segments per wave
     ResolvedPipeline res;
 };
 
@@ -61,7 +64,8 @@ struct smelt_hip_context {
     hipEvent_t ev_start = nullptr, ev_end = nullptr;
     bool batch_open = false;
     bool timing_valid = false;
-    hipModule_t module = nullptr;
+    std::vector<hipModule_t> modules;   // every code object loaded so far; kernels are looked up in load order
+    int matvec_engine = SMELT_HIP_MATVEC_AUTO;
     std::vector<Pipeline> pipelines;
     std::mutex pipeline_mutex;
     std::vector<SlotBuffer> slots;
@@ -1056,7 +1060,40 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "threadgroup exceeds 1024 threads");
     if (int e = validate_launch(ctx, *p, L, ws)) return e;
     hipFunction_t fn = p->fn;
-    if (p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
+    bool routed = false;
+    if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.grid[1] == 1) {
+        // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
+        // arguments, its own launch geometry (one workgroup per eight rows)
+        uint32_t rows = 0, cols = 0, group = 128;
+        auto U = [&](size_t i) { return L.args[i].value; };
+        switch (p->res.family) {
+            case kFamAffineMatvec: rows = U(5); cols = U(6); group = U(7); break;
+            case kFamAffineAdd: rows = U(6); cols = U(7); group = U(8); break;
+            case kFamAffineGateUp: rows = U(8); cols = U(9); group = U(10); break;
+            case kFamAffineBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); group = U(13); break;
+            case kFamSignedMatvec: rows = U(4); cols = U(5); break;
+            case kFamSignedAdd: rows = U(5); cols = U(6); break;
+            case kFamSignedGateUp: rows = U(6); cols = U(7); break;
+            case kFamBinaryPackedBank: rows = U(5) + U(6); cols = U(7); break;
+            case kFamBinaryPackedBank4: rows = U(7) + U(8) + U(9) + U(10); cols = U(11); break;
+            case kFamTerAffMatvec: rows = U(5); cols = U(6); break;
+            case kFamTerAffAdd: rows = U(6); cols = U(7); break;
+            case kFamTerAffGateUp: rows = U(8); cols = U(9); break;
+            case kFamTerAffBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); break;
+            default: break;
+        }
+        Mm1Plan plan;
+        if (rows > 0 && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
+                                 ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &plan) &&
+            p->fn_mm1[plan.nl]) {
+            fn = p->fn_mm1[plan.nl];
+            L.grid[0] = (rows + 7) / 8; L.grid[1] = 1; L.grid[2] = 1;
+            L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
+            L.lds = plan.lds;
+            routed = true;
+        }
+    }
+    if (!routed && p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
         // signed g128 matvec: large matrices run on the matrix cores (same bytes, same arguments + kw)
         const uint32_t rows = L.args[(size_t)p->res.rows_arg].value, cols = L.args[(size_t)p->res.cols_arg].value;
         const CodeLayout layout = code_layout(p->res.format);
@@ -1097,7 +1134,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         ctx->batch_open = true;
         ctx->timing_valid = false;
     }
-    if (p->fn_single && p->res.single_arg >= 0 && L.args[(size_t)p->res.single_arg].value == 1 && L.grid[1] == 1) fn = p->fn_single;
+    if (!routed && p->fn_single && p->res.single_arg >= 0 && L.args[(size_t)p->res.single_arg].value == 1 && L.grid[1] == 1) fn = p->fn_single;
     HIP_TRY(ctx, hipModuleLaunchKernel(fn, L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2],
                                        (unsigned)L.lds, ctx->stream, nullptr, config));
     return 1;
@@ -1190,7 +1227,7 @@ void smelt_hip_context_destroy(smelt_hip_context* ctx) {
         if (s.ptr) (void)hipFree(s.ptr);
     if (ctx->ws_partial) (void)hipFree(ctx->ws_partial);
     if (ctx->ws_counters) (void)hipFree(ctx->ws_counters);
-    if (ctx->module) (void)hipModuleUnload(ctx->module);
+    for (hipModule_t m : ctx->modules) (void)hipModuleUnload(m);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -1208,16 +1245,39 @@ int smelt_hip_set_activation_dtype(smelt_hip_context* ctx, int act_dtype) {
     return SMELT_HIP_OK;
 }
 
+int smelt_hip_set_matvec_engine(smelt_hip_context* ctx, int engine) {
+    if (!ctx || engine < SMELT_HIP_MATVEC_AUTO || engine > SMELT_HIP_MATVEC_VECTOR)
+        return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "matvec engine must be SMELT_HIP_MATVEC_AUTO, _MATRIX_CORE or _VECTOR");
+    ctx->matvec_engine = engine;
+    return SMELT_HIP_OK;
+}
+
 int smelt_hip_module_load(smelt_hip_context* ctx, const void* code_object, size_t bytes) {
     if (!ctx || !code_object || bytes == 0) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or empty code object");
-    if (ctx->module) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "a code object is already loaded");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    HIP_TRY(ctx, hipModuleLoadData(&ctx->module, code_object));
+    hipModule_t module = nullptr;
+    HIP_TRY(ctx, hipModuleLoadData(&module, code_object));
+    std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);
+    ctx->modules.push_back(module);
     return SMELT_HIP_OK;
 }
 
 int smelt_hip_module_load_file(smelt_hip_context* ctx, const char* path) {
     if (!ctx || !path) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or path");
+    if (DIR* dir = opendir(path)) {
+        // a directory: every code object of the build in it, in name order
+        std::vector<std::string> names;
+        while (const dirent* e = readdir(dir)) {
+            const std::string n = e->d_name;
+            if (n.size() > 6 && n.compare(n.size() - 6, 6, ".hsaco") == 0 && n.compare(0, 13, "smelt_kernels") == 0) names.push_back(n);
+        }
+        closedir(dir);
+        if (names.empty()) return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, std::string("no smelt_kernels*.hsaco under '") + path + "'");
+        std::sort(names.begin(), names.end());
+        for (const std::string& n : names)
+            if (int rc = smelt_hip_module_load_file(ctx, (std::string(path) + "/" + n).c_str())) return rc;
+        return SMELT_HIP_OK;
+    }
     std::ifstream f(path, std::ios::binary);
     if (!f) return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, std::string("cannot open code object '") + path + "'");
     std::vector<char> data((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
@@ -1227,7 +1287,18 @@ int smelt_hip_module_load_file(smelt_hip_context* ctx, const char* path) {
 
 int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int allow_missing, uint32_t* out_index) {
     if (!ctx || !entry) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or entry");
-    if (!ctx->module) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "load a code object before creating pipelines");
+    if (ctx->modules.empty()) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "load a code object before creating pipelines");
+    // a kernel lives in exactly one of the loaded code objects
+    auto find = [&](hipFunction_t* fn, const std::string& symbol) {
+        hipError_t last = hipErrorNotFound;
+        for (hipModule_t m : ctx->modules) {
+            last = hipModuleGetFunction(fn, m, symbol.c_str());
+            if (last == hipSuccess) break;
+        }
+        (void)hipGetLastError();   // a miss in one code object is not an error of the context
+        if (last != hipSuccess) *fn = nullptr;
+        return last;
+    };
     Pipeline p;
     p.entry = entry;
     std::string why;
@@ -1235,19 +1306,19 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
     if (st == kResolveMalformed) return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, why);
     if (st == kResolveUnknown && !allow_missing) return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, why);
     if (st == kResolveOk) {
-        hipError_t e = hipModuleGetFunction(&p.fn, ctx->module, p.res.symbol.c_str());
+        hipError_t e = find(&p.fn, p.res.symbol);
         if (e != hipSuccess) {
             if (!allow_missing)
                 return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "code object has no kernel '" + p.res.symbol + "' for pipeline '" + p.entry + "': " + hipGetErrorString(e));
         } else {
             p.ready = true;
-            if (!p.res.symbol_single.empty() &&
-                hipModuleGetFunction(&p.fn_single, ctx->module, p.res.symbol_single.c_str()) != hipSuccess)
-                p.fn_single = nullptr;
+            if (!p.res.symbol_single.empty() && find(&p.fn_single, p.res.symbol_single) != hipSuccess) p.fn_single = nullptr;
             if (!p.res.symbol_mm_stream.empty() &&
-                (hipModuleGetFunction(&p.fn_mm_stream, ctx->module, p.res.symbol_mm_stream.c_str()) != hipSuccess ||
-                 hipModuleGetFunction(&p.fn_mm_split, ctx->module, p.res.symbol_mm_split.c_str()) != hipSuccess))
+                (find(&p.fn_mm_stream, p.res.symbol_mm_stream) != hipSuccess || find(&p.fn_mm_split, p.res.symbol_mm_split) != hipSuccess))
                 p.fn_mm_stream = p.fn_mm_split = nullptr;
+            if (!p.res.mm1_prefix.empty())
+                for (uint32_t nl = 1; nl <= kMm1MaxSegments; ++nl)
+                    (void)find(&p.fn_mm1[nl], p.res.mm1_prefix + "nl" + std::to_string(nl) + "_" + p.res.mm1_tail);
         }
     }
     std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);

@@ -35,6 +35,7 @@ __global__ __launch_bounds__(256) void smelt_static_scratch_fill(uint32_t* words
 hipError_t clear_counters(void* base, size_t count, hipStream_t stream) {
     if (count == 0) return hipSuccess;
     const unsigned blocks = (unsigned)((count + 255) / 256 < 64 ? (count + 255) / 256 : 64);
+    (void)hipGetLastError();   // the launch's own status is wanted, not an earlier call's
     hipLaunchKernelGGL(smelt_static_scratch_fill, dim3(blocks), dim3(256), 0, stream,
                        static_cast<uint32_t*>(base), (uint32_t)count, 0u);
     return hipGetLastError();

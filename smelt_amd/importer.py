@@ -59,7 +59,7 @@ class Importer:
     def __init__(self, device: int = 0):
         self.lib = _lib()
         self.h = C.c_void_p()
-        rc = self.lib.smelt_hip_importer_create(device, rt.HSACO.encode(), C.byref(self.h))
+        rc = self.lib.smelt_hip_importer_create(device, rt.LIB_DIR.encode(), C.byref(self.h))
         if rc != 0:
             raise ImportError_(rc, self.lib.smelt_hip_importer_last_error(None).decode())
 

@@ -14,6 +14,13 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(HERE, "lib")
 HOST_LIB = os.path.join(LIB_DIR, "libsmelt_hip.so")
 HSACO = os.path.join(LIB_DIR, "smelt_kernels.hsaco")
+MATVEC_AUTO, MATVEC_MATRIX_CORE, MATVEC_VECTOR = 0, 1, 2
+
+
+def code_objects() -> list[str]:
+    """Every gfx950 code object of the build (smelt_kernels*.hsaco), in load order."""
+    import glob
+    return sorted(glob.glob(os.path.join(LIB_DIR, "smelt_kernels*.hsaco")))
 
 ACT_F16, ACT_BF16 = 0, 1
 SLOT_CUR, SLOT_ALT = -1, -2
@@ -104,6 +111,7 @@ def load_library() -> C.CDLL:
         "smelt_hip_context_destroy": (None, [vp]),
         "smelt_hip_last_error": (C.c_char_p, [vp]),
         "smelt_hip_set_activation_dtype": (i32, [vp, i32]),
+        "smelt_hip_set_matvec_engine": (i32, [vp, i32]),
         "smelt_hip_module_load": (i32, [vp, vp, sz]),
         "smelt_hip_module_load_file": (i32, [vp, C.c_char_p]),
         "smelt_hip_pipeline_create": (i32, [vp, C.c_char_p, i32, C.POINTER(u32)]),
@@ -169,7 +177,10 @@ class Context:
         self._pipelines: dict[str, int] = {}
         self.check(self.lib.smelt_hip_set_activation_dtype(self.h, act_dtype))
         if load_module:
-            self.check(self.lib.smelt_hip_module_load_file(self.h, HSACO.encode()))
+            self.check(self.lib.smelt_hip_module_load_file(self.h, LIB_DIR.encode()))
+
+    def set_matvec_engine(self, engine: int) -> None:
+        self.check(self.lib.smelt_hip_set_matvec_engine(self.h, engine))
 
     def close(self) -> None:
         if getattr(self, "h", None):

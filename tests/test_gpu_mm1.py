@@ -1,0 +1,172 @@
+"""GPU parity of the single-pass matrix-core matvec (the kernel large single-token records take):
+every format and both activation types against the oracle, through the C-ABI, with the engine
+forced to the matrix cores so that small, ragged and odd-width shapes exercise it too."""
+import numpy as np
+import pytest
+
+import fixtures as fx
+import gpu_harness as gh
+from oracle import oracle as so
+from smelt_amd import runtime as rt
+from test_gpu_matvec import run_affine, run_signed
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = rt.Context()
+    c.set_matvec_engine(rt.MATVEC_MATRIX_CORE)
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def vec():
+    c = rt.Context()
+    c.set_matvec_engine(rt.MATVEC_VECTOR)
+    yield c
+    c.close()
+
+
+# rows: multiples of 8, ragged tails, fewer than one tile; cols: one 16-byte piece per row, a partial
+# 128-byte segment, several segments per wave, several waves per row
+AFFINE_SHAPES = [(8, 32, 32), (5, 64, 64), (50, 1152, 64), (130, 3584, 64), (24, 2560, 128), (264, 5120, 64),
+                 (72, 17408, 64), (33, 9216, 32)]
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("shape", AFFINE_SHAPES)
+def test_affine_matrix_core_matvec(ctx, dtype, shape):
+    rows, cols, group = shape
+    packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=rows)
+    x = fx.synth_activation(1, cols, dtype, config=1, tensor=cols)
+    ref = so.affine_matvec(packed, scales, biases, fx.from_bits(x, dtype), rows, cols, group, dtype)
+    y = run_affine(ctx, packed, scales, biases, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    w = gh.check_outputs(y, ref, dtype, f"matrix-core affine {shape}")
+    print(f"\n  matrix-core affine {shape} dtype={dtype} max rel err {w:.2e}")
+
+
+def test_affine_matrix_core_exact_on_dyadic_fixture(ctx):
+    """KernelLab.swift:2829-2855 buffers: every partial sum is an exact dyadic rational, so the
+    matrix cores must give the oracle's bits too."""
+    rows, cols, group = 64, 1024, 64
+    packed, scales, biases, x = fx.kernel_lab_qmm_fixture(rows, cols, group, 1)
+    ref = so.affine_matvec(packed, scales, biases, fx.from_bits(x, fx.F16), rows, cols, group)
+    y = run_affine(ctx, packed, scales, biases, x, fx.F16, f"affine_matvec:{cols}:{group}", generic=True)
+    assert np.array_equal(y, ref.astype(np.float16).view(np.uint16))
+
+
+SIGNED_SHAPES = [(5, 128), (8, 256), (50, 1152), (1024, 5120), (264, 17408), (77, 9216)]
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")])
+@pytest.mark.parametrize("shape", SIGNED_SHAPES)
+def test_signed_matrix_core_matvec(ctx, fmt, name, dtype, shape):
+    rows, cols = shape
+    codes = fx.synth_signed_codes(fmt, rows, cols, config=2 + fmt, tensor=rows % 7)
+    scales = fx.synth_signed_scales(rows, cols, config=2 + fmt, tensor=rows % 7)
+    packed = fx.pack_signed_np(codes, fmt)
+    x = fx.synth_activation(1, cols, dtype, config=2 + fmt)
+    ref = so.signed_matvec(fmt, packed, scales, fx.from_bits(x, dtype), rows, cols, cols, 128)
+    y = run_signed(ctx, name, packed, scales, x, dtype, rows, cols)
+    w = gh.check_outputs(y, ref, dtype, f"matrix-core signed {name} {shape}")
+    print(f"\n  matrix-core {name} {shape} dtype={dtype} max rel err {w:.2e}")
+
+
+def test_ternary_matrix_core_reproduces_mlx_golden_bits(ctx):
+    """MLX v0.31.1 bit patterns held by SignedQuantKernelTests.swift:87-199: all partial sums of
+    these fixtures are exact in fp32, so the matrix-core kernel must reproduce them as well."""
+    g = fx.golden_vectors()
+    for key in ("ternary_qmv_mlx_k512", "ternary_qmv_mlx_k5120_m3"):
+        case = g[key]
+        codes, scales, x = fx.mlx_ternary_fixture(case["rows"], case["cols"], case["batch"], case["scale_unit"])
+        packed = fx.pack_signed_np(codes, fx.TERNARY2)
+        want = np.array([int(b, 16) for b in case["expected_bits"]], np.uint16).reshape(case["batch"], case["rows"])
+        for b in range(case["batch"]):   # the matrix-core kernel is the single-token one
+            y = run_signed(ctx, "ternary", packed, scales, x[b:b + 1], fx.F16, case["rows"], case["cols"])
+            assert np.array_equal(y[0], want[b]), (key, b)
+
+
+@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")])
+def test_signed_matrix_core_fused_forms_equal_staged(ctx, fmt, name):
+    rows, cols = 100, 2560
+    dtype = fx.BF16
+    gc = fx.synth_signed_codes(fmt, rows, cols, tensor=1)
+    uc = fx.synth_signed_codes(fmt, rows, cols, tensor=2)
+    gs = fx.synth_signed_scales(rows, cols, tensor=1)
+    us = fx.synth_signed_scales(rows, cols, tensor=2)
+    gp, up = fx.pack_signed_np(gc, fmt), fx.pack_signed_np(uc, fmt)
+    x = fx.synth_activation(1, cols, dtype, config=2)
+    g = run_signed(ctx, name, gp, gs, x, dtype, rows, cols)
+    u = run_signed(ctx, name, up, us, x, dtype, rows, cols)
+    res = fx.to_bits(fx.rng_for(2, 78).normal(0, 1, (1, rows)).astype(np.float32), dtype)
+    fused_add = run_signed(ctx, name, gp, gs, x, dtype, rows, cols, kind="add", residual=res)
+    assert np.array_equal(fused_add, so.narrow(fx.from_bits(g, dtype) + fx.from_bits(res, dtype), dtype))
+    fused = run_signed(ctx, name, gp, gs, x, dtype, rows, cols, kind="gate_up", second=(up, us))
+    staged = so.epilogue_signed_swiglu(g, u, so.BF16)
+    diff = np.abs(fused.astype(np.int32) - staged.astype(np.int32))
+    assert diff.max() <= 1, diff.max()   # the low-precision exp() is not pinned bit-exactly
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_affine_matrix_core_fused_forms_equal_staged(ctx, dtype):
+    rows, cols, group = 200, 5120, 64
+    gw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=4)
+    uw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=5)
+    x = fx.synth_activation(1, cols, dtype, config=1)
+    y = run_affine(ctx, *gw, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    res = fx.to_bits(fx.rng_for(1, 77).normal(0, 1, (1, rows)).astype(np.float32), dtype)
+    fused = run_affine(ctx, *gw, x, dtype, f"fused_affine_matvec_add:{cols}:{group}", residual=res, generic=True)
+    assert np.array_equal(fused, so.narrow(fx.from_bits(y, dtype) + fx.from_bits(res, dtype), dtype))
+    xf = fx.from_bits(x, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
+    u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
+    ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, so.BF16 if dtype == fx.BF16 else so.F16), dtype)
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*gw, *uw)]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(gh.X_SLOT, x)
+    ctx.alloc(gh.Y_SLOT, rows * 2)
+    bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
+    pipe = ctx.pipeline(f"fused_affine_gate_up_swiglu_c{cols}_r{rows}_g{group}_rows4" + gh.t_suffix(dtype))
+    ctx.encode_decode(rt.make_record(pipe, bufs, [], (512, 1, 1), (256, 1, 1)))
+    ctx.wait()
+    got = ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+    gh.check_outputs(got, ref, dtype, "matrix-core affine gate_up_swiglu", rel_tol=8e-3 if dtype == fx.BF16 else 4e-3)
+
+
+def test_engines_agree_within_tolerance_and_auto_switches_by_size(ctx, vec):
+    """The two engines differ in summation order only; AUTO keeps a small matrix on the vector
+    kernel (bit-identical to VECTOR) and moves a large one to the matrix cores (bit-identical to
+    MATRIX_CORE)."""
+    dtype = fx.BF16
+    auto = rt.Context()
+    try:
+        for rows, cols, large in ((256, 1024, False), (2048, 5120, True)):
+            w = fx.synth_affine(rows, cols, 64, dtype, config=1, tensor=3)
+            x = fx.synth_activation(1, cols, dtype, config=1, tensor=4)
+            name = f"affine_matvec:{cols}:64"
+            ym = run_affine(ctx, *w, x, dtype, name, generic=True)
+            yv = run_affine(vec, *w, x, dtype, name, generic=True)
+            ya = run_affine(auto, *w, x, dtype, name, generic=True)
+            ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
+            gh.check_outputs(ym, ref, dtype, "matrix-core")
+            gh.check_outputs(yv, ref, dtype, "vector")
+            assert np.array_equal(ya, ym if large else yv)
+    finally:
+        auto.close()
+
+
+def test_bf16_activations_beyond_the_fp16_range(ctx):
+    """bf16 activations enter the bf16 MFMA unconverted: magnitudes past 65504 are not clamped."""
+    rows, cols, group = 64, 1024, 64
+    dtype = fx.BF16
+    packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=8)
+    xf = fx.rng_for(1, 555).normal(0, 1, (1, cols)).astype(np.float32)
+    xf[0, ::37] *= 3.0e5
+    x = fx.to_bits(xf, dtype)
+    ref = so.affine_matvec(packed, scales, biases, fx.from_bits(x, dtype), rows, cols, group, dtype)
+    y = run_affine(ctx, packed, scales, biases, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    gh.check_outputs(y, ref, dtype, "matrix-core affine with |x| > 65504")

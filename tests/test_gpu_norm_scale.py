@@ -205,6 +205,9 @@ def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
     em.fused_norm_matvec(0, wg, cc.bind(X), cc.bind(NW), cc.bind(F4), cc.bind(SCR), up=wu)
     ctx = rt.Context(act_dtype=act)
     try:
+        # fused == unfused bit for bit holds between kernels of one engine: the norm-scale prologue
+        # exists on the vector-ALU kernels only, so the unfused records are kept there as well
+        ctx.set_matvec_engine(rt.MATVEC_VECTOR)
         em.install(ctx)
         ctx.upload_weights(0, image)
         x, w, _ = norm_inputs(1, hidden, dtype, seed=3)
