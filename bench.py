@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized matvec hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only step|layers|qmm|aux] [--engine auto|matrix|vector]
 
 A step is one pass over the decode-step matvec set of a 24-layer Qwen3.5-0.8B-shaped stack
 (BASELINE configs[1]): the q/k/v projection bank, o, fused gate+up, down (+residual) per layer and
@@ -10,13 +10,21 @@ tensors resident in HBM before the timed region.  The records are emitted by the
 emitters, captured once into a HIP graph and replayed; `value` is weight bytes (packed codes +
 scales + biases, counted once per step) divided by the step time.
 
-Prints one JSON line (see the fields at the bottom).  Nothing here runs on the CPU except the
-`cpu_baseline` leg, which times the scalar oracle on a bounded sample of the same workload.
+Side measurements (`extra`) follow the reference's kernel-lab protocol (KernelLab.swift:2738-2805,
+2965-2976): at least 200 timed launches per figure, median and p95.  One sample is one individually
+timed replay of a graph that holds back-to-back launches over rotating weight copies; "cold"
+figures rotate through at least 3 x 256 MB of distinct weights so that the 256 MB Infinity Cache
+cannot serve them, "warm" figures re-read one copy.
+
+Prints one JSON line.  Nothing here runs on the CPU except the `cpu_baseline` leg, which times the
+scalar oracle on a bounded sample of the same workload, and the one-off check of the lm_head
+argmax token against the oracle (outside every timed region).
 """
 from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -27,7 +35,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
-HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X published dense bf16 / fp16 matrix rate
+COLD_BYTES = 3 * (256 << 20)  # distinct weight bytes a cold rotation has to span
+MIN_TIMED_LAUNCHES = 200
 
 
 def synth_affine(rng, rows, cols, group, bf16):
@@ -38,13 +49,44 @@ def synth_affine(rng, rows, cols, group, bf16):
     return packed, bf16(s), bf16(b)
 
 
+def timed_replays(ctx, graph, launches, min_launches=MIN_TIMED_LAUNCHES, warm=2):
+    """Per-launch time of a graph's kernels: one sample = one individually timed replay divided by
+    its launch count; enough replays for `min_launches` timed launches."""
+    for _ in range(warm):
+        ctx.graph_time(graph, 1)
+    reps = max(8, math.ceil(min_launches / launches))
+    s = np.sort(np.array([ctx.graph_time(graph, 1) / launches for _ in range(reps)]))
+    p95 = s[min(len(s) - 1, math.ceil(0.95 * len(s)) - 1)]
+    return {"us_median": round(float(np.median(s)), 3), "us_p95": round(float(p95), 3), "us_min": round(float(s[0]), 3),
+            "timed_launches": int(reps * launches), "replays": int(reps)}
+
+
+def time_records(ctx, records, rounds=1, **kw):
+    """timed_replays() of a graph of `records` repeated `rounds` times."""
+    table = ctx.table(list(records) * rounds)
+    g, n = ctx.capture_decode(table)
+    out = timed_replays(ctx, g, n, **kw)
+    ctx.graph_destroy(g)
+    return out
+
+
+def rounds_for(launches, target=32):
+    """Rounds over a rotation per graph, so that the cost of starting a replay is spread over >= target launches."""
+    return max(1, math.ceil(target / launches))
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the 27B-layer and qmm side measurements")
+    ap.add_argument("--no-extra", action="store_true", help="skip every side measurement")
+    ap.add_argument("--only", choices=("step", "layers", "qmm", "aux"), default=None,
+                    help="the step plus one group of side measurements (layers: 27B-layer matvecs per weight format; "
+                         "qmm: 4B FFN token tiles; aux: config-0 cold/warm, cold step, quantiser, turbo_quant_h)")
+    ap.add_argument("--engine", choices=("auto", "matrix", "vector"), default="auto",
+                    help="single-token matvec engine (smelt_hip_set_matvec_engine); auto is what a package gets")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path has no cross-GPU part in this build "
@@ -55,31 +97,42 @@ def main() -> int:
     from smelt_amd import compiler as cc
     from smelt_amd import runtime as rt
 
+    engine = {"auto": rt.MATVEC_AUTO, "matrix": rt.MATVEC_MATRIX_CORE, "vector": rt.MATVEC_VECTOR}[args.engine]
     ctx = rt.Context(act_dtype=rt.ACT_BF16)
+    ctx.set_matvec_engine(engine)
     info = ctx.device_info()
     cus = info["compute_units"]
-    dtype = fx.BF16
     group, hidden, ffn, vocab, layers = 64, 1024, 3584, 151936, 24
+    groups = ("layers", "qmm", "aux") if args.only is None else () if args.only == "step" else (args.only,)
+    if args.no_extra:
+        groups = ()
+    want_cold_step = "aux" in groups
 
     # ---- weights.bin image of the workload ----------------------------------------------------
+    # set 0 is the step; sets 1 and 2 hold the same seeded tensors and exist so that a cold step can rotate
+    nsets = 3 if want_cold_step else 1
+    lm_copies = math.ceil(COLD_BYTES / (vocab * 576))  # copy 0 belongs to the step; the rest only rotate
     lay = cc.Layout()
-    per_layer = []
-    for _ in range(layers):
-        q, k, v = lay.affine_bank([2048, 512, 512], hidden, group)  # same-input projection bank
-        per_layer.append({
-            "q": q, "k": k, "v": v, "o": lay.affine(1024, hidden, group),
-            "gate": lay.affine(ffn, hidden, group), "up": lay.affine(ffn, hidden, group),
-            "down": lay.affine(hidden, ffn, group)})
-    lm_copies = 4  # copy 0 belongs to the step; 1..3 only rotate under the roofline measurement
+    sets = []
+    for _ in range(nsets):
+        per_layer = []
+        for _ in range(layers):
+            q, k, v = lay.affine_bank([2048, 512, 512], hidden, group)  # same-input projection bank
+            per_layer.append({
+                "q": q, "k": k, "v": v, "o": lay.affine(1024, hidden, group),
+                "gate": lay.affine(ffn, hidden, group), "up": lay.affine(ffn, hidden, group),
+                "down": lay.affine(hidden, ffn, group)})
+        sets.append(per_layer)
     lm_heads = [lay.affine(vocab, hidden, group) for _ in range(lm_copies)]
     image = np.zeros(lay.total_bytes, np.uint8)
     weight_bytes = 0
     tensor = 0
-    for L in per_layer:
-        for e in L.values():
-            t = synth_affine(fx.rng_for(1, tensor), e.rows, e.cols, group, fx.bf16_bits)
-            cc.write_affine(image, e, *t)
-            weight_bytes += e.size_bytes + e.scales_size_bytes + e.biases_size_bytes
+    for li in range(layers):
+        for key, e0 in sets[0][li].items():
+            t = synth_affine(fx.rng_for(1, tensor), e0.rows, e0.cols, group, fx.bf16_bits)
+            for s in sets:
+                cc.write_affine(image, s[li][key], *t)
+            weight_bytes += e0.size_bytes + e0.scales_size_bytes + e0.biases_size_bytes
             tensor += 1
     lm_t = synth_affine(fx.rng_for(1, tensor), vocab, hidden, group, fx.bf16_bits)
     for e in lm_heads:
@@ -90,20 +143,21 @@ def main() -> int:
     # ---- slots and records -----------------------------------------------------------------------
     W, H0, H1, QKV, ATT, ACT, KEYS, TOK = 0, 1, 2, 3, 4, 5, 6, 7
     em = cc.Emitter(rt.ACT_BF16, cus)
-    for L in per_layer:
-        # cur = hidden state in, alt = hidden state out; swapped after every layer
-        banked = em.bank_matvec(W, [L["q"], L["k"], L["v"]], cc.bind(rt.SLOT_CUR),
-                                [cc.bind(QKV, 0), cc.bind(QKV, 2048 * 2), cc.bind(QKV, 2560 * 2)])
-        assert banked
-        em.matvec(W, L["o"], cc.bind(ATT), cc.bind(rt.SLOT_ALT))
-        em.gate_up_swiglu(W, L["gate"], L["up"], cc.bind(rt.SLOT_ALT), cc.bind(ACT))
-        em.matvec_add(W, L["down"], cc.bind(ACT), cc.bind(rt.SLOT_ALT), cc.bind(rt.SLOT_CUR))
-        em.swap()
-    em.lm_head_argmax(W, lm_heads[0], cc.bind(rt.SLOT_CUR), cc.bind(KEYS), cc.bind(TOK))
-    step_records = len(em.records())
-    # roofline records: the lm_head kernel over rotating weight copies (4 x 87.5 MB > the 256 MB
-    # Infinity Cache, so every launch streams from HBM)
-    for e in lm_heads:
+    step_ends = []
+    for si, per_layer in enumerate(sets):
+        for L in per_layer:
+            # cur = hidden state in, alt = hidden state out; swapped after every layer
+            banked = em.bank_matvec(W, [L["q"], L["k"], L["v"]], cc.bind(rt.SLOT_CUR),
+                                    [cc.bind(QKV, 0), cc.bind(QKV, 2048 * 2), cc.bind(QKV, 2560 * 2)])
+            assert banked
+            em.matvec(W, L["o"], cc.bind(ATT), cc.bind(rt.SLOT_ALT))
+            em.gate_up_swiglu(W, L["gate"], L["up"], cc.bind(rt.SLOT_ALT), cc.bind(ACT))
+            em.matvec_add(W, L["down"], cc.bind(ACT), cc.bind(rt.SLOT_ALT), cc.bind(rt.SLOT_CUR))
+            em.swap()
+        em.lm_head_argmax(W, lm_heads[si], cc.bind(rt.SLOT_CUR), cc.bind(KEYS), cc.bind(TOK))
+        step_ends.append(len(em.records()))
+    rl_start = len(em.records())
+    for e in lm_heads:  # roofline records: the lm_head kernel over every rotating copy, input fixed
         em.lm_head_argmax(W, e, cc.bind(H0), cc.bind(KEYS), cc.bind(TOK))
     em.install(ctx)
     ctx.upload_weights(W, image)
@@ -117,8 +171,20 @@ def main() -> int:
     ctx.alloc(KEYS, max(em.argmax_partial_bytes, 8))
     ctx.alloc(TOK, 4)
     records = list(em.records())
-    step_table = ctx.table(records[:step_records])
+    step_table = ctx.table(records[:step_ends[0]])
     launches_per_step = sum(1 for r in step_table if r.op_kind == 0)
+
+    # ---- the full-size lm_head matvec + argmax against the oracle (outside every timed region) ------
+    ctx.interpret_decode(ctx.table(records[rl_start:rl_start + 2]))
+    ctx.wait()
+    lm_token = int(ctx.read(TOK, np.int32, 1)[0])
+    from oracle import oracle as so
+    logits = so.narrow(so.affine_matvec(*lm_t, fx.from_bits(x.reshape(1, -1), fx.BF16), vocab, hidden, group, so.BF16, threads=True), so.BF16)[0]
+    oracle_token = so.argmax16(logits)
+    # the two sides sum in different orders: a token whose 16-bit oracle logit equals the winner's is a tie
+    if lm_token != oracle_token and not (0 <= lm_token < vocab and logits[lm_token] == logits[oracle_token]):
+        print(f"lm_head argmax mismatch: GPU {lm_token}, oracle {oracle_token}", file=sys.stderr)
+        return 1
 
     # ---- timed region: K graph replays bracketed by synchronisation --------------------------------
     graph, launched = ctx.capture_decode(step_table, cur=H0, alt=H1)
@@ -134,32 +200,22 @@ def main() -> int:
     token = int(ctx.read(TOK, np.int32, 1)[0])
     ctx.graph_destroy(graph)
 
-    # ---- roofline of the dominant kernel (lm_head matvec + argmax, 30% of the step's bytes) ----------
-    rl_table = ctx.table([r for r in records[step_records:] if True])
-    # keep only the matvec+argmax records (every second record is the tiny key reduce)
-    # (eight rounds over the four copies per replay, so that the cost of starting a graph is spread
-    # over 32 launches and the figure is the kernel's own back-to-back cadence)
-    rl_only = ctx.table([r for i, r in enumerate(records[step_records:]) if i % 2 == 0] * 8)
-    g2, n2 = ctx.capture_decode(rl_only, cur=H0, alt=H1)
-    ctx.graph_time(g2, 5)
-    reps = 10
-    # five timed series of ten replays each; the median series is reported (clock ramps and other
-    # tenants of the memory system move single series by a few percent)
-    series = sorted(ctx.graph_time(g2, reps) / (reps * n2) for _ in range(5))
-    lm_us = series[2]
-    ctx.graph_destroy(g2)
+    # ---- roofline of the largest kernel of the step (lm_head matvec + argmax, 30% of its bytes) -------
+    # every second roofline record is the tiny key reduce; the graph holds the matvec+argmax launches only
+    rl_only = [r for i, r in enumerate(records[rl_start:]) if i % 2 == 0]
+    rl = time_records(ctx, rl_only, rounds=rounds_for(len(rl_only)))
+    lm_us = rl["us_median"]
     achieved = lm_bytes / lm_us / 1e3
+    traffic, traffic_source = committed_traffic()
     roofline = {"bound": "hbm", "kernel": "smelt_affine_matvec_argmax_single_bf16 (lm_head 151936x1024 u4 g64, fused argmax)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "bytes_per_launch": int(lm_bytes), "us_per_launch": round(lm_us, 3),
-                "us_per_launch_series": [round(v, 3) for v in series]}
-    del rl_table
-    roofline["traffic"] = committed_traffic()
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                "bytes_per_launch": int(lm_bytes), "us_per_launch": lm_us, "us_per_launch_p95": rl["us_p95"],
+                "timed_launches": rl["timed_launches"], "rotation_bytes": int(lm_bytes * lm_copies), "cache_state": "cold"}
 
     # One plain copy of known size: the calibration dispatch for HBM traffic counters (a counter
-    # run of this same command scales FETCH_SIZE / WRITE_SIZE of the lm_head kernel by what they
-    # read for this copy).
+    # run of this same command scales FETCH_SIZE / WRITE_SIZE of any kernel by what they read for
+    # this copy).
     CAL_SRC, CAL_DST, cal_bytes = 8, 9, 256 << 20
     ctx.alloc(CAL_SRC, cal_bytes)
     ctx.alloc(CAL_DST, cal_bytes)
@@ -170,12 +226,27 @@ def main() -> int:
     ctx.wait()
 
     extra = {}
-    if not args.no_extra:
-        extra = side_measurements(ctx, fx, cc, rt, cus)
+    if want_cold_step:
+        # the same step over three rotating weight sets: what a step costs when nothing of it is left
+        # in the Infinity Cache (the headline replays one 293 MB set, of which the cache keeps a part)
+        g, n = ctx.capture_decode(ctx.table(records[:step_ends[-1]]), cur=H0, alt=H1)
+        t = timed_replays(ctx, g, nsets, min_launches=60)
+        ctx.graph_destroy(g)
+        extra["config1_step_cold"] = {"ms_per_step": round(t["us_median"] / 1e3, 5), "ms_per_step_p95": round(t["us_p95"] / 1e3, 5),
+                                      "GBps": round(weight_bytes / t["us_median"] / 1e3, 1), "rotation_bytes": int(weight_bytes * nsets),
+                                      "steps_timed": t["timed_launches"]}
+    ctx.close()
+
+    if "layers" in groups:
+        extra.update(layer_measurements(fx, cc, rt, cus, engine))
+    if "qmm" in groups:
+        extra.update(qmm_measurements(fx, cc, rt, cus))
+    if "aux" in groups:
+        extra.update(aux_measurements(fx, cc, rt, cus, engine))
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(fx, per_layer, lm_heads[0], group)
+        cpu = cpu_baseline(fx, sets[0], lm_heads[0], group)
 
     out = {
         "metric": "qmatvec effective weight GB/s at M=1 (decode-step matvec set)",
@@ -185,147 +256,215 @@ def main() -> int:
         "config": {"workload": "configs[1]: 24-layer Qwen3.5-0.8B-shaped decode matvec set + 151936x1024 lm_head, "
                                "affine u4 g64, bf16 activations/scales, fp32 accumulate, M=1",
                    "weight_bytes_per_step": int(weight_bytes), "launches_per_step": launches_per_step,
-                   "replay": "hip graph", "device": info["name"].strip(), "compute_units": cus},
+                   "replay": "hip graph over one weight set (293 MB against a 256 MB Infinity Cache: partly warm)",
+                   "matvec_engine": args.engine, "device": info["name"].strip(), "compute_units": cus},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "wall_ms_timed_region": round(wall_ms, 3), "argmax_token": token,
+        "lm_head_argmax_check": {"gpu": lm_token, "oracle": oracle_token, "rows": vocab},
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(out))
-    ctx.close()
     return 0
 
 
 def committed_traffic():
     """HBM bytes per lm_head launch from the committed counter summary (two rocprofv3 --pmc runs of
-    this command, scaled by the copy calibration); None when no summary is present."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "lm_head_argmax_bf16_hbm_traffic.txt")
+    this command, scaled by the copy calibration) and where the figure comes from; None when absent."""
+    rel = os.path.join("profiles", "lm_head_argmax_bf16_hbm_traffic.txt")
     try:
-        for line in open(path):
+        for line in open(os.path.join(ROOT, rel)):
             if line.startswith("traffic_bytes_per_launch"):
-                return int(line.split("=")[1].split()[0])
+                return int(line.split("=")[1].split()[0]), f"committed counter summary {rel}; not measured by this run"
     except OSError:
         pass
-    return None
+    return None, None
 
 
-def side_measurements(ctx, fx, cc, rt, cus) -> dict:
-    """27B-layer binary / ternary / trit5 matvec sets, the 4B FFN qmm at M in {7,8,9,32,512}, the
-    affine 4-bit quantiser and a turbo_quant_h matvec.  Reported beside the headline; not part of `value`."""
+def signed_tensor(fx, rng, fmt, rows, cols, stride):
+    """Seeded codes + g128 fp16 scales of one signed matrix: bits p = 0.5; trits P(-1, 0, +1) = .3, .4, .3."""
+    if fmt == fx.BINARY1:
+        packed = rng.integers(0, 256, size=(rows, stride), dtype=np.uint8)
+    else:
+        u = rng.random(size=(rows, cols), dtype=np.float32)
+        codes = (u >= 0.3).astype(np.uint8) + (u >= 0.7).astype(np.uint8)
+        del u
+        packed = fx.pack_signed_np(codes, fmt, stride)
+        del codes
+    scales = fx.f16_bits(np.abs(rng.normal(0, 0.02, size=(rows, cols // 128))).astype(np.float32))
+    return packed, scales
+
+
+def layer_measurements(fx, cc, rt, cus, engine) -> dict:
+    """One 27B-shaped decoder layer (hidden 5120, FFN 17408, q/o 5120, k/v 1024) per weight format, as the
+    dispatch records a decode step holds: q/k/v (one bank launch where the format has a bank kernel),
+    o, fused gate+up+SwiGLU, down+residual.  Cold: the rotated layer copies span >= 768 MB."""
     out = {}
-    W, X, Y, ACT = 20, 21, 22, 23
-    shapes = [(17408, 5120), (17408, 5120), (5120, 17408), (5120, 5120), (5120, 5120), (1024, 5120), (1024, 5120)]
-    for name, wdtype, fmt in (("binary1", cc.BINARY1, fx.BINARY1), ("ternary2", cc.TERNARY2, fx.TERNARY2),
-                              ("trit5", cc.TRIT5, fx.TRIT5)):
+    W, X, XF, Y, RES, QKV = 20, 21, 22, 23, 24, 25
+    H, F, KV = 5120, 17408, 1024
+    formats = (("affine_u4_g64", None, None), ("binary1", cc.BINARY1, fx.BINARY1), ("ternary2", cc.TERNARY2, fx.TERNARY2),
+               ("trit5", cc.TRIT5, fx.TRIT5))
+    for name, wdtype, fmt in formats:
         c = rt.Context(act_dtype=rt.ACT_BF16)
+        c.set_matvec_engine(engine)
         lay = cc.Layout()
-        copies = 6  # rotate layer copies so launches stream from HBM rather than the Infinity Cache
-        ents = [[lay.signed(r, k, wdtype) for (r, k) in shapes] for _ in range(copies)]
+
+        def nbytes(*es):
+            return sum(e.size_bytes + e.scales_size_bytes + (e.biases_size_bytes if wdtype is None else 0) for e in es)
+
+        def make_layer():
+            if wdtype is None:
+                q, k, v = lay.affine_bank([H, KV, KV], H, 64)
+                mk = lambda r, k_: lay.affine(r, k_, 64)
+            else:
+                mk = lambda r, k_: lay.signed(r, k_, wdtype)
+                q, k, v = mk(H, H), mk(KV, H), mk(KV, H)
+            return {"q": q, "k": k, "v": v, "o": mk(H, H), "gate": mk(F, H), "up": mk(F, H), "down": mk(H, F)}
+
+        first = make_layer()
+        layer_bytes = nbytes(*first.values())
+        copies = math.ceil(COLD_BYTES / layer_bytes)
+        stack = [first] + [make_layer() for _ in range(copies - 1)]
         image = np.zeros(lay.total_bytes, np.uint8)
         rng = fx.rng_for(2, 0)
-        layer_bytes = 0
-        for ti, e0 in enumerate(ents[0]):
-            if fmt == fx.BINARY1:
-                packed = rng.integers(0, 256, size=(e0.rows, e0.packed_row_stride), dtype=np.uint8)
+        for key, e0 in first.items():
+            if wdtype is None:
+                t = synth_affine(rng, e0.rows, e0.cols, 64, fx.bf16_bits)
+                for L in stack:
+                    cc.write_affine(image, L[key], *t)
             else:
-                u = rng.random(size=(e0.rows, e0.cols), dtype=np.float32)
-                codes = (u >= 0.3).astype(np.uint8) + (u >= 0.7).astype(np.uint8)  # P(-1,0,+1) = .3,.4,.3
-                del u
-                packed = fx.pack_signed_np(codes, fmt, e0.packed_row_stride)
-                del codes
-            scales = fx.f16_bits(np.abs(rng.normal(0, 0.02, size=(e0.rows, e0.cols // 128))).astype(np.float32))
-            for layer in ents:  # every rotating copy holds the same seeded tensor
-                cc.write_signed(image, layer[ti], packed, scales)
-            layer_bytes += e0.size_bytes + e0.scales_size_bytes
+                t = signed_tensor(fx, rng, fmt, e0.rows, e0.cols, e0.packed_row_stride)
+                for L in stack:
+                    cc.write_signed(image, L[key], *t)
+            del t
         em = cc.Emitter(rt.ACT_BF16, cus)
-        for layer in ents:
-            for e in layer:
-                em.matvec(W, e, cc.bind(X), cc.bind(Y))
+        classes = {"qkv": [], "o": [], "gate_up": [], "down": []}
+        for L in stack:
+            marks = [len(em.records())]
+            outs = [cc.bind(QKV, 0), cc.bind(QKV, H * 2), cc.bind(QKV, (H + KV) * 2)]
+            try:
+                banked = em.bank_matvec(W, [L["q"], L["k"], L["v"]], cc.bind(X), outs)
+            except cc.EmitError:
+                banked = False
+            if not banked:
+                for key, o in zip(("q", "k", "v"), outs):
+                    em.matvec(W, L[key], cc.bind(X), o)
+            marks.append(len(em.records()))
+            em.matvec(W, L["o"], cc.bind(X), cc.bind(Y))
+            marks.append(len(em.records()))
+            em.gate_up_swiglu(W, L["gate"], L["up"], cc.bind(X), cc.bind(XF))
+            marks.append(len(em.records()))
+            em.matvec_add(W, L["down"], cc.bind(XF), cc.bind(Y), cc.bind(RES))
+            marks.append(len(em.records()))
+            for cls, a, b in zip(classes, marks[:-1], marks[1:]):
+                classes[cls].append((a, b))
+        class_bytes = {"qkv": nbytes(first["q"], first["k"], first["v"]), "o": nbytes(first["o"]),
+                       "gate_up": nbytes(first["gate"], first["up"]), "down": nbytes(first["down"])}
         em.install(c)
         c.upload_weights(W, image)
         del image
-        c.put(X, fx.bf16_bits(fx.rng_for(2, 1).normal(0, 1, 17408).astype(np.float32)))
-        c.alloc(Y, 17408 * 2)
-        table = em.records()
-        g, n = c.capture_decode(table)
-        c.graph_time(g, 3)
-        reps = 20
-        us = c.graph_time(g, reps) / (reps * copies)
-        per_kernel = {}
-        recs = list(table)
-        for (r, k), rec in zip(shapes[:3:2] + shapes[3:4] + shapes[5:6], [recs[0], recs[2], recs[3], recs[5]]):
-            t = c.benchmark_record(rec, warmup=5, iters=50)
-            e = [x for x in ents[0] if (x.rows, x.cols) == (r, k)][0]
-            b = e.size_bytes + e.scales_size_bytes
-            per_kernel[f"{r}x{k}"] = {"us_warm_median": round(float(np.median(t)), 2), "weight_bytes": int(b)}
-        c.graph_destroy(g)
-        views = None
-        if fmt in (fx.BINARY1, fx.TERNARY2):
-            # the same layer through signed activation views (i5): one view per distinct input
-            # (q/k/v share one, gate/up share one), every projection an integer popcount matvec
-            VP, VS = 24, 25
-            c.alloc(VP, 17408 // 128 * 5 * 16)
-            c.alloc(VS, 17408 // 128 * 2)
-            em2 = cc.Emitter(rt.ACT_BF16, cus)
-            for layer in ents:
-                for i, e in enumerate(layer):
-                    if i in (0, 2, 3, 5):   # gate (up shares it), down, q (k/v share it), o: a new input
-                        em2.activation_view(5, cc.bind(X), cc.bind(VP), cc.bind(VS), e.cols)
-                    em2.view_matvec(W, e, 5, cc.bind(VP), cc.bind(VS), cc.bind(Y))
-            remap = {i: c.pipeline(nm) for i, nm in enumerate(em2.pipelines)}
-            recs2 = list(em2.records())
-            for r in recs2:
-                r.pipeline = remap[r.pipeline]
-            g2, n2 = c.capture_decode(c.table(recs2))
-            c.graph_time(g2, 3)
-            us2 = c.graph_time(g2, reps) / (reps * copies)
-            c.graph_destroy(g2)
-            views = {"us_per_layer": round(us2, 2), "launches": n2 // copies, "planes": 5,
-                     "GBps": round(layer_bytes / us2 / 1e3, 1)}
-        out[f"bonsai27b_layer_{name}"] = {
-            "us_per_layer": round(us, 2), "weight_bytes": int(layer_bytes),
-            "GBps": round(layer_bytes / us / 1e3, 1), "pct_of_hbm_peak": round(100 * layer_bytes / us / 1e3 / HBM_PEAK_GBS, 2),
-            "launches": len(shapes), "kernels": per_kernel, "activation_views_i5": views}
+        c.put(X, fx.bf16_bits(fx.rng_for(2, 1).normal(0, 1, H).astype(np.float32)))
+        c.put(XF, fx.bf16_bits(fx.rng_for(2, 2).normal(0, 1, F).astype(np.float32)))
+        c.put(RES, fx.bf16_bits(fx.rng_for(2, 3).normal(0, 1, H).astype(np.float32)))
+        c.alloc(Y, H * 2)
+        c.alloc(QKV, (H + 2 * KV) * 2)
+        recs = list(em.records())
+        per_layer = len(recs) // copies
+        whole = time_records(c, recs, rounds=rounds_for(len(recs), 64))
+        layer_us, layer_p95 = whole["us_median"] * per_layer, whole["us_p95"] * per_layer
+        kernels = {}
+        for cls, spans in classes.items():
+            sel = [r for a, b in spans for r in recs[a:b]]
+            per = len(sel) // copies
+            t = time_records(c, sel, rounds=rounds_for(len(sel)))
+            us = t["us_median"] * per
+            kernels[cls] = {"launches": per, "weight_bytes": int(class_bytes[cls]), "us_median": round(us, 2),
+                            "us_p95": round(t["us_p95"] * per, 2), "GBps": round(class_bytes[cls] / us / 1e3, 1),
+                            "frac_of_hbm_peak": round(class_bytes[cls] / us / 1e3 / HBM_PEAK_GBS, 4),
+                            "timed_launches": t["timed_launches"]}
+        out[f"layer27b_{name}"] = {
+            "us_per_layer": round(layer_us, 2), "us_per_layer_p95": round(layer_p95, 2), "weight_bytes": int(layer_bytes),
+            "GBps": round(layer_bytes / layer_us / 1e3, 1), "frac_of_hbm_peak": round(layer_bytes / layer_us / 1e3 / HBM_PEAK_GBS, 4),
+            "launches_per_layer": per_layer, "rotation_bytes": int(layer_bytes * copies), "cache_state": "cold",
+            "timed_launches": whole["timed_launches"], "kernels": kernels}
         c.close()
-    # qmm: Qwen3.5-4B FFN (gate/up 2560->9216, down 9216->2560), affine u4 g64
+    return out
+
+
+def qmm_measurements(fx, cc, rt, cus) -> dict:
+    """Qwen3.5-4B FFN (gate/up 2560->9216, down 9216->2560), affine u4 g64, M tokens per launch; cold rotation."""
+    W, X, Y = 20, 21, 22
     c = rt.Context(act_dtype=rt.ACT_BF16)
     lay = cc.Layout()
-    copies = 4
+    one = 2 * 9216 * (1280 + 160) + 2560 * (4608 + 576)
+    copies = math.ceil(COLD_BYTES / one)
     ents = [[lay.affine(9216, 2560, 64), lay.affine(9216, 2560, 64), lay.affine(2560, 9216, 64)] for _ in range(copies)]
     image = np.zeros(lay.total_bytes, np.uint8)
     rng = fx.rng_for(4, 0)
+    tens = [synth_affine(rng, e.rows, e.cols, 64, fx.bf16_bits) for e in ents[0]]
     for layer in ents:
-        for e in layer:
-            cc.write_affine(image, e, *synth_affine(rng, e.rows, e.cols, 64, fx.bf16_bits))
+        for e, t in zip(layer, tens):
+            cc.write_affine(image, e, *t)
     c.upload_weights(W, image)
-    del image
+    del image, tens
     xs = fx.rng_for(4, 1).normal(0, 1, (512, 9216)).astype(np.float32)
     xs[:, fx.rng_for(4, 2).choice(9216, 92, replace=False)] *= 10.0
     c.put(X, fx.bf16_bits(xs))
     c.alloc(Y, 512 * 9216 * 2)
     layer_bytes = sum(e.size_bytes + e.scales_size_bytes + e.biases_size_bytes for e in ents[0])
+    assert layer_bytes == one
     qmm = {}
-    pipes_installed = 0
-    for M in (7, 8, 9, 32, 512):
+    for M in (1, 7, 8, 9, 16, 32, 128, 512):
         em = cc.Emitter(rt.ACT_BF16, cus)
         for layer in ents:
             for e in layer:
                 em.matvec(W, e, cc.bind(X), cc.bind(Y), batch=M)
-        names = em.pipelines
-        remap = {i: c.pipeline(nm) for i, nm in enumerate(names)}
+        remap = {i: c.pipeline(nm) for i, nm in enumerate(em.pipelines)}
         recs = list(em.records())
         for r in recs:
             r.pipeline = remap[r.pipeline]
-        table = c.table(recs)
-        g, n = c.capture_prefill(table, seq_len=M)
-        c.graph_time(g, 2)
-        reps = 10 if M < 512 else 3
-        us = c.graph_time(g, reps) / (reps * copies)
+        g, n = c.capture_prefill(c.table(recs), seq_len=M)
+        t = timed_replays(c, g, n, min_launches=MIN_TIMED_LAUNCHES)
         c.graph_destroy(g)
+        us = t["us_median"] * 3
         flops = 2.0 * M * sum(e.rows * e.cols for e in ents[0])
-        qmm[f"M={M}"] = {"us_per_ffn": round(us, 2), "TFLOPs": round(flops / us / 1e6, 2),
-                         "weight_GBps": round(layer_bytes / us / 1e3, 1)}
-        pipes_installed += len(names)
-    out["qwen35_4b_ffn_qmm"] = qmm
+        qmm[f"M={M}"] = {"us_per_ffn": round(us, 2), "us_per_ffn_p95": round(t["us_p95"] * 3, 2), "TFLOPs": round(flops / us / 1e6, 2),
+                         "frac_of_mfma_peak": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4), "weight_GBps": round(layer_bytes / us / 1e3, 1),
+                         "frac_of_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "timed_launches": t["timed_launches"],
+                         "pipeline": em.pipelines[0]}
+    c.close()
+    return {"qwen35_4b_ffn_qmm": {"cache_state": "cold", "rotation_bytes": int(layer_bytes * copies),
+                                  "weight_bytes_per_ffn": int(layer_bytes), **qmm}}
+
+
+def aux_measurements(fx, cc, rt, cus, engine) -> dict:
+    out = {}
+    W, X, Y, ACT = 20, 21, 22, 23
+    # config 0: one 3584 x 1024 affine matvec, cold (rotating copies) and warm (one copy re-read)
+    c = rt.Context(act_dtype=rt.ACT_BF16)
+    c.set_matvec_engine(engine)
+    lay = cc.Layout()
+    rows, cols = 3584, 1024
+    one = rows * 576
+    copies = math.ceil(COLD_BYTES / one)
+    ents = [lay.affine(rows, cols, 64) for _ in range(copies)]
+    image = np.zeros(lay.total_bytes, np.uint8)
+    t = synth_affine(fx.rng_for(0, 0), rows, cols, 64, fx.bf16_bits)
+    for e in ents:
+        cc.write_affine(image, e, *t)
+    em = cc.Emitter(rt.ACT_BF16, cus)
+    for e in ents:
+        em.matvec(W, e, cc.bind(X), cc.bind(Y))
+    em.install(c)
+    c.upload_weights(W, image)
+    del image
+    c.put(X, fx.bf16_bits(fx.rng_for(0, 1).normal(0, 1, cols).astype(np.float32)))
+    c.alloc(Y, rows * 2)
+    recs = list(em.records())
+    cold = time_records(c, recs)
+    warm = time_records(c, recs[:1], rounds=64)
+    out["config0_affine_matvec_3584x1024"] = {
+        "weight_bytes": one, "cold": {**cold, "GBps": round(one / cold["us_median"] / 1e3, 1), "rotation_bytes": one * copies},
+        "warm": {**warm, "GBps": round(one / warm["us_median"] / 1e3, 1)}}
     c.close()
     # weight import: affine 4-bit quantiser over a 9216 x 2560 tensor resident in HBM
     # (algorithmic bytes = source read + packed codes, scales and biases written)
@@ -389,9 +528,10 @@ def side_measurements(ctx, fx, cc, rt, cus) -> dict:
 
 
 def cpu_baseline(fx, per_layer, lm_head, group) -> dict:
-    """Scalar restatement of the reference's CPU dequant-matvec (the oracle), row-parallel over
-    the host cores with OpenMP, on a bounded sample of the same workload: the first layer's seven
-    matrices plus the first 16384 lm_head rows (about 25 MB of weights per pass)."""
+    """Scalar restatement of the reference's CPU dequant-matvec (the oracle) on a bounded sample of the
+    same workload: the first layer's seven matrices plus the first 16384 lm_head rows (about 12 MB of
+    weights per pass).  Reported threaded (OpenMP over rows, the host cores this process may use);
+    `single_thread` holds the same code on the same sample on one core."""
     from oracle import oracle as so
     sample = [(e.rows, e.cols) for e in per_layer[0].values()] + [(16384, lm_head.cols)]
     rng = fx.rng_for(1, 777)
@@ -401,21 +541,24 @@ def cpu_baseline(fx, per_layer, lm_head, group) -> dict:
     cores = len(os.sched_getaffinity(0))
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
 
-    def one_pass():
-        for (r, k), t in zip(sample, tensors):
-            so.affine_matvec(*t, xs[k], r, k, group, so.BF16, threads=True)
-
-    one_pass()
-    t0 = time.perf_counter()
-    passes = 0
-    while True:
+    def run(threads, budget):
+        def one_pass():
+            for (r, k), t in zip(sample, tensors):
+                so.affine_matvec(*t, xs[k], r, k, group, so.BF16, threads=threads)
         one_pass()
-        passes += 1
-        dt = time.perf_counter() - t0
-        if dt > 10.0:
-            break
-    gbs = nbytes * passes / dt / 1e9
+        t0 = time.perf_counter()
+        passes = 0
+        while True:
+            one_pass()
+            passes += 1
+            dt = time.perf_counter() - t0
+            if dt > budget:
+                return nbytes * passes / dt / 1e9, passes, dt
+
+    gbs1, p1, dt1 = run(False, 5.0)
+    gbs, passes, dt = run(True, 8.0)
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "single_thread": {"value": round(gbs1, 3), "unit": "GB/s", "cores": 1, "passes": p1, "seconds": round(dt1, 1)},
             "sample": f"{passes} passes over layer 0 (7 matrices) + 16384 lm_head rows = {nbytes} weight bytes/pass, "
                       f"{dt:.1f} s, scalar C restatement of the reference dequant-matvec, OpenMP over rows"}
 
