@@ -125,9 +125,12 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
 /* Which kernel a single-token quantized matvec record runs.  AUTO (the default): matrices of
  * 8M weights and more take the single-pass matrix-core kernel of the same pipeline, smaller ones
  * the vector-ALU kernel; MATRIX_CORE drops the size threshold (every shape the matrix-core kernel
- * can express takes it); VECTOR keeps every record on the vector-ALU kernels.  Results of the two
- * differ in summation order only.  No counterpart in the reference (one kernel per pipeline name
- * there); meant for A/B measurement and for tests. */
+ * can express takes it); VECTOR keeps every record on the vector-ALU kernels.  The same switch
+ * covers the skinny qmm records (up to 32 tokens per pass): AUTO and MATRIX_CORE run the streaming
+ * kernel of the pipeline (K split inside a workgroup, no workspace), VECTOR the split-K kernel the
+ * record's geometry describes (partial sums in the workspace).  Results of the alternatives differ
+ * in summation order only.  No counterpart in the reference (one kernel per pipeline name there);
+ * meant for A/B measurement and for tests. */
 enum { SMELT_HIP_MATVEC_AUTO = 0, SMELT_HIP_MATVEC_MATRIX_CORE = 1, SMELT_HIP_MATVEC_VECTOR = 2 };
 int smelt_hip_set_matvec_engine(smelt_hip_context *ctx, int engine);
 

@@ -1,0 +1,347 @@
+// Streaming small-batch quantized matmul for gfx950:  Y[M, N] = X[M, K] * W[N, K]^T for up to 16
+// tokens per pass, affine u4 weights with one scale group per 64 columns.
+//
+// At this batch the weights still stream from HBM once and the arithmetic is small; the kernel is
+// the multi-token form of the single-pass matvec.  A wave owns 16 * RT weight rows and, per round,
+// P pairs of scale groups (128 columns each); it issues every load of a round (scales first, then
+// activations and weights pair by pair) before it does anything else.  K is split over the waves
+// of a workgroup (up to sixteen) and, for long rows, over rounds; the waves' partial sums meet in
+// LDS and no workspace is used.
+//
+// Memory side: every load instruction covers whole runs of memory with adjacent lanes (four lanes
+// on the 64 bytes a row holds for a pair, sixteen lanes on the 256 bytes of a token), because a
+// load whose 64 lanes touch 64 different cache lines costs the memory pipeline four to eight
+// times the cycles.  The MFMA wants another lane order, so each pair goes through a wave-private
+// LDS buffer: written as loaded, read back in operand order.  LDS operations of one wave execute
+// in order, so the exchange needs no barrier.
+//
+// Arithmetic: v_mfma_f32_16x16x32_{f16,bf16}, tokens as the A operand (rows), sixteen weight rows
+// as the B operand (columns).
+//   * MFMA lane (n = lane % 16, q = lane / 16) takes the eight bytes of row n that hold columns
+//     16 q .. 16 q + 15 of a scale group: its two dwords are the lane's share of the B operands
+//     of the group's two MFMAs.  A packed dword becomes four operand registers with three shifts
+//     and four AND-ORs: codes (r, r + 4) of the dword land at one mantissa bit of the two halves
+//     of register r as (base + code), exact in the 16-bit float type.
+//   * The activations enter in their own type, unconverted; each 16-byte run is brought into the
+//     operand order of the codes (0, 4, 1, 5, 2, 6, 3, 7) with four byte permutes.
+//   * One more MFMA pair per group, against a B operand of ones, gives every lane the plain sum
+//     of its four tokens' activations over the group; with it
+//         y += s * sum((base + code) * x) + (b - base * s) * sum(x)
+//     applies the group's scale and bias in fp32 on the accumulators (each lane owns one weight
+//     row, so both are one scalar per lane).
+// Tokens past the batch and rows past the matrix re-read the last valid one and are never stored;
+// pairs past the end of a row re-read the last pair under a zero scale.
+#pragma once
+#include "mm1_matvec.hpp"
+
+namespace smelt {
+
+template <class ActT>
+struct QsCodes;
+template <>
+struct QsCodes<BF16> { static constexpr int kPos = 0; };   // base 128
+template <>
+struct QsCodes<F16> { static constexpr int kPos = 4; };    // base 64
+
+template <class ActT>
+struct QsOperand {
+    using E = Elem16<ActT>;
+    static constexpr int kPos = QsCodes<ActT>::kPos;
+    static constexpr uint32_t kMask = (0xFu << kPos) | (0xFu << (kPos + 16));
+    static constexpr uint32_t kBaseHalf = (uint32_t)(E::kExpBias + E::kMant - kPos) << E::kMant;
+    static constexpr uint32_t kBasePair = kBaseHalf | (kBaseHalf << 16);
+    static constexpr float kBase = (float)(1 << (E::kMant - kPos));
+    static constexpr uint32_t kOnePair = ((uint32_t)E::kExpBias << E::kMant) | ((uint32_t)E::kExpBias << (E::kMant + 16));
+    // eight codes of one dword -> B operand registers; register r holds codes (r, r + 4)
+    static __device__ __forceinline__ uint4_t codes(uint32_t c) {
+        uint32_t r[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int sh = 4 * j - kPos;
+            const uint32_t src = sh == 0 ? c : (sh > 0 ? c >> sh : c << -sh);
+            r[j] = and_or(src, kMask, kBasePair);
+        }
+        return uint4_t{r[0], r[1], r[2], r[3]};
+    }
+    // eight consecutive activations -> A operand registers in the order of the codes
+    static __device__ __forceinline__ uint4_t activations(const uint4_t& x) {
+        return uint4_t{__builtin_amdgcn_perm(x.z, x.x, 0x05040100u), __builtin_amdgcn_perm(x.z, x.x, 0x07060302u),
+                       __builtin_amdgcn_perm(x.w, x.y, 0x05040100u), __builtin_amdgcn_perm(x.w, x.y, 0x07060302u)};
+    }
+};
+
+// LDS: (scale, bias - base * scale) of every row of the tile and every group plus one zero column,
+// then one staging buffer per wave: 16 token rows of one pair (256 B + 16 B of padding each) and
+// 16 weight rows per tile (64 B + 8 B of padding each).  A wave's partial sums (1 KB per tile) go
+// to its own staging buffer once it is done with it.
+constexpr int kQsTokens = 16;          // tokens per pass (blockIdx.y)
+constexpr int kQsXStride = 272;        // bytes per staged token row
+constexpr int kQsWStride = 72;         // bytes per staged weight row
+__host__ __device__ constexpr size_t qms_scale_lds_bytes(int tiles, int groups) { return (size_t)tiles * 16 * (groups + 1) * 8; }
+__host__ __device__ constexpr size_t qms_wave_lds_bytes(int tiles) { return (size_t)16 * kQsXStride + (size_t)tiles * 16 * kQsWStride; }
+__host__ __device__ constexpr size_t qms_lds_bytes(int tiles, int groups, int waves) {
+    return qms_scale_lds_bytes(tiles, groups) + (size_t)waves * qms_wave_lds_bytes(tiles);
+}
+
+template <class ActT, class ScaleT, int NMAT, int RT, int XR, class Epi>
+__device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
+                                         const uint16_t* const (&B)[NMAT], const uint16_t* __restrict__ X, int batch,
+                                         int rows, int cols, const Epi& epi) {
+    using E = Elem16<ActT>;
+    using O = QsOperand<ActT>;
+    constexpr int T = NMAT * RT;   // 16-row tiles a wave multiplies by its slice of x
+    static_assert(qms_wave_lds_bytes(T) >= (size_t)T * 1024, "partial sums reuse the staging buffer");
+    static_assert(XR == 2 || XR == 4, "a pass stages eight or sixteen token rows");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int chunk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int kc = blockDim.x / kWave;
+    const int n = lane & 15, q = lane >> 4;
+    const int gt = cols >> 6;          // scale groups per row
+    const int npairs = gt >> 1;
+    const int rs = cols >> 1;          // bytes per packed row
+    const int row0 = blockIdx.x * (16 * RT);
+    const int m0 = blockIdx.y * kQsTokens;
+    const int last_tok = (batch < m0 + kQsTokens ? batch : m0 + kQsTokens) - 1;
+
+    // Nothing below predicates a load; loads return in issue order, so what is needed first is
+    // asked for first.
+    // ---- scales and biases of the tile: one run of eight groups of one row per thread ------------
+    const int runs = gt >> 3;
+    const int items = T * 16 * runs;
+    float2* lds_sb = reinterpret_cast<float2*>(smem);
+    const int sstride = gt + 1;
+    struct ScaleRun { uint4_t s, b; int at; };
+    auto load_scales = [&](int item) {
+        if (item > items - 1) item = items - 1;               // threads past the end repeat the last item
+        const int srow = item / runs, run = item - srow * runs;   // srow = (matrix * RT + tile) * 16 + row in tile
+        const int smat = srow / (16 * RT);
+        int r = row0 + (srow - smat * 16 * RT);
+        if (r > rows - 1) r = rows - 1;
+        const uint16_t* sp = S[0];
+        const uint16_t* bp = B[0];
+        if (NMAT > 1 && smat == 1) { sp = S[NMAT - 1]; bp = B[NMAT - 1]; }
+        ScaleRun out;
+        out.s = *reinterpret_cast<const uint4_t*>(sp + (size_t)r * gt + 8 * run);
+        out.b = *reinterpret_cast<const uint4_t*>(bp + (size_t)r * gt + 8 * run);
+        out.at = srow * sstride + 8 * run;
+        return out;
+    };
+    auto store_scales = [&](const ScaleRun& v) {
+        const uint32_t sd[4] = {v.s.x, v.s.y, v.s.z, v.s.w}, bd[4] = {v.b.x, v.b.y, v.b.z, v.b.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float s = ScaleT::widen((uint16_t)(e & 1 ? sd[e >> 1] >> 16 : sd[e >> 1] & 0xFFFFu));
+            const float b = ScaleT::widen((uint16_t)(e & 1 ? bd[e >> 1] >> 16 : bd[e >> 1] & 0xFFFFu));
+            lds_sb[v.at + e] = float2{s, __builtin_fmaf(-O::kBase, s, b)};
+        }
+    };
+    const ScaleRun first_run = load_scales((int)threadIdx.x);
+
+    unsigned char* stage = smem + qms_scale_lds_bytes(T, gt) + (size_t)chunk * qms_wave_lds_bytes(T);
+    unsigned char* stage_w = stage + 16 * kQsXStride;
+    // load side: sixteen lanes per token row, four lanes per weight row
+    const int x_tok = lane >> 4, x_piece = lane & 15;
+    const int w_row = lane >> 2, w_piece = lane & 3;
+    const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint4_t ones = {O::kOnePair, O::kOnePair, O::kOnePair, O::kOnePair};
+    float4_t acc[NMAT][RT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[m][t] = zero;
+
+    // One step = one pair of scale groups (128 columns): XR loads of activations (four token rows
+    // each) and one load per tile of weights.  Wave c takes pairs c, c + kc, c + 2 kc, ...
+    struct Step { uint4_t x[XR]; uint4_t w[NMAT][RT]; };
+    const uint16_t* x_base[XR];
+#pragma unroll
+    for (int r = 0; r < XR; ++r) {
+        int tok = m0 + 4 * r + x_tok;
+        if (tok > last_tok) tok = last_tok;
+        x_base[r] = X + (size_t)tok * cols + 8 * x_piece;
+    }
+    const uint8_t* w_base[NMAT][RT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            int r = row0 + 16 * t + w_row;
+            if (r > rows - 1) r = rows - 1;
+            w_base[m][t] = W[m] + (size_t)r * rs + 16 * w_piece;
+        }
+    auto issue = [&](Step& st, int pair) {
+        if (pair > npairs - 1) pair = npairs - 1;   // past the end: the last pair again, under a zero scale
+#pragma unroll
+        for (int r = 0; r < XR; ++r) st.x[r] = *reinterpret_cast<const uint4_t*>(x_base[r] + 128 * pair);
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int t = 0; t < RT; ++t) st.w[m][t] = *reinterpret_cast<const uint4_t*>(w_base[m][t] + 64 * pair);
+    };
+    // through the wave's staging buffer: written as loaded, read back in operand order
+    auto consume = [&](const Step& st, int pair) {
+#pragma unroll
+        for (int r = 0; r < XR; ++r)
+            *reinterpret_cast<uint4_t*>(stage + (4 * r + x_tok) * kQsXStride + 16 * x_piece) = st.x[r];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int t = 0; t < RT; ++t) {
+                unsigned char* at = stage_w + ((m * RT + t) * 16 + w_row) * kQsWStride + 16 * w_piece;
+                *reinterpret_cast<uint2_t*>(at) = uint2_t{st.w[m][t].x, st.w[m][t].y};
+                *reinterpret_cast<uint2_t*>(at + 8) = uint2_t{st.w[m][t].z, st.w[m][t].w};
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        int gi = 2 * pair;
+        if (gi > gt) gi = gt;   // the zero column (gt is even)
+        // with eight staged token rows, MFMA rows 8..15 re-read rows 0..7 (never stored)
+        const int xrow = XR == 4 ? n : (n & 7);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const unsigned char* xr = stage + xrow * kQsXStride + 128 * e + 32 * q;
+            const uint4_t a0 = O::activations(*reinterpret_cast<const uint4_t*>(xr));
+            const uint4_t a1 = O::activations(*reinterpret_cast<const uint4_t*>(xr + 16));
+            const float4_t xs = E::mfma(a1, ones, E::mfma(a0, ones, zero));
+            const int ge = gi + e < gt ? gi + e : gt;
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int t = 0; t < RT; ++t) {
+                    const uint2_t c = *reinterpret_cast<const uint2_t*>(stage_w + ((m * RT + t) * 16 + n) * kQsWStride + 32 * e + 8 * q);
+                    const float4_t d = E::mfma(a1, O::codes(c.y), E::mfma(a0, O::codes(c.x), zero));
+                    const float2 sb = lds_sb[((m * RT + t) * 16 + n) * sstride + ge];
+                    acc[m][t].x = __builtin_fmaf(sb.x, d.x, __builtin_fmaf(sb.y, xs.x, acc[m][t].x));
+                    acc[m][t].y = __builtin_fmaf(sb.x, d.y, __builtin_fmaf(sb.y, xs.y, acc[m][t].y));
+                    acc[m][t].z = __builtin_fmaf(sb.x, d.z, __builtin_fmaf(sb.y, xs.z, acc[m][t].z));
+                    acc[m][t].w = __builtin_fmaf(sb.x, d.w, __builtin_fmaf(sb.y, xs.w, acc[m][t].w));
+                }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    // One step is in flight while the other is consumed.  The first loads go out behind the scale
+    // loads; the scales reach LDS while they fly.
+    Step s0, s1;
+    int pair = chunk;
+    issue(s0, pair);
+    issue(s1, pair + kc);
+    store_scales(first_run);
+    // a tile with more runs than the workgroup has threads takes more passes
+    for (int base = (int)blockDim.x; base < items; base += (int)blockDim.x) store_scales(load_scales(base + (int)threadIdx.x));
+    if (threadIdx.x < T * 16) lds_sb[threadIdx.x * sstride + gt] = float2{0.0f, 0.0f};
+    __syncthreads();
+    for (; pair < npairs; pair += 2 * kc) {
+        consume(s0, pair);
+        issue(s0, pair + 2 * kc);
+        consume(s1, pair + kc);
+        issue(s1, pair + 3 * kc);
+    }
+
+    // ---- the kc waves of the workgroup, in wave order -------------------------------------------------
+    // each wave leaves its partial sums in its own staging buffer
+    {
+        float4_t* mine = reinterpret_cast<float4_t*>(stage);
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int t = 0; t < RT; ++t) mine[(m * RT + t) * kWave + lane] = acc[m][t];
+    }
+    __syncthreads();
+    if (chunk < RT) {
+        // wave t finishes tile t: lane (n, q) holds row 16 t + n of tokens 4 q .. 4 q + 3
+        const int t = chunk;
+        const unsigned char* first = smem + qms_scale_lds_bytes(T, gt);
+        float4_t sum[NMAT];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) sum[m] = zero;
+        for (int c = 0; c < kc; ++c)
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                const float4_t part = reinterpret_cast<const float4_t*>(first + (size_t)c * qms_wave_lds_bytes(T))[(m * RT + t) * kWave + lane];
+                sum[m].x += part.x; sum[m].y += part.y; sum[m].z += part.z; sum[m].w += part.w;
+            }
+        const int r = row0 + 16 * t + n;
+        if (r < rows) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int tok = m0 + 4 * q + v;
+                if (tok <= last_tok) {
+                    float val[NMAT];
+#pragma unroll
+                    for (int m = 0; m < NMAT; ++m) val[m] = v == 0 ? sum[m].x : (v == 1 ? sum[m].y : (v == 2 ? sum[m].z : sum[m].w));
+                    epi((size_t)tok * rows + r, val);
+                }
+            }
+        }
+    }
+}
+
+// ---- epilogues: (element index, values[NMAT]) -------------------------------------------------------
+template <class ActT>
+struct QsStore {
+    uint16_t* y;
+    __device__ __forceinline__ void operator()(size_t idx, const float (&v)[1]) const { y[idx] = ActT::narrow(v[0]); }
+};
+// matvec_out = narrow(acc); out = narrow(widen(matvec_out) + residual)
+template <class ActT>
+struct QsAdd {
+    uint16_t* mv;
+    const uint16_t* residual;
+    uint16_t* out;
+    __device__ __forceinline__ void operator()(size_t idx, const float (&v)[1]) const {
+        const uint16_t p = ActT::narrow(v[0]);
+        mv[idx] = p;
+        out[idx] = ActT::narrow(ActT::widen(p) + ActT::widen(residual[idx]));
+    }
+};
+template <class ActT>
+struct QsSwiglu {
+    uint16_t* y;
+    __device__ __forceinline__ void operator()(size_t idx, const float (&v)[2]) const {
+        const float g = v[0], u = v[1];
+        y[idx] = ActT::narrow(g / (1.0f + expf(-g)) * u);
+    }
+};
+
+}  // namespace smelt
+
+#define SMELT_QMS_KERNEL extern "C" __global__ __launch_bounds__(1024)
+
+// Argument lists of the skinny kernels of the same pipelines (the workspace pointers are unused).
+#define SMELT_AFFINE_QMS_PLAIN(T, ACT, SC, RTV, XRV)                                                \
+    SMELT_QMS_KERNEL void smelt_affine_qms_r##RTV##_x##XRV##_store_##T(                             \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* Y,    \
+        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {     \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        qms_body<ACT, SC, 1, RTV, XRV>(w, s, b, X, batch, rows, cols, QsStore<ACT>{Y});             \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_affine_qms_r##RTV##_x##XRV##_add_##T(                               \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* MV,   \
+        const uint16_t* RES, uint16_t* OUT, uint32_t batch, uint32_t rows, uint32_t cols,          \
+        uint32_t, uint32_t, float*, uint32_t*) {                                                   \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        qms_body<ACT, SC, 1, RTV, XRV>(w, s, b, X, batch, rows, cols, QsAdd<ACT>{MV, RES, OUT});    \
+    }
+
+#define SMELT_AFFINE_QMS_GATE_UP(T, ACT, SC, XRV)                                                   \
+    SMELT_QMS_KERNEL void smelt_affine_qms_r1_x##XRV##_gate_up_swiglu_##T(                          \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {                     \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        qms_body<ACT, SC, 2, 1, XRV>(w, s, b, X, batch, rows, cols, QsSwiglu<ACT>{Y});              \
+    }

@@ -218,15 +218,44 @@ void attach_mm1(ResolvedPipeline* r) {
     }
 }
 
+// The skinny qmm kernels that have a streaming form.
+void attach_qms(ResolvedPipeline* r) {
+    if (r->lds_variant != kSkinnyVariant) return;
+    const std::string t = act_suffix(r->act);
+    if (r->family == kFamAffineQmm) { r->qms_tail = "store_" + t; r->qms_nmat = 1; }
+    else if (r->family == kFamAffineQmmAdd) { r->qms_tail = "add_" + t; r->qms_nmat = 1; }
+    else if (r->family == kFamAffineQmmGateUp && r->symbol.find("swiglu") != std::string::npos) { r->qms_tail = "gate_up_swiglu_" + t; r->qms_nmat = 2; }
+}
+
 ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType default_act, size_t lds_limit,
                                      ResolvedPipeline* out, std::string* why);
 
 }  // namespace
 
+bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmsPlan* out) {
+    if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;
+    const uint32_t gt = cols / 64, npairs = gt / 2;
+    // Measured on MI355X at 2560- and 9216-column rows: about four steps per wave hide the memory
+    // round trips best, up to twelve waves; two row tiles per wave (half the activation traffic per
+    // weight byte) pay once a pass stages sixteen tokens and the matrix still fills the machine
+    // with 32-row workgroups.
+    const uint32_t rt = nmat == 1 && batch > 8 && rows >= 32 * 256 ? 2 : 1;
+    uint32_t kc = (npairs + 3) / 4;
+    if (kc < 2) kc = npairs < 2 ? 1 : 2;
+    if (kc > 12) kc = 12;
+    const uint32_t steps = (npairs + kc - 1) / kc;
+    kc = (npairs + steps - 1) / steps;   // same steps per wave, no idle wave
+    if (kc < rt) return false;
+    const uint32_t tiles = nmat * rt;
+    out->rt = rt; out->kc = kc;
+    out->lds = (size_t)tiles * 16 * (gt + 1) * 8 + (size_t)kc * (16 * 272 + (size_t)tiles * 16 * 72);
+    return out->lds <= lds_limit;
+}
+
 ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act,
                                size_t lds_limit, ResolvedPipeline* out, std::string* why) {
     const ResolveStatus st = resolve_pipeline_entry(entry_in, default_act, lds_limit, out, why);
-    if (st == kResolveOk) attach_mm1(out);
+    if (st == kResolveOk) { attach_mm1(out); attach_qms(out); }
     return st;
 }
 

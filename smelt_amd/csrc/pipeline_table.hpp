@@ -115,6 +115,10 @@ struct ResolvedPipeline {
     int mm1_layout = -1;             // CodeLayout of its weights
     uint32_t mm1_nmat = 1;
     bool workspace = false;          // kernel takes the context's (partials, counters) pointers last
+    // Streaming form of a skinny qmm pipeline, picked per launch by shape: the kernel is
+    // "smelt_affine_qms_r<R>_x<X>_" + qms_tail for R row tiles per wave and 4 X staged token rows.
+    std::string qms_tail;
+    uint32_t qms_nmat = 1;
 };
 
 constexpr uint32_t kSkinnyVariant = 32;
@@ -157,5 +161,15 @@ struct Mm1Plan {
 };
 bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
               bool force, Mm1Plan* out);
+
+// Launch plan of the streaming skinny qmm: workgroups of `kc` waves over 16 * rt rows each, 16 tokens
+// per grid row; wave c takes the pairs of scale groups c, c + kc, ...  False when the shape has no
+// such kernel.
+constexpr uint32_t kQmsMaxRowTiles = 4;
+struct QmsPlan {
+    uint32_t rt = 0, kc = 0;
+    size_t lds = 0;
+};
+bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmsPlan* out);
 
 }  // namespace smelt_host

@@ -45,6 +45,7 @@ struct Pipeline {
     hipFunction_t fn_single = nullptr;  // used when the record's batch argument is 1
     hipFunction_t fn_mm_stream = nullptr, fn_mm_split = nullptr;  // matrix-core variants picked by shape
     hipFunction_t fn_mm1[kMm1MaxSegments + 1] = {};               // single-pass matrix-core matvec, by segments per wave
+    hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
     ResolvedPipeline res;
 };
 
@@ -1093,6 +1094,20 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             routed = true;
         }
     }
+    if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR) {
+        // skinny qmm: the streaming kernel of the same pipeline, same arguments, its own launch
+        // geometry (16 * rt rows per workgroup, 16 tokens per grid row); it uses no workspace
+        const size_t o = p->res.family == kFamAffineQmm ? 5 : (p->res.family == kFamAffineQmmAdd ? 7 : 8);
+        const uint32_t batch = L.args[o].value, rows = L.args[o + 1].value, cols = L.args[o + 2].value, group = L.args[o + 3].value;
+        QmsPlan plan;
+        if (batch > 0 && qms_plan(rows, cols, group, p->res.qms_nmat, batch, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
+            fn = p->fn_qms[plan.rt][batch > 8];
+            L.grid[0] = (rows + 16 * plan.rt - 1) / (16 * plan.rt); L.grid[1] = (batch + 15) / 16; L.grid[2] = 1;
+            L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
+            L.lds = plan.lds;
+            routed = true;
+        }
+    }
     if (!routed && p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
         // signed g128 matvec: large matrices run on the matrix cores (same bytes, same arguments + kw)
         const uint32_t rows = L.args[(size_t)p->res.rows_arg].value, cols = L.args[(size_t)p->res.cols_arg].value;
@@ -1319,6 +1334,10 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
             if (!p.res.mm1_prefix.empty())
                 for (uint32_t nl = 1; nl <= kMm1MaxSegments; ++nl)
                     (void)find(&p.fn_mm1[nl], p.res.mm1_prefix + "nl" + std::to_string(nl) + "_" + p.res.mm1_tail);
+            if (!p.res.qms_tail.empty())
+                for (uint32_t rt = 1; rt <= kQmsMaxRowTiles; ++rt)
+                    for (uint32_t wide = 0; wide < 2; ++wide)
+                        (void)find(&p.fn_qms[rt][wide], "smelt_affine_qms_r" + std::to_string(rt) + (wide ? "_x4_" : "_x2_") + p.res.qms_tail);
         }
     }
     std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);

@@ -16,6 +16,7 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def ctx():
     c = rt.Context()
+    c.set_matvec_engine(rt.MATVEC_VECTOR)   # keeps skinny records on the split-K kernels tested here
     yield c
     c.close()
 

@@ -30,6 +30,7 @@ def _run(ctx, encode, w_offs, x_bits, rows, cols, ksplit, pipe_name, nmat_bufs):
 def test_static_scratch_matches_allocated_workspace_twice_in_a_row():
     dtype = fx.BF16
     ctx = rt.Context()
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)   # the split-K kernels: the ones that use the scratch
     try:
         # first call: 13 tokens on 416 x 2560 split 4 ways (13 row tiles x 4 partials)
         # second call: 5 tokens on the first 100 rows of a 1536-column matrix split 3 ways
@@ -56,6 +57,7 @@ def test_static_scratch_matches_allocated_workspace_twice_in_a_row():
 def test_static_scratch_rejects_partials_beyond_its_size():
     dtype = fx.F16
     ctx = rt.Context()
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)
     try:
         # 4096 workgroup partials of 4 KB fit; 140 row tiles x 32 splits = 4480 do not.  The context's
         # own 64 MB workspace takes the same record.
