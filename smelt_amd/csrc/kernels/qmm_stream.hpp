@@ -345,3 +345,233 @@ struct QsSwiglu {
         const uint16_t* const b[2] = {gB, uB};                                                     \
         qms_body<ACT, SC, 2, 1, XRV>(w, s, b, X, batch, rows, cols, QsSwiglu<ACT>{Y});              \
     }
+
+// ---- token-tile form: prefill chunks ------------------------------------------------------------
+// The same arithmetic for many tokens.  A workgroup of four waves (two along the rows, two along
+// the tokens) owns 32 * RT weight rows times 32 * TB tokens and walks K one pair of scale groups
+// at a time.  Per step the 256 threads bring the tile's activations (in the operand order of the
+// codes), packed weights and (scale, bias - base * scale) pairs into one of two LDS buffers,
+// shared by the four waves, while the other buffer is multiplied; the global loads run two or four
+// steps ahead in registers.  Each wave unpacks a 16-row B operand once per step and group and
+// reuses it for its TB token blocks.
+namespace smelt {
+
+constexpr int kQtThreads = 256;
+__host__ __device__ constexpr size_t qmt_buffer_bytes(int nmat, int rt, int tb) {
+    return (size_t)32 * tb * kQsXStride + (size_t)nmat * 32 * rt * kQsWStride + (size_t)nmat * 32 * rt * 2 * 8;
+}
+__host__ __device__ constexpr size_t qmt_lds_bytes(int nmat, int rt, int tb) { return 2 * qmt_buffer_bytes(nmat, rt, tb); }
+
+template <class ActT, class ScaleT, int NMAT, int RT, int TB, class Epi>
+__device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
+                                         const uint16_t* const (&B)[NMAT], const uint16_t* __restrict__ X, int batch,
+                                         int rows, int cols, const Epi& epi) {
+    using E = Elem16<ActT>;
+    using O = QsOperand<ActT>;
+    constexpr int BN = 32 * RT, BM = 32 * TB;           // rows (per matrix) and tokens of the workgroup tile
+    constexpr int XI = BM * 16 / kQtThreads;            // 16-byte activation loads per thread and step
+    constexpr int WROWS = NMAT * BN;                    // staged weight rows
+    constexpr int WI = (WROWS * 4 + kQtThreads - 1) / kQtThreads;   // 16-byte weight loads per thread and step
+    static_assert(BM * 16 % kQtThreads == 0 && WROWS <= kQtThreads, "staging assignment");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    constexpr size_t kBuf = qmt_buffer_bytes(NMAT, RT, TB);
+    constexpr size_t kOffW = (size_t)BM * kQsXStride, kOffS = kOffW + (size_t)WROWS * kQsWStride;   // within a buffer
+    constexpr int D = XI + WI <= 6 ? 4 : 2;            // steps in flight in registers
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int wn = wave & 1, wm = wave >> 1;
+    const int n = lane & 15, q = lane >> 4;
+    const int gt = cols >> 6, npairs = gt >> 1, rs = cols >> 1;
+    const int row0 = blockIdx.x * BN;
+    const int m0 = blockIdx.y * BM;
+    const int last_tok = (batch < m0 + BM ? batch : m0 + BM) - 1;
+
+    // staging assignment: sixteen lanes per token row, four lanes per weight row, one thread per
+    // staged row for the scales (staged row = (matrix * 2 + row half) * 16 RT + row in half)
+    const uint16_t* x_src[XI];
+    int x_dst[XI];
+#pragma unroll
+    for (int j = 0; j < XI; ++j) {
+        const int item = tid + kQtThreads * j, t = item >> 4, piece = item & 15;
+        int tok = m0 + t;
+        if (tok > last_tok) tok = last_tok;
+        x_src[j] = X + (size_t)tok * cols + 8 * piece;
+        x_dst[j] = t * kQsXStride + 16 * piece;
+    }
+    const uint8_t* w_src[WI];
+    int w_dst[WI];
+#pragma unroll
+    for (int j = 0; j < WI; ++j) {
+        int item = tid + kQtThreads * j;
+        if (item > WROWS * 4 - 1) item = WROWS * 4 - 1;
+        const int sr = item >> 2, piece = item & 3, m = sr / BN;
+        int r = row0 + (sr - m * BN);
+        if (r > rows - 1) r = rows - 1;
+        w_src[j] = (NMAT > 1 && m == 1 ? W[NMAT - 1] : W[0]) + (size_t)r * rs + 16 * piece;
+        w_dst[j] = sr * kQsWStride + 16 * piece;
+    }
+    const uint16_t* s_src;
+    const uint16_t* b_src;
+    {
+        int sr = tid;
+        if (sr > WROWS - 1) sr = WROWS - 1;
+        const int m = sr / BN;
+        int r = row0 + (sr - m * BN);
+        if (r > rows - 1) r = rows - 1;
+        s_src = (NMAT > 1 && m == 1 ? S[NMAT - 1] : S[0]) + (size_t)r * gt;
+        b_src = (NMAT > 1 && m == 1 ? B[NMAT - 1] : B[0]) + (size_t)r * gt;
+    }
+    const int s_dst = tid < WROWS ? tid : WROWS - 1;
+
+    struct Step { uint4_t x[XI]; uint4_t w[WI]; uint32_t s, b; };
+    auto issue = [&](Step& st, int pair) {
+        st.s = *reinterpret_cast<const uint32_t*>(s_src + 2 * pair);
+        st.b = *reinterpret_cast<const uint32_t*>(b_src + 2 * pair);
+#pragma unroll
+        for (int j = 0; j < XI; ++j) st.x[j] = *reinterpret_cast<const uint4_t*>(x_src[j] + 128 * pair);
+#pragma unroll
+        for (int j = 0; j < WI; ++j) st.w[j] = *reinterpret_cast<const uint4_t*>(w_src[j] + 64 * pair);
+    };
+    auto stage = [&](const Step& st, unsigned char* buf) {
+        float2* lds_sc = reinterpret_cast<float2*>(buf + kOffS);   // [staged row][2]
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float s = ScaleT::widen((uint16_t)(e ? st.s >> 16 : st.s & 0xFFFFu));
+            const float b = ScaleT::widen((uint16_t)(e ? st.b >> 16 : st.b & 0xFFFFu));
+            lds_sc[s_dst * 2 + e] = float2{s, __builtin_fmaf(-O::kBase, s, b)};
+        }
+#pragma unroll
+        for (int j = 0; j < XI; ++j) *reinterpret_cast<uint4_t*>(buf + x_dst[j]) = O::activations(st.x[j]);
+#pragma unroll
+        for (int j = 0; j < WI; ++j) {
+            *reinterpret_cast<uint2_t*>(buf + kOffW + w_dst[j]) = uint2_t{st.w[j].x, st.w[j].y};
+            *reinterpret_cast<uint2_t*>(buf + kOffW + w_dst[j] + 8) = uint2_t{st.w[j].z, st.w[j].w};
+        }
+    };
+
+    const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint4_t ones = {O::kOnePair, O::kOnePair, O::kOnePair, O::kOnePair};
+    float4_t acc[NMAT][RT][TB];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int u = 0; u < TB; ++u) acc[m][t][u] = zero;
+
+    auto multiply = [&](const unsigned char* buf) {
+        const float2* lds_sc = reinterpret_cast<const float2*>(buf + kOffS);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            uint4_t a0[TB], a1[TB];
+            float4_t xs[TB];
+#pragma unroll
+            for (int u = 0; u < TB; ++u) {
+                const unsigned char* xr = buf + ((wm * TB + u) * 16 + n) * kQsXStride + 128 * e + 32 * q;
+                a0[u] = *reinterpret_cast<const uint4_t*>(xr);
+                a1[u] = *reinterpret_cast<const uint4_t*>(xr + 16);
+                xs[u] = E::mfma(a1[u], ones, E::mfma(a0[u], ones, zero));
+            }
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int t = 0; t < RT; ++t) {
+                    const int sr = ((m * 2 + wn) * RT + t) * 16 + n;
+                    const uint2_t c = *reinterpret_cast<const uint2_t*>(buf + kOffW + sr * kQsWStride + 32 * e + 8 * q);
+                    const uint4_t b0 = O::codes(c.x), b1 = O::codes(c.y);
+                    const float2 sb = lds_sc[sr * 2 + e];
+#pragma unroll
+                    for (int u = 0; u < TB; ++u) {
+                        const float4_t d = E::mfma(a1[u], b1, E::mfma(a0[u], b0, zero));
+                        acc[m][t][u].x = __builtin_fmaf(sb.x, d.x, __builtin_fmaf(sb.y, xs[u].x, acc[m][t][u].x));
+                        acc[m][t][u].y = __builtin_fmaf(sb.x, d.y, __builtin_fmaf(sb.y, xs[u].y, acc[m][t][u].y));
+                        acc[m][t][u].z = __builtin_fmaf(sb.x, d.z, __builtin_fmaf(sb.y, xs[u].z, acc[m][t][u].z));
+                        acc[m][t][u].w = __builtin_fmaf(sb.x, d.w, __builtin_fmaf(sb.y, xs[u].w, acc[m][t][u].w));
+                    }
+                }
+        }
+    };
+
+    // Loads past the last pair repeat it (staged into the idle buffer, never multiplied), so that no
+    // load sits under a branch.
+    const int last_pair = npairs - 1;
+    Step st[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) issue(st[d], d < last_pair ? d : last_pair);
+    stage(st[0], smem);
+    issue(st[0], D < last_pair ? D : last_pair);
+    __syncthreads();
+    for (int base = 0; base < npairs; base += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int pair = base + d;
+            if (pair >= npairs) break;
+            // the next step's tile goes into the other buffer (everyone left it at the last barrier)
+            stage(st[(d + 1) % D], smem + ((d + 1) & 1) * kBuf);
+            issue(st[(d + 1) % D], pair + 1 + D < last_pair ? pair + 1 + D : last_pair);
+            multiply(smem + (d & 1) * kBuf);
+            __syncthreads();
+        }
+    }
+
+    // lane (n, q) holds row n of tile t and tokens 4 q .. 4 q + 3 of block u
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const int r = row0 + (wn * RT + t) * 16 + n;
+        if (r < rows) {
+#pragma unroll
+            for (int u = 0; u < TB; ++u)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int tok = m0 + (wm * TB + u) * 16 + 4 * q + v;
+                    if (tok <= last_tok) {
+                        float val[NMAT];
+#pragma unroll
+                        for (int m = 0; m < NMAT; ++m)
+                            val[m] = v == 0 ? acc[m][t][u].x : (v == 1 ? acc[m][t][u].y : (v == 2 ? acc[m][t][u].z : acc[m][t][u].w));
+                        epi((size_t)tok * rows + r, val);
+                    }
+                }
+        }
+    }
+}
+
+}  // namespace smelt
+
+#define SMELT_QMT_KERNEL extern "C" __global__ __launch_bounds__(256)
+
+// Argument lists of the token-slab qmm kernels of the same pipelines, plus the two workspace
+// pointers of the skinny ones (unused).
+#define SMELT_AFFINE_QMT_PLAIN(T, ACT, SC, RTV, TBV)                                               \
+    SMELT_QMT_KERNEL void smelt_affine_qmt_r##RTV##_t##TBV##_store_##T(                            \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* Y,    \
+        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {                        \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        qmt_body<ACT, SC, 1, RTV, TBV>(w, s, b, X, batch, rows, cols, QsStore<ACT>{Y});            \
+    }                                                                                              \
+    SMELT_QMT_KERNEL void smelt_affine_qmt_r##RTV##_t##TBV##_add_##T(                              \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* MV,   \
+        const uint16_t* RES, uint16_t* OUT, uint32_t batch, uint32_t rows, uint32_t cols,          \
+        uint32_t, uint32_t, float*, uint32_t*) {                                                                      \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        qmt_body<ACT, SC, 1, RTV, TBV>(w, s, b, X, batch, rows, cols, QsAdd<ACT>{MV, RES, OUT});   \
+    }
+
+#define SMELT_AFFINE_QMT_GATE_UP(T, ACT, SC, RTV, TBV)                                             \
+    SMELT_QMT_KERNEL void smelt_affine_qmt_r##RTV##_t##TBV##_gate_up_swiglu_##T(                   \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {                                        \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        qmt_body<ACT, SC, 2, RTV, TBV>(w, s, b, X, batch, rows, cols, QsSwiglu<ACT>{Y});           \
+    }

@@ -220,7 +220,6 @@ void attach_mm1(ResolvedPipeline* r) {
 
 // The skinny qmm kernels that have a streaming form.
 void attach_qms(ResolvedPipeline* r) {
-    if (r->lds_variant != kSkinnyVariant) return;
     const std::string t = act_suffix(r->act);
     if (r->family == kFamAffineQmm) { r->qms_tail = "store_" + t; r->qms_nmat = 1; }
     else if (r->family == kFamAffineQmmAdd) { r->qms_tail = "add_" + t; r->qms_nmat = 1; }
@@ -231,6 +230,18 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
                                      ResolvedPipeline* out, std::string* why);
 
 }  // namespace
+
+bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmtPlan* out) {
+    // Measured on MI355X at the 4B FFN shapes: up to 128 tokens the streaming kernel's 16-token
+    // passes are as fast or faster (the weights of the later passes come from cache); beyond, the
+    // shared activation tile wins.  64 rows x 64 tokens per workgroup keeps the 2560-row matrix on
+    // every compute unit; larger tiles measured no faster at 512 tokens.
+    if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch <= 128) return false;
+    out->rt = nmat == 2 ? 1 : 2;
+    out->tb = 2;
+    out->lds = 2 * ((size_t)32 * out->tb * 272 + (size_t)nmat * 32 * out->rt * 72 + (size_t)nmat * 32 * out->rt * 16);   // two buffers
+    return out->lds <= lds_limit;
+}
 
 bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmsPlan* out) {
     if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;

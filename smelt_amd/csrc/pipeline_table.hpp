@@ -172,4 +172,12 @@ struct QmsPlan {
 };
 bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmsPlan* out);
 
+// Launch plan of the token-tile qmm: workgroups of four waves over 32 * rt rows (per matrix) and
+// 32 * tb tokens.  False when the shape has no such kernel or too few tokens to pay for the tiles.
+struct QmtPlan {
+    uint32_t rt = 0, tb = 0;
+    size_t lds = 0;
+};
+bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmtPlan* out);
+
 }  // namespace smelt_host

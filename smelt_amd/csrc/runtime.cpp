@@ -45,6 +45,7 @@ struct Pipeline {
     hipFunction_t fn_single = nullptr;  // used when the record's batch argument is 1
     hipFunction_t fn_mm_stream = nullptr, fn_mm_split = nullptr;  // matrix-core variants picked by shape
     hipFunction_t fn_mm1[kMm1MaxSegments + 1] = {};               // single-pass matrix-core matvec, by segments per wave
+    hipFunction_t fn_qmt[5][5] = {};                              // token-tile qmm, by row tiles and token blocks per wave
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
     ResolvedPipeline res;
 };
@@ -1061,7 +1062,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY, "threadgroup exceeds 1024 threads");
     if (int e = validate_launch(ctx, *p, L, ws)) return e;
     hipFunction_t fn = p->fn;
-    bool routed = false;
+    bool routed = false, qms_routed = false;
     if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.grid[1] == 1) {
         // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
         // arguments, its own launch geometry (one workgroup per eight rows)
@@ -1099,13 +1100,23 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         // geometry (16 * rt rows per workgroup, 16 tokens per grid row); it uses no workspace
         const size_t o = p->res.family == kFamAffineQmm ? 5 : (p->res.family == kFamAffineQmmAdd ? 7 : 8);
         const uint32_t batch = L.args[o].value, rows = L.args[o + 1].value, cols = L.args[o + 2].value, group = L.args[o + 3].value;
+        QmtPlan tplan;
+        if (qmt_plan(rows, cols, group, p->res.qms_nmat, batch, ctx->lds_limit, &tplan) && p->fn_qmt[tplan.rt][tplan.tb]) {
+            fn = p->fn_qmt[tplan.rt][tplan.tb];
+            L.grid[0] = (rows + 32 * tplan.rt - 1) / (32 * tplan.rt); L.grid[1] = (batch + 32 * tplan.tb - 1) / (32 * tplan.tb); L.grid[2] = 1;
+            L.block[0] = 256; L.block[1] = 1; L.block[2] = 1;
+            L.lds = tplan.lds;
+            routed = true;
+            qms_routed = true;
+        }
         QmsPlan plan;
-        if (batch > 0 && qms_plan(rows, cols, group, p->res.qms_nmat, batch, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
+        if (!routed && batch > 0 && qms_plan(rows, cols, group, p->res.qms_nmat, batch, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
             fn = p->fn_qms[plan.rt][batch > 8];
             L.grid[0] = (rows + 16 * plan.rt - 1) / (16 * plan.rt); L.grid[1] = (batch + 15) / 16; L.grid[2] = 1;
             L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
             L.lds = plan.lds;
             routed = true;
+            qms_routed = true;
         }
     }
     if (!routed && p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
@@ -1136,7 +1147,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             pos += 4;
         }
     }
-    if (p->res.workspace) {
+    if (p->res.workspace || qms_routed) {
+        // (the streaming qmm declares the two workspace pointers of the skinny kernels and ignores them)
         pos = (pos + 7) & ~(size_t)7;
         memcpy(kernarg + pos, &ws.partial, 8);
         memcpy(kernarg + pos + 8, &ws.counters, 8);
@@ -1334,6 +1346,10 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
             if (!p.res.mm1_prefix.empty())
                 for (uint32_t nl = 1; nl <= kMm1MaxSegments; ++nl)
                     (void)find(&p.fn_mm1[nl], p.res.mm1_prefix + "nl" + std::to_string(nl) + "_" + p.res.mm1_tail);
+            if (!p.res.qms_tail.empty())
+                for (uint32_t rt = 1; rt <= 4; ++rt)
+                    for (uint32_t tb = 2; tb <= 4; tb += 2)
+                        (void)find(&p.fn_qmt[rt][tb], "smelt_affine_qmt_r" + std::to_string(rt) + "_t" + std::to_string(tb) + "_" + p.res.qms_tail);
             if (!p.res.qms_tail.empty())
                 for (uint32_t rt = 1; rt <= kQmsMaxRowTiles; ++rt)
                     for (uint32_t wide = 0; wide < 2; ++wide)

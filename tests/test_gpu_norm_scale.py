@@ -249,7 +249,9 @@ def run_qmm(ctx, entry, dtype, batch, bufs_fn, rows, grid_w, bt, batch_index):
 @pytest.mark.parametrize("batch,suffix,bt", [(14, "_batched_full", 16), (37, "_batched_full", 16), (70, "_batched_full_b64", 64)])
 def test_norm_scale_qmm_equals_plain_qmm_on_the_stored_rows(ctx, dtype, batch, suffix, bt):
     """agent_norm_scale_affine_qmm_fixed_batched_full (lut_matvec.metal:8496-8530): per-token scales,
-    normalised rows stored, and the product equal to the plain qmm run on those rows bit for bit."""
+    normalised rows stored, and the product equal to the plain qmm run on those rows bit for bit
+    (the plain record kept on the token-slab kernel the fused form shares its tile code with)."""
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)
     rows, cols, group = 1000, 1024, 64
     weights = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=2)
     x, w, rs = norm_inputs(batch, cols, dtype, seed=batch)
@@ -269,6 +271,7 @@ def test_norm_scale_qmm_equals_plain_qmm_on_the_stored_rows(ctx, dtype, batch, s
     staged = run_qmm(ctx, "affine_matvec" + shape + suffix, dtype, batch,
                      lambda: [(0, 0, ow), (0, 1, os_), (0, 2, ob), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)],
                      rows, (rows + 63) // 64, bt, 5)
+    ctx.set_matvec_engine(rt.MATVEC_AUTO)
     assert np.array_equal(fused, staged)
     ref = so.affine_matvec(*weights, fx.from_bits(xn, dtype), rows, cols, group, dtype)
     gh.check_outputs(fused, ref, dtype, "norm_scale qmm")
@@ -290,9 +293,11 @@ def test_norm_scale_gate_up_qmm_and_geglu_qmm(ctx, act):
                     lambda: [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0)] + [(0, 3 + i, o) for i, o in enumerate(offs)] +
                             [(gh.Y_SLOT, 9, 0)], rows, (rows + 63) // 64, bt, 10)
     ctx.put(gh.X_SLOT, xn)
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)   # the staged record on the token-slab kernel the fused form shares its tile code with
     staged = run_qmm(ctx, f"fused_affine_gate_up_{act}" + shape, dtype, batch,
                      lambda: [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)],
                      rows, (rows + 63) // 64, bt, 8)
+    ctx.set_matvec_engine(rt.MATVEC_AUTO)
     assert np.array_equal(fused, staged)
     xf = fx.from_bits(xn, dtype)
     g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)

@@ -14,6 +14,7 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def ctx():
     c = rt.Context()
+    c.set_matvec_engine(rt.MATVEC_VECTOR)   # keeps qmm records on the token-slab kernels tested here
     yield c
     c.close()
 

@@ -176,3 +176,98 @@ def test_stream_qmm_fused_add_and_gate_up(ctx, dtype):
     sd = so.BF16 if dtype == fx.BF16 else so.F16
     ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, sd), dtype)
     gh.check_outputs(y, ref, dtype, "stream gate_up_swiglu", rel_tol=8e-3 if dtype == fx.BF16 else 4e-3)
+
+
+# ---- token-tile form: more than 128 tokens; up to there, 16-token passes of the streaming kernel ------
+
+def qmm_full(ctx, w, x_bits, dtype, rows, cols, bt=64):
+    """A token-slab qmm record as the emitter writes it for prefill chunks (64-row slabs, bt-token grid rows)."""
+    batch = x_bits.shape[0]
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in w]
+    ctx.upload_weights(0, wf.image())
+    ctx.put(gh.X_SLOT, x_bits)
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+    pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g64_batched_full_b{bt}" + gh.t_suffix(dtype))
+    bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+    rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], ((rows + 63) // 64, bt, 1), (256, 1, 1),
+                         grid_kinds=(0, rt.GRID_SEQ_LEN_CEIL_DIV, 0))
+    assert ctx.encode_prefill(rec, seq_len=batch) == 1
+    ctx.wait()
+    return ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("batch", [49, 64, 100, 129, 300])
+def test_tile_qmm_4b_shapes(ctx, dtype, batch):
+    """Qwen3.5-4B-shaped slab (K=2560, 392 rows: ragged last row tile), ragged last token tile."""
+    rows, cols = 392, 2560
+    w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=0)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=batch, outlier_frac=0.01)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype, threads=True)
+    y = qmm_full(ctx, w, x, dtype, rows, cols)
+    worst = gh.check_outputs(y, ref, dtype, f"tile qmm M={batch}")
+    print(f"\n  tile qmm M={batch} dtype={dtype} max rel err {worst:.2e}")
+
+
+@pytest.mark.parametrize("shape", [(200, 9216, 512), (8200, 1024, 96), (40, 512, 170), (2600, 2560, 520)])
+def test_tile_qmm_shapes(ctx, split_k, shape):
+    """Long rows at a 512-token chunk, many rows in several 16-token passes, a matrix smaller than
+    one tile, and ragged row and token tiles; against the oracle and the token-slab kernel."""
+    rows, cols, batch = shape
+    dtype = fx.BF16
+    w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=rows % 11)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=cols % 13, outlier_frac=0.01)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype, threads=True)
+    y = qmm_full(ctx, w, x, dtype, rows, cols)
+    gh.check_outputs(y, ref, dtype, f"tile qmm {shape}")
+    assert np.array_equal(y, qmm_full(ctx, w, x, dtype, rows, cols))
+    gh.check_outputs(qmm_full(split_k, w, x, dtype, rows, cols), ref, dtype, f"slab qmm {shape}")
+
+
+def test_tile_qmm_is_exact_where_the_sums_are(ctx):
+    rows, cols, group, batch = 64, 1024, 64, 150
+    packed, scales, biases, x = fx.kernel_lab_qmm_fixture(rows, cols, group, batch)
+    ref = so.affine_matvec(packed, scales, biases, fx.from_bits(x, fx.F16), rows, cols, group)
+    y = qmm_full(ctx, (packed, scales, biases), x, fx.F16, rows, cols)
+    assert np.array_equal(y, ref.astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_tile_qmm_fused_add_and_gate_up(ctx, dtype):
+    rows, cols, batch = 200, 2560, 140
+    gw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=3)
+    uw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=4)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=8)
+    res = fx.to_bits(fx.rng_for(4, 79).normal(0, 1, (batch, rows)).astype(np.float32), dtype)
+    plain = qmm_full(ctx, gw, x, dtype, rows, cols)
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*gw, *uw)]
+    ctx.upload_weights(0, wf.image())
+    ctx.put(gh.X_SLOT, x)
+    ctx.put(gh.RES_SLOT, res)
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+    ctx.alloc(gh.AUX_SLOT, batch * rows * 2)
+    t = gh.t_suffix(dtype)
+    grid = ((rows + 63) // 64, (batch + 63) // 64, 1)
+    pipe = ctx.pipeline(f"fused_affine_matvec_add_c{cols}_r{rows}_g64_batched_full_b64" + t)
+    bufs = [(0, i, offs[i]) for i in range(3)] + [(gh.X_SLOT, 3, 0), (gh.AUX_SLOT, 4, 0), (gh.RES_SLOT, 5, 0), (gh.Y_SLOT, 6, 0)]
+    rec = rt.make_record(pipe, bufs, [(7, batch)], grid, (256, 1, 1))
+    assert ctx.encode_prefill(rec, seq_len=batch) == 1
+    ctx.wait()
+    mv = ctx.read(gh.AUX_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    out = ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    assert np.array_equal(mv, plain)                       # fused == staged, bit for bit
+    assert np.array_equal(out, so.narrow(fx.from_bits(plain, dtype) + fx.from_bits(res, dtype), dtype))
+    pipe = ctx.pipeline(f"fused_affine_gate_up_swiglu_c{cols}_r{rows}_g64_batched_full_b64" + t)
+    bufs = [(0, i, offs[i]) for i in range(6)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
+    rec = rt.make_record(pipe, bufs, [(8, batch)], grid, (256, 1, 1))
+    assert ctx.encode_prefill(rec, seq_len=batch) == 1
+    ctx.wait()
+    y = ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    xf = fx.from_bits(x, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, 64, dtype)
+    u = so.affine_matvec(*uw, xf, rows, cols, 64, dtype)
+    sd = so.BF16 if dtype == fx.BF16 else so.F16
+    ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, sd), dtype)
+    gh.check_outputs(y, ref, dtype, "tile gate_up_swiglu", rel_tol=8e-3 if dtype == fx.BF16 else 4e-3)
