@@ -23,6 +23,10 @@ def build_affine_table(dtype):
     tensors = {}
     for i, (name, e) in enumerate((("q", wq), ("gate", wg), ("up", wu), ("down", wd), ("lm_head", wl))):
         t = fx.synth_affine(e.rows, e.cols, group, dtype, config=1, tensor=20 + i)
+        if name in ("down", "lm_head"):
+            # the chain multiplies magnitudes up; the two deep tensors are scaled by 2^-6 (exact in
+            # both 16-bit types) so that every intermediate and every logit stays inside fp16
+            t = (t[0], fx.to_bits(fx.from_bits(t[1], dtype) / 64.0, dtype), fx.to_bits(fx.from_bits(t[2], dtype) / 64.0, dtype))
         cc.write_affine(image, e, *t)
         tensors[name] = t
     em = cc.Emitter(rt.ACT_BF16 if dtype == fx.BF16 else rt.ACT_F16)
@@ -33,6 +37,7 @@ def build_affine_table(dtype):
     return em, image, tensors, (hidden, qdim, ffn, vocab, group)
 
 
+@pytest.mark.filterwarnings("error::RuntimeWarning")   # an fp16 overflow in the reference chain would be one
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 def test_affine_decode_table_eager_and_graph(dtype):
     em, image, tensors, (hidden, qdim, ffn, vocab, group) = build_affine_table(dtype)
@@ -187,5 +192,41 @@ def test_affine_projection_bank_equals_independent_matvecs():
         ctx.wait()
         a, b = ctx.read(2, np.uint16, total), ctx.read(3, np.uint16, total)
         assert a.any() and np.array_equal(a, b)
+    finally:
+        ctx.close()
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_lm_head_argmax_full_vocabulary(dtype):
+    """The tied lm_head of the decode-step configuration at its real size (151936 x 1024, affine u4
+    g64): the token the fused matvec + argmax returns is the oracle's argmax over all 151936 16-bit
+    logits.  The two sides sum in different orders, so a token whose oracle logit has the winner's
+    16-bit value counts as the tie it is (lowest index wins only among bit-identical logits)."""
+    vocab, hidden, group = 151936, 1024, 64
+    lay = cc.Layout()
+    wl = lay.affine(vocab, hidden, group)
+    w = fx.synth_affine(vocab, hidden, group, dtype, config=1, tensor=168)
+    image = np.zeros(lay.total_bytes, np.uint8)
+    cc.write_affine(image, wl, *w)
+    act = rt.ACT_BF16 if dtype == fx.BF16 else rt.ACT_F16
+    ctx = rt.Context(act_dtype=act)
+    try:
+        em = cc.Emitter(act, ctx.device_info()["compute_units"])
+        em.lm_head_argmax(0, wl, cc.bind(H_SLOT), cc.bind(KEY_SLOT), cc.bind(TOK_SLOT))
+        em.install(ctx)
+        ctx.upload_weights(0, image)
+        ctx.alloc(KEY_SLOT, max(em.argmax_partial_bytes, 8))
+        ctx.alloc(TOK_SLOT, 4)
+        for seed in (9000, 9001, 9002):
+            x = fx.to_bits(fx.rng_for(1, seed).normal(0, 1, (1, hidden)).astype(np.float32), dtype)
+            ctx.put(H_SLOT, x)
+            ctx.interpret_decode(em.records())
+            ctx.wait()
+            tok = int(ctx.read(TOK_SLOT, np.int32, 1)[0])
+            logits = so.narrow(so.affine_matvec(*w, fx.from_bits(x, dtype), vocab, hidden, group, dtype, threads=True), dtype)[0]
+            want = so.argmax16(logits)
+            assert 0 <= tok < vocab
+            assert tok == want or logits[tok] == logits[want], (seed, tok, want)
+            print(f"\n  lm_head dtype={dtype} seed={seed}: token {tok} (oracle {want})")
     finally:
         ctx.close()

@@ -170,3 +170,21 @@ def test_bf16_activations_beyond_the_fp16_range(ctx):
     ref = so.affine_matvec(packed, scales, biases, fx.from_bits(x, dtype), rows, cols, group, dtype)
     y = run_affine(ctx, packed, scales, biases, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
     gh.check_outputs(y, ref, dtype, "matrix-core affine with |x| > 65504")
+
+
+def test_vector_engine_converts_bf16_activations_to_fp16(vec):
+    """The vector-ALU kernels feed v_dot2_f32_f16: bf16 activations are converted to fp16 on staging,
+    exact for |x| in [2^-14, 65504] and saturating beyond.  Pinned here: with |x| > 65504 the kernel
+    matches the oracle run on the clamped activations, not on the raw ones."""
+    rows, cols, group = 64, 1024, 64
+    dtype = fx.BF16
+    packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=8)
+    xf = fx.rng_for(1, 555).normal(0, 1, (1, cols)).astype(np.float32)
+    xf[0, ::37] *= 3.0e5
+    x = fx.to_bits(xf, dtype)
+    raw = fx.from_bits(x, dtype)
+    clamped = np.clip(raw, -65504.0, 65504.0)
+    y = run_affine(vec, packed, scales, biases, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    gh.check_outputs(y, so.affine_matvec(packed, scales, biases, clamped, rows, cols, group, dtype), dtype, "vector engine, clamped reference")
+    ref_raw = so.affine_matvec(packed, scales, biases, raw, rows, cols, group, dtype)
+    assert np.abs(fx.from_bits(y, dtype) - ref_raw).max() > 0.1 * np.abs(ref_raw).max()
