@@ -317,7 +317,7 @@ def layer_measurements(fx, cc, rt, cus, engine) -> dict:
                 mk = lambda r, k_: lay.affine(r, k_, 64)
             else:
                 mk = lambda r, k_: lay.signed(r, k_, wdtype)
-                q, k, v = mk(H, H), mk(KV, H), mk(KV, H)
+                q, k, v = lay.signed_bank([H, KV, KV], H, wdtype)
             return {"q": q, "k": k, "v": v, "o": mk(H, H), "gate": mk(F, H), "up": mk(F, H), "down": mk(H, F)}
 
         first = make_layer()

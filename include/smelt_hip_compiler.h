@@ -92,6 +92,10 @@ int smelt_layout_make_signed_entry(int rows, int cols, int dtype, int group_size
  * entry; a bank kernel then walks the members as one virtual row space. */
 int smelt_layout_make_affine_bank(const int *member_rows, int members, int cols, int group_size,
                                   uint64_t *offset_io, SmeltWeightEntryC *out_members);
+/* The same bank for signed members (binary1, ternary2, trit5): one contiguous code slab, then one
+ * 128-byte-aligned scale slab. */
+int smelt_layout_make_signed_bank(const int *member_rows, int members, int cols, int dtype, int group_size,
+                                  uint64_t *offset_io, SmeltWeightEntryC *out_members);
 /* dense fp16/bf16/fp32/int32 entry, 16-byte aligned (:700-737) */
 int smelt_layout_make_dense_entry(int rows, int cols, int dtype, uint64_t *offset_io,
                                   SmeltWeightEntryC *out);

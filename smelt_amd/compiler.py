@@ -66,6 +66,7 @@ def lib() -> C.CDLL:
         "smelt_layout_make_signed_entry": (i32, [i32, i32, i32, i32, u64p, we]),
         "smelt_layout_make_dense_entry": (i32, [i32, i32, i32, u64p, we]),
         "smelt_layout_make_affine_bank": (i32, [C.POINTER(i32), i32, i32, i32, u64p, we]),
+        "smelt_layout_make_signed_bank": (i32, [C.POINTER(i32), i32, i32, i32, i32, u64p, we]),
         "smelt_emit_bank_matvec": (i32, [vp, i32, we, i32, Binding, C.POINTER(Binding)]),
         "smelt_route_decode_affine": (i32, [i32, i32, i32, i32, i32, C.POINTER(Route)]),
         "smelt_route_prefill_affine": (i32, [i32, i32, i32, i32, i32, i32, C.POINTER(Route)]),
@@ -146,6 +147,15 @@ class Layout:
         rows = (C.c_int * n)(*member_rows)
         out = (WeightEntry * n)()
         self._check(lib().smelt_layout_make_affine_bank(rows, n, cols, group, C.byref(self.offset), out))
+        members = [WeightEntry.from_buffer_copy(bytes(out[i])) for i in range(n)]
+        self.entries.extend(members)
+        return members
+
+    def signed_bank(self, member_rows, cols, dtype, group=128) -> list[WeightEntry]:
+        n = len(member_rows)
+        rows = (C.c_int * n)(*member_rows)
+        out = (WeightEntry * n)()
+        self._check(lib().smelt_layout_make_signed_bank(rows, n, cols, dtype, group, C.byref(self.offset), out))
         members = [WeightEntry.from_buffer_copy(bytes(out[i])) for i in range(n)]
         self.entries.extend(members)
         return members

@@ -357,6 +357,39 @@ int smelt_layout_make_affine_bank(const int* member_rows, int members, int cols,
     return SMELT_HIP_OK;
 }
 
+int smelt_layout_make_signed_bank(const int* member_rows, int members, int cols, int dtype, int group_size, uint64_t* offset_io, SmeltWeightEntryC* out) {
+    if (!member_rows || !offset_io || !out || members < 2 || members > 4 || cols <= 0 || group_size <= 0 || !signed_dtype(dtype)) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    const int padded = (cols + group_size - 1) / group_size * group_size;
+    uint64_t stride;
+    if (dtype == SMELT_DTYPE_TRIT5) stride = (uint64_t)((((cols + 4) / 5) + 15) & ~15);
+    else stride = (uint64_t)((padded * (dtype == SMELT_DTYPE_BINARY1 ? 1 : 2) + 7) / 8);
+    const uint64_t groups = (uint64_t)(padded / group_size);
+    uint64_t total_rows = 0;
+    for (int m = 0; m < members; ++m) {
+        if (member_rows[m] <= 0) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+        total_rows += (uint64_t)member_rows[m];
+    }
+    const uint64_t packed0 = align_to(*offset_io, 128);
+    const uint64_t scales0 = align_to(packed0 + total_rows * stride, 128);
+    *offset_io = scales0 + total_rows * groups * 2;
+    uint64_t before = 0;
+    for (int m = 0; m < members; ++m) {
+        SmeltWeightEntryC& e = out[m];
+        memset(&e, 0, sizeof(e));
+        e.rows = member_rows[m]; e.cols = cols;
+        e.dtype = dtype;
+        e.group_size = group_size;
+        e.packed_row_stride = (int32_t)stride;
+        e.padded_cols = padded;
+        e.offset = packed0 + before * stride;
+        e.size_bytes = (uint64_t)e.rows * stride;
+        e.scales_offset = scales0 + before * groups * 2;
+        e.scales_size_bytes = (uint64_t)e.rows * groups * 2;
+        before += (uint64_t)e.rows;
+    }
+    return SMELT_HIP_OK;
+}
+
 int smelt_layout_make_dense_entry(int rows, int cols, int dtype, uint64_t* offset_io, SmeltWeightEntryC* out) {
     if (!offset_io || !out || rows <= 0 || cols <= 0) return SMELT_HIP_ERR_INVALID_ARGUMENT;
     int bpe = 0;
@@ -971,9 +1004,23 @@ int smelt_emit_bank_matvec(smelt_emitter* e, int weights_slot, const SmeltWeight
         e->records.push_back(rb.r);
         return SMELT_HIP_OK;
     }
-    if (family != SMELT_FAMILY_TERNARY2) return 1;  // banks exist for affine and ternary members
+    if (family != SMELT_FAMILY_TERNARY2 && family != SMELT_FAMILY_BINARY1) return 1;  // banks exist for affine, binary and ternary members
     for (int m = 0; m < count; ++m)
         if (int rc = check_signed_entry(e, &members[m])) return rc;
+    if (family == SMELT_FAMILY_BINARY1) {
+        // binary packed bank (C S x y0..y3 rows0..rows3 cols)
+        const MatvecGeometry g = matvec_geometry(signed_row_stride(kFmtBinary1, (uint32_t)first.cols), (int)rows, 4, e->compute_units);
+        rb.buffer(0, weights_slot, first.offset);
+        rb.buffer(1, weights_slot, first.scales_offset);
+        rb.buffer(2, input);
+        for (int m = 0; m < 4; ++m) rb.buffer((uint8_t)(3 + m), outputs[m < count ? m : 0]);
+        for (int m = 0; m < 4; ++m) rb.constant((uint8_t)(7 + m), m < count ? (uint32_t)members[m].rows : 0u);
+        rb.constant(11, (uint32_t)first.cols);
+        rb.grid((uint32_t)g.grid_w, 1, 1, 256);
+        rb.r.pipeline = e->pipeline_index("signed_binary_packed_bank4_matvec_g128_rows8");
+        e->records.push_back(rb.r);
+        return SMELT_HIP_OK;
+    }
     const MatvecGeometry g = matvec_geometry(signed_row_stride(kFmtTernary2, (uint32_t)first.cols), (int)rows, 4, e->compute_units);
     rb.buffer(0, weights_slot, first.offset);
     rb.buffer(1, weights_slot, first.scales_offset);

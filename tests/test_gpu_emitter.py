@@ -196,6 +196,56 @@ def test_affine_projection_bank_equals_independent_matvecs():
         ctx.close()
 
 
+@pytest.mark.parametrize("engine", [rt.MATVEC_VECTOR, rt.MATVEC_MATRIX_CORE])
+@pytest.mark.parametrize("fmt,wdtype", [(fx.BINARY1, cc.BINARY1), (fx.TERNARY2, cc.TERNARY2), (fx.TRIT5, cc.TRIT5)])
+def test_signed_projection_bank(fmt, wdtype, engine):
+    """q|k|v of a signed format laid out as one bank: contiguous code and scale slabs, one dispatch
+    for binary and ternary members (no bank kernel exists for trit5: the emitter says so and the
+    members run one by one); every member against the oracle, on both matvec engines."""
+    hidden = 1280
+    member_rows = [520, 136, 128]
+    lay = cc.Layout()
+    members = lay.signed_bank(member_rows, hidden, wdtype)
+    assert members[1].offset == members[0].offset + members[0].size_bytes
+    assert members[2].scales_offset == members[1].scales_offset + members[1].scales_size_bytes
+    assert members[0].offset % 128 == 0 and members[0].scales_offset % 128 == 0
+    image = np.zeros(lay.total_bytes, np.uint8)
+    tensors = []
+    for i, e in enumerate(members):
+        codes = fx.synth_signed_codes(fmt, e.rows, hidden, config=2 + fmt, tensor=i)
+        scales = fx.synth_signed_scales(e.rows, hidden, config=2 + fmt, tensor=i)
+        packed = fx.pack_signed_np(codes, fmt, e.packed_row_stride)
+        cc.write_signed(image, e, packed, scales)
+        tensors.append((packed, scales))
+    dtype = fx.BF16
+    ctx = rt.Context(act_dtype=rt.ACT_BF16)
+    ctx.set_matvec_engine(engine)
+    try:
+        em = cc.Emitter(rt.ACT_BF16)
+        outs = [cc.bind(2, 0), cc.bind(2, 520 * 2), cc.bind(2, 656 * 2)]
+        banked = em.bank_matvec(0, members, cc.bind(1), outs)
+        assert banked == (fmt != fx.TRIT5)
+        if not banked:
+            for e, o in zip(members, outs):
+                em.matvec(0, e, cc.bind(1), o)
+        em.install(ctx)
+        ctx.upload_weights(0, image)
+        x = fx.synth_activation(1, hidden, dtype, config=2, tensor=43)
+        ctx.put(1, x)
+        total = sum(member_rows)
+        ctx.alloc(2, total * 2)
+        assert ctx.interpret_decode(em.records()) == (1 if banked else 3)
+        ctx.wait()
+        y = ctx.read(2, np.uint16, total)
+        at = 0
+        for (packed, scales), e in zip(tensors, members):
+            ref = so.signed_matvec(fmt, packed, scales, fx.from_bits(x, dtype), e.rows, hidden, hidden, 128)
+            gh.check_outputs(y[at:at + e.rows].reshape(1, -1), ref, dtype, f"bank member of {e.rows} rows")
+            at += e.rows
+    finally:
+        ctx.close()
+
+
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 def test_lm_head_argmax_full_vocabulary(dtype):
     """The tied lm_head of the decode-step configuration at its real size (151936 x 1024, affine u4
