@@ -223,7 +223,13 @@ int smelt_hip_benchmark_record(smelt_hip_context *ctx, const SmeltDispatchRecord
 
 /* Launch-bound tables (about a thousand records per token, SmeltRuntime.swift:3251-3275) are
  * captured once into a HIP graph and replayed; the analogue of the reference's indirect
- * command buffer replay. */
+ * command buffer replay.  A graph holds what the capture resolved: device addresses of the
+ * slots (cur / alt included), byte offsets and constants derived from `position` (decode) or
+ * `seq_len` / `start_pos` (prefill), grids derived from seq_len.  It therefore stays valid only
+ * while no slot it binds is re-allocated or re-uploaded, and replays the position it was
+ * captured with: a table whose records carry position-dependent offsets or constants needs one
+ * capture per position (a table of matvec / qmm records carries none).  Destroy a graph before
+ * freeing the slots it names. */
 int smelt_hip_graph_capture_decode(smelt_hip_context *ctx, const SmeltDispatchRecord *table,
                                    size_t count, int cur0, int alt0, int32_t position,
                                    smelt_hip_graph **out);
