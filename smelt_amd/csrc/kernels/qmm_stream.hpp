@@ -539,7 +539,9 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
 
 }  // namespace smelt
 
-#define SMELT_QMT_KERNEL extern "C" __global__ __launch_bounds__(256)
+// Two waves per SIMD at least: that caps the kernel at 256 registers, all of them VGPRs, so the MFMA results land where
+// the fp32 FMAs read them (with the whole 512-register file on offer the compiler parks them in AGPRs and copies).
+#define SMELT_QMT_KERNEL extern "C" __global__ __launch_bounds__(256, 2)
 
 // Argument lists of the token-slab qmm kernels of the same pipelines, plus the two workspace
 // pointers of the skinny ones (unused).

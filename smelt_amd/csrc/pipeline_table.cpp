@@ -235,10 +235,13 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     // Measured on MI355X at the 4B FFN shapes: up to 128 tokens the streaming kernel's 16-token
     // passes are as fast or faster (the weights of the later passes come from cache); beyond, the
     // shared activation tile wins.  64 rows x 64 tokens per workgroup keeps the 2560-row matrix on
-    // every compute unit; larger tiles measured no faster at 512 tokens.
+    // every compute unit; 128-token tiles measured no faster.
     if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch <= 128) return false;
     out->rt = nmat == 2 ? 1 : 2;
     out->tb = 2;
+    // 128-row tiles once they still give every compute unit two workgroups (measured: 502 against 425 TFLOP/s at 1024
+    // tokens on the 9216-row matrix, equal at 256)
+    if (nmat == 1 && (uint64_t)((rows + 127) / 128) * ((batch + 63) / 64) >= 512) out->rt = 4;
     out->lds = 2 * ((size_t)32 * out->tb * 272 + (size_t)nmat * 32 * out->rt * 72 + (size_t)nmat * 32 * out->rt * 16);   // two buffers
     return out->lds <= lds_limit;
 }
