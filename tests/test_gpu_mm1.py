@@ -188,3 +188,86 @@ def test_vector_engine_converts_bf16_activations_to_fp16(vec):
     gh.check_outputs(y, so.affine_matvec(packed, scales, biases, clamped, rows, cols, group, dtype), dtype, "vector engine, clamped reference")
     ref_raw = so.affine_matvec(packed, scales, biases, raw, rows, cols, group, dtype)
     assert np.abs(fx.from_bits(y, dtype) - ref_raw).max() > 0.1 * np.abs(ref_raw).max()
+
+
+def test_ternary_affine_names_on_both_engines(ctx, vec):
+    """signed_ternary_affine_{matvec, matvec_add, gate_up_swiglu}_g128_rows8 (the production ternary
+    names: codes, scales, scales again, x, y): the matrix-core kernels against the oracle and the
+    vector kernels, ragged row count."""
+    dtype = fx.BF16
+    rows, cols = 203, 2560
+    gc = fx.synth_signed_codes(fx.TERNARY2, rows, cols, config=3, tensor=5)
+    uc = fx.synth_signed_codes(fx.TERNARY2, rows, cols, config=3, tensor=6)
+    gs = fx.synth_signed_scales(rows, cols, config=3, tensor=5)
+    us = fx.synth_signed_scales(rows, cols, config=3, tensor=6)
+    gp, up = fx.pack_signed_np(gc, fx.TERNARY2), fx.pack_signed_np(uc, fx.TERNARY2)
+    x = fx.synth_activation(1, cols, dtype, config=3, tensor=7)
+    res = fx.to_bits(fx.rng_for(3, 80).normal(0, 1, (1, rows)).astype(np.float32), dtype)
+    xf = fx.from_bits(x, dtype)
+    g_ref = so.signed_matvec(so.TERNARY2, gp, gs, xf, rows, cols, cols, 128)
+    u_ref = so.signed_matvec(so.TERNARY2, up, us, xf, rows, cols, cols, 128)
+    got = {}
+    for name, c in (("matrix", ctx), ("vector", vec)):
+        wf = gh.WeightFile()
+        ogp, ogs, oup, ous = wf.add(gp), wf.add(gs), wf.add(up), wf.add(us)
+        c.upload_weights(0, wf.image())
+        c.put(gh.X_SLOT, x)
+        c.put(gh.RES_SLOT, res)
+        for s in (gh.Y_SLOT, gh.AUX_SLOT, gh.AUX2_SLOT):
+            c.alloc(s, rows * 2)
+        grid = ((rows + 7) // 8, 1, 1)
+
+        def run(pipe, bufs, consts):
+            c.encode_decode(rt.make_record(c.pipeline(pipe + gh.t_suffix(dtype)), bufs, consts, grid, (256, 1, 1)))
+            c.wait()
+
+        run("signed_ternary_affine_matvec_g128_rows8",
+            [(0, 0, ogp), (0, 1, ogs), (0, 2, ogs), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)], [(5, rows), (6, cols)])
+        run("signed_ternary_affine_matvec_add_g128_rows8",
+            [(0, 0, ogp), (0, 1, ogs), (0, 2, ogs), (gh.X_SLOT, 3, 0), (gh.AUX_SLOT, 4, 0), (gh.RES_SLOT, 5, 0)], [(6, rows), (7, cols)])
+        run("signed_ternary_affine_gate_up_swiglu_g128_rows8",
+            [(0, 0, ogp), (0, 1, ogs), (0, 2, ogs), (0, 3, oup), (0, 4, ous), (0, 5, ous), (gh.X_SLOT, 6, 0), (gh.AUX2_SLOT, 7, 0)],
+            [(8, rows), (9, cols)])
+        y = c.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+        ya = c.read(gh.AUX_SLOT, np.uint16, rows).reshape(1, rows)
+        yg = c.read(gh.AUX2_SLOT, np.uint16, rows).reshape(1, rows)
+        gh.check_outputs(y, g_ref, dtype, f"ternary-affine matvec ({name})")
+        assert np.array_equal(ya, so.narrow(fx.from_bits(y, dtype) + fx.from_bits(res, dtype), dtype))
+        staged = so.epilogue_signed_swiglu(so.narrow(g_ref, dtype), so.narrow(u_ref, dtype), so.BF16)
+        assert np.abs(yg.astype(np.int32) - staged.astype(np.int32)).max() <= 2, name
+        got[name] = y
+    assert np.abs(got["matrix"].astype(np.int32) - got["vector"].astype(np.int32)).max() <= 1
+
+
+def test_affine_bank4_on_the_matrix_cores(ctx, vec):
+    """affine_bank4_matvec:K:G over q|k|v: the matrix-core bank kernel gives each member the bits of
+    its own matrix-core matvec, and the oracle's values."""
+    dtype = fx.BF16
+    cols, group = 2560, 64
+    member_rows = [264, 72, 61]
+    rows = sum(member_rows)
+    w = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=9)
+    x = fx.synth_activation(1, cols, dtype, config=1, tensor=10)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, group, dtype)
+    whole = run_affine(ctx, *w, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    gh.check_outputs(whole, ref, dtype, "matrix-core matvec over the whole slab")
+    for c in (ctx, vec):
+        wf = gh.WeightFile()
+        offs = [wf.add(a) for a in w]
+        c.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+        c.put(gh.X_SLOT, x)
+        outs = [gh.Y_SLOT, gh.AUX_SLOT, gh.AUX2_SLOT]
+        for s, r in zip(outs, member_rows):
+            c.alloc(s, r * 2)
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0)] + [(outs[min(i, 2)], 4 + i, 0) for i in range(4)]
+        consts = [(8 + i, member_rows[i] if i < 3 else 0) for i in range(4)]
+        pipe = c.pipeline(f"affine_bank4_matvec:{cols}:{group}" + gh.t_suffix(dtype))
+        c.encode_decode(rt.make_record(pipe, bufs, consts, ((rows + 7) // 8, 1, 1), (256, 1, 1)))
+        c.wait()
+        start = 0
+        for s, r in zip(outs, member_rows):
+            y = c.read(s, np.uint16, r).reshape(1, r)
+            gh.check_outputs(y, ref[:, start:start + r], dtype, "bank member")
+            if c is ctx:
+                assert np.array_equal(y, whole[:, start:start + r])
+            start += r
