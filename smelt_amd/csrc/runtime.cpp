@@ -1063,29 +1063,38 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     if (int e = validate_launch(ctx, *p, L, ws)) return e;
     hipFunction_t fn = p->fn;
     bool routed = false, qms_routed = false;
+    // the re-routed kernels fetch codes, scales, biases and activations 16 bytes at a time: the
+    // first `n` arguments (the read-only operands) have to sit on 16-byte boundaries, as the layouts
+    // the library writes do; a record that binds them elsewhere keeps the kernel its name describes
+    auto aligned16 = [&](size_t n) {
+        for (size_t i = 0; i < n && i < L.args.size(); ++i)
+            if (L.args[i].kind == 'P' && (reinterpret_cast<uintptr_t>(L.args[i].ptr) & 15u)) return false;
+        return true;
+    };
     if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.grid[1] == 1) {
         // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
         // arguments, its own launch geometry (one workgroup per eight rows)
         uint32_t rows = 0, cols = 0, group = 128;
+        size_t ro = 0;   // leading read-only operands (codes, scales[, biases], ..., x)
         auto U = [&](size_t i) { return L.args[i].value; };
         switch (p->res.family) {
-            case kFamAffineMatvec: rows = U(5); cols = U(6); group = U(7); break;
-            case kFamAffineAdd: rows = U(6); cols = U(7); group = U(8); break;
-            case kFamAffineGateUp: rows = U(8); cols = U(9); group = U(10); break;
-            case kFamAffineBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); group = U(13); break;
-            case kFamSignedMatvec: rows = U(4); cols = U(5); break;
-            case kFamSignedAdd: rows = U(5); cols = U(6); break;
-            case kFamSignedGateUp: rows = U(6); cols = U(7); break;
-            case kFamBinaryPackedBank: rows = U(5) + U(6); cols = U(7); break;
-            case kFamBinaryPackedBank4: rows = U(7) + U(8) + U(9) + U(10); cols = U(11); break;
-            case kFamTerAffMatvec: rows = U(5); cols = U(6); break;
-            case kFamTerAffAdd: rows = U(6); cols = U(7); break;
-            case kFamTerAffGateUp: rows = U(8); cols = U(9); break;
-            case kFamTerAffBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); break;
+            case kFamAffineMatvec: rows = U(5); cols = U(6); group = U(7); ro = 4; break;
+            case kFamAffineAdd: rows = U(6); cols = U(7); group = U(8); ro = 4; break;
+            case kFamAffineGateUp: rows = U(8); cols = U(9); group = U(10); ro = 7; break;
+            case kFamAffineBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); group = U(13); ro = 4; break;
+            case kFamSignedMatvec: rows = U(4); cols = U(5); ro = 3; break;
+            case kFamSignedAdd: rows = U(5); cols = U(6); ro = 3; break;
+            case kFamSignedGateUp: rows = U(6); cols = U(7); ro = 5; break;
+            case kFamBinaryPackedBank: rows = U(5) + U(6); cols = U(7); ro = 3; break;
+            case kFamBinaryPackedBank4: rows = U(7) + U(8) + U(9) + U(10); cols = U(11); ro = 3; break;
+            case kFamTerAffMatvec: rows = U(5); cols = U(6); ro = 4; break;
+            case kFamTerAffAdd: rows = U(6); cols = U(7); ro = 4; break;
+            case kFamTerAffGateUp: rows = U(8); cols = U(9); ro = 7; break;
+            case kFamTerAffBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); ro = 4; break;
             default: break;
         }
         Mm1Plan plan;
-        if (rows > 0 && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
+        if (rows > 0 && aligned16(ro) && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
                                  ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &plan) &&
             p->fn_mm1[plan.nl]) {
             fn = p->fn_mm1[plan.nl];
@@ -1095,7 +1104,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             routed = true;
         }
     }
-    if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR) {
+    if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
+        aligned16(p->res.family == kFamAffineQmmGateUp ? 7 : 4)) {
         // skinny qmm: the streaming kernel of the same pipeline, same arguments, its own launch
         // geometry (16 * rt rows per workgroup, 16 tokens per grid row); it uses no workspace
         const size_t o = p->res.family == kFamAffineQmm ? 5 : (p->res.family == kFamAffineQmmAdd ? 7 : 8);

@@ -271,3 +271,31 @@ def test_affine_bank4_on_the_matrix_cores(ctx, vec):
             if c is ctx:
                 assert np.array_equal(y, whole[:, start:start + r])
             start += r
+
+
+def test_operands_off_a_16_byte_boundary_keep_the_vector_kernel(ctx, vec):
+    """The matrix-core kernels fetch scales and biases 16 bytes at a time; a record that binds a
+    scale plane 2 bytes past a boundary is served by the kernel its pipeline names (bit-identical to
+    the vector engine), not faulted on."""
+    dtype = fx.BF16
+    rows, cols, group = 96, 2560, 64
+    packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=12)
+    x = fx.synth_activation(1, cols, dtype, config=1, tensor=13)
+    ref = so.affine_matvec(packed, scales, biases, fx.from_bits(x, dtype), rows, cols, group, dtype)
+    image = np.zeros(1 << 20, np.uint8)
+    o_w, o_s, o_b = 0, 256 * 1024 + 2, 512 * 1024
+    for off, a in ((o_w, packed), (o_s, scales), (o_b, biases)):
+        b = np.ascontiguousarray(a).view(np.uint8).ravel()
+        image[off:off + b.size] = b
+    out = []
+    for c in (ctx, vec):
+        c.upload_weights(gh.WEIGHTS_SLOT, image)
+        c.put(gh.X_SLOT, x)
+        c.alloc(gh.Y_SLOT, rows * 2)
+        pipe = c.pipeline(f"affine_matvec:{cols}:{group}" + gh.t_suffix(dtype))
+        bufs = [(0, 0, o_w), (0, 1, o_s), (0, 2, o_b), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+        c.encode_decode(rt.make_record(pipe, bufs, [(5, rows)], ((rows + 7) // 8, 1, 1), (256, 1, 1)))
+        c.wait()
+        out.append(c.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows))
+    gh.check_outputs(out[0], ref, dtype, "misaligned scale plane")
+    assert np.array_equal(out[0], out[1])
