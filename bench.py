@@ -86,7 +86,8 @@ def main() -> int:
                     help="the step plus one group of side measurements (layers: 27B-layer matvecs per weight format; "
                          "qmm: 4B FFN token tiles; aux: config-0 cold/warm, cold step, quantiser, turbo_quant_h)")
     ap.add_argument("--engine", choices=("auto", "matrix", "vector"), default="auto",
-                    help="single-token matvec engine (smelt_hip_set_matvec_engine); auto is what a package gets")
+                    help="kernel choice (smelt_hip_set_matvec_engine): auto is what a package gets; vector keeps every record on the "
+                         "kernel its pipeline name describes (vector-ALU matvec, split-K / slab qmm)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path has no cross-GPU part in this build "
@@ -240,7 +241,7 @@ def main() -> int:
     if "layers" in groups:
         extra.update(layer_measurements(fx, cc, rt, cus, engine))
     if "qmm" in groups:
-        extra.update(qmm_measurements(fx, cc, rt, cus))
+        extra.update(qmm_measurements(fx, cc, rt, cus, engine))
     if "aux" in groups:
         extra.update(aux_measurements(fx, cc, rt, cus, engine))
 
@@ -390,10 +391,11 @@ def layer_measurements(fx, cc, rt, cus, engine) -> dict:
     return out
 
 
-def qmm_measurements(fx, cc, rt, cus) -> dict:
+def qmm_measurements(fx, cc, rt, cus, engine) -> dict:
     """Qwen3.5-4B FFN (gate/up 2560->9216, down 9216->2560), affine u4 g64, M tokens per launch; cold rotation."""
     W, X, Y = 20, 21, 22
     c = rt.Context(act_dtype=rt.ACT_BF16)
+    c.set_matvec_engine(engine)
     lay = cc.Layout()
     one = 2 * 9216 * (1280 + 160) + 2560 * (4608 + 576)
     copies = math.ceil(COLD_BYTES / one)
