@@ -32,6 +32,7 @@
 // Tokens past the batch and rows past the matrix re-read the last valid one and are never stored;
 // pairs past the end of a row re-read the last pair under a zero scale.
 #pragma once
+#include <type_traits>
 #include "mm1_matvec.hpp"
 
 namespace smelt {
@@ -347,69 +348,87 @@ struct QsSwiglu {
     }
 
 // ---- token-tile form: prefill chunks ------------------------------------------------------------
-// The same arithmetic for many tokens.  A workgroup of four waves (two along the rows, two along
-// the tokens) owns 32 * RT weight rows times 32 * TB tokens and walks K one pair of scale groups
-// at a time.  Per step the 256 threads bring the tile's activations (in the operand order of the
-// codes), packed weights and (scale, bias - base * scale) pairs into one of two LDS buffers,
-// shared by the four waves, while the other buffer is multiplied; the global loads run two or four
-// steps ahead in registers.  Each wave unpacks a 16-row B operand once per step and group and
-// reuses it for its TB token blocks.
+// The same arithmetic for many tokens.  A workgroup of four waves (two along the rows, two along the
+// tokens) owns 32 * RT weight rows times 32 * TB tokens and walks K one pair of scale groups at a time.
+// Per step the threads bring the tile's activations (stored in the operand order of the codes), packed
+// weights and (scale, bias - base * scale) pairs into one of two LDS buffers, shared by the waves, while
+// the other buffer is multiplied; the global loads run two steps ahead in registers (buffer loads: a
+// uniform descriptor per tensor, a 32-bit offset per thread), the scales for four steps at a time
+// (16 bytes per row and tensor).  Each wave unpacks a 16-row B operand once per step and group and reuses
+// it for its TB token blocks.  With KW = 2 the workgroup has eight waves: the second four take the second
+// scale group of every step, and the two halves of K meet in LDS at the end; that halves the time of a
+// workgroup when the matrix has too few tiles to give every compute unit two.
 namespace smelt {
 
 constexpr int kQtThreads = 256;
-__host__ __device__ constexpr size_t qmt_buffer_bytes(int nmat, int rt, int tb) {
-    return (size_t)32 * tb * kQsXStride + (size_t)nmat * 32 * rt * kQsWStride + (size_t)nmat * 32 * rt * 2 * 8;
+// one buffer of a tile of bn rows (per matrix) times bm tokens
+__host__ __device__ constexpr size_t qmt_buffer_bytes(int nmat, int bn, int bm) {
+    return (size_t)bm * kQsXStride + (size_t)nmat * bn * kQsWStride + (size_t)nmat * bn * 2 * 8;
 }
-__host__ __device__ constexpr size_t qmt_lds_bytes(int nmat, int rt, int tb) { return 2 * qmt_buffer_bytes(nmat, rt, tb); }
+__host__ __device__ constexpr size_t qmt_lds_bytes(int nmat, int bn, int bm) { return 2 * qmt_buffer_bytes(nmat, bn, bm); }
 
-template <class ActT, class ScaleT, int NMAT, int RT, int TB, class Epi>
+template <class ActT, class ScaleT, int NMAT, int RT, int TB, int KW, class Epi>
 __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
                                          const uint16_t* const (&B)[NMAT], const uint16_t* __restrict__ X, int batch,
-                                         int rows, int cols, const Epi& epi) {
+                                         int rows, int cols, float* ws_partial, uint32_t* ws_counters, const Epi& epi) {
     using E = Elem16<ActT>;
     using O = QsOperand<ActT>;
+    static_assert(KW == 1 || KW == 2, "one or two waves along K");
     constexpr int BN = 32 * RT, BM = 32 * TB;           // rows (per matrix) and tokens of the workgroup tile
-    constexpr int XI = BM * 16 / kQtThreads;            // 16-byte activation loads per thread and step
+    constexpr int NT = kQtThreads * KW;                 // threads of the workgroup
+    constexpr int XI = BM * 16 / NT;                    // 16-byte activation loads per thread and step
     constexpr int WROWS = NMAT * BN;                    // staged weight rows
-    constexpr int WI = (WROWS * 4 + kQtThreads - 1) / kQtThreads;   // 16-byte weight loads per thread and step
-    static_assert(BM * 16 % kQtThreads == 0 && WROWS <= kQtThreads, "staging assignment");
+    constexpr int WI = (WROWS * 4 + NT - 1) / NT;       // 16-byte weight loads per thread and step
+    static_assert(BM * 16 % NT == 0 && WROWS <= NT, "staging assignment");
+    // a weight load of NT threads covers NT / 4 staged rows: all of one matrix
+    static_assert(NMAT == 1 || BN % (NT / 4) == 0 || WI == 1, "a weight load stays within one matrix, or there is only one");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    constexpr size_t kBuf = qmt_buffer_bytes(NMAT, RT, TB);
+    constexpr size_t kBuf = qmt_buffer_bytes(NMAT, BN, BM);
     constexpr size_t kOffW = (size_t)BM * kQsXStride, kOffS = kOffW + (size_t)WROWS * kQsWStride;   // within a buffer
-    constexpr int D = XI + WI <= 6 ? 4 : 2;            // steps in flight in registers
+    constexpr int D = 2;                                // steps in flight in registers
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-    const int wn = wave & 1, wm = wave >> 1;
+    const int wn = wave & 1, wm = (wave >> 1) & 1, wk = wave >> 2;
     const int n = lane & 15, q = lane >> 4;
-    const int gt = cols >> 6, npairs = gt >> 1, rs = cols >> 1;
+    const int gt = cols >> 6, rs = cols >> 1;
+    // gridDim.z workgroups share a tile: each takes a run of blocks of four steps (cols is a multiple of 512)
+    const int nblocks = gt >> 3, ksplit = gridDim.z, ks = blockIdx.z;
+    const int first_block = (int)((long)nblocks * ks / ksplit), end_block = (int)((long)nblocks * (ks + 1) / ksplit);
+    const int first_pair = 4 * first_block, npairs = 4 * end_block;   // this workgroup's steps: [first_pair, npairs)
     const int row0 = blockIdx.x * BN;
     const int m0 = blockIdx.y * BM;
     const int last_tok = (batch < m0 + BM ? batch : m0 + BM) - 1;
 
     // staging assignment: sixteen lanes per token row, four lanes per weight row, one thread per
     // staged row for the scales (staged row = (matrix * 2 + row half) * 16 RT + row in half)
-    const uint16_t* x_src[XI];
-    int x_dst[XI];
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(X), 0, 0xFFFFFFFF, 0x00027000);
+    __amdgpu_buffer_rsrc_t w_rsrc[NMAT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) w_rsrc[m] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(W[m]), 0, 0xFFFFFFFF, 0x00027000);
+    int x_off[XI], x_dst[XI];
 #pragma unroll
     for (int j = 0; j < XI; ++j) {
-        const int item = tid + kQtThreads * j, t = item >> 4, piece = item & 15;
+        const int item = tid + NT * j, t = item >> 4, piece = item & 15;
         int tok = m0 + t;
         if (tok > last_tok) tok = last_tok;
-        x_src[j] = X + (size_t)tok * cols + 8 * piece;
+        x_off[j] = (tok * cols + 8 * piece) * 2;
         x_dst[j] = t * kQsXStride + 16 * piece;
     }
-    const uint8_t* w_src[WI];
-    int w_dst[WI];
+    // a single weight load that spans both matrices takes its matrix from a pointer per thread
+    constexpr bool kSplitLoad = NMAT > 1 && BN % (NT / 4) != 0;
+    int w_off[WI], w_dst[WI];
+    const uint8_t* w_ptr = nullptr;
 #pragma unroll
     for (int j = 0; j < WI; ++j) {
-        int item = tid + kQtThreads * j;
+        int item = tid + NT * j;
         if (item > WROWS * 4 - 1) item = WROWS * 4 - 1;
         const int sr = item >> 2, piece = item & 3, m = sr / BN;
         int r = row0 + (sr - m * BN);
         if (r > rows - 1) r = rows - 1;
-        w_src[j] = (NMAT > 1 && m == 1 ? W[NMAT - 1] : W[0]) + (size_t)r * rs + 16 * piece;
+        w_off[j] = r * rs + 16 * piece;
         w_dst[j] = sr * kQsWStride + 16 * piece;
+        if (kSplitLoad) w_ptr = (m == 1 ? W[NMAT - 1] : W[0]) + w_off[j];
     }
     const uint16_t* s_src;
     const uint16_t* b_src;
@@ -424,21 +443,29 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
     }
     const int s_dst = tid < WROWS ? tid : WROWS - 1;
 
-    struct Step { uint4_t x[XI]; uint4_t w[WI]; uint32_t s, b; };
+    struct Step { uint4_t x[XI]; uint4_t w[WI]; };
+    struct Scales { uint4_t s, b; };   // eight groups (four steps) of one staged row
     auto issue = [&](Step& st, int pair) {
-        st.s = *reinterpret_cast<const uint32_t*>(s_src + 2 * pair);
-        st.b = *reinterpret_cast<const uint32_t*>(b_src + 2 * pair);
 #pragma unroll
-        for (int j = 0; j < XI; ++j) st.x[j] = *reinterpret_cast<const uint4_t*>(x_src[j] + 128 * pair);
+        for (int j = 0; j < XI; ++j) st.x[j] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_off[j], 256 * pair, 0);
 #pragma unroll
-        for (int j = 0; j < WI; ++j) st.w[j] = *reinterpret_cast<const uint4_t*>(w_src[j] + 64 * pair);
+        for (int j = 0; j < WI; ++j) {
+            constexpr int per = NT / 4;   // staged rows per load
+            const int m = NMAT == 1 || kSplitLoad ? 0 : ((per * j) / BN < NMAT ? (per * j) / BN : NMAT - 1);
+            if (kSplitLoad) st.w[j] = *reinterpret_cast<const uint4_t*>(w_ptr + 64 * pair);
+            else st.w[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc[m], w_off[j], 64 * pair, 0);
+        }
     };
-    auto stage = [&](const Step& st, unsigned char* buf) {
+    auto issue_scales = [&](Scales& sc, int block) {
+        sc.s = *reinterpret_cast<const uint4_t*>(s_src + 8 * block);
+        sc.b = *reinterpret_cast<const uint4_t*>(b_src + 8 * block);
+    };
+    auto stage = [&](const Step& st, uint32_t sp, uint32_t bp, unsigned char* buf) {
         float2* lds_sc = reinterpret_cast<float2*>(buf + kOffS);   // [staged row][2]
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const float s = ScaleT::widen((uint16_t)(e ? st.s >> 16 : st.s & 0xFFFFu));
-            const float b = ScaleT::widen((uint16_t)(e ? st.b >> 16 : st.b & 0xFFFFu));
+            const float s = ScaleT::widen((uint16_t)(e ? sp >> 16 : sp & 0xFFFFu));
+            const float b = ScaleT::widen((uint16_t)(e ? bp >> 16 : bp & 0xFFFFu));
             lds_sc[s_dst * 2 + e] = float2{s, __builtin_fmaf(-O::kBase, s, b)};
         }
 #pragma unroll
@@ -463,7 +490,8 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
     auto multiply = [&](const unsigned char* buf) {
         const float2* lds_sc = reinterpret_cast<const float2*>(buf + kOffS);
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
+        for (int ee = 0; ee < 2 / KW; ++ee) {
+            const int e = KW == 2 ? wk : ee;
             uint4_t a0[TB], a1[TB];
             float4_t xs[TB];
 #pragma unroll
@@ -494,26 +522,116 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
     };
 
     // Loads past the last pair repeat it (staged into the idle buffer, never multiplied), so that no
-    // load sits under a branch.
-    const int last_pair = npairs - 1;
+    // load sits under a branch.  `sc` holds the scales of the block of four steps being staged; it is
+    // reloaded as soon as the block's last step is staged, one step before its next use.
+    const int last_pair = npairs - 1, last_block = end_block - 1;
     Step st[D];
+    Scales sc;
+    issue_scales(sc, first_block);
 #pragma unroll
-    for (int d = 0; d < D; ++d) issue(st[d], d < last_pair ? d : last_pair);
-    stage(st[0], smem);
-    issue(st[0], D < last_pair ? D : last_pair);
+    for (int d = 0; d < D; ++d) issue(st[d], first_pair + d < last_pair ? first_pair + d : last_pair);
+    stage(st[0], sc.s.x, sc.b.x, smem);
+    issue(st[0], first_pair + D < last_pair ? first_pair + D : last_pair);
     __syncthreads();
-    for (int base = 0; base < npairs; base += D) {
+    for (int base = first_pair; base < npairs; base += 4) {
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
+        for (int d = 0; d < 4; ++d) {
             const int pair = base + d;
-            if (pair >= npairs) break;
             // the next step's tile goes into the other buffer (everyone left it at the last barrier)
-            stage(st[(d + 1) % D], smem + ((d + 1) & 1) * kBuf);
+            unsigned char* to = smem + ((d + 1) & 1) * kBuf;
+            if (d == 0) stage(st[(d + 1) % D], sc.s.y, sc.b.y, to);
+            if (d == 1) stage(st[(d + 1) % D], sc.s.z, sc.b.z, to);
+            if (d == 2) {
+                stage(st[(d + 1) % D], sc.s.w, sc.b.w, to);
+                const int block = (base >> 2) + 1;
+                issue_scales(sc, block < last_block ? block : last_block);
+            }
+            if (d == 3) stage(st[(d + 1) % D], sc.s.x, sc.b.x, to);
             issue(st[(d + 1) % D], pair + 1 + D < last_pair ? pair + 1 + D : last_pair);
             multiply(smem + (d & 1) * kBuf);
             __syncthreads();
         }
     }
+
+    constexpr int NV = NMAT * RT * TB * 4;   // accumulator values per lane
+    if constexpr (KW == 2) {
+        // the two halves of every step meet in LDS (all waves are past the last barrier of the loop):
+        // value j of lane l of wave pair p at [(p * NV + j) * 64 + l]
+        static_assert((size_t)4 * NV * kWave * sizeof(float) <= 2 * kBuf, "reduction fits the staging buffers");
+        float* red = reinterpret_cast<float*>(smem) + (size_t)(wave & 3) * NV * kWave + lane;
+        if (wk == 1) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int t = 0; t < RT; ++t)
+#pragma unroll
+                    for (int u = 0; u < TB; ++u) {
+                        float* at = red + (size_t)((m * RT + t) * TB + u) * 4 * kWave;
+                        at[0] = acc[m][t][u].x; at[kWave] = acc[m][t][u].y; at[2 * kWave] = acc[m][t][u].z; at[3 * kWave] = acc[m][t][u].w;
+                    }
+        }
+        __syncthreads();
+        if (wk == 0) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int t = 0; t < RT; ++t)
+#pragma unroll
+                    for (int u = 0; u < TB; ++u) {
+                        const float* at = red + (size_t)((m * RT + t) * TB + u) * 4 * kWave;
+                        acc[m][t][u].x += at[0]; acc[m][t][u].y += at[kWave]; acc[m][t][u].z += at[2 * kWave]; acc[m][t][u].w += at[3 * kWave];
+                    }
+        }
+    }
+    if (ksplit > 1) {
+        // Workgroup partials meet in the workspace; the last to arrive adds them in slice order, so the
+        // result does not depend on the order of arrival.  Partials are written and read with agent-scope
+        // relaxed atomics (coherent across the compute dies without cache write-backs), value j of thread t
+        // at [j * 256 + t].  A workgroup's stores are complete before its arrival is counted, and the last
+        // arrival reads only after its count returned.  The counter is left at zero for the next launch.
+        __shared__ uint32_t last_flag;
+        const size_t tile = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
+        float* mine = ws_partial + (tile * ksplit + ks) * NV * kQtThreads + tid;
+        if (wk == 0) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int t = 0; t < RT; ++t)
+#pragma unroll
+                    for (int u = 0; u < TB; ++u) {
+                        float* at = mine + (size_t)((m * RT + t) * TB + u) * 4 * kQtThreads;
+                        __hip_atomic_store(at, acc[m][t][u].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(at + kQtThreads, acc[m][t][u].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(at + 2 * kQtThreads, acc[m][t][u].z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(at + 3 * kQtThreads, acc[m][t][u].w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+        }
+        __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wave's stores are acknowledged
+        __syncthreads();
+        if (tid == 0) last_flag = atomicAdd(ws_counters + tile, 1u) == (uint32_t)(ksplit - 1) ? 1u : 0u;
+        __syncthreads();
+        if (!last_flag) return;
+        if (wk == 0) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int t = 0; t < RT; ++t)
+#pragma unroll
+                    for (int u = 0; u < TB; ++u) {
+                        float4_t sum = zero;
+                        for (int c = 0; c < ksplit; ++c) {
+                            const float* at = ws_partial + (tile * ksplit + c) * NV * kQtThreads + tid + (size_t)((m * RT + t) * TB + u) * 4 * kQtThreads;
+                            sum.x += __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            sum.y += __hip_atomic_load(at + kQtThreads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            sum.z += __hip_atomic_load(at + 2 * kQtThreads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            sum.w += __hip_atomic_load(at + 3 * kQtThreads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                        acc[m][t][u] = sum;
+                    }
+        }
+        if (tid == 0) ws_counters[tile] = 0u;
+    }
+    if (wk != 0) return;
 
     // lane (n, q) holds row n of tile t and tokens 4 q .. 4 q + 3 of block u
 #pragma unroll
@@ -539,41 +657,42 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
 
 }  // namespace smelt
 
-// Two waves per SIMD at least: that caps the kernel at 256 registers, all of them VGPRs, so the MFMA results land where
-// the fp32 FMAs read them (with the whole 512-register file on offer the compiler parks them in AGPRs and copies).
-#define SMELT_QMT_KERNEL extern "C" __global__ __launch_bounds__(256, 2)
+// Two workgroups per compute unit at least (the second launch-bound is in waves per SIMD): that caps the kernel at 256
+// (four waves) or 128 (eight waves) registers, all of them VGPRs, so the MFMA results land where the fp32 FMAs read them
+// (with the whole 512-register file on offer the compiler parks them in AGPRs and copies).
+#define SMELT_QMT_KERNEL(KWV) extern "C" __global__ __launch_bounds__(256 * KWV, 2 * KWV)
 
 // Argument lists of the token-slab qmm kernels of the same pipelines, plus the two workspace
-// pointers of the skinny ones (unused).
-#define SMELT_AFFINE_QMT_PLAIN(T, ACT, SC, RTV, TBV)                                               \
-    SMELT_QMT_KERNEL void smelt_affine_qmt_r##RTV##_t##TBV##_store_##T(                            \
+// pointers of the skinny ones (used when gridDim.z workgroups split K).
+#define SMELT_AFFINE_QMT_PLAIN(T, ACT, SC, RTV, TBV, KWV)                                          \
+    SMELT_QMT_KERNEL(KWV) void smelt_affine_qmt_r##RTV##_t##TBV##_k##KWV##_store_##T(              \
         const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* Y,    \
-        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {                        \
+        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t, uint32_t, float* WSP, uint32_t* WSC) { \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {W};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
         const uint16_t* const b[1] = {B};                                                          \
-        qmt_body<ACT, SC, 1, RTV, TBV>(w, s, b, X, batch, rows, cols, QsStore<ACT>{Y});            \
+        qmt_body<ACT, SC, 1, RTV, TBV, KWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsStore<ACT>{Y}); \
     }                                                                                              \
-    SMELT_QMT_KERNEL void smelt_affine_qmt_r##RTV##_t##TBV##_add_##T(                              \
+    SMELT_QMT_KERNEL(KWV) void smelt_affine_qmt_r##RTV##_t##TBV##_k##KWV##_add_##T(                \
         const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* MV,   \
         const uint16_t* RES, uint16_t* OUT, uint32_t batch, uint32_t rows, uint32_t cols,          \
-        uint32_t, uint32_t, float*, uint32_t*) {                                                                      \
+        uint32_t, uint32_t, float* WSP, uint32_t* WSC) {                                           \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {W};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
         const uint16_t* const b[1] = {B};                                                          \
-        qmt_body<ACT, SC, 1, RTV, TBV>(w, s, b, X, batch, rows, cols, QsAdd<ACT>{MV, RES, OUT});   \
+        qmt_body<ACT, SC, 1, RTV, TBV, KWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsAdd<ACT>{MV, RES, OUT}); \
     }
 
-#define SMELT_AFFINE_QMT_GATE_UP(T, ACT, SC, RTV, TBV)                                             \
-    SMELT_QMT_KERNEL void smelt_affine_qmt_r##RTV##_t##TBV##_gate_up_swiglu_##T(                   \
+#define SMELT_AFFINE_QMT_GATE_UP(T, ACT, SC, RTV, TBV, KWV)                                        \
+    SMELT_QMT_KERNEL(KWV) void smelt_affine_qmt_r##RTV##_t##TBV##_k##KWV##_gate_up_swiglu_##T(     \
         const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
         const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
-        uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {                                        \
+        uint32_t rows, uint32_t cols, uint32_t, uint32_t, float* WSP, uint32_t* WSC) {             \
         using namespace smelt;                                                                     \
         const uint8_t* const w[2] = {gW, uW};                                                      \
         const uint16_t* const s[2] = {gS, uS};                                                     \
         const uint16_t* const b[2] = {gB, uB};                                                     \
-        qmt_body<ACT, SC, 2, RTV, TBV>(w, s, b, X, batch, rows, cols, QsSwiglu<ACT>{Y});           \
+        qmt_body<ACT, SC, 2, RTV, TBV, KWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsSwiglu<ACT>{Y}); \
     }

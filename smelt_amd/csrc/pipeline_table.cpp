@@ -231,18 +231,40 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
 
 }  // namespace
 
-bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmtPlan* out) {
-    // Measured on MI355X at the 4B FFN shapes: up to 128 tokens the streaming kernel's 16-token
-    // passes are as fast or faster (the weights of the later passes come from cache); beyond, the
-    // shared activation tile wins.  64 rows x 64 tokens per workgroup keeps the 2560-row matrix on
-    // every compute unit; 128-token tiles measured no faster.
-    if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch <= 128) return false;
-    out->rt = nmat == 2 ? 1 : 2;
+bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
+              size_t lds_limit, QmtPlan* out) {
+    // Measured on MI355X at the 4B FFN shapes: below 128 tokens the streaming kernel's 16-token
+    // passes are as fast or faster (the weights of the later passes come from cache); from there on the
+    // shared activation tile wins (128 tokens: 22 against 27 us on 9216 x 2560, 29 against 38 on 2560 x 9216).
+    if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch < 128) return false;
+    // buffer loads address the activations and each weight matrix with 32-bit byte offsets
+    if ((uint64_t)batch * cols * 2 >= (1ull << 31) || (uint64_t)rows * (cols / 2) >= (1ull << 31)) return false;
+    // 96 rows x 64 tokens per workgroup and eight waves (two along K) measured best at 256 to 1024 tokens on
+    // the 9216 x 2560 and 2560 x 9216 matrices (48 / 63 us at 512 tokens against 57 / 77 with 64-row and 57 / 83
+    // with 128-row tiles of four waves); 64-row tiles when the 96-row ones would leave a quarter of the compute
+    // units without a workgroup (2560 rows at 256 tokens: 51 against 62 us).
+    const uint32_t token_blocks = (batch + 63) / 64;
     out->tb = 2;
-    // 128-row tiles once they still give every compute unit two workgroups (measured: 502 against 425 TFLOP/s at 1024
-    // tokens on the 9216-row matrix, equal at 256)
-    if (nmat == 1 && (uint64_t)((rows + 127) / 128) * ((batch + 63) / 64) >= 512) out->rt = 4;
-    out->lds = 2 * ((size_t)32 * out->tb * 272 + (size_t)nmat * 32 * out->rt * 72 + (size_t)nmat * 32 * out->rt * 16);   // two buffers
+    out->kw = 2;
+    if (nmat == 2) {
+        out->rt = 1;
+    } else {
+        const uint64_t tiles3 = (uint64_t)((rows + 95) / 96) * token_blocks;
+        out->rt = tiles3 * 4 >= (uint64_t)compute_units * 3 ? 3 : 2;
+    }
+    out->bn = 32 * out->rt;
+    out->bm = 32 * out->tb;
+    const uint64_t tiles = (uint64_t)((rows + out->bn - 1) / out->bn) * token_blocks;
+    // few tiles and long rows: workgroups share a tile along K so that every compute unit has about two, each
+    // with at least six blocks of 512 columns (2560 x 9216: 58 against 64 us at 512 tokens with two, 34 against
+    // 50 us at 256 tokens with three; splitting the 2560-column matrix only cost time)
+    out->ksplit = (uint32_t)((2ull * compute_units + tiles / 2) / tiles);
+    if (out->ksplit > cols / 512 / 6) out->ksplit = cols / 512 / 6;
+    if (out->ksplit < 1) out->ksplit = 1;
+    out->partial_bytes = out->ksplit > 1 ? (size_t)tiles * out->ksplit * nmat * out->rt * out->tb * 4 * 256 * sizeof(float) : 0;
+    out->counter_bytes = out->ksplit > 1 ? (size_t)tiles * sizeof(uint32_t) : 0;
+    // two buffers of: token rows, weight rows, scale pairs
+    out->lds = 2 * ((size_t)out->bm * 272 + (size_t)nmat * out->bn * 72 + (size_t)nmat * out->bn * 16);
     return out->lds <= lds_limit;
 }
 

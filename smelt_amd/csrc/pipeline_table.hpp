@@ -172,12 +172,16 @@ struct QmsPlan {
 };
 bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmsPlan* out);
 
-// Launch plan of the token-tile qmm: workgroups of four waves over 32 * rt rows (per matrix) and
+// Launch plan of the token-tile qmm: workgroups of 4 * kw waves over 32 * rt rows (per matrix) and
 // 32 * tb tokens.  False when the shape has no such kernel or too few tokens to pay for the tiles.
 struct QmtPlan {
-    uint32_t rt = 0, tb = 0;
+    uint32_t rt = 0, tb = 0, kw = 1;           // row tiles and token blocks per wave, waves along K
+    uint32_t bn = 0, bm = 0;                   // rows (per matrix) and tokens of a workgroup tile
+    uint32_t ksplit = 1;                       // workgroups that share a tile (grid z); above 1 they meet in the workspace
+    size_t partial_bytes = 0, counter_bytes = 0;   // workspace the split needs
     size_t lds = 0;
 };
-bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmtPlan* out);
+bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
+              size_t lds_limit, QmtPlan* out);
 
 }  // namespace smelt_host

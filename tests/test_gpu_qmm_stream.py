@@ -178,7 +178,7 @@ def test_stream_qmm_fused_add_and_gate_up(ctx, dtype):
     gh.check_outputs(y, ref, dtype, "stream gate_up_swiglu", rel_tol=8e-3 if dtype == fx.BF16 else 4e-3)
 
 
-# ---- token-tile form: more than 128 tokens; up to there, 16-token passes of the streaming kernel ------
+# ---- token-tile form: 128 tokens and more; below, 16-token passes of the streaming kernel ------
 
 def qmm_full(ctx, w, x_bits, dtype, rows, cols, bt=64):
     """A token-slab qmm record as the emitter writes it for prefill chunks (64-row slabs, bt-token grid rows)."""
@@ -198,7 +198,7 @@ def qmm_full(ctx, w, x_bits, dtype, rows, cols, bt=64):
 
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
-@pytest.mark.parametrize("batch", [49, 64, 100, 129, 300])
+@pytest.mark.parametrize("batch", [49, 64, 100, 127, 128, 129, 300])
 def test_tile_qmm_4b_shapes(ctx, dtype, batch):
     """Qwen3.5-4B-shaped slab (K=2560, 392 rows: ragged last row tile), ragged last token tile."""
     rows, cols = 392, 2560
@@ -210,10 +210,13 @@ def test_tile_qmm_4b_shapes(ctx, dtype, batch):
     print(f"\n  tile qmm M={batch} dtype={dtype} max rel err {worst:.2e}")
 
 
-@pytest.mark.parametrize("shape", [(200, 9216, 512), (8200, 1024, 96), (40, 512, 170), (2600, 2560, 520)])
+@pytest.mark.parametrize("shape", [(200, 9216, 512), (8200, 1024, 96), (40, 512, 170), (2600, 2560, 520), (2560, 9216, 256),
+                                   (1000, 6144, 200)])
 def test_tile_qmm_shapes(ctx, split_k, shape):
-    """Long rows at a 512-token chunk, many rows in several 16-token passes, a matrix smaller than
-    one tile, and ragged row and token tiles; against the oracle and the token-slab kernel."""
+    """Long rows at a 512-token chunk (three workgroups share each tile along K), many rows in several
+    16-token passes, a matrix smaller than one tile, ragged row and token tiles, the 4B down projection
+    at 256 tokens (64-row tiles, three-way split), a two-way split with uneven halves; against the oracle
+    and the token-slab kernel, and twice in a row (the split leaves its counters at zero)."""
     rows, cols, batch = shape
     dtype = fx.BF16
     w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=rows % 11)
