@@ -247,7 +247,10 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     out->tb = 2;
     out->kw = 2;
     if (nmat == 2) {
-        out->rt = 1;
+        // gate and up together (9216 x 2560 each): four waves; 64 rows of each matrix per workgroup once that
+        // leaves three workgroups per compute unit (105 against 110 us at 512 tokens), 32 below (60 against 63 at 256)
+        out->kw = 1;
+        out->rt = (uint64_t)((rows + 63) / 64) * token_blocks >= 3ull * compute_units ? 2 : 1;
     } else {
         const uint64_t tiles3 = (uint64_t)((rows + 95) / 96) * token_blocks;
         out->rt = tiles3 * 4 >= (uint64_t)compute_units * 3 ? 3 : 2;
