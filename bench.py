@@ -218,12 +218,26 @@ def main() -> int:
                 "bytes_per_launch": int(lm_bytes), "us_per_launch": lm_us, "us_per_launch_p95": rl["us_p95"],
                 "timed_launches": rl["timed_launches"], "rotation_bytes": int(lm_bytes * lm_copies), "cache_state": "cold"}
 
-    # One plain copy of known size: the calibration dispatch for HBM traffic counters (a counter
-    # run of this same command scales FETCH_SIZE / WRITE_SIZE of any kernel by what they read for
-    # this copy).
+    # What a plain read of the same bytes reaches on this part: a kernel that only loads each lm_head copy
+    # (16 bytes per lane, four loads in flight) over the same rotation.  Reported beside the roofline; the
+    # fraction above stays against the published peak.
     CAL_SRC, CAL_DST, cal_bytes = 8, 9, 256 << 20
     ctx.alloc(CAL_SRC, cal_bytes)
     ctx.alloc(CAL_DST, cal_bytes)
+    rd = ctx.pipeline("read_u128")
+    lm_span = lm_bytes // 16 * 16
+    reads = [rt.make_record(rd, [(W, 0, e.offset), (CAL_DST, 1, 0)], [(2, lm_span // 16)], (cus * 16, 1, 1), (256, 1, 1))
+             for e in lm_heads]
+    try:
+        rs = time_records(ctx, reads, rounds=rounds_for(len(reads)))
+        roofline["plain_read_same_bytes"] = {"us_per_launch": rs["us_median"], "GBps": round(lm_span / rs["us_median"] / 1e3, 1),
+                                             "lm_head_rate_over_it": round(rs["us_median"] / lm_us, 3)}
+    except rt.SmeltHipError as err:   # reported, never fatal for the headline
+        roofline["plain_read_same_bytes"] = {"error": err.message}
+
+    # One plain copy of known size: the calibration dispatch for HBM traffic counters (a counter
+    # run of this same command scales FETCH_SIZE / WRITE_SIZE of any kernel by what they read for
+    # this copy).
     cp = ctx.pipeline("copy_u128")
     cal = rt.make_record(cp, [(CAL_SRC, 0, 0), (CAL_DST, 1, 0)], [(2, cal_bytes // 16)], (cus * 16, 1, 1), (256, 1, 1))
     for _ in range(2):

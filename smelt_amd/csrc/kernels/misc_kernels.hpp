@@ -198,4 +198,26 @@ extern "C" __global__ __launch_bounds__(256) void smelt_copy_u128(const smelt::u
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
+
+// Plain device read of n16 16-byte elements (grid-stride, four loads in flight per thread): every
+// thread folds what it read into one element of dst (dst[global thread id], inside the first n16
+// elements).  What this kernel reaches on a buffer is what a weight-streaming kernel can hope for
+// on the same bytes.
+extern "C" __global__ __launch_bounds__(256) void smelt_read_u128(const smelt::uint4_t* __restrict__ src,
+                                                                  smelt::uint4_t* __restrict__ dst,
+                                                                  uint32_t n16) {
+    const uint32_t stride = gridDim.x * blockDim.x, first = blockIdx.x * blockDim.x + threadIdx.x;
+    smelt::uint4_t acc = {0u, 0u, 0u, 0u};
+    uint32_t i = first;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const smelt::uint4_t a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+        acc.x ^= a.x ^ b.x ^ c.x ^ d.x; acc.y ^= a.y ^ b.y ^ c.y ^ d.y;
+        acc.z ^= a.z ^ b.z ^ c.z ^ d.z; acc.w ^= a.w ^ b.w ^ c.w ^ d.w;
+    }
+    for (; i < n16; i += stride) {
+        const smelt::uint4_t a = src[i];
+        acc.x ^= a.x; acc.y ^= a.y; acc.z ^= a.z; acc.w ^= a.w;
+    }
+    if (first < n16) dst[first] = acc;
+}
 #endif
