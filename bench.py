@@ -390,21 +390,39 @@ def layer_measurements(fx, cc, rt, cus, engine) -> dict:
         per_layer = len(recs) // copies
         whole = time_records(c, recs, rounds=rounds_for(len(recs), 64))
         layer_us, layer_p95 = whole["us_median"] * per_layer, whole["us_p95"] * per_layer
+        # beside every class: one launch of a kernel that only reads the same weights (read_u128), over the
+        # same rotation: the time the memory system needs to hand a reader those bytes
+        def extent(es):
+            lo = min(e.offset for e in es)
+            hi = max(max(e.offset + e.size_bytes, e.scales_offset + e.scales_size_bytes,
+                         e.biases_offset + e.biases_size_bytes if wdtype is None else 0) for e in es)
+            return lo, (hi - lo) // 16
+        members = {"qkv": ("q", "k", "v"), "o": ("o",), "gate_up": ("gate", "up"), "down": ("down",)}
+        rd = c.pipeline("read_u128")
+        SINK = 26
+        c.alloc(SINK, max(extent([L[k] for k in ks])[1] for L in stack[:1] for ks in members.values()) * 16 + 4096)
         kernels = {}
         for cls, spans in classes.items():
             sel = [r for a, b in spans for r in recs[a:b]]
             per = len(sel) // copies
             t = time_records(c, sel, rounds=rounds_for(len(sel)))
             us = t["us_median"] * per
+            reads = []
+            for L in stack:
+                lo, n16 = extent([L[k] for k in members[cls]])
+                reads.append(rt.make_record(rd, [(W, 0, lo), (SINK, 1, 0)], [(2, n16)], (cus * 16, 1, 1), (256, 1, 1)))
+            tr = time_records(c, reads, rounds=rounds_for(len(reads)))
             kernels[cls] = {"launches": per, "weight_bytes": int(class_bytes[cls]), "us_median": round(us, 2),
                             "us_p95": round(t["us_p95"] * per, 2), "GBps": round(class_bytes[cls] / us / 1e3, 1),
                             "frac_of_hbm_peak": round(class_bytes[cls] / us / 1e3 / HBM_PEAK_GBS, 4),
-                            "timed_launches": t["timed_launches"]}
+                            "timed_launches": t["timed_launches"],
+                            "plain_read_us": round(tr["us_median"], 2), "rate_over_plain_read": round(tr["us_median"] / us, 3)}
         out[f"layer27b_{name}"] = {
             "us_per_layer": round(layer_us, 2), "us_per_layer_p95": round(layer_p95, 2), "weight_bytes": int(layer_bytes),
             "GBps": round(layer_bytes / layer_us / 1e3, 1), "frac_of_hbm_peak": round(layer_bytes / layer_us / 1e3 / HBM_PEAK_GBS, 4),
             "launches_per_layer": per_layer, "rotation_bytes": int(layer_bytes * copies), "cache_state": "cold",
-            "timed_launches": whole["timed_launches"], "kernels": kernels}
+            "timed_launches": whole["timed_launches"],
+            "plain_read_us_per_layer": round(sum(k["plain_read_us"] for k in kernels.values()), 2), "kernels": kernels}
         c.close()
     return out
 

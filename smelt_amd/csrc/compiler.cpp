@@ -1004,12 +1004,13 @@ int smelt_emit_bank_matvec(smelt_emitter* e, int weights_slot, const SmeltWeight
         e->records.push_back(rb.r);
         return SMELT_HIP_OK;
     }
-    if (family != SMELT_FAMILY_TERNARY2 && family != SMELT_FAMILY_BINARY1) return 1;  // banks exist for affine, binary and ternary members
+    if (family != SMELT_FAMILY_TERNARY2 && family != SMELT_FAMILY_BINARY1 && family != SMELT_FAMILY_TRIT5) return 1;  // banks exist for these
     for (int m = 0; m < count; ++m)
         if (int rc = check_signed_entry(e, &members[m])) return rc;
-    if (family == SMELT_FAMILY_BINARY1) {
-        // binary packed bank (C S x y0..y3 rows0..rows3 cols)
-        const MatvecGeometry g = matvec_geometry(signed_row_stride(kFmtBinary1, (uint32_t)first.cols), (int)rows, 4, e->compute_units);
+    if (family == SMELT_FAMILY_BINARY1 || family == SMELT_FAMILY_TRIT5) {
+        // binary packed bank (C S x y0..y3 rows0..rows3 cols); five-digit-byte rows take the same bindings
+        const bool trit5 = family == SMELT_FAMILY_TRIT5;
+        const MatvecGeometry g = matvec_geometry(signed_row_stride(trit5 ? kFmtTrit5 : kFmtBinary1, (uint32_t)first.cols), (int)rows, 4, e->compute_units);
         rb.buffer(0, weights_slot, first.offset);
         rb.buffer(1, weights_slot, first.scales_offset);
         rb.buffer(2, input);
@@ -1017,7 +1018,7 @@ int smelt_emit_bank_matvec(smelt_emitter* e, int weights_slot, const SmeltWeight
         for (int m = 0; m < 4; ++m) rb.constant((uint8_t)(7 + m), m < count ? (uint32_t)members[m].rows : 0u);
         rb.constant(11, (uint32_t)first.cols);
         rb.grid((uint32_t)g.grid_w, 1, 1, 256);
-        rb.r.pipeline = e->pipeline_index("signed_binary_packed_bank4_matvec_g128_rows8");
+        rb.r.pipeline = e->pipeline_index(trit5 ? "signed_trit5_packed_bank4_matvec_g128_rows8" : "signed_binary_packed_bank4_matvec_g128_rows8");
         e->records.push_back(rb.r);
         return SMELT_HIP_OK;
     }

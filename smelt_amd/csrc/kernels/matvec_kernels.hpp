@@ -604,6 +604,20 @@ using u32 = uint32_t;
 // Binary projection banks on the direct (fp16 activation) path, signed_quant.metal:2638-2935:
 //   packed bank   one code slab whose rows belong to 2 or 4 consumers in order
 //   dual/virtual  two separate matrices driven as one row space (rows of the first, then the second)
+// Five-digit-byte projection bank: the binary packed bank's argument list over trit5 rows (this format is
+// not in the reference; the bank is what lets q, k and v share one launch as they do for the other formats).
+#define SMELT_TRIT5_BANK_KERNELS(T, ACT)                                                          \
+    SMELT_KERNEL void smelt_signed_trit5_packed_bank4_matvec_##T(                                 \
+        const u8* C, const u16* S, const u16* X, u16* y0, u16* y1, u16* y2, u16* y3, u32 rows0,   \
+        u32 rows1, u32 rows2, u32 rows3, u32 cols) {                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        matvec_body<FmtTrit5, ACT, F16, 4, 1, 1>(mats, X, rows0 + rows1 + rows2 + rows3, cols,    \
+                                                 packed_row_stride<FmtTrit5>(cols, 128), 128, 0, 1, \
+                                                 epi);                                            \
+    }
+
 #define SMELT_BINARY_BANK_KERNELS(T, ACT)                                                         \
     SMELT_KERNEL void smelt_signed_binary_packed_bank_matvec_##T(                                 \
         const u8* C, const u16* S, const u16* X, u16* y0, u16* y1, u32 rows0, u32 rows1,          \

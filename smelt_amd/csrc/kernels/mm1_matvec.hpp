@@ -75,8 +75,12 @@ struct M1Codes {
     static constexpr int kFields = 32 / WIDTH;          // columns per dword
     static constexpr int kPairs = kFields / 2;
     static constexpr int kFPD = kPairs / 4;             // MFMAs (operand fragments) per dword
+    static constexpr int kDW = 4;                       // dwords of codes in one lane's 16 bytes
+    static constexpr bool kDecode = false;              // the 16 bytes are the codes themselves
     static constexpr int kFPL = 4 * kFPD;               // per 16-byte piece
     static constexpr int kPieceCols = 4 * kFields;      // columns of one lane's 16 bytes
+    // bytes of one packed row of a g128 format (rows are padded to whole groups)
+    static __host__ __device__ constexpr int row_stride(int cols) { return (cols + 127) / 128 * 128 * 4 / kFields; }
     static constexpr int kPasses = (kPairs + P::kPerPass - 1) / P::kPerPass;
     static __device__ __forceinline__ constexpr int mant_pos(int j) { return P::kMLo + WIDTH * (j % P::kPerPass); }
     // right shift (left when negative) that brings the codes of a pass to their mantissa positions
@@ -113,6 +117,34 @@ struct M1Ter2 : M1Codes<2, ActT> {
     static constexpr bool kHasBias = false;
     static constexpr float kSemMul = 1.0f, kOffset = 1.0f;
 };
+// The 243-entry decode table of the five-digit bytes (five 2-bit codes, digit i at bits 2i..2i+1; invalid
+// bytes decode to five semantic zeros), built at compile time.
+struct Trit5Lut {
+    uint16_t e[256];
+    constexpr Trit5Lut() : e() {
+        for (unsigned b = 0; b < 256; ++b) {
+            unsigned v = b, code = 0;
+            for (int i = 0; i < 5; ++i) { code |= (v % 3u) << (2 * i); v /= 3u; }
+            e[b] = b >= 243u ? 0x0155u : (uint16_t)code;
+        }
+    }
+};
+__device__ __constant__ constexpr Trit5Lut kTrit5Lut{};
+
+// trit5: the 16 bytes of a lane hold 80 base-3 digits, decoded through the 243-entry table into five
+// dwords of ternary2 codes.  A 128-byte row segment is 640 columns, five scale groups: a piece spans up
+// to two of them, and the kernel keeps the two apart (see the job).
+template <class ActT>
+struct M1Trit5 : M1Codes<2, ActT> {
+    using Base = M1Codes<2, ActT>;
+    static constexpr bool kHasBias = false;
+    static constexpr float kSemMul = 1.0f, kOffset = 1.0f;
+    static constexpr int kDW = 5;
+    static constexpr bool kDecode = true;
+    static constexpr int kFPL = 5 * Base::kFPD;
+    static constexpr int kPieceCols = 5 * Base::kFields;
+    static __host__ __device__ constexpr int row_stride(int cols) { return (((cols + 4) / 5) + 15) & ~15; }
+};
 template <class ActT>
 struct M1U4 : M1Codes<4, ActT> {
     static constexpr bool kHasBias = true;
@@ -124,12 +156,13 @@ struct M1U4 : M1Codes<4, ActT> {
 //             folded-out constant and the plain sum of x (8 B), then one piece of zero fragments;
 //   then the scale rows (and bias rows) of the workgroup's eight rows, one block per matrix and
 //   plane; then the waves' partial sums [wave][matrix][8] (fp32).
-__host__ __device__ constexpr size_t mm1_wave_lds_bytes(int frags_per_piece, int nl) {
-    return (size_t)nl * 8 * frags_per_piece * 16 + (size_t)nl * 8 * 8 + (size_t)frags_per_piece * 16;
+//   (five-dword pieces: per dword the folded-out constant, 4 B; and a 512-byte decode table at the end)
+__host__ __device__ constexpr size_t mm1_wave_lds_bytes(int frags_per_piece, int nl, int dw = 4) {
+    return (size_t)nl * 8 * frags_per_piece * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) + (size_t)frags_per_piece * 16;
 }
-__host__ __device__ constexpr size_t mm1_lds_bytes(int frags_per_piece, int nl, int waves, int nmat, int gpr, bool has_bias) {
-    return (size_t)waves * mm1_wave_lds_bytes(frags_per_piece, nl) + (size_t)nmat * (has_bias ? 2 : 1) * 8 * gpr * 2 +
-           (size_t)waves * nmat * 32;
+__host__ __device__ constexpr size_t mm1_lds_bytes(int frags_per_piece, int nl, int waves, int nmat, int gpr, bool has_bias, int dw = 4) {
+    return (size_t)waves * mm1_wave_lds_bytes(frags_per_piece, nl, dw) + (size_t)nmat * (has_bias ? 2 : 1) * 8 * gpr * 2 +
+           (size_t)waves * nmat * 32 + (dw == 4 ? 0 : 512);
 }
 
 __device__ __forceinline__ float quad_sum(float v) {
@@ -143,11 +176,14 @@ template <class F, class ActT, class ScaleT, int NMAT, int NL, class Epi>
 __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint16_t* __restrict__ x_all, int rows,
                                          int cols, int row_stride, int group, const Epi& epi) {
     using E = Elem16<ActT>;
-    constexpr int FPD = F::kFPD, FPL = F::kFPL, FIELDS = F::kFields, PAIRS = F::kPairs;
-    constexpr int NITEMS = NL * 32;                        // staging items of a wave: 8 pieces x 4 dwords per segment
+    constexpr int FPD = F::kFPD, FPL = F::kFPL, FIELDS = F::kFields, PAIRS = F::kPairs, DW = F::kDW;
+    constexpr int NITEMS = NL * 8 * DW;                    // staging items of a wave: 8 pieces x DW dwords per segment
     constexpr int ITEMS = (NITEMS + kWave - 1) / kWave;    // per lane
     constexpr int PLANES = F::kHasBias ? 2 : 1;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
+    // five-digit bytes: the 512-byte decode table sits at the start of LDS (a lookup address is the byte
+    // value times two), everything else behind it
+    unsigned char* const smem = smem_all + (F::kDecode ? 512 : 0);
     const int lane = threadIdx.x & (kWave - 1);
     const int chunk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int kc = blockDim.x / kWave;
@@ -188,16 +224,22 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // ---- 2. this wave's slice of x ---------------------------------------------------------------
     // One item = the columns of one packed dword; item it = 4 * (piece within the run) + dword.
     uint32_t xe[ITEMS][FIELDS / 2];
+    int item_piece[ITEMS], item_dword[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         int it = lane + k * kWave;
         if (it > NITEMS - 1) it = NITEMS - 1;
-        int col0 = (piece0 + (it >> 2)) * F::kPieceCols + (it & 3) * FIELDS;
+        item_piece[k] = DW == 4 ? it >> 2 : (it * 52429) >> 18;   // it / 5 for it < 2^14
+        item_dword[k] = it - DW * item_piece[k];
+        int col0 = (piece0 + item_piece[k]) * F::kPieceCols + item_dword[k] * FIELDS;
+        // a dword past the end of the row (five-dword pieces end inside a piece) multiplies zeros
+        const bool past = DW != 4 && col0 > cols - FIELDS;
         if (col0 > cols - FIELDS) col0 = cols - FIELDS;   // cols is a multiple of kFields
 #pragma unroll
         for (int v = 0; v < FIELDS / 8; ++v) {
             const uint4_t t = *reinterpret_cast<const uint4_t*>(x + col0 + 8 * v);
-            xe[k][4 * v] = t.x; xe[k][4 * v + 1] = t.y; xe[k][4 * v + 2] = t.z; xe[k][4 * v + 3] = t.w;
+            xe[k][4 * v] = past ? 0u : t.x; xe[k][4 * v + 1] = past ? 0u : t.y;
+            xe[k][4 * v + 2] = past ? 0u : t.z; xe[k][4 * v + 3] = past ? 0u : t.w;
         }
     }
     // ---- 3. every weight load of the job -------------------------------------------------------------
@@ -220,7 +262,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     }
 
     // ---- 4. scales into LDS ----------------------------------------------------------------------------
-    const size_t wave_bytes = mm1_wave_lds_bytes(FPL, NL);
+    const size_t wave_bytes = mm1_wave_lds_bytes(FPL, NL, DW);
     uint4_t* lds_scales = reinterpret_cast<uint4_t*>(smem + (size_t)kc * wave_bytes);
 #pragma unroll
     for (int m = 0; m < NMAT; ++m)
@@ -237,16 +279,20 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // 2v, 2v+1 of fragment t = columns 4t+v, 4t+v+kPairs).  The four items of a 16-byte piece sit
     // in the four lanes of a quad, which add up their sum(base * x) and sum(x).
     uint4_t* wfrag = reinterpret_cast<uint4_t*>(smem + (size_t)chunk * wave_bytes);
-    float* wsum = reinterpret_cast<float*>(wfrag + (size_t)NL * 8 * FPL);   // [piece][2]: constant, sum x
-    uint4_t* wzero = reinterpret_cast<uint4_t*>(wsum + NL * 16);            // FPL zero fragments
+    float* wsum = reinterpret_cast<float*>(wfrag + (size_t)NL * 8 * FPL);   // [piece][2]: constant, sum x ([piece][DW]: constants)
+    uint4_t* wzero = reinterpret_cast<uint4_t*>(wsum + (DW == 4 ? NL * 16 : NL * 8 * DW));   // FPL zero fragments
+    // decode table of the five-digit bytes, copied from constant memory; visible after the barrier below
+    uint16_t* lut = reinterpret_cast<uint16_t*>(smem_all);
+    if constexpr (F::kDecode) {
+        for (uint32_t i = threadIdx.x; i < 128; i += blockDim.x)
+            reinterpret_cast<uint32_t*>(lut)[i] = reinterpret_cast<const uint32_t*>(kTrit5Lut.e)[i];
+    }
     if (lane < FPL) wzero[lane] = uint4_t{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         // lanes past the last item hold the last item again (whole quads of them: d == 3) and store
         // the same fragments again
-        int it = lane + k * kWave;
-        if (it > NITEMS - 1) it = NITEMS - 1;
-        const int pl = it >> 2, d = it & 3;
+        const int pl = item_piece[k], d = item_dword[k], it = pl * DW + d;
         float cb = 0.0f, xs = 0.0f;
         constexpr uint32_t kOnes = F::both((uint32_t)E::kExpBias << E::kMant);   // (1.0, 1.0)
         uint32_t fr[PAIRS];
@@ -257,21 +303,38 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             cb = E::dot2k(fr[j], F::base_pair(j), cb);
             xs = E::dot2k(fr[j], kOnes, xs);
         }
-        cb = quad_sum(cb);
-        xs = quad_sum(xs);
+        if constexpr (DW == 4) {
+            cb = quad_sum(cb);
+            xs = quad_sum(xs);
+        }
 #pragma unroll
         for (int t = 0; t < FPD; ++t)
             wfrag[(size_t)pl * FPL + d * FPD + t] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
-        if (d == 0) *reinterpret_cast<float2*>(wsum + 2 * pl) = float2{__builtin_fmaf(F::kOffset, xs, cb), xs};
+        if constexpr (DW == 4) {
+            if (d == 0) *reinterpret_cast<float2*>(wsum + 2 * pl) = float2{__builtin_fmaf(F::kOffset, xs, cb), xs};
+        } else {
+            wsum[it] = __builtin_fmaf(F::kOffset, xs, cb);   // one constant per dword: the job adds them per scale group
+        }
     }
     __syncthreads();   // scales of every wave, fragments of this one
 
     // ---- 6. the job --------------------------------------------------------------------------------
     // A-operand lanes 20q and 20q + 1 (token slots 4q and 4q + 1 in k-block q: the two halves of
-    // the segment) read fragments; the other fifty-six read the zero fragments, so no lane is
-    // masked off.
-    const int a_half = n - 4 * q;
-    const bool a_live = a_half == 0 || a_half == 1;
+    // the segment) read fragments; the others read the zero fragments, so no lane is masked off.
+    // Five-dword pieces span up to two scale groups (a segment is five groups, eight pieces of five
+    // dwords: piece p starts at dword 5p of forty, a group is eight dwords): the dwords of a piece's
+    // second group go to token slots 4q + 2 and 4q + 3 instead, i.e. for those dwords A lanes 20q + 2
+    // and 20q + 3 are the ones that read fragments.
+    const int a_slot = n - 4 * q;                       // 0..3 for the lanes that ever read fragments
+    const bool a_valid = DW == 4 ? (a_slot == 0 || a_slot == 1) : (a_slot >= 0 && a_slot < 4);
+    const int a_half = a_slot & 1, a_second = a_slot >> 1;
+    const int a_piece = 4 * a_half + q;                 // piece of the segment this lane feeds
+    auto first_group_dwords = [](int piece_in_segment) {
+        if (DW == 4) return 4;
+        const int left = 8 - ((5 * piece_in_segment) & 7);
+        return left < 5 ? left : 5;
+    };
+    const int a_split = first_group_dwords(a_piece);
     const uint16_t* lds_s16 = reinterpret_cast<const uint16_t*>(lds_scales);
     float y[NMAT];
 #pragma unroll
@@ -281,35 +344,70 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         float4_t acc[NMAT];
 #pragma unroll
         for (int m = 0; m < NMAT; ++m) acc[m] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        const uint4_t* pf = a_live ? wfrag + (size_t)(i * 8 + 4 * a_half + q) * FPL : wzero;
+        // the codes of this segment: as loaded, or decoded here (in load order, before the transpose)
+        uint32_t cd[NMAT][DW];
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
+        for (int m = 0; m < NMAT; ++m) {
+            if constexpr (F::kDecode) {
+                FmtTrit5::decode(codes[m][i], lut, cd[m]);
+            } else {
+                cd[m][0] = codes[m][i].x; cd[m][1] = codes[m][i].y; cd[m][2] = codes[m][i].z; cd[m][3] = codes[m][i].w;
+            }
+        }
+        const uint4_t* piece_frags = wfrag + (size_t)(i * 8 + a_piece) * FPL;
+#pragma unroll
+        for (int d = 0; d < DW; ++d) {
+            const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
+            const uint4_t* pf = a_live ? piece_frags + d * FPD : wzero;
             uint4_t afr[FPD];
 #pragma unroll
-            for (int f = 0; f < FPD; ++f) afr[f] = pf[d * FPD + f];
+            for (int f = 0; f < FPD; ++f) afr[f] = pf[f];
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) {
-                const uint4_t lw = codes[m][i];
-                const uint32_t cw = (uint32_t)__builtin_amdgcn_ds_bpermute(xpose, (int)(d == 0 ? lw.x : (d == 1 ? lw.y : (d == 2 ? lw.z : lw.w))));
+                const uint32_t cw = (uint32_t)__builtin_amdgcn_ds_bpermute(xpose, (int)cd[m][d]);
                 uint4_t ops[FPD];
                 F::operands(cw, ops);
 #pragma unroll
                 for (int f = 0; f < FPD; ++f) acc[m] = E::mfma(afr[f], ops[f], acc[m]);
             }
         }
-        const float2 cs = *reinterpret_cast<const float2*>(wsum + 2 * (i * 8 + 4 * hh + q));
         const int piece = piece0 + i * 8 + 4 * hh + q;
         const bool piece_ok = piece < pieces;
         const int g = ((piece_ok ? piece : pieces - 1) * F::kPieceCols) >> gshift;
+        if constexpr (DW == 4) {
+            const float2 cs = *reinterpret_cast<const float2*>(wsum + 2 * (i * 8 + 4 * hh + q));
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m) {
-            const int sidx = (m * PLANES) * (8 * gpr) + rn * gpr + g;
-            const float sv = F::kSemMul * ScaleT::widen(lds_s16[sidx]);
-            const float dotp = hh ? acc[m].y : acc[m].x;   // token slot 4q + hh
-            y[m] = __builtin_fmaf(piece_ok ? sv : 0.0f, dotp - cs.x, y[m]);
-            if (F::kHasBias) {
-                const float bv = ScaleT::widen(lds_s16[sidx + 8 * gpr]);
-                y[m] = __builtin_fmaf(piece_ok ? bv : 0.0f, cs.y, y[m]);
+            for (int m = 0; m < NMAT; ++m) {
+                const int sidx = (m * PLANES) * (8 * gpr) + rn * gpr + g;
+                const float sv = F::kSemMul * ScaleT::widen(lds_s16[sidx]);
+                const float dotp = hh ? acc[m].y : acc[m].x;   // token slot 4q + hh
+                y[m] = __builtin_fmaf(piece_ok ? sv : 0.0f, dotp - cs.x, y[m]);
+                if (F::kHasBias) {
+                    const float bv = ScaleT::widen(lds_s16[sidx + 8 * gpr]);
+                    y[m] = __builtin_fmaf(piece_ok ? bv : 0.0f, cs.y, y[m]);
+                }
+            }
+        } else {
+            // the folded-out constants of the piece's dwords, per scale group
+            const int split = first_group_dwords(4 * hh + q);
+            const float* cdw = wsum + (i * 8 + 4 * hh + q) * DW;
+            float c_first = 0.0f, c_second = 0.0f;
+#pragma unroll
+            for (int d = 0; d < DW; ++d) {
+                const float c = cdw[d];
+                c_first += d < split ? c : 0.0f;
+                c_second += d < split ? 0.0f : c;
+            }
+            const int g2 = g + 1 < gpr ? g + 1 : gpr - 1;   // unused (its sums are zero) when the piece has one group
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                const int srow = (m * PLANES) * (8 * gpr) + rn * gpr;
+                const float s1 = F::kSemMul * ScaleT::widen(lds_s16[srow + g]);
+                const float s2 = F::kSemMul * ScaleT::widen(lds_s16[srow + g2]);
+                const float d1 = hh ? acc[m].y : acc[m].x;   // token slot 4q + hh: first group
+                const float d2 = hh ? acc[m].w : acc[m].z;   // token slot 4q + 2 + hh: second group
+                y[m] = __builtin_fmaf(piece_ok ? s1 : 0.0f, d1 - c_first, y[m]);
+                y[m] = __builtin_fmaf(piece_ok ? s2 : 0.0f, d2 - c_second, y[m]);
             }
         }
     }
@@ -358,7 +456,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
         EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
         mm1_body<F, ACT, F16, 1, NLV>(mats, X, rows, cols,                                   \
-                                           (cols + 127) / 128 * 128 * 4 / F::kFields, 128, epi);  \
+                                           F::row_stride((int)cols), 128, epi);  \
     }                                                                                             \
     SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_matvec_add_##T(              \
         const u8* C, const u16* S, const u16* X, u16* Y, const u16* res, u32 rows, u32 cols) {    \
@@ -367,7 +465,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
         EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
         mm1_body<F, ACT, F16, 1, NLV>(mats, X, rows, cols,                                   \
-                                           (cols + 127) / 128 * 128 * 4 / F::kFields, 128, epi);  \
+                                           F::row_stride((int)cols), 128, epi);  \
     }                                                                                             \
     SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_gate_up_swiglu_##T(          \
         const u8* gC, const u16* gS, const u8* uC, const u16* uS, const u16* X, u16* Y, u32 rows, \
@@ -377,7 +475,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
         EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
         mm1_body<F, ACT, F16, 2, NLV>(mats, X, rows, cols,                                   \
-                                           (cols + 127) / 128 * 128 * 4 / F::kFields, 128, epi);  \
+                                           F::row_stride((int)cols), 128, epi);  \
     }
 
 // Affine 4-bit: argument lists of the vector-ALU kernels of the same pipelines.
@@ -471,4 +569,17 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
         mm1_body<M1Bin<ACT>, ACT, F16, 1, NLV>(mats, X, rows0 + rows1 + rows2 + rows3, cols,      \
                                                cols / 8, 128, epi);                               \
+    }
+
+
+#define SMELT_TRIT5_MM1_BANK(T, ACT, NLV)                                                         \
+    SMELT_MM1_KERNEL void smelt_signed_trit5_mm1_nl##NLV##_packed_bank4_matvec_##T(               \
+        const u8* C, const u16* S, const u16* X, u16* y0, u16* y1, u16* y2, u16* y3, u32 rows0,   \
+        u32 rows1, u32 rows2, u32 rows3, u32 cols) {                                              \
+        using namespace smelt;                                                                    \
+        using F = M1Trit5<ACT>;                                                                   \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
+        mm1_body<F, ACT, F16, 1, NLV>(mats, X, rows0 + rows1 + rows2 + rows3, cols,               \
+                                      F::row_stride((int)cols), 128, epi);                        \
     }

@@ -18,3 +18,10 @@
 
 SMELT_MM1_EVERY_NL(f16, smelt::F16)
 SMELT_MM1_EVERY_NL(bf16, smelt::BF16)
+
+#define SMELT_MM1_TRIT5(T, ACT)                                                                   \
+    SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 1) SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 2) \
+    SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 3)                                    \
+    SMELT_TRIT5_MM1_BANK(T, ACT, 1) SMELT_TRIT5_MM1_BANK(T, ACT, 2) SMELT_TRIT5_MM1_BANK(T, ACT, 3)
+SMELT_MM1_TRIT5(f16, smelt::F16)
+SMELT_MM1_TRIT5(bf16, smelt::BF16)

@@ -13,3 +13,5 @@ SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, f16, smelt::F16)
 SMELT_SIGNED_KERNELS(trit5, smelt::FmtTrit5, bf16, smelt::BF16)
 SMELT_BINARY_BANK_KERNELS(f16, smelt::F16)
 SMELT_BINARY_BANK_KERNELS(bf16, smelt::BF16)
+SMELT_TRIT5_BANK_KERNELS(f16, smelt::F16)
+SMELT_TRIT5_BANK_KERNELS(bf16, smelt::BF16)

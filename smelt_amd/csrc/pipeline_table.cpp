@@ -149,22 +149,25 @@ uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
 
 bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
               bool force, Mm1Plan* out) {
-    uint32_t row_stride, frags, nl_max;
+    uint32_t row_stride, frags, nl_max, dw = 4;
     switch (layout) {
         case kCodesU4: row_stride = cols / 2; frags = 4; nl_max = 6; break;
         case kCodesTernary2: row_stride = (cols + 127u) / 128u * 32u; frags = 8; nl_max = 3; break;
         case kCodesBinary1: row_stride = (cols + 127u) / 128u * 16u; frags = 16; nl_max = 3; break;
+        // five digits per byte: a 16-byte piece is five dwords of sixteen columns, a 128-byte segment five groups
+        case kCodesTrit5: if (cols % 16 != 0) return false; row_stride = (((cols + 4u) / 5u) + 15u) & ~15u; frags = 10; nl_max = 3; dw = 5; break;
         default: return false;
     }
     if (rows == 0 || cols == 0 || row_stride % 16 != 0 || group < 32 || (group & (group - 1))) return false;
     if (layout != kCodesU4 && group != 128) return false;
     // small matrices are launch-bound either way and stay where they are tuned
-    if (!force && (uint64_t)rows * cols < (8u << 20)) return false;
+    // (five-digit bytes: the vector kernel decodes through the same table at twice the cost, so the bar is lower)
+    if (!force && (uint64_t)rows * cols < (layout == kCodesTrit5 ? (2u << 20) : (8u << 20))) return false;
     const uint32_t pieces = row_stride / 16, nseg = (pieces + 7) / 8, gpr = (cols + group - 1) / group;
     const uint32_t planes = layout == kCodesU4 ? 2 : 1;
     auto lds_of = [&](uint32_t kc, uint32_t nl) {
-        const size_t wave = (size_t)nl * 8 * frags * 16 + (size_t)nl * 8 * 8 + (size_t)frags * 16;
-        return kc * wave + (size_t)nmat * planes * 8 * gpr * 2 + (size_t)kc * nmat * 32;
+        const size_t wave = (size_t)nl * 8 * frags * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) + (size_t)frags * 16;
+        return kc * wave + (size_t)nmat * planes * 8 * gpr * 2 + (size_t)kc * nmat * 32 + (dw == 4 ? 0 : 512);   // + decode table
     };
     Mm1Plan best;
     uint32_t best_waste = ~0u;
@@ -201,6 +204,10 @@ void attach_mm1(ResolvedPipeline* r) {
         {"smelt_signed_ternary_matvec_", "smelt_signed_ternary_mm1_", "matvec_", kCodesTernary2, 1},
         {"smelt_signed_ternary_matvec_add_", "smelt_signed_ternary_mm1_", "matvec_add_", kCodesTernary2, 1},
         {"smelt_signed_ternary_gate_up_swiglu_", "smelt_signed_ternary_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},
+        {"smelt_signed_trit5_matvec_", "smelt_signed_trit5_mm1_", "matvec_", kCodesTrit5, 1},
+        {"smelt_signed_trit5_matvec_add_", "smelt_signed_trit5_mm1_", "matvec_add_", kCodesTrit5, 1},
+        {"smelt_signed_trit5_gate_up_swiglu_", "smelt_signed_trit5_mm1_", "gate_up_swiglu_", kCodesTrit5, 2},
+        {"smelt_signed_trit5_packed_bank4_matvec_", "smelt_signed_trit5_mm1_", "packed_bank4_matvec_", kCodesTrit5, 1},
         {"smelt_teraff_matvec_", "smelt_teraff_mm1_", "matvec_", kCodesTernary2, 1},
         {"smelt_teraff_matvec_add_", "smelt_teraff_mm1_", "matvec_add_", kCodesTernary2, 1},
         {"smelt_teraff_gate_up_swiglu_", "smelt_teraff_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},
@@ -801,6 +808,9 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
     }
     if (entry == "signed_binary_packed_bank4_matvec_g128_rows8") {
         out->family = kFamBinaryPackedBank4; out->format = kFmtBinary1; out->symbol = "smelt_signed_binary_packed_bank4_matvec_" + t; out->kinds = "PPPPPPPUUUUU"; return kResolveOk;
+    }
+    if (entry == "signed_trit5_packed_bank4_matvec_g128_rows8") {   // same bindings over five-digit-byte rows
+        out->family = kFamBinaryPackedBank4; out->format = kFmtTrit5; out->symbol = "smelt_signed_trit5_packed_bank4_matvec_" + t; out->kinds = "PPPPPPPUUUUU"; return kResolveOk;
     }
     if (entry == "signed_binary_dual_matvec_g128_rows8" || entry == "signed_binary_virtual_bank_matvec_g128_rows8") {
         out->family = kFamBinaryTwoMatrix; out->format = kFmtBinary1; out->symbol = "smelt_signed_binary_two_matrix_matvec_" + t; out->kinds = "PPPPPPPUUU"; return kResolveOk;

@@ -200,8 +200,8 @@ def test_affine_projection_bank_equals_independent_matvecs():
 @pytest.mark.parametrize("fmt,wdtype", [(fx.BINARY1, cc.BINARY1), (fx.TERNARY2, cc.TERNARY2), (fx.TRIT5, cc.TRIT5)])
 def test_signed_projection_bank(fmt, wdtype, engine):
     """q|k|v of a signed format laid out as one bank: contiguous code and scale slabs, one dispatch
-    for binary and ternary members (no bank kernel exists for trit5: the emitter says so and the
-    members run one by one); every member against the oracle, on both matvec engines."""
+    (binary, ternary and five-digit-byte members alike); every member against the oracle, on both
+    matvec engines."""
     hidden = 1280
     member_rows = [520, 136, 128]
     lay = cc.Layout()
@@ -224,7 +224,7 @@ def test_signed_projection_bank(fmt, wdtype, engine):
         em = cc.Emitter(rt.ACT_BF16)
         outs = [cc.bind(2, 0), cc.bind(2, 520 * 2), cc.bind(2, 656 * 2)]
         banked = em.bank_matvec(0, members, cc.bind(1), outs)
-        assert banked == (fmt != fx.TRIT5)
+        assert banked
         if not banked:
             for e, o in zip(members, outs):
                 em.matvec(0, e, cc.bind(1), o)

@@ -60,14 +60,28 @@ def test_affine_matrix_core_exact_on_dyadic_fixture(ctx):
 SIGNED_SHAPES = [(5, 128), (8, 256), (50, 1152), (1024, 5120), (264, 17408), (77, 9216)]
 
 
+def pack_signed(codes, fmt, garbage_padding=False):
+    """Packed rows at the stride the kernels expect (trit5: five digits per byte, rows padded to 16 bytes).
+    With garbage_padding the trit5 bytes past the last column's byte hold arbitrary valid digit bytes."""
+    if fmt != fx.TRIT5:
+        return fx.pack_signed_np(codes, fmt)
+    cols = codes.shape[1]
+    stride = (((cols + 4) // 5) + 15) // 16 * 16
+    packed = fx.pack_signed_np(codes, fmt, stride)
+    used = (cols + 4) // 5
+    if garbage_padding and used < stride:
+        packed[:, used:] = fx.rng_for(3, cols).integers(0, 243, (codes.shape[0], stride - used), dtype=np.uint8)
+    return packed
+
+
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
-@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")])
+@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary"), (fx.TRIT5, "trit5")])
 @pytest.mark.parametrize("shape", SIGNED_SHAPES)
 def test_signed_matrix_core_matvec(ctx, fmt, name, dtype, shape):
     rows, cols = shape
     codes = fx.synth_signed_codes(fmt, rows, cols, config=2 + fmt, tensor=rows % 7)
     scales = fx.synth_signed_scales(rows, cols, config=2 + fmt, tensor=rows % 7)
-    packed = fx.pack_signed_np(codes, fmt)
+    packed = pack_signed(codes, fmt, garbage_padding=True)
     x = fx.synth_activation(1, cols, dtype, config=2 + fmt)
     ref = so.signed_matvec(fmt, packed, scales, fx.from_bits(x, dtype), rows, cols, cols, 128)
     y = run_signed(ctx, name, packed, scales, x, dtype, rows, cols)
@@ -89,7 +103,7 @@ def test_ternary_matrix_core_reproduces_mlx_golden_bits(ctx):
             assert np.array_equal(y[0], want[b]), (key, b)
 
 
-@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")])
+@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary"), (fx.TRIT5, "trit5")])
 def test_signed_matrix_core_fused_forms_equal_staged(ctx, fmt, name):
     rows, cols = 100, 2560
     dtype = fx.BF16
@@ -97,7 +111,7 @@ def test_signed_matrix_core_fused_forms_equal_staged(ctx, fmt, name):
     uc = fx.synth_signed_codes(fmt, rows, cols, tensor=2)
     gs = fx.synth_signed_scales(rows, cols, tensor=1)
     us = fx.synth_signed_scales(rows, cols, tensor=2)
-    gp, up = fx.pack_signed_np(gc, fmt), fx.pack_signed_np(uc, fmt)
+    gp, up = pack_signed(gc, fmt), pack_signed(uc, fmt)
     x = fx.synth_activation(1, cols, dtype, config=2)
     g = run_signed(ctx, name, gp, gs, x, dtype, rows, cols)
     u = run_signed(ctx, name, up, us, x, dtype, rows, cols)
