@@ -39,6 +39,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X published dense bf16 / fp16 matrix rate
 COLD_BYTES = 3 * (256 << 20)  # distinct weight bytes a cold rotation has to span
 MIN_TIMED_LAUNCHES = 200
+PLAIN_READ = True     # time read_u128 over the same bytes beside the kernels (--no-plain-read clears it)
 
 
 def synth_affine(rng, rows, cols, group, bf16):
@@ -82,6 +83,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip every side measurement")
+    ap.add_argument("--no-plain-read", action="store_true",
+                    help="skip the plain-read reference launches (profiler runs: fewer graph replays, and the "
+                         "read_u128 dispatches stay out of the per-kernel tables)")
     ap.add_argument("--only", choices=("step", "layers", "qmm", "aux"), default=None,
                     help="the step plus one group of side measurements (layers: 27B-layer matvecs per weight format; "
                          "qmm: 4B FFN token tiles; aux: config-0 cold/warm, cold step, quantiser, turbo_quant_h)")
@@ -99,6 +103,8 @@ def main() -> int:
     from smelt_amd import runtime as rt
 
     engine = {"auto": rt.MATVEC_AUTO, "matrix": rt.MATVEC_MATRIX_CORE, "vector": rt.MATVEC_VECTOR}[args.engine]
+    global PLAIN_READ
+    PLAIN_READ = not args.no_plain_read
     ctx = rt.Context(act_dtype=rt.ACT_BF16)
     ctx.set_matvec_engine(engine)
     info = ctx.device_info()
@@ -229,6 +235,8 @@ def main() -> int:
     reads = [rt.make_record(rd, [(W, 0, e.offset), (CAL_DST, 1, 0)], [(2, lm_span // 16)], (cus * 16, 1, 1), (256, 1, 1))
              for e in lm_heads]
     try:
+        if not PLAIN_READ:
+            raise rt.SmeltHipError(0, "skipped (--no-plain-read)")
         rs = time_records(ctx, reads, rounds=rounds_for(len(reads)))
         roofline["plain_read_same_bytes"] = {"us_per_launch": rs["us_median"], "GBps": round(lm_span / rs["us_median"] / 1e3, 1),
                                              "lm_head_rate_over_it": round(rs["us_median"] / lm_us, 3)}
@@ -411,18 +419,20 @@ def layer_measurements(fx, cc, rt, cus, engine) -> dict:
             for L in stack:
                 lo, n16 = extent([L[k] for k in members[cls]])
                 reads.append(rt.make_record(rd, [(W, 0, lo), (SINK, 1, 0)], [(2, n16)], (cus * 16, 1, 1), (256, 1, 1)))
-            tr = time_records(c, reads, rounds=rounds_for(len(reads)))
+            tr = time_records(c, reads, rounds=rounds_for(len(reads))) if PLAIN_READ else None
             kernels[cls] = {"launches": per, "weight_bytes": int(class_bytes[cls]), "us_median": round(us, 2),
                             "us_p95": round(t["us_p95"] * per, 2), "GBps": round(class_bytes[cls] / us / 1e3, 1),
                             "frac_of_hbm_peak": round(class_bytes[cls] / us / 1e3 / HBM_PEAK_GBS, 4),
                             "timed_launches": t["timed_launches"],
-                            "plain_read_us": round(tr["us_median"], 2), "rate_over_plain_read": round(tr["us_median"] / us, 3)}
+                            "plain_read_us": round(tr["us_median"], 2) if tr else None,
+                            "rate_over_plain_read": round(tr["us_median"] / us, 3) if tr else None}
         out[f"layer27b_{name}"] = {
             "us_per_layer": round(layer_us, 2), "us_per_layer_p95": round(layer_p95, 2), "weight_bytes": int(layer_bytes),
             "GBps": round(layer_bytes / layer_us / 1e3, 1), "frac_of_hbm_peak": round(layer_bytes / layer_us / 1e3 / HBM_PEAK_GBS, 4),
             "launches_per_layer": per_layer, "rotation_bytes": int(layer_bytes * copies), "cache_state": "cold",
             "timed_launches": whole["timed_launches"],
-            "plain_read_us_per_layer": round(sum(k["plain_read_us"] for k in kernels.values()), 2), "kernels": kernels}
+            "plain_read_us_per_layer": round(sum(k["plain_read_us"] for k in kernels.values()), 2) if PLAIN_READ else None,
+            "kernels": kernels}
         c.close()
     return out
 
