@@ -126,10 +126,12 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * 8M weights and more take the single-pass matrix-core kernel of the same pipeline, smaller ones
  * the vector-ALU kernel; MATRIX_CORE drops the size threshold (every shape the matrix-core kernel
  * can express takes it); VECTOR keeps every record on the vector-ALU kernels.  The same switch
- * covers the skinny qmm records (up to 32 tokens per pass): AUTO and MATRIX_CORE run the streaming
- * kernel of the pipeline (K split inside a workgroup, no workspace), VECTOR the split-K kernel the
- * record's geometry describes (partial sums in the workspace).  Results of the alternatives differ
- * in summation order only.  No counterpart in the reference (one kernel per pipeline name there);
+ * covers the qmm records: AUTO and MATRIX_CORE run the streaming kernel of the pipeline below 128
+ * tokens (K split inside a workgroup, no workspace) and the token-tile kernel from 128 tokens on
+ * (matrices with few tiles and long rows split K across workgroups: partial sums in the
+ * workspace, added in a fixed order), VECTOR the split-K or token-slab kernel the record's geometry
+ * describes (split-K: partial sums in the workspace).  Results of the alternatives differ in
+ * summation order only.  No counterpart in the reference (one kernel per pipeline name there);
  * meant for A/B measurement and for tests. */
 enum { SMELT_HIP_MATVEC_AUTO = 0, SMELT_HIP_MATVEC_MATRIX_CORE = 1, SMELT_HIP_MATVEC_VECTOR = 2 };
 int smelt_hip_set_matvec_engine(smelt_hip_context *ctx, int engine);
@@ -186,11 +188,13 @@ int smelt_hip_encode_prefill_record(smelt_hip_context *ctx, const SmeltDispatchR
 /* No counterpart in the reference.  For callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the same as
  * smelt_hip_encode_prefill_record, except that kernels which split K across workgroups (the
- * "_batched_skinny" qmm pipelines) keep their partial sums and arrival counters in a file-scope
- * device array of the library instead of the workspace a context allocates, and the call itself
- * allocates and frees nothing.  A record whose partials need more than
- * SMELT_HIP_STATIC_SCRATCH_BYTES (4 KB per workgroup and matrix) or more than 16384 row tiles is
- * rejected with SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY.  Each GPU holds one copy of the array for the
+ * "_batched_skinny" qmm pipelines under the VECTOR engine, the token-tile qmm otherwise) keep their
+ * partial sums and arrival counters in a file-scope device array of the library instead of the
+ * workspace a context allocates, and the call itself allocates and frees nothing.  A
+ * "_batched_skinny" record whose partials need more than SMELT_HIP_STATIC_SCRATCH_BYTES (4 KB per
+ * workgroup and matrix) or more than 16384 row tiles is rejected with
+ * SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY; the token-tile kernel does not split K when its partials do
+ * not fit.  Each GPU holds one copy of the array for the
  * life of the process, shared by every context on it: calls that overlap on one GPU (two streams)
  * race; calls on one stream are ordered. */
 #define SMELT_HIP_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
