@@ -1,6 +1,7 @@
 """GPU parity of the allocation-free entry point: smelt_hip_encode_prefill_record_static_scratch
 against smelt_hip_encode_prefill_record on the split-K skinny qmm, bit for bit, on two calls in a
-row (the second with a smaller input), plus the size limit."""
+row (the second with a smaller input), plus the size limit; and on a token-slab record whose tiles
+the token-tile kernel splits along K (its partial sums then live in the same static array)."""
 import numpy as np
 import pytest
 
@@ -74,5 +75,38 @@ def test_static_scratch_rejects_partials_beyond_its_size():
         y = _run(ctx, ctx.encode_prefill, offs, x, rows, cols, ksplit, name, 1)
         ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
         gh.check_outputs(y, ref, dtype, "allocated workspace takes the larger record")
+    finally:
+        ctx.close()
+
+
+def test_static_scratch_holds_the_token_tile_kernels_partials():
+    """200 x 9216 at 300 and then 140 tokens: few tiles and long rows, so three workgroups share each
+    tile along K; their partials go to the static array in one call and to the context's workspace in
+    the other, and the results are the same bits."""
+    dtype = fx.BF16
+    ctx = rt.Context()
+    try:
+        rows, cols = 200, 9216
+        w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=34)
+        wf = gh.WeightFile()
+        offs = [wf.add(a) for a in w]
+        ctx.upload_weights(0, wf.image())
+        pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g64_batched_full_b64@bf16")
+        for batch in (300, 140):
+            x = fx.synth_activation(batch, cols, dtype, config=4, tensor=200 + batch)
+            ctx.put(gh.X_SLOT, x)
+            ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+            bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+            rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], ((rows + 63) // 64, 64, 1), (256, 1, 1),
+                                 grid_kinds=(0, rt.GRID_SEQ_LEN_CEIL_DIV, 0))
+            outs = []
+            for encode in (ctx.encode_prefill, ctx.encode_prefill_static_scratch, ctx.encode_prefill_static_scratch):
+                print(f"\n  token-tile split case batch={batch} via {encode.__name__}", flush=True)
+                assert encode(rec, seq_len=batch) == 1
+                ctx.wait()
+                outs.append(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows))
+            assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[2])
+            ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype, threads=True)
+            gh.check_outputs(outs[1], ref, dtype, f"static-scratch token-tile qmm M={batch}")
     finally:
         ctx.close()
