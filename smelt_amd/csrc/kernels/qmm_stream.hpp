@@ -367,14 +367,19 @@ __host__ __device__ constexpr size_t qmt_buffer_bytes(int nmat, int bn, int bm) 
 }
 __host__ __device__ constexpr size_t qmt_lds_bytes(int nmat, int bn, int bm) { return 2 * qmt_buffer_bytes(nmat, bn, bm); }
 
-template <class ActT, class ScaleT, int NMAT, int RT, int TB, int KW, class Epi>
+template <class ActT, class ScaleT, int NMAT, int RT, int TB, int KW, bool PERWAVE, class Epi>
 __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
                                          const uint16_t* const (&B)[NMAT], const uint16_t* __restrict__ X, int batch,
                                          int rows, int cols, float* ws_partial, uint32_t* ws_counters, const Epi& epi) {
     using E = Elem16<ActT>;
     using O = QsOperand<ActT>;
     static_assert(KW == 1 || KW == 2, "one or two waves along K");
-    constexpr int BN = 32 * RT, BM = 32 * TB;           // rows (per matrix) and tokens of the workgroup tile
+    // PERWAVE (two matrices): the two waves along the rows take one matrix each (RT row tiles of it) instead
+    // of half the rows of both, so a wave's loop is that of the one-matrix kernel; gate and up of an element
+    // meet in LDS at the end.
+    static_assert(!PERWAVE || NMAT == 2, "one matrix per wave is for gate and up");
+    constexpr int AM = PERWAVE ? 1 : NMAT;              // matrices a wave accumulates
+    constexpr int BN = (PERWAVE ? 16 : 32) * RT, BM = 32 * TB;   // rows (per matrix) and tokens of the workgroup tile
     constexpr int NT = kQtThreads * KW;                 // threads of the workgroup
     constexpr int XI = BM * 16 / NT;                    // 16-byte activation loads per thread and step
     constexpr int WROWS = NMAT * BN;                    // staged weight rows
@@ -479,9 +484,9 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
 
     const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
     const uint4_t ones = {O::kOnePair, O::kOnePair, O::kOnePair, O::kOnePair};
-    float4_t acc[NMAT][RT][TB];
+    float4_t acc[AM][RT][TB];
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m)
+    for (int m = 0; m < AM; ++m)
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
@@ -502,10 +507,10 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
                 xs[u] = E::mfma(a1[u], ones, E::mfma(a0[u], ones, zero));
             }
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m)
+            for (int m = 0; m < AM; ++m)
 #pragma unroll
                 for (int t = 0; t < RT; ++t) {
-                    const int sr = ((m * 2 + wn) * RT + t) * 16 + n;
+                    const int sr = PERWAVE ? (wn * RT + t) * 16 + n : ((m * 2 + wn) * RT + t) * 16 + n;
                     const uint2_t c = *reinterpret_cast<const uint2_t*>(buf + kOffW + sr * kQsWStride + 32 * e + 8 * q);
                     const uint4_t b0 = O::codes(c.x), b1 = O::codes(c.y);
                     const float2 sb = lds_sc[sr * 2 + e];
@@ -553,7 +558,7 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         }
     }
 
-    constexpr int NV = NMAT * RT * TB * 4;   // accumulator values per lane
+    constexpr int NV = AM * RT * TB * 4;   // accumulator values per lane
     if constexpr (KW == 2) {
         // the two halves of every step meet in LDS (all waves are past the last barrier of the loop):
         // value j of lane l of wave pair p at [(p * NV + j) * 64 + l]
@@ -561,7 +566,7 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         float* red = reinterpret_cast<float*>(smem) + (size_t)(wave & 3) * NV * kWave + lane;
         if (wk == 1) {
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m)
+            for (int m = 0; m < AM; ++m)
 #pragma unroll
                 for (int t = 0; t < RT; ++t)
 #pragma unroll
@@ -573,7 +578,7 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         __syncthreads();
         if (wk == 0) {
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m)
+            for (int m = 0; m < AM; ++m)
 #pragma unroll
                 for (int t = 0; t < RT; ++t)
 #pragma unroll
@@ -594,7 +599,7 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         float* mine = ws_partial + (tile * ksplit + ks) * NV * kQtThreads + tid;
         if (wk == 0) {
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m)
+            for (int m = 0; m < AM; ++m)
 #pragma unroll
                 for (int t = 0; t < RT; ++t)
 #pragma unroll
@@ -613,7 +618,7 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         if (!last_flag) return;
         if (wk == 0) {
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m)
+            for (int m = 0; m < AM; ++m)
 #pragma unroll
                 for (int t = 0; t < RT; ++t)
 #pragma unroll
@@ -633,6 +638,44 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
     }
     if (wk != 0) return;
 
+    if constexpr (PERWAVE) {
+        // the waves that hold up hand their sums to the waves that hold gate of the same elements:
+        // value j of lane l of token half wm at [(wm * NV + j) * 64 + l]
+        static_assert((size_t)2 * NV * kWave * sizeof(float) <= 2 * kBuf, "the exchange fits the staging buffers");
+        float* xch = reinterpret_cast<float*>(smem) + (size_t)wm * NV * kWave + lane;
+        asm volatile("s_barrier" ::: "memory");   // the four waves that are left: everyone is done with LDS
+        if (wn == 1) {
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int u = 0; u < TB; ++u) {
+                    float* at = xch + (size_t)(t * TB + u) * 4 * kWave;
+                    at[0] = acc[0][t][u].x; at[kWave] = acc[0][t][u].y; at[2 * kWave] = acc[0][t][u].z; at[3 * kWave] = acc[0][t][u].w;
+                }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (wn == 1) return;
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            const int r = row0 + t * 16 + n;
+            if (r < rows) {
+#pragma unroll
+                for (int u = 0; u < TB; ++u) {
+                    const float* at = xch + (size_t)(t * TB + u) * 4 * kWave;
+                    const float up[4] = {at[0], at[kWave], at[2 * kWave], at[3 * kWave]};
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int tok = m0 + (wm * TB + u) * 16 + 4 * q + v;
+                        if (tok <= last_tok) {
+                            const float val[2] = {v == 0 ? acc[0][t][u].x : (v == 1 ? acc[0][t][u].y : (v == 2 ? acc[0][t][u].z : acc[0][t][u].w)), up[v]};
+                            epi((size_t)tok * rows + r, val);
+                        }
+                    }
+                }
+            }
+        }
+        return;
+    } else {
     // lane (n, q) holds row n of tile t and tokens 4 q .. 4 q + 3 of block u
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
@@ -653,6 +696,7 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
                 }
         }
     }
+    }
 }
 
 }  // namespace smelt
@@ -672,7 +716,7 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         const uint8_t* const w[1] = {W};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
         const uint16_t* const b[1] = {B};                                                          \
-        qmt_body<ACT, SC, 1, RTV, TBV, KWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsStore<ACT>{Y}); \
+        qmt_body<ACT, SC, 1, RTV, TBV, KWV, false>(w, s, b, X, batch, rows, cols, WSP, WSC, QsStore<ACT>{Y}); \
     }                                                                                              \
     SMELT_QMT_KERNEL(KWV) void smelt_affine_qmt_r##RTV##_t##TBV##_k##KWV##_add_##T(                \
         const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* MV,   \
@@ -682,11 +726,11 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         const uint8_t* const w[1] = {W};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
         const uint16_t* const b[1] = {B};                                                          \
-        qmt_body<ACT, SC, 1, RTV, TBV, KWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsAdd<ACT>{MV, RES, OUT}); \
+        qmt_body<ACT, SC, 1, RTV, TBV, KWV, false>(w, s, b, X, batch, rows, cols, WSP, WSC, QsAdd<ACT>{MV, RES, OUT}); \
     }
 
-#define SMELT_AFFINE_QMT_GATE_UP(T, ACT, SC, RTV, TBV, KWV)                                        \
-    SMELT_QMT_KERNEL(KWV) void smelt_affine_qmt_r##RTV##_t##TBV##_k##KWV##_gate_up_swiglu_##T(     \
+#define SMELT_AFFINE_QMT_GATE_UP(T, ACT, SC, RTV, TBV, KWV, PWV, TAG)                                        \
+    SMELT_QMT_KERNEL(KWV) void smelt_affine_qmt_##TAG##RTV##_t##TBV##_k##KWV##_gate_up_swiglu_##T(     \
         const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
         const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
         uint32_t rows, uint32_t cols, uint32_t, uint32_t, float* WSP, uint32_t* WSC) {             \
@@ -694,5 +738,5 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         const uint8_t* const w[2] = {gW, uW};                                                      \
         const uint16_t* const s[2] = {gS, uS};                                                     \
         const uint16_t* const b[2] = {gB, uB};                                                     \
-        qmt_body<ACT, SC, 2, RTV, TBV, KWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsSwiglu<ACT>{Y}); \
+        qmt_body<ACT, SC, 2, RTV, TBV, KWV, PWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsSwiglu<ACT>{Y}); \
     }

@@ -253,16 +253,19 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     const uint32_t token_blocks = (batch + 63) / 64;
     out->tb = 2;
     out->kw = 2;
+    out->per_wave = false;
     if (nmat == 2) {
-        // gate and up together (9216 x 2560 each): four waves; 64 rows of each matrix per workgroup once that
-        // leaves three workgroups per compute unit (105 against 110 us at 512 tokens), 32 below (60 against 63 at 256)
-        out->kw = 1;
-        out->rt = (uint64_t)((rows + 63) / 64) * token_blocks >= 3ull * compute_units ? 2 : 1;
+        // gate and up together (9216 x 2560 each): 64 rows of each matrix per workgroup of four waves once that
+        // leaves three workgroups per compute unit (104 us at 512 tokens, 170 at 1024); below, the two waves along
+        // the rows take one matrix each, 48 rows of it, eight waves: the loop of the one-matrix kernel (54 us at
+        // 256 tokens against 61; 106 / 185 at 512 / 1024)
+        if ((uint64_t)((rows + 63) / 64) * token_blocks >= 3ull * compute_units) { out->rt = 2; out->kw = 1; }
+        else { out->per_wave = true; out->rt = 3; }
     } else {
         const uint64_t tiles3 = (uint64_t)((rows + 95) / 96) * token_blocks;
         out->rt = tiles3 * 4 >= (uint64_t)compute_units * 3 ? 3 : 2;
     }
-    out->bn = 32 * out->rt;
+    out->bn = (out->per_wave ? 16 : 32) * out->rt;
     out->bm = 32 * out->tb;
     const uint64_t tiles = (uint64_t)((rows + out->bn - 1) / out->bn) * token_blocks;
     // few tiles and long rows: workgroups share a tile along K so that every compute unit has about two, each
@@ -271,7 +274,7 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     out->ksplit = (uint32_t)((2ull * compute_units + tiles / 2) / tiles);
     if (out->ksplit > cols / 512 / 6) out->ksplit = cols / 512 / 6;
     if (out->ksplit < 1) out->ksplit = 1;
-    out->partial_bytes = out->ksplit > 1 ? (size_t)tiles * out->ksplit * nmat * out->rt * out->tb * 4 * 256 * sizeof(float) : 0;
+    out->partial_bytes = out->ksplit > 1 ? (size_t)tiles * out->ksplit * (out->per_wave ? 1 : nmat) * out->rt * out->tb * 4 * 256 * sizeof(float) : 0;
     out->counter_bytes = out->ksplit > 1 ? (size_t)tiles * sizeof(uint32_t) : 0;
     // two buffers of: token rows, weight rows, scale pairs
     out->lds = 2 * ((size_t)out->bm * 272 + (size_t)nmat * out->bn * 72 + (size_t)nmat * out->bn * 16);

@@ -176,6 +176,7 @@ bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
 // 32 * tb tokens.  False when the shape has no such kernel or too few tokens to pay for the tiles.
 struct QmtPlan {
     uint32_t rt = 0, tb = 0, kw = 1;           // row tiles and token blocks per wave, waves along K
+    bool per_wave = false;                     // two matrices: one per wave along the rows (16 * rt rows of each per workgroup)
     uint32_t bn = 0, bm = 0;                   // rows (per matrix) and tokens of a workgroup tile
     uint32_t ksplit = 1;                       // workgroups that share a tile (grid z); above 1 they meet in the workspace
     size_t partial_bytes = 0, counter_bytes = 0;   // workspace the split needs

@@ -46,6 +46,7 @@ struct Pipeline {
     hipFunction_t fn_mm_stream = nullptr, fn_mm_split = nullptr;  // matrix-core variants picked by shape
     hipFunction_t fn_mm1[kMm1MaxSegments + 1] = {};               // single-pass matrix-core matvec, by segments per wave
     hipFunction_t fn_qmt[5][5][3] = {};                           // token-tile qmm, by row tiles and token blocks per wave and waves along K
+    hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
     ResolvedPipeline res;
 };
@@ -1111,8 +1112,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         const size_t o = p->res.family == kFamAffineQmm ? 5 : (p->res.family == kFamAffineQmmAdd ? 7 : 8);
         const uint32_t batch = L.args[o].value, rows = L.args[o + 1].value, cols = L.args[o + 2].value, group = L.args[o + 3].value;
         QmtPlan tplan;
-        if (qmt_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &tplan) && p->fn_qmt[tplan.rt][tplan.tb][tplan.kw]) {
-            fn = p->fn_qmt[tplan.rt][tplan.tb][tplan.kw];
+        if (qmt_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &tplan) && (tplan.per_wave ? p->fn_qmt_per_wave : p->fn_qmt)[tplan.rt][tplan.tb][tplan.kw]) {
+            fn = (tplan.per_wave ? p->fn_qmt_per_wave : p->fn_qmt)[tplan.rt][tplan.tb][tplan.kw];
             // a split that the workspace of this call cannot hold is not taken
             const uint32_t ksplit = tplan.partial_bytes <= ws.partial_bytes && tplan.counter_bytes <= ws.counter_bytes ? tplan.ksplit : 1;
             L.grid[0] = (rows + tplan.bn - 1) / tplan.bn; L.grid[1] = (batch + tplan.bm - 1) / tplan.bm; L.grid[2] = ksplit;
@@ -1362,7 +1363,11 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
                 for (uint32_t rt = 1; rt <= 4; ++rt)
                     for (uint32_t tb = 2; tb <= 4; tb += 2)
                         for (uint32_t kw = 1; kw <= 2; ++kw)
-                            (void)find(&p.fn_qmt[rt][tb][kw], "smelt_affine_qmt_r" + std::to_string(rt) + "_t" + std::to_string(tb) + "_k" + std::to_string(kw) + "_" + p.res.qms_tail);
+                        {
+                            const std::string rest = std::to_string(rt) + "_t" + std::to_string(tb) + "_k" + std::to_string(kw) + "_" + p.res.qms_tail;
+                            (void)find(&p.fn_qmt[rt][tb][kw], "smelt_affine_qmt_r" + rest);
+                            (void)find(&p.fn_qmt_per_wave[rt][tb][kw], "smelt_affine_qmt_w" + rest);
+                        }
             if (!p.res.qms_tail.empty())
                 for (uint32_t rt = 1; rt <= kQmsMaxRowTiles; ++rt)
                     for (uint32_t wide = 0; wide < 2; ++wide)

@@ -274,3 +274,30 @@ def test_tile_qmm_fused_add_and_gate_up(ctx, dtype):
     sd = so.BF16 if dtype == fx.BF16 else so.F16
     ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, sd), dtype)
     gh.check_outputs(y, ref, dtype, "tile gate_up_swiglu", rel_tol=8e-3 if dtype == fx.BF16 else 4e-3)
+
+
+def test_tile_qmm_gate_up_on_a_grid_that_fills_the_machine(ctx):
+    """6144 rows at 512 tokens: enough 64-row tiles for three workgroups per compute unit, which is where
+    the gate+up record takes the four-wave kernel with both matrices in every wave (the smaller grids of
+    the test above take the one-matrix-per-wave kernel)."""
+    dtype = fx.BF16
+    rows, cols, batch = 6144, 512, 512
+    gw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=13)
+    uw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=14)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=18)
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*gw, *uw)]
+    ctx.upload_weights(0, wf.image())
+    ctx.put(gh.X_SLOT, x)
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+    pipe = ctx.pipeline(f"fused_affine_gate_up_swiglu_c{cols}_r{rows}_g64_batched_full_b64@bf16")
+    bufs = [(0, i, offs[i]) for i in range(6)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
+    rec = rt.make_record(pipe, bufs, [(8, batch)], ((rows + 63) // 64, (batch + 63) // 64, 1), (256, 1, 1))
+    assert ctx.encode_prefill(rec, seq_len=batch) == 1
+    ctx.wait()
+    y = ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+    xf = fx.from_bits(x, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, 64, dtype, threads=True)
+    u = so.affine_matvec(*uw, xf, rows, cols, 64, dtype, threads=True)
+    ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, so.BF16), dtype)
+    gh.check_outputs(y, ref, dtype, "tile gate_up_swiglu, full grid", rel_tol=8e-3)
