@@ -479,9 +479,22 @@ def qmm_measurements(fx, cc, rt, cus, engine) -> dict:
                          "frac_of_mfma_peak": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4), "weight_GBps": round(layer_bytes / us / 1e3, 1),
                          "frac_of_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "timed_launches": t["timed_launches"],
                          "pipeline": em.pipelines[0]}
+    # what a reader gets for the same three launches: read_u128 over each matrix of the same rotating copies
+    plain = None
+    if PLAIN_READ:
+        SINK = 23
+        c.alloc(SINK, max(e.size_bytes + e.scales_size_bytes + e.biases_size_bytes for e in ents[0]) + 4096)
+        rd = c.pipeline("read_u128")
+        reads = [rt.make_record(rd, [(W, 0, e.offset), (SINK, 1, 0)],
+                                [(2, (e.biases_offset + e.biases_size_bytes - e.offset) // 16)], (cus * 16, 1, 1), (256, 1, 1))
+                 for layer in ents for e in layer]
+        tr = time_records(c, reads, rounds=rounds_for(len(reads)))
+        plain = round(tr["us_median"] * 3, 2)
+        for v in qmm.values():
+            v["rate_over_plain_read"] = round(plain / v["us_per_ffn"], 3)
     c.close()
     return {"qwen35_4b_ffn_qmm": {"cache_state": "cold", "rotation_bytes": int(layer_bytes * copies),
-                                  "weight_bytes_per_ffn": int(layer_bytes), **qmm}}
+                                  "weight_bytes_per_ffn": int(layer_bytes), "plain_read_us_per_ffn": plain, **qmm}}
 
 
 def aux_measurements(fx, cc, rt, cus, engine) -> dict:
