@@ -242,6 +242,26 @@ def main() -> int:
                                              "lm_head_rate_over_it": round(rs["us_median"] / lm_us, 3)}
     except rt.SmeltHipError as err:   # reported, never fatal for the headline
         roofline["plain_read_same_bytes"] = {"error": err.message}
+    # ... and of the whole step: one read launch per matvec launch (the bank, o, gate+up, down of every layer,
+    # the lm_head), same order, same graph form
+    step_read = None
+    if PLAIN_READ:
+        def extent(es):
+            lo = min(e.offset for e in es)
+            hi = max(e.biases_offset + e.biases_size_bytes for e in es)
+            return lo, (hi - lo) // 16
+        spans = []
+        for L in sets[0]:
+            spans += [extent([L["q"], L["k"], L["v"]]), extent([L["o"]]), extent([L["gate"], L["up"]]), extent([L["down"]])]
+        spans.append(extent([lm_heads[0]]))
+        step_reads = [rt.make_record(rd, [(W, 0, lo), (CAL_DST, 1, 0)], [(2, n16)], (cus * 16, 1, 1), (256, 1, 1)) for lo, n16 in spans]
+        g2, n2 = ctx.capture_decode(ctx.table(step_reads), cur=H0, alt=H1)
+        for _ in range(3):
+            ctx.graph_launch(g2)
+        ctx.wait()
+        rd_us = ctx.graph_time(g2, 50) / 50
+        ctx.graph_destroy(g2)
+        step_read = {"launches": n2, "ms": round(rd_us / 1e3, 5), "step_rate_over_it": round(rd_us / 1e3 / ms_per_step, 3)}
 
     # One plain copy of known size: the calibration dispatch for HBM traffic counters (a counter
     # run of this same command scales FETCH_SIZE / WRITE_SIZE of any kernel by what they read for
@@ -253,6 +273,8 @@ def main() -> int:
     ctx.wait()
 
     extra = {}
+    if step_read:
+        extra["config1_step_plain_read"] = step_read
     if want_cold_step:
         # the same step over three rotating weight sets: what a step costs when nothing of it is left
         # in the Infinity Cache (the headline replays one 293 MB set, of which the cache keeps a part)
