@@ -223,6 +223,26 @@ size_t smelt_emitter_argmax_partial_bytes(const smelt_emitter *e);
 int smelt_hip_resolve_pipeline_name(const char *entry, int default_act, char *symbol,
                                     size_t symbol_cap, char *kinds, size_t kinds_cap);
 
+/* Launch plans of the kernels a record is re-routed to, without a device (no counterpart in the
+ * reference: one kernel per pipeline name there; for tests and for integrators who want to know
+ * what a record will run).  Each writes its answer as unsigned 32-bit fields and returns 1 when
+ * the shape takes the kernel, 0 when it keeps the kernel its pipeline names, negative on error.
+ *
+ * smelt_hip_plan_qmm: an affine g64 qmm record (plain, +add: nmat 1; gate+up: nmat 2) of `batch`
+ * tokens.  out[0] = 1 streaming kernel, 2 token-tile kernel; out[1] row tiles per wave;
+ * out[2] waves along K (streaming: waves of the workgroup); out[3] = 1 when the two matrices go to
+ * separate waves; out[4] workgroups that share a tile along K; out[5..7] grid; out[8] threads;
+ * out[9] LDS bytes; out[10] workspace bytes of the K split (low 32 bits).
+ *
+ * smelt_hip_plan_matvec: a single-token matvec of code layout 0 affine u4, 1 binary1, 2 ternary2,
+ * 3 trit5.  out[0] 128-byte segments per wave; out[1] waves per workgroup; out[2] workgroups;
+ * out[3] threads; out[4] LDS bytes. */
+int smelt_hip_plan_qmm(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch,
+                       uint32_t compute_units, size_t lds_limit, size_t workspace_bytes,
+                       uint32_t out[11]);
+int smelt_hip_plan_matvec(int code_layout, uint32_t rows, uint32_t cols, uint32_t group,
+                          uint32_t nmat, size_t lds_limit, int force, uint32_t out[5]);
+
 #ifdef __cplusplus
 }
 #endif

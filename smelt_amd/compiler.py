@@ -55,7 +55,7 @@ def lib() -> C.CDLL:
     l = rt.load_library()
     if _declared:
         return l
-    vp, i32, sz = C.c_void_p, C.c_int, C.c_size_t
+    vp, i32, u32, sz = C.c_void_p, C.c_int, C.c_uint32, C.c_size_t
     we, u64p = C.POINTER(WeightEntry), C.POINTER(C.c_uint64)
     sig = {
         "smelt_dtype_name": (C.c_char_p, [i32]),
@@ -95,6 +95,8 @@ def lib() -> C.CDLL:
         "smelt_emitter_pipeline_name": (C.c_char_p, [vp, sz]),
         "smelt_emitter_argmax_partial_bytes": (sz, [vp]),
         "smelt_hip_resolve_pipeline_name": (i32, [C.c_char_p, i32, C.c_char_p, sz, C.c_char_p, sz]),
+        "smelt_hip_plan_qmm": (i32, [u32, u32, u32, u32, u32, u32, sz, sz, C.POINTER(u32)]),
+        "smelt_hip_plan_matvec": (i32, [i32, u32, u32, u32, u32, sz, i32, C.POINTER(u32)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(l, name)
@@ -207,6 +209,30 @@ def resolve_pipeline_name(entry: str, act=rt.ACT_F16):
     kinds = C.create_string_buffer(64)
     rc = lib().smelt_hip_resolve_pipeline_name(entry.encode(), act, sym, 128, kinds, 64)
     return rc, sym.value.decode(), kinds.value.decode()
+
+
+QMM_PLAN_FIELDS = ("kernel", "row_tiles", "k_waves", "per_wave", "ksplit", "grid_x", "grid_y", "grid_z",
+                   "threads", "lds", "workspace")
+MATVEC_PLAN_FIELDS = ("segments", "waves", "workgroups", "threads", "lds")
+LAYOUT_U4, LAYOUT_BINARY1, LAYOUT_TERNARY2, LAYOUT_TRIT5 = range(4)
+
+
+def plan_qmm(rows, cols, group, nmat, batch, compute_units=256, lds_limit=160 * 1024, workspace_bytes=1 << 30):
+    """Launch plan of an affine qmm record, or None when it keeps the kernel its pipeline names."""
+    out = (C.c_uint32 * 11)()
+    rc = lib().smelt_hip_plan_qmm(rows, cols, group, nmat, batch, compute_units, lds_limit, workspace_bytes, out)
+    if rc < 0:
+        raise ValueError(f"smelt_hip_plan_qmm: {rc}")
+    return dict(zip(QMM_PLAN_FIELDS, out)) if rc else None
+
+
+def plan_matvec(layout, rows, cols, group, nmat=1, lds_limit=160 * 1024, force=False):
+    """Launch plan of the single-pass matrix-core matvec, or None when the shape stays on its own kernel."""
+    out = (C.c_uint32 * 5)()
+    rc = lib().smelt_hip_plan_matvec(layout, rows, cols, group, nmat, lds_limit, int(force), out)
+    if rc < 0:
+        raise ValueError(f"smelt_hip_plan_matvec: {rc}")
+    return dict(zip(MATVEC_PLAN_FIELDS, out)) if rc else None
 
 
 class EmitError(RuntimeError):

@@ -1072,6 +1072,38 @@ const char* smelt_emitter_pipeline_name(const smelt_emitter* e, size_t index) {
 }
 size_t smelt_emitter_argmax_partial_bytes(const smelt_emitter* e) { return e ? e->argmax_partial_bytes : 0; }
 
+int smelt_hip_plan_qmm(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
+                       size_t lds_limit, size_t workspace_bytes, uint32_t out[11]) {
+    if (!out) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    memset(out, 0, 11 * sizeof(uint32_t));
+    smelt_host::QmtPlan t;
+    if (smelt_host::qmt_plan(rows, cols, group, nmat, batch, compute_units, lds_limit, &t)) {
+        const uint32_t ksplit = t.partial_bytes <= workspace_bytes ? t.ksplit : 1;
+        out[0] = 2; out[1] = t.rt; out[2] = t.kw; out[3] = t.per_wave ? 1u : 0u; out[4] = ksplit;
+        out[5] = (rows + t.bn - 1) / t.bn; out[6] = (batch + t.bm - 1) / t.bm; out[7] = ksplit;
+        out[8] = 256 * t.kw; out[9] = (uint32_t)t.lds; out[10] = ksplit > 1 ? (uint32_t)t.partial_bytes : 0u;
+        return 1;
+    }
+    smelt_host::QmsPlan q;
+    if (batch > 0 && smelt_host::qms_plan(rows, cols, group, nmat, batch, lds_limit, &q)) {
+        out[0] = 1; out[1] = q.rt; out[2] = q.kc; out[4] = 1;
+        out[5] = (rows + 16 * q.rt - 1) / (16 * q.rt); out[6] = (batch + 15) / 16; out[7] = 1;
+        out[8] = 64 * q.kc; out[9] = (uint32_t)q.lds;
+        return 1;
+    }
+    return 0;
+}
+
+int smelt_hip_plan_matvec(int code_layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
+                          int force, uint32_t out[5]) {
+    if (!out || code_layout < 0 || code_layout > 3) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    memset(out, 0, 5 * sizeof(uint32_t));
+    smelt_host::Mm1Plan p;
+    if (!smelt_host::mm1_plan((smelt_host::CodeLayout)code_layout, rows, cols, group, nmat, lds_limit, force != 0, &p)) return 0;
+    out[0] = p.nl; out[1] = p.kc; out[2] = (rows + 7) / 8; out[3] = 64 * p.kc; out[4] = (uint32_t)p.lds;
+    return 1;
+}
+
 int smelt_hip_resolve_pipeline_name(const char* entry, int default_act, char* symbol, size_t symbol_cap, char* kinds, size_t kinds_cap) {
     if (!entry) return SMELT_HIP_ERR_INVALID_ARGUMENT;
     ResolvedPipeline r;

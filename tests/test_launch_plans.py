@@ -1,0 +1,94 @@
+"""Launch plans of the kernels a record is re-routed to (smelt_hip_plan_qmm / smelt_hip_plan_matvec):
+the rules of the choice, checked over a sweep of shapes without a device."""
+import itertools
+
+import pytest
+
+from smelt_amd import compiler as cc
+
+CUS, LDS = 256, 160 * 1024
+SHAPES = [(9216, 2560), (2560, 9216), (17408, 5120), (5120, 17408), (5120, 5120), (1024, 5120),
+          (1000, 6144), (64, 512), (151936, 2560), (24, 1024)]
+BATCHES = [1, 2, 7, 8, 9, 16, 31, 32, 33, 64, 127, 128, 129, 200, 256, 512, 1024, 4096]
+
+
+def ceil_div(a, b):
+    return (a + b - 1) // b
+
+
+@pytest.mark.parametrize("nmat", [1, 2])
+def test_qmm_plans_cover_the_output_and_fit_the_machine(nmat):
+    for (rows, cols), batch in itertools.product(SHAPES, BATCHES):
+        p = cc.plan_qmm(rows, cols, 64, nmat, batch, CUS, LDS)
+        assert p is not None, (rows, cols, batch)
+        assert p["lds"] <= LDS and p["threads"] <= 1024 and p["threads"] % 64 == 0
+        if p["kernel"] == 1:       # streaming: 16 * rt rows, 16 tokens per workgroup, no workspace
+            assert batch < 128 or cols % 512
+            assert p["grid_x"] * 16 * p["row_tiles"] >= rows > (p["grid_x"] - 1) * 16 * p["row_tiles"]
+            assert p["grid_y"] == ceil_div(batch, 16) and p["grid_z"] == 1 and p["workspace"] == 0
+            assert p["threads"] == 64 * p["k_waves"]
+        else:                      # token tiles: 64 tokens, 32 * rt rows (16 * rt of each matrix when split by wave)
+            assert p["kernel"] == 2 and batch >= 128 and cols % 512 == 0
+            bn = (16 if p["per_wave"] else 32) * p["row_tiles"]
+            assert p["grid_x"] == ceil_div(rows, bn) and p["grid_y"] == ceil_div(batch, 64)
+            assert p["threads"] == 256 * p["k_waves"]
+            assert p["per_wave"] == 0 or nmat == 2
+            # a K slice is at least six 512-column blocks; a split needs room for its partial sums
+            assert 1 <= p["ksplit"] == p["grid_z"] <= max(1, cols // 512 // 6)
+            assert (p["workspace"] > 0) == (p["ksplit"] > 1)
+            if p["ksplit"] > 1:
+                tiles = p["grid_x"] * p["grid_y"]
+                assert tiles < 2 * CUS              # only grids that leave the machine short are split
+                assert p["workspace"] >= tiles * p["ksplit"] * bn * 64 * 4 * nmat // (2 if p["per_wave"] else 1) // 2
+
+
+def test_qmm_k_split_needs_the_workspace():
+    with_ws = cc.plan_qmm(2560, 9216, 64, 1, 512, CUS, LDS)
+    assert with_ws["ksplit"] > 1
+    without = cc.plan_qmm(2560, 9216, 64, 1, 512, CUS, LDS, workspace_bytes=with_ws["workspace"] - 1)
+    assert without["ksplit"] == 1 and without["grid_z"] == 1 and without["workspace"] == 0
+    assert {k: without[k] for k in ("kernel", "row_tiles", "k_waves", "grid_x", "grid_y", "lds")} == \
+           {k: with_ws[k] for k in ("kernel", "row_tiles", "k_waves", "grid_x", "grid_y", "lds")}
+
+
+def test_qmm_plan_rejects_what_no_kernel_takes():
+    assert cc.plan_qmm(1024, 1024, 32, 1, 64) is None      # group 32 has no streaming form
+    assert cc.plan_qmm(1024, 1024, 64, 1, 0) is None
+    assert cc.plan_qmm(1024, 1000, 64, 1, 64) is None      # ragged K
+    # a small LDS budget: the plan shrinks or gives up, never overshoots
+    for limit in (16 << 10, 32 << 10, 64 << 10):
+        p = cc.plan_qmm(9216, 2560, 64, 2, 512, CUS, limit)
+        assert p is None or p["lds"] <= limit
+
+
+@pytest.mark.parametrize("layout,group", [(cc.LAYOUT_U4, 64), (cc.LAYOUT_BINARY1, 128), (cc.LAYOUT_TERNARY2, 128),
+                                          (cc.LAYOUT_TRIT5, 128)])
+def test_matvec_plans(layout, group):
+    bytes_per_row = {cc.LAYOUT_U4: lambda c: c // 2, cc.LAYOUT_BINARY1: lambda c: ceil_div(c, 128) * 16,
+                     cc.LAYOUT_TERNARY2: lambda c: ceil_div(c, 128) * 32,
+                     cc.LAYOUT_TRIT5: lambda c: (ceil_div(c, 5) + 15) // 16 * 16}[layout]
+    for rows, cols in SHAPES:
+        for nmat in (1, 2):
+            p = cc.plan_matvec(layout, rows, cols, group, nmat, LDS, force=True)
+            if p is None:
+                continue
+            segments = ceil_div(bytes_per_row(cols), 128)
+            assert p["waves"] <= 16 and p["threads"] == 64 * p["waves"] and p["lds"] <= LDS
+            assert p["waves"] * p["segments"] >= segments > (p["waves"] - 1) * p["segments"]
+            assert p["workgroups"] == ceil_div(rows, 8)
+    # the 27B layer's matrices take the kernel by default in every format
+    for rows, cols in [(17408, 5120), (5120, 17408), (5120, 5120)]:
+        assert cc.plan_matvec(layout, rows, cols, group) is not None
+    # small matrices stay on the vector kernels unless forced (five-digit bytes from 2M weights, the rest from 8M)
+    small = cc.plan_matvec(layout, 1024, 2560, group)
+    assert (small is not None) == (layout == cc.LAYOUT_TRIT5)
+    assert cc.plan_matvec(layout, 256, 2560, group) is None
+    assert cc.plan_matvec(layout, 256, 2560, group, force=True) is not None
+
+
+def test_matvec_plan_rejects_bad_arguments():
+    with pytest.raises(ValueError):
+        cc.plan_matvec(7, 1024, 1024, 64)
+    assert cc.plan_matvec(cc.LAYOUT_BINARY1, 8192, 8192, 64) is None     # signed formats are g128 only
+    assert cc.plan_matvec(cc.LAYOUT_TRIT5, 8192, 8200, 128) is None      # rows of five-digit bytes: 16-column multiples
+    assert cc.plan_matvec(cc.LAYOUT_U4, 8192, 8192, 48) is None
