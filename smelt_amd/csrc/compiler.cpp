@@ -101,7 +101,8 @@ bool hip_has_kernel(const SmeltMatvecCell& c, int family) {
     if (c.activation == SMELT_ACT_FP32) return false;
     // GeGLU: affine only (single-token kernel and the MFMA slab kernel)
     if (c.fusion == SMELT_FUSION_GATE_UP_GEGLU) return family == SMELT_FAMILY_AFFINE_U4;
-    if (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_DUAL_MATVEC) return false;
+    // prompt rows of the dual matvec: the per-token "_batched" form and the token tiles of "_batched_verify_b4"
+    if (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_DUAL_MATVEC) return family == SMELT_FAMILY_AFFINE_U4;
     if (c.shape == SMELT_SHAPE_GEMM && c.fusion == SMELT_FUSION_GATE_UP_SWIGLU && family == SMELT_FAMILY_TERNARY2) return false;
     return true;
 }

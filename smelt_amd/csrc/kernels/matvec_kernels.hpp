@@ -101,6 +101,22 @@ struct EpiDual : EpiBase {
     }
 };
 
+// two projections, each rounded to the activation type and added to its own residual in that type
+// (fused_dual_affine_matvec_add_fixed_rows4, lut_matvec.metal:4660-4733)
+template <class ActT>
+struct EpiDualAdd : EpiBase {
+    uint16_t* y1;
+    uint16_t* y2;
+    const uint16_t* r1;
+    const uint16_t* r2;
+    int rows;
+    __device__ __forceinline__ void operator()(int b, int row, const float* v) const {
+        const size_t at = (size_t)b * rows + row;
+        y1[at] = ActT::narrow(ActT::widen(ActT::narrow(v[0])) + ActT::widen(r1[at]));
+        y2[at] = ActT::narrow(ActT::widen(ActT::narrow(v[1])) + ActT::widen(r2[at]));
+    }
+};
+
 // ---- workgroup body ------------------------------------------------------------------------
 //
 // A wave walks its row tiles (grid-stride, so any grid covers every row) as a flat sequence of
@@ -319,6 +335,17 @@ using u32 = uint32_t;
                                              packed_row_stride<FmtU4>(cols, group), group,        \
                                              blockIdx.y, blockIdx.y + 1, epi);                    \
     }                                                                                             \
+    SMELT_KERNEL void smelt_affine_dual_matvec_add_##T(                                           \
+        const u8* W1, const u16* S1, const u16* B1, const u8* W2, const u16* S2, const u16* B2,   \
+        const u16* x, u16* y1, u16* y2, const u16* r1, const u16* r2, u32 rows, u32 cols,         \
+        u32 group) {                                                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
+        EpiDualAdd<ACT> epi{{}, y1, y2, r1, r2, (int)rows};                                       \
+        matvec_body<FmtU4, ACT, SC, 2, 1, 2>(mats, x, rows, cols,                                 \
+                                             packed_row_stride<FmtU4>(cols, group), group,        \
+                                             blockIdx.y, blockIdx.y + 1, epi);                    \
+    }                                                                                             \
     SMELT_KERNEL_W5 void smelt_affine_gate_up_geglu_##T(                                          \
         const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
         const u16* x, u16* y, u32 rows, u32 cols, u32 group) {                                    \
@@ -464,6 +491,20 @@ using u32 = uint32_t;
         using namespace smelt;                                                                    \
         const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
         EpiGeglu<ACT> epi{{}, Y, (int)rows};                                                      \
+        const u32 lo = blockIdx.y * batch_tile;                                                   \
+        if (lo >= batch) return;                                                                  \
+        const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \
+        matvec_body<FmtU4, ACT, SC, 2, MBV, 2>(mats, X, rows, cols,                               \
+                                               packed_row_stride<FmtU4>(cols, group), group, lo,  \
+                                               hi, epi);                                          \
+    }                                                                                             \
+    SMELT_KERNEL void smelt_affine_dual_matvec_batched_mb##MBV##_##T(                             \
+        const u8* W1, const u16* S1, const u16* B1, const u8* W2, const u16* S2, const u16* B2,   \
+        const u16* X, u16* Y1, u16* Y2, u32 batch, u32 rows, u32 cols, u32 group,                 \
+        u32 batch_tile) {                                                                         \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
+        EpiDual<ACT> epi{{}, Y1, Y2, (int)rows};                                                  \
         const u32 lo = blockIdx.y * batch_tile;                                                   \
         if (lo >= batch) return;                                                                  \
         const u32 hi = lo + batch_tile < batch ? lo + batch_tile : batch;                         \

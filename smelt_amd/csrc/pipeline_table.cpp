@@ -400,6 +400,7 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
         {"fused_affine_matvec_add", kFamAffineAdd},
         {"fused_affine_gate_up_swiglu", kFamAffineGateUp},
         {"fused_dual_affine_matvec", kFamAffineDual},
+        {"fused_dual_affine_matvec_add", kFamAffineDualAdd},
         {"fused_affine_gate_up_geglu", kFamAffineGateUp},
         {"norm_scale_affine_matvec", kFamNormScaleAffineMatvec},
         {"norm_add_scale_affine_matvec", kFamNormAddScaleAffineMatvec},
@@ -441,7 +442,8 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
         if (suffix == "_batched") bt = 8;
         else if (suffix == "_batched_skinny") { bt = 32; full = true; skinny = true; }
         else if (suffix == "_batched_tile3") bt = 3;
-        else if (suffix == "_batched_tile4" || suffix == "_batched_ext_b4") bt = 4;
+        // "_batched_verify_b4": the generated small-batch kernels (SmeltGeneratedKernelVariants.swift:17-35), token tiles of 4
+        else if (suffix == "_batched_tile4" || suffix == "_batched_ext_b4" || suffix == "_batched_verify_b4") bt = 4;
         else if (suffix == "_batched_ext_b5" || suffix == "_batched_sg4_bt5") bt = 5;
         else if (suffix == "_batched_full") { bt = 16; full = true; }
         else if (starts_with(suffix, "_batched_full_b") && parse_uint(suffix.substr(15), &bt) && bt >= 1 && bt <= 4096) { full = true; }
@@ -473,6 +475,7 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
                 case kFamAffineAdd: out->symbol = "smelt_affine_matvec_add_" + t; out->kinds = "PPPPPPUUU"; break;
                 case kFamAffineGateUp: out->symbol = "smelt_affine_gate_up_swiglu_" + t; out->kinds = "PPPPPPPPUUU"; break;
                 case kFamAffineDual: out->symbol = "smelt_affine_dual_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; break;
+                case kFamAffineDualAdd: out->symbol = "smelt_affine_dual_matvec_add_" + t; out->kinds = "PPPPPPPPPPPUUU"; break;
                 case kFamNormScaleAffineMatvec: out->symbol = "smelt_norm_scale_affine_matvec_" + t; out->kinds = "PPPPPPPPUUU"; break;
                 case kFamNormScaleAffineGateUp: out->symbol = std::string("smelt_") + a.prefix + "_" + t; out->kinds = "PPPPPPPPPPUUU"; break;
                 case kFamNormAddScaleAffineMatvec: out->symbol = "smelt_norm_add_scale_affine_matvec_" + t; out->kinds = "PPPPPPPPPUUU"; break;
@@ -485,7 +488,7 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
             if (prologue && want_mfma) { *why = "no matrix-core form of '" + entry + "'"; return kResolveUnknown; }
             out->appended = {rows, cols, group};
             const uint32_t nmat = a.m1 == kFamAffineGateUp ? 2 : 1;
-            if (a.m1 != kFamAffineDual && !prologue && !strstr(a.prefix, "geglu"))
+            if (a.m1 != kFamAffineDual && a.m1 != kFamAffineDualAdd && !prologue && !strstr(a.prefix, "geglu"))
                 if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, 1, nmat, lds_limit) : 0) {
                     out->mfma_kw = kw;
                     out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_" : (a.m1 == kFamAffineAdd ? "smelt_affine_mm_matvec_add_" : "smelt_affine_mm_gate_up_swiglu_")) + (kw == 1 ? "stream_" : "split_") + t;
@@ -495,9 +498,20 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
             return kResolveOk;
         }
         const bool geglu = strstr(a.prefix, "geglu") != nullptr;
-        if (a.m1 == kFamNormAddScaleAffineMatvec || a.m1 == kFamNormScaleAffineDual) {
+        if (a.m1 == kFamNormAddScaleAffineMatvec || a.m1 == kFamNormScaleAffineDual || a.m1 == kFamAffineDualAdd) {
             *why = "no batched HIP kernel for '" + entry + "'";
             return kResolveUnknown;
+        }
+        if (a.m1 == kFamAffineDual) {
+            // token tiles of two same-shape projections (fused_dual_affine_matvec_fixed_ext, lut_matvec.metal:3816-3922)
+            if (want_mfma || full || suffix != "_batched_verify_b4") { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
+            const uint32_t mbv = pick_mb(kCodesU4, row_stride, 4, lds_limit);
+            out->lds_variant = mbv;
+            out->family = kFamAffineDualBatched;
+            out->symbol = "smelt_affine_dual_matvec_batched_mb" + std::to_string(mbv) + "_" + t;
+            out->kinds = "PPPPPPPPPUUUUU";
+            out->appended = {rows, cols, group, bt};
+            return kResolveOk;
         }
         if (a.m1 == kFamAffineGateUp && geglu && !want_mfma && (suffix == "_batched" || suffix == "_batched_bt4_sg4")) {
             // small-batch GeGLU (lut_matvec.metal:8342-8364, 8752-8753): token tiles of 3 and 4

@@ -88,6 +88,8 @@ enum FamilyId {
     kFamBiasAddBatched,          // in bias out rows                             (threads grid, grid.y = token)
     kFamNormScaleAffineQmm,      // rs X nw XN W S B Y batch | rows cols group batch_tile          (MFMA slabs)
     kFamNormScaleAffineQmmGateUp,// rs X nw gW gS gB uW uS uB Y batch | rows cols group batch_tile
+    kFamAffineDualAdd,           // W1 S1 B1 W2 S2 B2 x y1 y2 res1 res2 | rows cols group          (grid.y = token)
+    kFamAffineDualBatched,       // W1 S1 B1 W2 S2 B2 X Y1 Y2 batch | rows cols group batch_tile
     kFamCount
 };
 

@@ -156,7 +156,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
                                    r.family == kFamNormScaleAffineQmm || r.family == kFamNormScaleAffineQmmGateUp ||
                                    r.family == kFamNormAddScaleAffineMatvec || r.family == kFamNormScaleAffineDual ||
                                    r.family == kFamFusedNormAffineMatvec || r.family == kFamFusedNormAffineGateUp;
-    const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec || norm_scale_matvec;
+    const bool matvec_like = r.family <= kFamAffineBank4 || plane_matvec || lut_matvec || norm_scale_matvec ||
+                             r.family == kFamAffineDualAdd || r.family == kFamAffineDualBatched;
     const bool skinny = r.lds_variant == kSkinnyVariant &&
                         (r.family == kFamAffineQmm || r.family == kFamAffineQmmAdd || r.family == kFamAffineQmmGateUp);
     if (matvec_like) {
@@ -209,15 +210,17 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
             break;
         }
         case kFamAffineGateUp:
+        case kFamAffineDualAdd:
         case kFamAffineDual: {
-            const size_t o = r.family == kFamAffineDual ? 9 : 8;
+            const size_t o = r.family == kFamAffineDualAdd ? 11 : (r.family == kFamAffineDual ? 9 : 8);
             const size_t rows = U(o), cols = U(o + 1), group = U(o + 2);
             if (int e = check_affine_shape(rows, cols, group)) return e;
             affine(0, 1, 2, rows, cols, group);
             affine(3, 4, 5, rows, cols, group);
             need[6] = gy * cols * 2; align[6] = 16;
             need[7] = gy * rows * 2; written[7] = true;
-            if (r.family == kFamAffineDual) { need[8] = gy * rows * 2; written[8] = true; }
+            if (r.family != kFamAffineGateUp) { need[8] = gy * rows * 2; written[8] = true; }
+            if (r.family == kFamAffineDualAdd) need[9] = need[10] = gy * rows * 2;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
             mm_cols = cols; mm_nmat = 2;
             break;
@@ -335,16 +338,18 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
             break;
         }
         case kFamAffineBatched:
+        case kFamAffineDualBatched:
         case kFamAffineGateUpBatched: {
-            const size_t o = r.family == kFamAffineGateUpBatched ? 8 : 5;
+            const size_t o = r.family == kFamAffineDualBatched ? 9 : (r.family == kFamAffineGateUpBatched ? 8 : 5);
             const size_t batch = U(o), rows = U(o + 1), cols = U(o + 2), group = U(o + 3), bt = U(o + 4);
             if (int e = check_affine_shape(rows, cols, group)) return e;
             if (bt == 0 || gy * bt < batch) return bad_geom("grid height * batch tile does not cover the batch");
             affine(0, 1, 2, rows, cols, group);
             size_t xi = 3, yi = 4;
-            if (r.family == kFamAffineGateUpBatched) { affine(3, 4, 5, rows, cols, group); xi = 6; yi = 7; }
+            if (r.family != kFamAffineBatched) { affine(3, 4, 5, rows, cols, group); xi = 6; yi = 7; }
             need[xi] = batch * cols * 2; align[xi] = 16;
             need[yi] = batch * rows * 2; written[yi] = true;
+            if (r.family == kFamAffineDualBatched) { need[8] = batch * rows * 2; written[8] = true; }
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), r.lds_variant);
             mm_cols = cols; mm_tokens = std::min<size_t>(8, std::min(batch, bt)); mm_nmat = r.family == kFamAffineGateUpBatched ? 2 : 1;
             break;

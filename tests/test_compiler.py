@@ -48,6 +48,7 @@ def test_gateway_has_no_holes_and_never_defaults():
     assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, cc.GEMM, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_OK
     assert cc.select(cc.ACT_FP16, cc.BINARY1, fusion=cc.FUSION_GATE_UP_GEGLU, hip_backend=True)[0] == cc.SELECT_NOT_MEANINGFUL
+    assert cc.select(cc.ACT_FP16, cc.AFFINE_U4, cc.GEMM, fusion=cc.FUSION_DUAL, hip_backend=True)[0] == cc.SELECT_OK
 
 
 def test_weight_layout_alignment_sizes_and_no_overlap():
@@ -162,6 +163,16 @@ def test_pipeline_names_resolve_to_kernels_with_the_reference_binding_counts():
     assert cc.resolve_pipeline_name("fused_lut_matvec:1024:4")[0] == -3    # fewer than 8 rows per table
     assert cc.resolve_pipeline_name("tqh_matvec_batched")[1:] == ("smelt_tqh_matvec_f16", "PPPPUUU")
     assert cc.resolve_pipeline_name("u4_lut_qmm")[0] == -4
+    # the compiler's generated variants (SmeltGeneratedKernelVariants.swift:17-35, 66-68)
+    assert cc.resolve_pipeline_name("affine_matvec_c2560_r9216_g64_batched_verify_b4")[1:] == ("smelt_affine_matvec_batched_mb4_f16", "PPPPPUUUUU")
+    assert cc.resolve_pipeline_name("fused_affine_gate_up_swiglu_c2560_r9216_g64_batched_verify_b4")[1:] == \
+        ("smelt_affine_gate_up_swiglu_batched_mb4_f16", "PPPPPPPPUUUUU")
+    assert cc.resolve_pipeline_name("fused_dual_affine_matvec_c2048_r16_g64_batched_verify_b4@bf16")[1:] == \
+        ("smelt_affine_dual_matvec_batched_mb4_bf16", "PPPPPPPPPUUUUU")
+    assert cc.resolve_pipeline_name("fused_dual_affine_matvec_add_c2048_r256_g64_rows4")[1:] == \
+        ("smelt_affine_dual_matvec_add_f16", "PPPPPPPPPPPUUU")
+    assert cc.resolve_pipeline_name("fused_dual_affine_matvec_add_c2048_r256_g64_batched")[0] == -4
+    assert cc.resolve_pipeline_name("fused_dual_affine_matvec_c2048_r16_g64_batched_full")[0] == -4
     assert cc.resolve_pipeline_name("rms_norm_1pw_from_fp32")[1:] == ("smelt_rms_norm_1pw_from_fp32_f16", "PPPUF")
     assert cc.resolve_pipeline_name("rms_norm_gated_d128")[1] == "smelt_rms_norm_gated_f16"
     assert cc.resolve_pipeline_name("rms_norm_head_f32")[0] == -4          # fp32 trunk kernels are out of scope

@@ -436,3 +436,71 @@ def test_dual_matvec_per_token_and_small_batch_geglu(ctx):
         assert ctx.encode_decode(rt.make_record(pipe, bufs, [(8, batch)], (rows // 8, (batch + bt - 1) // bt, 1), (256, 1, 1))) == 1
         ctx.wait()
         assert np.array_equal(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), single), suffix
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_generated_small_batch_and_dual_add_names(ctx, dtype):
+    """The compiler's generated variants (SmeltGeneratedKernelVariants.swift:17-35, 66-68):
+    `_batched_verify_b4` forms of the matvec, gate+up+SwiGLU and dual matvec (token tiles of 4, the token
+    count at the binding after the outputs; lut_matvec.metal:3816-3922) and the decode dual matvec with two
+    residuals (`fused_dual_affine_matvec_add_*_rows4`, :4660-4733).  Per token they are the single-token
+    kernels' bits; the residual form is checked against the oracle's round-then-add."""
+    rows, cols, group, batch = 264, 1024, 64, 6
+    w1 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=20)
+    w2 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=21)
+    x = fx.synth_activation(batch, cols, dtype, config=1, tensor=73)
+    s1 = run_affine(ctx, *w1, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    s2 = run_affine(ctx, *w2, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    shape = f"c{cols}_r{rows}_g{group}"
+    tiles = (batch + 3) // 4
+
+    got = run_affine(ctx, *w1, x, dtype, f"affine_matvec_{shape}_batched_verify_b4", batched=True, batch_tile=4)
+    assert np.array_equal(got, s1)
+
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*w1, *w2)]
+    image = wf.image()
+    weights = [(0, i, o) for i, o in enumerate(offs)]
+
+    # gate+up+SwiGLU, tiles of 4 tokens against the single-token fused kernel
+    single = np.stack([run_gate_up(ctx, w1, w2, dtype, f"fused_affine_gate_up_swiglu:{cols}:{group}", [(8, rows)], x[b:b + 1])[0]
+                       for b in range(batch)])
+    ctx.upload_weights(gh.WEIGHTS_SLOT, image)
+    ctx.put(gh.X_SLOT, x); ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+    pipe = ctx.pipeline(f"fused_affine_gate_up_swiglu_{shape}_batched_verify_b4" + gh.t_suffix(dtype))
+    rec = rt.make_record(pipe, weights + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)], [(8, batch)], ((rows + 7) // 8, tiles, 1), (64, 1, 1))
+    assert ctx.encode_decode(rec) == 1
+    ctx.wait()
+    assert np.array_equal(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), single)
+
+    # dual matvec, tiles of 4 tokens; a grid one tile short is refused
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2); ctx.alloc(gh.AUX_SLOT, batch * rows * 2)
+    pipe = ctx.pipeline(f"fused_dual_affine_matvec_{shape}_batched_verify_b4" + gh.t_suffix(dtype))
+    bufs = weights + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0), (gh.AUX_SLOT, 8, 0)]
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, [(9, batch)], ((rows + 7) // 8, tiles, 1), (64, 1, 1))) == 1
+    ctx.wait()
+    assert np.array_equal(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), s1)
+    assert np.array_equal(ctx.read(gh.AUX_SLOT, np.uint16, batch * rows).reshape(batch, rows), s2)
+    with pytest.raises(rt.SmeltHipError):
+        ctx.encode_decode(rt.make_record(pipe, bufs, [(9, batch)], ((rows + 7) // 8, tiles - 1, 1), (64, 1, 1)))
+
+    # decode dual matvec with a residual per output (each output may alias its residual)
+    r1 = fx.to_bits(fx.rng_for(5, 1).normal(0, 1, (1, rows)).astype(np.float32), dtype)
+    r2 = fx.to_bits(fx.rng_for(5, 2).normal(0, 1, (1, rows)).astype(np.float32), dtype)
+    ctx.put(gh.X_SLOT, x[:1]); ctx.put(gh.Y_SLOT, r1); ctx.alloc(gh.AUX_SLOT, rows * 2); ctx.put(gh.AUX2_SLOT, r2)
+    pipe = ctx.pipeline(f"fused_dual_affine_matvec_add_{shape}_rows4" + gh.t_suffix(dtype))
+    bufs = weights + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0), (gh.AUX_SLOT, 8, 0), (gh.Y_SLOT, 9, 0), (gh.AUX2_SLOT, 10, 0)]
+    assert ctx.encode_decode(rt.make_record(pipe, bufs, [], (rows // 4, 1, 1), (64, 1, 1))) == 1
+    ctx.wait()
+    odt = so.F16 if dtype == fx.F16 else so.BF16
+    xf = fx.from_bits(x[:1], dtype)
+    a1 = so.affine_matvec(*w1, xf, rows, cols, group, dtype)
+    a2 = so.affine_matvec(*w2, xf, rows, cols, group, dtype)
+    y1 = ctx.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows)
+    y2 = ctx.read(gh.AUX_SLOT, np.uint16, rows).reshape(1, rows)
+    # the projections agree with the oracle to tolerance; rounded to the activation type and added to the residual
+    # in that type they are the fused kernel's bits (the oracle's epilogue on the GPU's own projections)
+    gh.check_outputs(s1[:1], a1, dtype, "dual, first projection")
+    gh.check_outputs(s2[:1], a2, dtype, "dual, second projection")
+    assert np.array_equal(y1, so.epilogue_residual_add(fx.from_bits(s1[:1], dtype), r1, odt))
+    assert np.array_equal(y2, so.epilogue_residual_add(fx.from_bits(s2[:1], dtype), r2, odt))
