@@ -157,8 +157,15 @@ struct M1U4 : M1Codes<4, ActT> {
 //   then the scale rows (and bias rows) of the workgroup's eight rows, one block per matrix and
 //   plane; then the waves' partial sums [wave][matrix][8] (fp32).
 //   (five-dword pieces: per dword the folded-out constant, 4 B; and a 512-byte decode table at the end)
+//   Four-dword pieces hold a power-of-two number of fragments, which would put the eight pieces of a
+//   segment (read together, one per A-operand lane) on the same LDS banks: their stride is one
+//   fragment longer.  Five-dword pieces (160 bytes) spread over the banks by themselves.
+__host__ __device__ constexpr int mm1_piece_stride(int frags_per_piece, int dw = 4) {
+    return dw == 4 ? frags_per_piece + 1 : frags_per_piece;
+}
 __host__ __device__ constexpr size_t mm1_wave_lds_bytes(int frags_per_piece, int nl, int dw = 4) {
-    return (size_t)nl * 8 * frags_per_piece * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) + (size_t)frags_per_piece * 16;
+    return (size_t)nl * 8 * mm1_piece_stride(frags_per_piece, dw) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) +
+           (size_t)frags_per_piece * 16;
 }
 __host__ __device__ constexpr size_t mm1_lds_bytes(int frags_per_piece, int nl, int waves, int nmat, int gpr, bool has_bias, int dw = 4) {
     return (size_t)waves * mm1_wave_lds_bytes(frags_per_piece, nl, dw) + (size_t)nmat * (has_bias ? 2 : 1) * 8 * gpr * 2 +
@@ -177,6 +184,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
                                          int cols, int row_stride, int group, const Epi& epi) {
     using E = Elem16<ActT>;
     constexpr int FPD = F::kFPD, FPL = F::kFPL, FIELDS = F::kFields, PAIRS = F::kPairs, DW = F::kDW;
+    constexpr int PSTRIDE = mm1_piece_stride(FPL, DW);     // fragments from one piece to the next in LDS
     constexpr int NITEMS = NL * 8 * DW;                    // staging items of a wave: 8 pieces x DW dwords per segment
     constexpr int ITEMS = (NITEMS + kWave - 1) / kWave;    // per lane
     constexpr int PLANES = F::kHasBias ? 2 : 1;
@@ -279,7 +287,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // 2v, 2v+1 of fragment t = columns 4t+v, 4t+v+kPairs).  The four items of a 16-byte piece sit
     // in the four lanes of a quad, which add up their sum(base * x) and sum(x).
     uint4_t* wfrag = reinterpret_cast<uint4_t*>(smem + (size_t)chunk * wave_bytes);
-    float* wsum = reinterpret_cast<float*>(wfrag + (size_t)NL * 8 * FPL);   // [piece][2]: constant, sum x ([piece][DW]: constants)
+    float* wsum = reinterpret_cast<float*>(wfrag + (size_t)NL * 8 * PSTRIDE);   // [piece][2]: constant, sum x ([piece][DW]: constants)
     uint4_t* wzero = reinterpret_cast<uint4_t*>(wsum + (DW == 4 ? NL * 16 : NL * 8 * DW));   // FPL zero fragments
     // decode table of the five-digit bytes, copied from constant memory; visible after the barrier below
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem_all);
@@ -309,7 +317,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         }
 #pragma unroll
         for (int t = 0; t < FPD; ++t)
-            wfrag[(size_t)pl * FPL + d * FPD + t] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
+            wfrag[(size_t)pl * PSTRIDE + d * FPD + t] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
         if constexpr (DW == 4) {
             if (d == 0) *reinterpret_cast<float2*>(wsum + 2 * pl) = float2{__builtin_fmaf(F::kOffset, xs, cb), xs};
         } else {
@@ -354,7 +362,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
                 cd[m][0] = codes[m][i].x; cd[m][1] = codes[m][i].y; cd[m][2] = codes[m][i].z; cd[m][3] = codes[m][i].w;
             }
         }
-        const uint4_t* piece_frags = wfrag + (size_t)(i * 8 + a_piece) * FPL;
+        const uint4_t* piece_frags = wfrag + (size_t)(i * 8 + a_piece) * PSTRIDE;
 #pragma unroll
         for (int d = 0; d < DW; ++d) {
             const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
