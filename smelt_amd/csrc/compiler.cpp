@@ -1075,7 +1075,7 @@ size_t smelt_emitter_argmax_partial_bytes(const smelt_emitter* e) { return e ? e
 
 int smelt_hip_plan_qmm(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
                        size_t lds_limit, size_t workspace_bytes, uint32_t out[11]) {
-    if (!out) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (!out || nmat < 1 || nmat > 2) return SMELT_HIP_ERR_INVALID_ARGUMENT;
     memset(out, 0, 11 * sizeof(uint32_t));
     smelt_host::QmtPlan t;
     if (smelt_host::qmt_plan(rows, cols, group, nmat, batch, compute_units, lds_limit, &t)) {
@@ -1097,7 +1097,7 @@ int smelt_hip_plan_qmm(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nm
 
 int smelt_hip_plan_matvec(int code_layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
                           int force, uint32_t out[5]) {
-    if (!out || code_layout < 0 || code_layout > 3) return SMELT_HIP_ERR_INVALID_ARGUMENT;
+    if (!out || code_layout < 0 || code_layout > 3 || nmat < 1 || nmat > 2) return SMELT_HIP_ERR_INVALID_ARGUMENT;
     memset(out, 0, 5 * sizeof(uint32_t));
     smelt_host::Mm1Plan p;
     if (!smelt_host::mm1_plan((smelt_host::CodeLayout)code_layout, rows, cols, group, nmat, lds_limit, force != 0, &p)) return 0;

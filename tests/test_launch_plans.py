@@ -89,6 +89,10 @@ def test_matvec_plans(layout, group):
 def test_matvec_plan_rejects_bad_arguments():
     with pytest.raises(ValueError):
         cc.plan_matvec(7, 1024, 1024, 64)
+    with pytest.raises(ValueError):
+        cc.plan_matvec(cc.LAYOUT_U4, 1024, 1024, 64, nmat=3)
+    with pytest.raises(ValueError):
+        cc.plan_qmm(1024, 1024, 64, 0, 64)
     assert cc.plan_matvec(cc.LAYOUT_BINARY1, 8192, 8192, 64) is None     # signed formats are g128 only
     assert cc.plan_matvec(cc.LAYOUT_TRIT5, 8192, 8200, 128) is None      # rows of five-digit bytes: 16-column multiples
     assert cc.plan_matvec(cc.LAYOUT_U4, 8192, 8192, 48) is None
