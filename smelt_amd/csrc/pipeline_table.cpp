@@ -173,7 +173,16 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     Mm1Plan best;
     uint32_t best_waste = ~0u;
     const uint32_t tolerated = nseg / 10 > 1 ? nseg / 10 : 1;
-    for (uint32_t nl = nl_max; nl >= 1; --nl) {
+    // Segments per wave, in order of preference.  Affine 4-bit rows are long (a 5120-column row is twenty
+    // segments): as many segments per wave as the kernels have.  The signed formats measured best with two
+    // (binary 27B layer 33.5 -> 31.5 us, five-digit bytes 50.2 -> 47.6 against three; one or four and more
+    // were slower), then three where two would need more than sixteen waves.
+    static const uint32_t kLongRows[] = {6, 5, 4, 3, 2, 1}, kSigned[] = {2, 3, 1};
+    const uint32_t* order = layout == kCodesU4 ? kLongRows : kSigned;
+    const uint32_t norder = layout == kCodesU4 ? 6 : 3;
+    for (uint32_t o = 0; o < norder; ++o) {
+        const uint32_t nl = order[o];
+        if (nl > nl_max || (nl > nseg && nl > 1)) continue;
         const uint32_t kc = (nseg + nl - 1) / nl;
         if (kc > 16 || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
         const size_t lds = lds_of(kc, nl);
