@@ -162,7 +162,8 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     if (layout != kCodesU4 && group != 128) return false;
     // small matrices are launch-bound either way and stay where they are tuned
     // (five-digit bytes: the vector kernel decodes through the same table at twice the cost, so the bar is lower)
-    if (!force && (uint64_t)rows * cols < (layout == kCodesTrit5 ? (2u << 20) : (8u << 20))) return false;
+    // (affine: from 1M weights, see the short walk below)
+    if (!force && (uint64_t)rows * cols < (layout == kCodesTrit5 ? (2u << 20) : (layout == kCodesU4 ? (1u << 20) : (8u << 20)))) return false;
     const uint32_t pieces = row_stride / 16, nseg = (pieces + 7) / 8, gpr = (cols + group - 1) / group;
     const uint32_t planes = layout == kCodesU4 ? 2 : 1;
     auto lds_of = [&](uint32_t kc, uint32_t nl) {
@@ -180,11 +181,17 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     static const uint32_t kLongRows[] = {6, 5, 4, 3, 2, 1}, kSigned[] = {2, 3, 1};
     const uint32_t* order = layout == kCodesU4 ? kLongRows : kSigned;
     const uint32_t norder = layout == kCodesU4 ? 6 : 3;
+    // Affine matrices below 8M weights (a 0.8B model's projections) are a launch and one memory round trip:
+    // the more waves share a row the shorter that trip, so the fewest segments per wave that eight waves cover
+    // (config-1 step 0.366 -> 0.346 ms against the vector kernels)
+    static const uint32_t kShortWalk[] = {1, 2, 3, 4, 5, 6};
+    const bool small_affine = layout == kCodesU4 && (uint64_t)rows * cols < (8u << 20);
+    if (small_affine) order = kShortWalk;
     for (uint32_t o = 0; o < norder; ++o) {
         const uint32_t nl = order[o];
         if (nl > nl_max || (nl > nseg && nl > 1)) continue;
         const uint32_t kc = (nseg + nl - 1) / nl;
-        if (kc > 16 || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
+        if (kc > (small_affine ? 8u : 16u) || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
         const size_t lds = lds_of(kc, nl);
         if (lds > lds_limit) continue;
         const uint32_t waste = kc * nl - nseg;

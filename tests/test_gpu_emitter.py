@@ -160,8 +160,10 @@ def test_signed_layer_table_decode_and_prefill(wdtype):
         ctx.close()
 
 
-def test_affine_projection_bank_equals_independent_matvecs():
-    """One bank dispatch over q|k|v gives the bits of three independent dispatches."""
+@pytest.mark.parametrize("engine", [rt.MATVEC_VECTOR, rt.MATVEC_MATRIX_CORE])
+def test_affine_projection_bank_equals_independent_matvecs(engine):
+    """One bank dispatch over q|k|v gives the bits of three independent dispatches (on either engine; AUTO picks
+    per matrix size, and the bank is larger than its members)."""
     hidden, group = 1024, 64
     member_rows = [2048, 512, 520]
     lay = cc.Layout()
@@ -183,6 +185,7 @@ def test_affine_projection_bank_equals_independent_matvecs():
             em.matvec(0, e, cc.bind(1), o)
         assert not em.bank_matvec(0, [members[0], lone], cc.bind(1), outs[:2])   # not contiguous: no bank
         em.install(ctx)
+        ctx.set_matvec_engine(engine)
         ctx.upload_weights(0, image)
         ctx.put(1, fx.synth_activation(1, hidden, fx.F16, config=1, tensor=41))
         total = sum(member_rows)

@@ -18,6 +18,16 @@ def ctx():
     c.close()
 
 
+@pytest.fixture
+def vector_ctx(ctx):
+    """The module's context on the vector-ALU kernels: comparisons that are bit for bit between a fused kernel and
+    its staged pair hold there; under AUTO an affine matrix from 1M weights takes the single-pass matrix-core
+    kernel, whose order of accumulation differs (same tolerance against the oracle)."""
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)
+    yield ctx
+    ctx.set_matvec_engine(rt.MATVEC_AUTO)
+
+
 def run_affine(ctx, packed, scales, biases, x_bits, dtype, entry, *, residual=None, grid=None,
                tg=256, generic=False, batched=False, batch_tile=8):
     rows, cols = packed.shape[0], packed.shape[1] * 2
@@ -200,7 +210,8 @@ def test_signed_fused_add_and_gate_up_equal_staged(ctx, fmt, name):
     assert diff.max() <= 1, diff.max()
 
 
-def test_affine_gate_up_swiglu_and_dual(ctx):
+def test_affine_gate_up_swiglu_and_dual(vector_ctx):
+    ctx = vector_ctx
     rows, cols, group = 3584, 1024, 64
     dtype = fx.F16
     gw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=4)

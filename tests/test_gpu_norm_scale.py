@@ -26,6 +26,16 @@ def ctx():
     c.close()
 
 
+@pytest.fixture
+def vector_ctx(ctx):
+    """The module's context on the vector-ALU kernels: comparisons that are bit for bit between a fused kernel and
+    its staged pair hold there; under AUTO an affine matrix from 1M weights takes the single-pass matrix-core
+    kernel, whose order of accumulation differs (same tolerance against the oracle)."""
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)
+    yield ctx
+    ctx.set_matvec_engine(rt.MATVEC_AUTO)
+
+
 def norm_inputs(batch, cols, dtype, seed):
     rng = np.random.default_rng(seed)
     x = fx.to_bits(rng.normal(0, 2.0, (batch, cols)).astype(np.float32), dtype)
@@ -58,7 +68,8 @@ def run_norm_scale_matvec(ctx, weights, x, w, rs, dtype, entry, consts, batch_ti
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 @pytest.mark.parametrize("rows,cols,group", [(2048, 1536, 128), (777, 1056, 32), (6144, 1024, 64)])
-def test_norm_scale_matvec_equals_staged_pair(ctx, dtype, rows, cols, group):
+def test_norm_scale_matvec_equals_staged_pair(vector_ctx, dtype, rows, cols, group):
+    ctx = vector_ctx
     weights = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=3)
     x, w, rs = norm_inputs(1, cols, dtype, seed=rows)
     xn_ref = so.norm_scale_input(x[0], rs[0], w, dtype)
@@ -116,7 +127,8 @@ def run_gate_up(ctx, gw, uw, dtype, entry, consts, x, norm=None):
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 @pytest.mark.parametrize("act", ["swiglu", "geglu"])
-def test_norm_scale_gate_up_equals_staged_pair(ctx, dtype, act):
+def test_norm_scale_gate_up_equals_staged_pair(vector_ctx, dtype, act):
+    ctx = vector_ctx
     rows, cols, group = 3584, 1024, 64
     gw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=4)
     uw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=5)
@@ -362,10 +374,11 @@ def test_norm_scale_dual_matvec_per_token(ctx, rows):
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 @pytest.mark.parametrize("threads", [64, 256])
-def test_norm_fused_into_matvec_and_gate_up(ctx, dtype, threads):
+def test_norm_fused_into_matvec_and_gate_up(vector_ctx, dtype, threads):
     """atomic_norm_affine_matvec / _gate_up_swiglu (fused_norm_matvec.metal:19-297): the norm's scale is
     computed inside the consumer.  The scale lands in scratch[0] with the ready flag in scratch[1]; the
     stored row and the products equal the scale-only + norm-scale pair run with that scale."""
+    ctx = vector_ctx
     rows, cols, group = 1024, 2048, 64
     weights = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=8)
     uw = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=9)
