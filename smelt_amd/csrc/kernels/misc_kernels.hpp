@@ -220,4 +220,36 @@ extern "C" __global__ __launch_bounds__(256) void smelt_read_u128(const smelt::u
     }
     if (first < n16) dst[first] = acc;
 }
+
+// The same read with the streaming (non-temporal) hint the weight kernels use and U loads in flight
+// per thread, and without the per-thread store of read_u128 (8 MB of writes per launch at 2048 workgroups).  Together with the launch grid (workgroups per compute unit) these are the knobs of a
+// reader; the benchmark sweeps them to find what the memory system hands a kernel at each launch size.
+template <int U>
+__device__ __forceinline__ void smelt_read_stream(const smelt::uint4_t* __restrict__ src, smelt::uint4_t* __restrict__ dst, uint32_t n16) {
+    const uint32_t stride = gridDim.x * blockDim.x, first = blockIdx.x * blockDim.x + threadIdx.x;
+    smelt::uint4_t acc = {0u, 0u, 0u, 0u};
+    uint32_t i = first;
+    for (; i + (U - 1) * stride < n16; i += U * stride) {
+        smelt::uint4_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < U; ++u) { acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w; }
+    }
+    for (; i < n16; i += stride) {
+        const smelt::uint4_t a = __builtin_nontemporal_load(src + i);
+        acc.x ^= a.x; acc.y ^= a.y; acc.z ^= a.z; acc.w ^= a.w;
+    }
+    // a reader writes nothing: the store below keeps the loads alive and (almost) never executes
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5EED1E55u && first < n16) dst[first] = acc;
+}
+extern "C" __global__ __launch_bounds__(256) void smelt_read_u128_nt4(const smelt::uint4_t* __restrict__ src, smelt::uint4_t* __restrict__ dst, uint32_t n16) {
+    smelt_read_stream<4>(src, dst, n16);
+}
+extern "C" __global__ __launch_bounds__(256) void smelt_read_u128_nt8(const smelt::uint4_t* __restrict__ src, smelt::uint4_t* __restrict__ dst, uint32_t n16) {
+    smelt_read_stream<8>(src, dst, n16);
+}
+extern "C" __global__ __launch_bounds__(256) void smelt_read_u128_nt16(const smelt::uint4_t* __restrict__ src, smelt::uint4_t* __restrict__ dst, uint32_t n16) {
+    smelt_read_stream<16>(src, dst, n16);
+}
 #endif

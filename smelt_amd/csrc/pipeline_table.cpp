@@ -853,6 +853,9 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
     if (entry == "signed_normalize_mlx_scales") { out->family = kFamSignedMlxScales; out->symbol = "smelt_signed_normalize_mlx_scales"; out->kinds = "PPPPUU"; return kResolveOk; }
     if (entry == "copy_u128") { out->family = kFamCopy; out->symbol = "smelt_copy_u128"; out->kinds = "PPU"; return kResolveOk; }
     if (entry == "read_u128") { out->family = kFamCopy; out->symbol = "smelt_read_u128"; out->kinds = "PPU"; return kResolveOk; }
+    if (entry == "read_u128_nt4" || entry == "read_u128_nt8" || entry == "read_u128_nt16") {
+        out->family = kFamCopy; out->symbol = "smelt_" + entry; out->kinds = "PPU"; return kResolveOk;
+    }
     if (entry == "argmax_key_reduce") { out->family = kFamArgmaxReduce; out->symbol = "smelt_argmax_key_reduce"; out->kinds = "PPU"; return kResolveOk; }
 
     *why = "no HIP kernel named '" + entry + "'";
