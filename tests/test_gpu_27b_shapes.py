@@ -1,7 +1,7 @@
 """GPU parity at the full 27B-layer shapes (hidden 5120, FFN 17408): every weight format through the
-kernel a package gets by default (AUTO engine: the single-pass matrix-core matvec for affine u4, binary
-and ternary; the vector kernels for trit5) against the OpenMP oracle, plain matvec, +residual and fused
-gate+up where the shape has one.  Seeded tensors as the benchmark's configurations 2 and 3 draw them."""
+kernel a package gets by default (AUTO engine: the single-pass matrix-core matvec for affine u4, binary,
+ternary and trit5) against the OpenMP oracle, plain matvec, +residual and fused gate+up where the shape
+has one.  Seeded tensors as the benchmark's configurations 2 and 3 draw them."""
 import numpy as np
 import pytest
 
@@ -67,7 +67,7 @@ def test_signed_27b_shapes(ctx, fmt, name, shape):
     y = run_signed(ctx, name, packed, scales, x, dtype, rows, cols)
     worst = gh.check_outputs(y, ref, dtype, f"{name} {shape}")
     print(f"\n  {name} {shape} max rel err {worst:.2e}")
-    if shape == (F, H) and fmt != fx.TRIT5:   # gate and up share the input: the fused SwiGLU form
+    if shape == (F, H):   # gate and up share the input: the fused SwiGLU form
         up = signed_tensor(fmt, rows, cols, 2)
         u_ref = so.signed_matvec(fmt, *up, xf, rows, cols, cols, 128, threads=True)
         u = run_signed(ctx, name, *up, x, dtype, rows, cols)

@@ -5,6 +5,7 @@ import pytest
 
 import fixtures as fx
 import gpu_harness as gh
+from gpu_harness import SIGNED_SWIGLU_STEPS
 from oracle import oracle as so
 from smelt_amd import compiler as cc
 from smelt_amd import runtime as rt
@@ -70,7 +71,7 @@ def test_affine_decode_table_eager_and_graph(dtype):
         g = so.affine_matvec(*tensors["gate"], xf, ffn, hidden, group, dtype)
         u = so.affine_matvec(*tensors["up"], xf, ffn, hidden, group, dtype)
         act_ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, dtype), dtype)
-        gh.check_outputs(act.reshape(1, -1), act_ref, dtype, "gate_up", rel_tol=4e-3)
+        gh.check_outputs(act.reshape(1, -1), gh.swiglu_unrounded(g, u), dtype, "gate_up")
         # downstream references consume the GPU's own upstream bits, as the next kernel does
         d = so.affine_matvec(*tensors["down"], fx.from_bits(act.reshape(1, -1), dtype), hidden, ffn, group, dtype)
         out_ref = fx.from_bits(so.epilogue_residual_add(d, res, dtype), dtype)
@@ -141,8 +142,7 @@ def test_signed_layer_table_decode_and_prefill(wdtype):
         g = so.narrow(so.signed_matvec(ofmt, *t["gate"], xf[:1], ffn, hidden, hidden, 128), fx.F16)
         u = so.narrow(so.signed_matvec(ofmt, *t["up"], xf[:1], ffn, hidden, hidden, 128), fx.F16)
         act = ctx.read(FFN_SLOT, np.uint16, ffn)
-        act_ref = fx.from_bits(so.epilogue_signed_swiglu(g, u, so.F16), fx.F16)
-        gh.check_outputs(act.reshape(1, -1), act_ref, fx.F16, "signed gate_up", rel_tol=6e-3)
+        gh.check_steps(act.reshape(1, -1), so.epilogue_signed_swiglu(g, u, so.F16).reshape(1, -1), fx.F16, "signed gate_up", max_steps=SIGNED_SWIGLU_STEPS)
         d = so.signed_matvec(ofmt, *t["down"], fx.from_bits(act.reshape(1, -1), fx.F16), hidden, ffn, ffn, 128)
         out_ref = fx.from_bits(so.epilogue_residual_add(d, res, so.F16), fx.F16)
         gh.check_outputs(ctx.read(OUT_SLOT, np.uint16, hidden).reshape(1, -1), out_ref, fx.F16, "down+add")

@@ -248,7 +248,8 @@ def test_whole_layer_record_list_eager_and_graph():
         assert ctx.interpret_decode(table) == 6
         ctx.wait()
         eager_h, eager_qkv = ctx.read(H, np.uint16, hidden), ctx.read(QKV, np.uint16, 3072)
-        gh.check_outputs(eager_qkv, so.widen(ref_qkv, odt), dtype, "layer q/k/v", rel_tol=8e-3)
+        # the normed row feeding q/k/v can sit one step of the 16-bit type from the oracle's (sum of squares in another order)
+        gh.check_steps(eager_qkv, np.asarray(ref_qkv).reshape(np.shape(eager_qkv)), dtype, "layer q/k/v", max_steps=2, min_exact=0.9)
         # six chained kernels with bf16 values between them: a last-place flip of one activation
         # moves every downstream sum a little, so the end of the chain is compared in norm
         gh_, rh = fx.from_bits(eager_h, dtype).astype(np.float64), so.widen(ref_h, odt).astype(np.float64)

@@ -143,8 +143,10 @@ def test_norm_scale_gate_up_equals_staged_pair(vector_ctx, dtype, act):
     g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
     u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
     epi = so.epilogue_affine_swiglu if act == "swiglu" else so.epilogue_geglu
-    ref = fx.from_bits(epi(g, u, dtype), dtype)
-    gh.check_outputs(fused, ref, dtype, f"norm_scale gate_up {act}", rel_tol=4e-3 if dtype == fx.F16 else 1.6e-2)
+    if act == "swiglu":
+        gh.check_outputs(fused, gh.swiglu_unrounded(g, u), dtype, f"norm_scale gate_up {act}")
+    else:   # GeGLU rounds gate and up to the 16-bit type before the activation: counted in output steps
+        gh.check_steps(fused, epi(g, u, dtype).reshape(np.shape(fused)), dtype, f"norm_scale gate_up {act}", max_steps=gh.GEGLU_STEPS)
 
 
 def test_geglu_fixed_name_and_clamps(ctx):
@@ -240,10 +242,12 @@ def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
         rs2 = float(ctx.read(SCR, np.float32, 1)[0])
         assert abs(rs2 - rs) <= 2e-6 * rs and ctx.read(SCR, np.uint32, 2)[1] == 1
         assert np.array_equal(ctx.read(XN2, np.uint16, hidden), so.norm_scale_input(x[0], rs2, w, dtype))
-        gh.check_outputs(ctx.read(Q3, np.uint16, rows).reshape(1, rows), fx.from_bits(ctx.read(Q, np.uint16, rows), dtype).reshape(1, rows),
-                         dtype, "fused norm matvec against the pair", rel_tol=4e-3 if dtype == fx.F16 else 1.6e-2)
-        gh.check_outputs(ctx.read(F4, np.uint16, ffn).reshape(1, ffn), fx.from_bits(ctx.read(F1, np.uint16, ffn), dtype).reshape(1, ffn),
-                         dtype, "fused norm gate+up against the pair", rel_tol=4e-3 if dtype == fx.F16 else 1.6e-2)
+        # the consumer forms the norm scale itself (another summation order): a staged activation can sit one
+        # step of the 16-bit type away, which moves an output by whole steps too
+        gh.check_steps(ctx.read(Q3, np.uint16, rows).reshape(1, rows), ctx.read(Q, np.uint16, rows).reshape(1, rows),
+                       dtype, "fused norm matvec against the pair", max_steps=2, min_exact=0.9)
+        gh.check_steps(ctx.read(F4, np.uint16, ffn).reshape(1, ffn), ctx.read(F1, np.uint16, ffn).reshape(1, ffn),
+                       dtype, "fused norm gate+up against the pair", max_steps=2, min_exact=0.9)
     finally:
         ctx.close()
 
@@ -315,7 +319,10 @@ def test_norm_scale_gate_up_qmm_and_geglu_qmm(ctx, act):
     g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
     u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
     epi = so.epilogue_affine_swiglu if act == "swiglu" else so.epilogue_geglu
-    gh.check_outputs(fused, fx.from_bits(epi(g, u, dtype), dtype), dtype, f"gate_up {act} qmm", rel_tol=4e-3)
+    if act == "swiglu":
+        gh.check_outputs(fused, gh.swiglu_unrounded(g, u), dtype, f"gate_up {act} qmm")
+    else:
+        gh.check_steps(fused, epi(g, u, dtype).reshape(np.shape(fused)), dtype, f"gate_up {act} qmm", max_steps=gh.GEGLU_STEPS)
 
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])

@@ -118,7 +118,7 @@ def test_affine_qmm_fused_add_and_gate_up(ctx):
     g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
     u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
     ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, so.F16), fx.F16)
-    gh.check_outputs(y, ref, dtype, "qmm gate_up_swiglu", rel_tol=4e-3)
+    gh.check_outputs(y, gh.swiglu_unrounded(g, u), dtype, "qmm gate_up_swiglu")
     assert plain_u.shape == plain.shape
 
 
