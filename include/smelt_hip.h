@@ -253,6 +253,10 @@ int smelt_hip_graph_time(smelt_hip_context *ctx, smelt_hip_graph *graph, int ite
 int smelt_hip_device_info(smelt_hip_context *ctx, char *name, size_t name_cap, int *compute_units,
                           size_t *lds_per_block, size_t *hbm_bytes);
 
+/* Free and total device memory as the runtime reports them (hipMemGetInfo).  No counterpart in the reference;
+ * for callers and tests that must see that an entry point allocated nothing. */
+int smelt_hip_memory_info(smelt_hip_context *ctx, size_t *free_bytes, size_t *total_bytes);
+
 #ifdef __cplusplus
 }
 #endif

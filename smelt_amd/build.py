@@ -52,7 +52,13 @@ def build_kernels() -> list[str]:
         return out
 
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
-        return list(pool.map(one, KERNEL_UNITS))
+        built = list(pool.map(one, KERNEL_UNITS))
+    # the runtime loads exactly the code objects this build made
+    with open(os.path.join(LIB, "smelt_kernels.manifest"), "w") as f:
+        f.write("# code objects of this build, one per line\n")
+        for unit in KERNEL_UNITS:
+            f.write(unit + ".hsaco\n")
+    return built
 
 
 def build_host() -> str:

@@ -108,6 +108,7 @@ struct Arg {
     uint32_t value = 0;
     char* ptr = nullptr;
     size_t avail = 0;  // bytes from ptr to the end of its slot
+    size_t need = 0;   // bytes the pipeline's own kernel touches (set by validate_launch)
     bool writable = false;
 };
 
@@ -130,6 +131,9 @@ struct Launch {
     uint32_t grid[3];
     uint32_t block[3];
     size_t lds = 0;
+    // split-K workspace the pipeline's own kernel needs; checked once the kernel that actually runs is
+    // known (the streaming kernel a skinny record is re-routed to needs none)
+    size_t ws_partial_need = 0, ws_counter_need = 0;
 };
 
 size_t cdiv(size_t a, size_t b) { return (a + b - 1) / b; }
@@ -442,10 +446,8 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
                 const uint32_t ksplit = (uint32_t)(L.grid[0] / tiles);
                 L.lds = qmm_skinny_lds_bytes((uint32_t)cols, ksplit, nmat, (uint32_t)std::min(batch, bt), L.block[0] / 64);
                 if (ksplit > 1) {
-                    if ((size_t)L.grid[0] * gy * nmat * 4096 > ws.partial_bytes || tiles * gy * 4 > ws.counter_bytes)
-                        return bad_geom("split-K partials (" + std::to_string((size_t)L.grid[0] * gy * nmat * 4096) + " bytes, " +
-                                        std::to_string(tiles * gy) + " counters) exceed the workspace (" +
-                                        std::to_string(ws.partial_bytes) + " bytes, " + std::to_string(ws.counter_bytes / 4) + " counters)");
+                    L.ws_partial_need = (size_t)L.grid[0] * gy * nmat * 4096;
+                    L.ws_counter_need = tiles * gy * 4;
                 }
                 break;
             }
@@ -873,6 +875,7 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
         return bad_geom("needs " + std::to_string(L.lds) + " bytes of LDS, device allows " + std::to_string(ctx->lds_limit));
     for (size_t i = 0; i < L.args.size(); ++i) {
         if (L.args[i].kind != 'P') continue;
+        L.args[i].need = need[i];
         if (need[i] > L.args[i].avail)
             return fail(ctx, SMELT_HIP_ERR_OUT_OF_RANGE,
                         "pipeline '" + p.entry + "': argument " + std::to_string(i) + " needs " +
@@ -1077,6 +1080,13 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             if (L.args[i].kind == 'P' && (reinterpret_cast<uintptr_t>(L.args[i].ptr) & 15u)) return false;
         return true;
     };
+    // ... and in whole 16-byte pieces: a plane whose validated extent ends inside a piece (rows * groups * 2
+    // not a multiple of 16) must have the rest of that piece inside its slot as well
+    auto whole_pieces = [&](size_t n) {
+        for (size_t i = 0; i < n && i < L.args.size(); ++i)
+            if (L.args[i].kind == 'P' && ((L.args[i].need + 15) & ~(size_t)15) > L.args[i].avail) return false;
+        return true;
+    };
     if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.grid[1] == 1) {
         // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
         // arguments, its own launch geometry (one workgroup per eight rows)
@@ -1100,7 +1110,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             default: break;
         }
         Mm1Plan plan;
-        if (rows > 0 && aligned16(ro) && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
+        if (rows > 0 && aligned16(ro) && whole_pieces(ro) && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
                                  ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &plan) &&
             p->fn_mm1[plan.nl]) {
             fn = p->fn_mm1[plan.nl];
@@ -1111,7 +1121,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         }
     }
     if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
-        aligned16(p->res.family == kFamAffineQmmGateUp ? 7 : 4)) {
+        aligned16(p->res.family == kFamAffineQmmGateUp ? 7 : 4) && whole_pieces(p->res.family == kFamAffineQmmGateUp ? 7 : 4)) {
         // skinny qmm: the streaming kernel of the same pipeline, same arguments, its own launch
         // geometry (16 * rt rows per workgroup, 16 tokens per grid row); it uses no workspace
         const size_t o = p->res.family == kFamAffineQmm ? 5 : (p->res.family == kFamAffineQmmAdd ? 7 : 8);
@@ -1137,6 +1147,11 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             qms_routed = true;
         }
     }
+    if (!qms_routed && (L.ws_partial_need > ws.partial_bytes || L.ws_counter_need > ws.counter_bytes))
+        return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY,
+                    "pipeline '" + p->entry + "': split-K partials (" + std::to_string(L.ws_partial_need) + " bytes, " +
+                        std::to_string(L.ws_counter_need / 4) + " counters) exceed the workspace (" + std::to_string(ws.partial_bytes) +
+                        " bytes, " + std::to_string(ws.counter_bytes / 4) + " counters)");
     if (!routed && p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
         // signed g128 matvec: large matrices run on the matrix cores (same bytes, same arguments + kw)
         const uint32_t rows = L.args[(size_t)p->res.rows_arg].value, cols = L.args[(size_t)p->res.cols_arg].value;
@@ -1312,11 +1327,25 @@ int smelt_hip_module_load_file(smelt_hip_context* ctx, const char* path) {
     if (DIR* dir = opendir(path)) {
         // a directory: every code object of the build in it, in name order
         std::vector<std::string> names;
-        while (const dirent* e = readdir(dir)) {
-            const std::string n = e->d_name;
-            if (n.size() > 6 && n.compare(n.size() - 6, 6, ".hsaco") == 0 && n.compare(0, 13, "smelt_kernels") == 0) names.push_back(n);
-        }
         closedir(dir);
+        // the build writes the list of its code objects next to them: load exactly those, so that a code
+        // object left behind by an older build is never picked up (and never wins a duplicate symbol)
+        {
+            std::ifstream manifest(std::string(path) + "/smelt_kernels.manifest");
+            std::string line;
+            while (manifest && std::getline(manifest, line)) {
+                while (!line.empty() && (line.back() == '\r' || line.back() == ' ')) line.pop_back();
+                if (!line.empty() && line[0] != '#') names.push_back(line);
+            }
+        }
+        if (names.empty()) {   // no manifest: every smelt_kernels*.hsaco of the directory
+            dir = opendir(path);
+            while (const dirent* e = dir ? readdir(dir) : nullptr) {
+                const std::string n = e->d_name;
+                if (n.size() > 6 && n.compare(n.size() - 6, 6, ".hsaco") == 0 && n.compare(0, 13, "smelt_kernels") == 0) names.push_back(n);
+            }
+            if (dir) closedir(dir);
+        }
         if (names.empty()) return fail(ctx, SMELT_HIP_ERR_INVALID_PACKAGE, std::string("no smelt_kernels*.hsaco under '") + path + "'");
         std::sort(names.begin(), names.end());
         for (const std::string& n : names)
@@ -1334,9 +1363,14 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
     if (!ctx || !entry) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or entry");
     if (ctx->modules.empty()) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "load a code object before creating pipelines");
     // a kernel lives in exactly one of the loaded code objects
+    std::vector<hipModule_t> modules;
+    {
+        std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);   // smelt_hip_module_load appends under this lock
+        modules = ctx->modules;
+    }
     auto find = [&](hipFunction_t* fn, const std::string& symbol) {
         hipError_t last = hipErrorNotFound;
-        for (hipModule_t m : ctx->modules) {
+        for (hipModule_t m : modules) {
             last = hipModuleGetFunction(fn, m, symbol.c_str());
             if (last == hipSuccess) break;
         }
@@ -1364,15 +1398,16 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
             if (!p.res.mm1_prefix.empty())
                 for (uint32_t nl = 1; nl <= kMm1MaxSegments; ++nl)
                     (void)find(&p.fn_mm1[nl], p.res.mm1_prefix + "nl" + std::to_string(nl) + "_" + p.res.mm1_tail);
-            if (!p.res.qms_tail.empty())
-                for (uint32_t rt = 1; rt <= 4; ++rt)
-                    for (uint32_t tb = 2; tb <= 4; tb += 2)
-                        for (uint32_t kw = 1; kw <= 2; ++kw)
-                        {
-                            const std::string rest = std::to_string(rt) + "_t" + std::to_string(tb) + "_k" + std::to_string(kw) + "_" + p.res.qms_tail;
-                            (void)find(&p.fn_qmt[rt][tb][kw], "smelt_affine_qmt_r" + rest);
-                            (void)find(&p.fn_qmt_per_wave[rt][tb][kw], "smelt_affine_qmt_w" + rest);
-                        }
+            if (!p.res.qms_tail.empty()) {
+                // the variants qmt_plan can return: (row tiles, token blocks, waves along K), one matrix per wave or not
+                static const struct { uint32_t rt, tb, kw; bool per_wave; } kQmtVariants[] = {
+                    {2, 2, 2, false}, {3, 2, 2, false}, {2, 2, 1, false}, {3, 2, 2, true}};
+                for (const auto& v : kQmtVariants) {
+                    const std::string rest = std::to_string(v.rt) + "_t" + std::to_string(v.tb) + "_k" + std::to_string(v.kw) + "_" + p.res.qms_tail;
+                    if (v.per_wave) (void)find(&p.fn_qmt_per_wave[v.rt][v.tb][v.kw], "smelt_affine_qmt_w" + rest);
+                    else (void)find(&p.fn_qmt[v.rt][v.tb][v.kw], "smelt_affine_qmt_r" + rest);
+                }
+            }
             if (!p.res.qms_tail.empty())
                 for (uint32_t rt = 1; rt <= kQmsMaxRowTiles; ++rt)
                     for (uint32_t wide = 0; wide < 2; ++wide)
@@ -1642,6 +1677,16 @@ int smelt_hip_device_info(smelt_hip_context* ctx, char* name, size_t name_cap, i
     if (compute_units) *compute_units = ctx->props.multiProcessorCount;
     if (lds_per_block) *lds_per_block = ctx->lds_limit;
     if (hbm_bytes) *hbm_bytes = ctx->props.totalGlobalMem;
+    return SMELT_HIP_OK;
+}
+
+int smelt_hip_memory_info(smelt_hip_context* ctx, size_t* free_bytes, size_t* total_bytes) {
+    if (!ctx) return fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    size_t f = 0, t = 0;
+    HIP_TRY(ctx, hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
     return SMELT_HIP_OK;
 }
 

@@ -8,6 +8,7 @@
 // kernel, a fill or a copy.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 
@@ -24,7 +25,7 @@ constexpr int kMaxDevices = 64;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 // device address of `scratch` on each device, filled by static_scratch_prepare
-void* g_scratch_ptr[kMaxDevices] = {};
+std::atomic<void*> g_scratch_ptr[kMaxDevices] = {};
 std::mutex g_scratch_mutex;
 
 __global__ __launch_bounds__(256) void smelt_static_scratch_fill(uint32_t* words, uint32_t count, uint32_t value) {
@@ -51,7 +52,7 @@ int static_scratch_prepare(int device, hipStream_t stream, std::string* why) {
         return SMELT_HIP_ERR_INVALID_ARGUMENT;
     }
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (g_scratch_ptr[device]) return SMELT_HIP_OK;
+    if (g_scratch_ptr[device].load(std::memory_order_acquire)) return SMELT_HIP_OK;
     // the caller has made `device` current
     void* ptr = nullptr;
     hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
@@ -65,7 +66,7 @@ int static_scratch_prepare(int device, hipStream_t stream, std::string* why) {
         *why = std::string("clearing the static scratch: ") + hipGetErrorString(e);
         return SMELT_HIP_ERR_HIP;
     }
-    g_scratch_ptr[device] = ptr;
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
     return SMELT_HIP_OK;
 }
 
@@ -78,19 +79,21 @@ int smelt_hip_encode_prefill_record_static_scratch(smelt_hip_context* ctx, const
     using namespace smelt_host;
     if (!ctx || !rec) return context_fail(ctx, SMELT_HIP_ERR_INVALID_ARGUMENT, "null context or record");
     const int device = context_device(ctx);
-    void* base = device >= 0 && device < kMaxDevices ? g_scratch_ptr[device] : nullptr;
+    void* base = device >= 0 && device < kMaxDevices ? g_scratch_ptr[device].load(std::memory_order_acquire) : nullptr;
     if (!base) return context_fail(ctx, SMELT_HIP_ERR_HIP, "the static scratch was not set up on this device");
+    {
+        const hipError_t e = hipSetDevice(device);   // the array's address belongs to this device
+        if (e != hipSuccess) return context_fail(ctx, SMELT_HIP_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
+    }
     SplitKWorkspace ws;
     ws.counters = base;
     ws.counter_bytes = kCounterBytes;
     ws.partial = static_cast<unsigned char*>(base) + kCounterBytes;
     ws.partial_bytes = kPartialBytes;
-    // The counters must be zero when a split-K launch starts.  A finished launch leaves them so; the
-    // array is shared by everything on this GPU, so they are cleared again here rather than trusted.
-    if (rec->op_kind == SMELT_OP_DISPATCH) {
-        const hipError_t e = clear_counters(ws.counters, kCounterBytes / 4, context_stream(ctx));
-        if (e != hipSuccess) return context_fail(ctx, SMELT_HIP_ERR_HIP, std::string("clearing the static scratch: ") + hipGetErrorString(e));
-    }
+    // The counters must be zero when a split-K launch starts.  They are cleared once per device at set-up and
+    // every split-K kernel leaves the counters it used at zero when it finishes, so a call launches nothing
+    // but the record's own kernel (records that do not split K never touch them).  Calls that overlap on one
+    // GPU share the array and race; that is the caller's to avoid.
     return encode_prefill_with_workspace(ctx, rec, cur, alt, seq_len, start_pos, ws);
 }
 

@@ -142,6 +142,7 @@ def load_library() -> C.CDLL:
         "smelt_hip_graph_time": (i32, [vp, vp, i32, C.POINTER(C.c_float)]),
         "smelt_hip_device_info": (i32, [vp, C.c_char_p, sz, C.POINTER(i32), C.POINTER(sz),
                                         C.POINTER(sz)]),
+        "smelt_hip_memory_info": (i32, [vp, C.POINTER(sz), C.POINTER(sz)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -301,6 +302,12 @@ class Context:
 
     def graph_destroy(self, g) -> None:
         self.lib.smelt_hip_graph_destroy(self.h, g)
+
+    def memory_info(self) -> tuple[int, int]:
+        """(free, total) device bytes as hipMemGetInfo reports them."""
+        free, total = C.c_size_t(), C.c_size_t()
+        self.check(self.lib.smelt_hip_memory_info(self.h, C.byref(free), C.byref(total)))
+        return free.value, total.value
 
     def device_info(self) -> dict:
         name = C.create_string_buffer(256)

@@ -55,6 +55,40 @@ def test_static_scratch_matches_allocated_workspace_twice_in_a_row():
         ctx.close()
 
 
+def test_static_scratch_call_allocates_nothing():
+    """Free device memory (hipMemGetInfo) is the same before and after calls of the allocation-free entry point,
+    and a call launches one kernel: the record's own."""
+    dtype = fx.BF16
+    ctx = rt.Context()
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)
+    try:
+        rows, cols, batch, ksplit = 416, 2560, 13, 4
+        w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=31)
+        x = fx.synth_activation(batch, cols, dtype, config=4, tensor=131)
+        wf = gh.WeightFile()
+        offs = [wf.add(a) for a in w]
+        ctx.upload_weights(0, wf.image())
+        ctx.put(gh.X_SLOT, x)
+        ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+        pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g64_batched_skinny@bf16")
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+        tiles = (rows + 31) // 32
+        rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], (tiles * ksplit, 32, 1), (256, 1, 1),
+                             grid_kinds=(0, rt.GRID_SEQ_LEN_CEIL_DIV, 0))
+        assert ctx.encode_prefill_static_scratch(rec, seq_len=batch) == 1     # first call: whatever lazy set-up there is
+        ctx.wait()
+        free_before, _ = ctx.memory_info()
+        for _ in range(5):
+            assert ctx.encode_prefill_static_scratch(rec, seq_len=batch) == 1
+        ctx.wait()
+        free_after, _ = ctx.memory_info()
+        assert free_after == free_before, (free_before, free_after)
+        ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype)
+        gh.check_outputs(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), ref, dtype, "static scratch after repeated calls")
+    finally:
+        ctx.close()
+
+
 def test_static_scratch_rejects_partials_beyond_its_size():
     dtype = fx.F16
     ctx = rt.Context()
