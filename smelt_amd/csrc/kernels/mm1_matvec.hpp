@@ -264,9 +264,13 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
                 codes[m][i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(mats[m].codes + (size_t)ld_row * row_stride + (size_t)piece * 16));
         }
     }
+    // the epilogue's operand, by every lane of every wave (clamped to the tile's rows): under a branch
+    // the load brings its own wait on everything issued before it, and wave 0 would stage x only
+    // after all its weights have arrived
     uint16_t res = 0;
     if constexpr (Epi::kPrefetch) {
-        if (chunk == 0 && lane < 8 && row0 + lane < rows) res = epi.prefetch(token, row0 + lane);
+        const int rr = row0 + (lane & 7);
+        res = epi.prefetch(token, rr < rows ? rr : rows - 1);
     }
 
     // ---- 4. scales into LDS ----------------------------------------------------------------------------
