@@ -132,7 +132,11 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * (matrices with few tiles and long rows split K across workgroups: partial sums in the
  * workspace, added in a fixed order), VECTOR the split-K or token-slab kernel the record's geometry
  * describes (split-K: partial sums in the workspace).  Results of the alternatives differ in
- * summation order only.  No counterpart in the reference (one kernel per pipeline name there);
+ * summation order only.  Consequence under AUTO: the records of one model run on two summation
+ * orders, e.g. a matvec at one token (matrix-core kernel) and its batched-verify form (vector
+ * kernel) agree to one step of the output type but not bit for bit; a caller that compares such
+ * rows bit for bit pins one engine.  On one engine a fused kernel and the staged pair it
+ * replaces are bit-identical.  No counterpart in the reference (one kernel per pipeline name there);
  * meant for A/B measurement and for tests. */
 enum { SMELT_HIP_MATVEC_AUTO = 0, SMELT_HIP_MATVEC_MATRIX_CORE = 1, SMELT_HIP_MATVEC_VECTOR = 2 };
 int smelt_hip_set_matvec_engine(smelt_hip_context *ctx, int engine);
@@ -141,7 +145,9 @@ int smelt_hip_set_matvec_engine(smelt_hip_context *ctx, int engine);
  * image produced by hipcc --genco, loaded with hipModuleLoadData.  The kernels ship as several
  * code objects (smelt_kernels*.hsaco); load every one of them before creating pipelines. */
 int smelt_hip_module_load(smelt_hip_context *ctx, const void *code_object, size_t bytes);
-/* `path` names one code object, or a directory: then every smelt_kernels*.hsaco in it is loaded. */
+/* `path` names one code object, or a directory: then the code objects its smelt_kernels.manifest
+ * lists (one file name per line, written by the build) are loaded, or, without a manifest, every
+ * smelt_kernels*.hsaco in it. */
 int smelt_hip_module_load_file(smelt_hip_context *ctx, const char *path);
 
 /* pipelineFunction(for:library:) + makePipelineState: SmeltRuntime.swift:6229-6306.
