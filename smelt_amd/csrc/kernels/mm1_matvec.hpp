@@ -179,9 +179,13 @@ __device__ __forceinline__ float quad_sum(float v) {
 
 // One workgroup = one tile of eight rows; its kc waves split K: wave `chunk` owns the 128-byte
 // segments [chunk * NL, chunk * NL + NL) of every row of the tile.
-template <class F, class ActT, class ScaleT, int NMAT, int NL, class Epi>
+// NORM: 0 = x is multiplied as it is; 1 = the norm-scale prologue (what is multiplied is
+// narrow((x * rs[token]) * (1 + weight)), the bits a staged norm would have stored; workgroup 0 also
+// stores that row to ns.out); 2 = the same followed by the residual add of the norm_add_scale form.
+template <class F, class ActT, class ScaleT, int NMAT, int NL, class Epi, int NORM = 0>
 __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint16_t* __restrict__ x_all, int rows,
-                                         int cols, int row_stride, int group, const Epi& epi) {
+                                         int cols, int row_stride, int group, const Epi& epi,
+                                         const NormScale& ns = NormScale{}) {
     using E = Elem16<ActT>;
     constexpr int FPD = F::kFPD, FPL = F::kFPL, FIELDS = F::kFields, PAIRS = F::kPairs, DW = F::kDW;
     constexpr int PSTRIDE = mm1_piece_stride(FPL, DW);     // fragments from one piece to the next in LDS
@@ -245,7 +249,29 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         if (col0 > cols - FIELDS) col0 = cols - FIELDS;   // cols is a multiple of kFields
 #pragma unroll
         for (int v = 0; v < FIELDS / 8; ++v) {
-            const uint4_t t = *reinterpret_cast<const uint4_t*>(x + col0 + 8 * v);
+            uint4_t t = *reinterpret_cast<const uint4_t*>(x + col0 + 8 * v);
+            if constexpr (NORM != 0) {
+                // eight activations through the prologue, each rounded as the staged norm rounds it
+                const float rs = ns.rs[token];
+                const uint4_t w8 = *reinterpret_cast<const uint4_t*>(ns.weight + col0 + 8 * v);
+                uint4_t r8 = uint4_t{0u, 0u, 0u, 0u};
+                if constexpr (NORM == 2) r8 = *reinterpret_cast<const uint4_t*>(ns.residual + (size_t)token * cols + col0 + 8 * v);
+                uint32_t out[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t pair = 0;
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        uint16_t e = norm_scale_value<ActT>((uint16_t)(t[j] >> (16 * h)), rs, (uint16_t)(w8[j] >> (16 * h)));
+                        if constexpr (NORM == 2) e = ActT::narrow(ActT::widen(e) + ActT::widen((uint16_t)(r8[j] >> (16 * h))));
+                        pair |= (uint32_t)e << (16 * h);
+                    }
+                    out[j] = pair;
+                }
+                t = uint4_t{out[0], out[1], out[2], out[3]};
+                // (lanes past the last item hold the last item again and store the same bits again)
+                if (blockIdx.x == 0 && ns.out != nullptr) *reinterpret_cast<uint4_t*>(ns.out + (size_t)token * cols + col0 + 8 * v) = t;
+            }
             xe[k][4 * v] = past ? 0u : t.x; xe[k][4 * v + 1] = past ? 0u : t.y;
             xe[k][4 * v + 2] = past ? 0u : t.z; xe[k][4 * v + 3] = past ? 0u : t.w;
         }
@@ -526,6 +552,81 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         EpiBank4<ACT> epi{{}, {y0, y1, y2, y3}, {rows0, rows1, rows2, rows3}};                    \
         mm1_body<M1U4<ACT>, ACT, SC, 1, NLV>(mats, X, rows0 + rows1 + rows2 + rows3, cols,        \
                                              cols / 2, group, epi);                               \
+    }
+
+// The other fused affine forms of the vector-ALU kernels, same argument lists: two projections of one
+// input, GeGLU, and the norm-scale prologue in front of a projection, a pair or a gate+up.
+#define SMELT_AFFINE_MM1_FUSED(T, ACT, SC, NLV)                                                   \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_dual_matvec_##T(                             \
+        const u8* W1, const u16* S1, const u16* B1, const u8* W2, const u16* S2, const u16* B2,   \
+        const u16* X, u16* y1, u16* y2, u32 rows, u32 cols, u32 group) {                          \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
+        EpiDual<ACT> epi{{}, y1, y2, (int)rows};                                                  \
+        mm1_body<M1U4<ACT>, ACT, SC, 2, NLV>(mats, X, rows, cols, cols / 2, group, epi);          \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_dual_matvec_add_##T(                         \
+        const u8* W1, const u16* S1, const u16* B1, const u8* W2, const u16* S2, const u16* B2,   \
+        const u16* X, u16* y1, u16* y2, const u16* r1, const u16* r2, u32 rows, u32 cols,         \
+        u32 group) {                                                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
+        EpiDualAdd<ACT> epi{{}, y1, y2, r1, r2, (int)rows};                                       \
+        mm1_body<M1U4<ACT>, ACT, SC, 2, NLV>(mats, X, rows, cols, cols / 2, group, epi);          \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_gate_up_geglu_##T(                           \
+        const u8* gW, const u16* gS, const u16* gB, const u8* uW, const u16* uS, const u16* uB,   \
+        const u16* X, u16* Y, u32 rows, u32 cols, u32 group) {                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiGeglu<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<M1U4<ACT>, ACT, SC, 2, NLV>(mats, X, rows, cols, cols / 2, group, epi);          \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_norm_scale_matvec_##T(                       \
+        const float* rs, const u16* X, const u16* nw, u16* xn, const u8* W, const u16* S,         \
+        const u16* B, u16* Y, u32 rows, u32 cols, u32 group) {                                    \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<M1U4<ACT>, ACT, SC, 1, NLV, EpiStore<ACT>, 1>(mats, X, rows, cols, cols / 2, group, epi, \
+                                                               NormScale{rs, nw, xn});            \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_norm_add_scale_matvec_##T(                   \
+        const float* rs, const u16* X, const u16* nw, const u16* res, u16* xn, const u8* W,       \
+        const u16* S, const u16* B, u16* Y, u32 rows, u32 cols, u32 group) {                      \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<M1U4<ACT>, ACT, SC, 1, NLV, EpiStore<ACT>, 2>(mats, X, rows, cols, cols / 2, group, epi, \
+                                                               NormScale{rs, nw, xn, res});       \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_norm_scale_dual_matvec_##T(                  \
+        const float* rs, const u16* X, const u16* nw, const u8* W1, const u16* S1, const u16* B1, \
+        const u8* W2, const u16* S2, const u16* B2, u16* y1, u16* y2, u32 rows, u32 cols,         \
+        u32 group) {                                                                              \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{W1, S1, B1}, {W2, S2, B2}};                                     \
+        EpiDual<ACT> epi{{}, y1, y2, (int)rows};                                                  \
+        mm1_body<M1U4<ACT>, ACT, SC, 2, NLV, EpiDual<ACT>, 1>(mats, X, rows, cols, cols / 2, group, epi, \
+                                                              NormScale{rs, nw, nullptr});        \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_norm_scale_gate_up_swiglu_##T(               \
+        const float* rs, const u16* X, const u16* nw, const u8* gW, const u16* gS, const u16* gB, \
+        const u8* uW, const u16* uS, const u16* uB, u16* Y, u32 rows, u32 cols, u32 group) {      \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiAffineSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        mm1_body<M1U4<ACT>, ACT, SC, 2, NLV, EpiAffineSwiglu<ACT>, 1>(mats, X, rows, cols, cols / 2, group, \
+                                                                      epi, NormScale{rs, nw, nullptr}); \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_norm_scale_gate_up_geglu_##T(                \
+        const float* rs, const u16* X, const u16* nw, const u8* gW, const u16* gS, const u16* gB, \
+        const u8* uW, const u16* uS, const u16* uB, u16* Y, u32 rows, u32 cols, u32 group) {      \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gW, gS, gB}, {uW, uS, uB}};                                     \
+        EpiGeglu<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<M1U4<ACT>, ACT, SC, 2, NLV, EpiGeglu<ACT>, 1>(mats, X, rows, cols, cols / 2, group, epi, \
+                                                               NormScale{rs, nw, nullptr});       \
     }
 
 // Ternary "affine" pipelines bind the scale plane a second time where MLX binds a bias plane; it

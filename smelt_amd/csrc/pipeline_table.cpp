@@ -213,6 +213,14 @@ void attach_mm1(ResolvedPipeline* r) {
         {"smelt_affine_matvec_add_", "smelt_affine_mm1_", "matvec_add_", kCodesU4, 1},
         {"smelt_affine_gate_up_swiglu_", "smelt_affine_mm1_", "gate_up_swiglu_", kCodesU4, 2},
         {"smelt_affine_bank4_matvec_", "smelt_affine_mm1_", "bank4_matvec_", kCodesU4, 1},
+        {"smelt_affine_dual_matvec_", "smelt_affine_mm1_", "dual_matvec_", kCodesU4, 2},
+        {"smelt_affine_dual_matvec_add_", "smelt_affine_mm1_", "dual_matvec_add_", kCodesU4, 2},
+        {"smelt_affine_gate_up_geglu_", "smelt_affine_mm1_", "gate_up_geglu_", kCodesU4, 2},
+        {"smelt_norm_scale_affine_matvec_", "smelt_affine_mm1_", "norm_scale_matvec_", kCodesU4, 1},
+        {"smelt_norm_add_scale_affine_matvec_", "smelt_affine_mm1_", "norm_add_scale_matvec_", kCodesU4, 1},
+        {"smelt_norm_scale_affine_dual_matvec_", "smelt_affine_mm1_", "norm_scale_dual_matvec_", kCodesU4, 2},
+        {"smelt_norm_scale_affine_gate_up_swiglu_", "smelt_affine_mm1_", "norm_scale_gate_up_swiglu_", kCodesU4, 2},
+        {"smelt_norm_scale_affine_gate_up_geglu_", "smelt_affine_mm1_", "norm_scale_gate_up_geglu_", kCodesU4, 2},
         {"smelt_signed_binary_matvec_", "smelt_signed_binary_mm1_", "matvec_", kCodesBinary1, 1},
         {"smelt_signed_binary_matvec_add_", "smelt_signed_binary_mm1_", "matvec_add_", kCodesBinary1, 1},
         {"smelt_signed_binary_gate_up_swiglu_", "smelt_signed_binary_mm1_", "gate_up_swiglu_", kCodesBinary1, 2},

@@ -1075,15 +1075,15 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     // the re-routed kernels fetch codes, scales, biases and activations 16 bytes at a time: the
     // first `n` arguments (the read-only operands) have to sit on 16-byte boundaries, as the layouts
     // the library writes do; a record that binds them elsewhere keeps the kernel its name describes
-    auto aligned16 = [&](size_t n) {
-        for (size_t i = 0; i < n && i < L.args.size(); ++i)
+    auto aligned16 = [&](size_t n, size_t first = 0) {
+        for (size_t i = first; i < n && i < L.args.size(); ++i)
             if (L.args[i].kind == 'P' && (reinterpret_cast<uintptr_t>(L.args[i].ptr) & 15u)) return false;
         return true;
     };
     // ... and in whole 16-byte pieces: a plane whose validated extent ends inside a piece (rows * groups * 2
     // not a multiple of 16) must have the rest of that piece inside its slot as well
-    auto whole_pieces = [&](size_t n) {
-        for (size_t i = 0; i < n && i < L.args.size(); ++i)
+    auto whole_pieces = [&](size_t n, size_t first = 0) {
+        for (size_t i = first; i < n && i < L.args.size(); ++i)
             if (L.args[i].kind == 'P' && ((L.args[i].need + 15) & ~(size_t)15) > L.args[i].avail) return false;
         return true;
     };
@@ -1092,8 +1092,17 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         // arguments, its own launch geometry (one workgroup per eight rows)
         uint32_t rows = 0, cols = 0, group = 128;
         size_t ro = 0;   // leading read-only operands (codes, scales[, biases], ..., x)
+        size_t skip = 0; // ... behind this many leading arguments that are not fetched 16 bytes at a time
         auto U = [&](size_t i) { return L.args[i].value; };
         switch (p->res.family) {
+            case kFamAffineDual: rows = U(9); cols = U(10); group = U(11); ro = 7; break;
+            case kFamAffineDualAdd: rows = U(11); cols = U(12); group = U(13); ro = 7; break;
+            // norm-scale prologue: the fp32 scale comes first; x, the norm weight, [the residual,] the
+            // normalised row (stored 16 bytes at a time by workgroup 0) and the planes follow
+            case kFamNormScaleAffineMatvec: rows = U(8); cols = U(9); group = U(10); skip = 1; ro = 6; break;
+            case kFamNormAddScaleAffineMatvec: rows = U(9); cols = U(10); group = U(11); skip = 1; ro = 7; break;
+            case kFamNormScaleAffineDual: rows = U(11); cols = U(12); group = U(13); skip = 1; ro = 8; break;
+            case kFamNormScaleAffineGateUp: rows = U(10); cols = U(11); group = U(12); skip = 1; ro = 8; break;
             case kFamAffineMatvec: rows = U(5); cols = U(6); group = U(7); ro = 4; break;
             case kFamAffineAdd: rows = U(6); cols = U(7); group = U(8); ro = 4; break;
             case kFamAffineGateUp: rows = U(8); cols = U(9); group = U(10); ro = 7; break;
@@ -1110,7 +1119,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             default: break;
         }
         Mm1Plan plan;
-        if (rows > 0 && aligned16(ro) && whole_pieces(ro) && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
+        if (rows > 0 && aligned16(skip + ro, skip) && whole_pieces(skip + ro, skip) && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
                                  ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &plan) &&
             p->fn_mm1[plan.nl]) {
             fn = p->fn_mm1[plan.nl];

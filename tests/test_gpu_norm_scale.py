@@ -28,9 +28,9 @@ def ctx():
 
 @pytest.fixture
 def vector_ctx(ctx):
-    """The module's context on the vector-ALU kernels: comparisons that are bit for bit between a fused kernel and
-    its staged pair hold there; under AUTO an affine matrix from 1M weights takes the single-pass matrix-core
-    kernel, whose order of accumulation differs (same tolerance against the oracle)."""
+    """The module's context on the vector-ALU kernels: a fused kernel and its staged pair are bit for bit equal on
+    one engine (tests/test_gpu_mm1_fused.py makes the same comparisons on the matrix cores); a per-token batched
+    form runs the vector kernel whatever the engine, so comparing it with a single-token record needs this."""
     ctx.set_matvec_engine(rt.MATVEC_VECTOR)
     yield ctx
     ctx.set_matvec_engine(rt.MATVEC_AUTO)
@@ -87,8 +87,11 @@ def test_norm_scale_matvec_equals_staged_pair(vector_ctx, dtype, rows, cols, gro
 
 
 @pytest.mark.parametrize("batch,tile", [(3, 8), (8, 8), (11, 8)])
-def test_norm_scale_matvec_batched_rows_use_their_own_scale(ctx, batch, tile):
-    """Per-token scale scalePtr[token] (lut_matvec.metal:4318-4322); every row equals the batch-1 kernel."""
+def test_norm_scale_matvec_batched_rows_use_their_own_scale(vector_ctx, batch, tile):
+    """Per-token scale scalePtr[token] (lut_matvec.metal:4318-4322); every row equals the batch-1 kernel (on one
+    engine: under AUTO the batch-1 record of this 5M-weight matrix takes the matrix-core kernel and the token tiles
+    the vector kernel, equal to one output step only)."""
+    ctx = vector_ctx
     rows, cols, group, dtype = 2048, 2560, 128, fx.F16
     weights = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=1)
     x, w, rs = norm_inputs(batch, cols, dtype, seed=batch)
