@@ -19,7 +19,7 @@ LIB = os.path.join(HERE, "lib")
 HSACO = os.path.join(LIB, "smelt_kernels.hsaco")
 # every translation unit under csrc/kernels becomes one code object; the runtime loads them all
 KERNEL_UNITS = ["smelt_kernels", "smelt_kernels_batched_f16", "smelt_kernels_batched_bf16",
-                "smelt_kernels_signed", "smelt_kernels_planes", "smelt_kernels_mfma", "smelt_kernels_qmm",
+                "smelt_kernels_signed", "smelt_kernels_planes", "smelt_kernels_qmm",
                 "smelt_kernels_layer", "smelt_kernels_mm1", "smelt_kernels_mm1f", "smelt_kernels_qms", "smelt_kernels_qmt"]
 HOST_LIB = os.path.join(LIB, "libsmelt_hip.so")
 

@@ -109,34 +109,6 @@ size_t qmm_skinny_lds_bytes(uint32_t cols, uint32_t ksplit, uint32_t nmat, uint3
     return stage > reduce ? stage : reduce;
 }
 
-size_t mfma_matvec_lds_bytes(CodeLayout layout, uint32_t cols, uint32_t tokens, uint32_t nmat, uint32_t waves, uint32_t kw) {
-    // operand fragments [windows][fragments per window][tokens] x 16 B (tokens rounded up to a
-    // power of two, at most 8), one zero slot, per-window corrections (and activation sums for
-    // affine) for 8 token slots, wave partials when K is split over waves, then (1 KB aligned) the
-    // code rings: two 4 KB items per wave and matrix
-    const uint32_t window = layout == kCodesU4 ? 64 : 128, frags = layout == kCodesU4 ? 8 : 16;
-    uint32_t shift = 0;
-    while ((1u << shift) < tokens && shift < 3) ++shift;
-    const size_t nwin = cols / window;
-    size_t bytes = ((nwin * frags * 16) << shift) + 16 + nwin * 32 * (layout == kCodesU4 ? 2 : 1);
-    if (kw > 1) bytes += (size_t)waves * nmat * 1024;
-    return ((bytes + 1023) & ~(size_t)1023) + (size_t)waves * nmat * 2 * 4096;
-}
-
-uint32_t mfma_matvec_kw(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t tokens, uint32_t nmat, size_t lds_limit) {
-    // One scale group per window and whole ring items (128 bytes per row) along K; matrices under
-    // 8M weights are latency-bound and gain nothing from it.
-    if (layout != kCodesU4 && layout != kCodesTernary2 && layout != kCodesBinary1) return 0;
-    const uint32_t window = layout == kCodesU4 ? 64 : 128;
-    const uint32_t item_cols = layout == kCodesU4 ? 256 : (layout == kCodesTernary2 ? 512 : 1024);
-    if (group != window || cols == 0 || cols % item_cols != 0 || (uint64_t)rows * cols < (8u << 20)) return 0;
-    const uint32_t tiles = (rows + 31) / 32, items = cols / item_cols;
-    uint32_t kw = tiles >= 2048 ? 1 : (tiles >= 1024 ? 2 : 4);
-    while (kw > items) kw /= 2;  // every wave of a tile needs at least one item
-    if (mfma_matvec_lds_bytes(layout, cols, tokens, nmat, 4, kw) > lds_limit) return 0;
-    return kw;
-}
-
 uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
     const uint32_t padded = (cols + 127u) / 128u * 128u;
     switch (f) {
@@ -449,19 +421,15 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
             const size_t n_alias = strlen(alias);
             if (suffix.size() >= n_alias && suffix.compare(suffix.size() - n_alias, n_alias, alias) == 0) suffix.resize(suffix.size() - n_alias);
         }
-        // "_mfma" after the variant suffix asks for the matrix-core matvec of the same pipeline
-        bool want_mfma = false;
+        // ("_mfma" after the variant suffix once asked for a ring-buffered matrix-core matvec; that engine is gone,
+        // the single-pass matrix-core kernels are picked per launch under the pipeline's own name)
         if (suffix.size() >= 5 && suffix.compare(suffix.size() - 5, 5, "_mfma") == 0) {
-            want_mfma = true;
-            suffix.resize(suffix.size() - 5);
+            *why = "no HIP kernel for '" + entry + "' (the '_mfma' opt-in names are withdrawn)";
+            return kResolveUnknown;
         }
         // the norm-scale dual kernel's "_batched" form takes its token from grid.y, like the single-token kernels
         const bool m1 = suffix.empty() || suffix == "_rows4" || suffix == "_rows8" || suffix == "_rows4_sg1" ||
                         ((a.m1 == kFamNormScaleAffineDual || a.m1 == kFamAffineDual) && suffix == "_batched");
-        if (want_mfma && mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 2, lds_limit) == 0) {
-            *why = "matrix-core matvec needs group 64, cols % 256 == 0 and at least 8M weights: '" + entry + "'";
-            return kResolveMalformed;
-        }
         uint32_t bt = 0;
         bool full = false, skinny = false;
         if (suffix == "_batched") bt = 8;
@@ -483,14 +451,6 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
             out->single_arg = 5;
             out->kinds = "PPPPPUFUUUU";
             out->appended = {rows, cols, group, bt};
-            if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, 1, 1, lds_limit) : 0) {
-                out->mfma_kw = kw;
-                out->symbol_single.clear();
-                out->single_arg = -1;
-                out->symbol = std::string("smelt_affine_mm_matvec_argmax_") + (kw == 1 ? "stream_" : "split_") + t;
-                out->kinds += "U";
-                out->appended.push_back(kw);
-            }
             return kResolveOk;
         }
         if (m1) {
@@ -510,16 +470,7 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
             if (a.m1 == kFamAffineGateUp && strstr(a.prefix, "geglu")) out->symbol = "smelt_affine_gate_up_geglu_" + t;
             const bool prologue = a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp ||
                                   a.m1 == kFamNormAddScaleAffineMatvec || a.m1 == kFamNormScaleAffineDual;
-            if (prologue && want_mfma) { *why = "no matrix-core form of '" + entry + "'"; return kResolveUnknown; }
             out->appended = {rows, cols, group};
-            const uint32_t nmat = a.m1 == kFamAffineGateUp ? 2 : 1;
-            if (a.m1 != kFamAffineDual && a.m1 != kFamAffineDualAdd && !prologue && !strstr(a.prefix, "geglu"))
-                if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, 1, nmat, lds_limit) : 0) {
-                    out->mfma_kw = kw;
-                    out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_" : (a.m1 == kFamAffineAdd ? "smelt_affine_mm_matvec_add_" : "smelt_affine_mm_gate_up_swiglu_")) + (kw == 1 ? "stream_" : "split_") + t;
-                    out->kinds += "U";
-                    out->appended.push_back(kw);
-                }
             return kResolveOk;
         }
         const bool geglu = strstr(a.prefix, "geglu") != nullptr;
@@ -529,7 +480,7 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
         }
         if (a.m1 == kFamAffineDual) {
             // token tiles of two same-shape projections (fused_dual_affine_matvec_fixed_ext, lut_matvec.metal:3816-3922)
-            if (want_mfma || full || suffix != "_batched_verify_b4") { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
+            if (full || suffix != "_batched_verify_b4") { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
             const uint32_t mbv = pick_mb(kCodesU4, row_stride, 4, lds_limit);
             out->lds_variant = mbv;
             out->family = kFamAffineDualBatched;
@@ -538,7 +489,7 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
             out->appended = {rows, cols, group, bt};
             return kResolveOk;
         }
-        if (a.m1 == kFamAffineGateUp && geglu && !want_mfma && (suffix == "_batched" || suffix == "_batched_bt4_sg4")) {
+        if (a.m1 == kFamAffineGateUp && geglu && (suffix == "_batched" || suffix == "_batched_bt4_sg4")) {
             // small-batch GeGLU (lut_matvec.metal:8342-8364, 8752-8753): token tiles of 3 and 4
             bt = suffix == "_batched" ? 3 : 4;
             const uint32_t mbv = pick_mb(kCodesU4, row_stride, 4, lds_limit);
@@ -552,7 +503,7 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
         if (a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp || geglu) {
             // prologue and GeGLU forms: the MFMA slab kernel for "_batched_full", the vector-ALU
             // token tile for the plain "_batched" matvec, nothing else
-            if (want_mfma || skinny || (!full && a.m1 != kFamNormScaleAffineMatvec)) {
+            if (skinny || (!full && a.m1 != kFamNormScaleAffineMatvec)) {
                 *why = "no batched HIP kernel for '" + entry + "'";
                 return kResolveUnknown;
             }
@@ -603,12 +554,6 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
         else if (a.m1 == kFamAffineGateUp) { out->family = kFamAffineGateUpBatched; out->symbol = "smelt_affine_gate_up_swiglu_batched_" + mbs; out->kinds = "PPPPPPPPUUUUU"; }
         else { *why = "no batched HIP kernel for '" + entry + "'"; return kResolveUnknown; }
         out->appended = {rows, cols, group, bt};
-        if (const uint32_t kw = want_mfma ? mfma_matvec_kw(kCodesU4, rows, cols, group, std::min(bt, 8u), a.m1 == kFamAffineGateUp ? 2 : 1, lds_limit) : 0) {
-            out->mfma_kw = kw;
-            out->symbol = std::string(a.m1 == kFamAffineMatvec ? "smelt_affine_mm_matvec_batched_" : "smelt_affine_mm_gate_up_swiglu_batched_") + (kw == 1 ? "stream_" : "split_") + t;
-            out->kinds += "U";
-            out->appended.push_back(kw);
-        }
         return kResolveOk;
     }
 
@@ -642,18 +587,6 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
             out->format = s.fmt;
             out->symbol = std::string(s.sym) + t;
             out->kinds = s.kinds;
-            // matrix-core variants, chosen per launch from the record's rows and cols
-            const bool add = s.fam == kFamSignedAdd || s.fam == kFamTerAffAdd;
-            if ((s.fam == kFamSignedMatvec || add || s.fam == kFamTerAffMatvec) && s.fmt != kFmtTrit5) {
-                const std::string stem = (s.fam == kFamTerAffMatvec || s.fam == kFamTerAffAdd)
-                                             ? "smelt_teraff_mm_matvec_"
-                                             : std::string("smelt_signed_") + (s.fmt == kFmtBinary1 ? "binary" : "ternary") + "_mm_matvec_";
-                out->symbol_mm_stream = stem + (add ? "add_stream_" : "stream_") + t;
-                out->symbol_mm_split = stem + (add ? "add_split_" : "split_") + t;
-                const int first_const = (int)std::string(s.kinds).find('U');
-                out->rows_arg = first_const;
-                out->cols_arg = first_const + 1;
-            }
             return kResolveOk;
         }
     }

@@ -108,9 +108,6 @@ struct ResolvedPipeline {
                                      // or kSkinnyVariant for the split-K skinny kernels
     std::string symbol_single;       // optional kernel for launches whose batch argument is 1
     int single_arg = -1;             // index of that batch argument
-    std::string symbol_mm_stream, symbol_mm_split;  // optional matrix-core kernels picked per launch by shape
-    int rows_arg = -1, cols_arg = -1;               // where that launch finds rows and cols
-    uint32_t mfma_kw = 0;            // > 0: matrix-core matvec variant, waves that share a row tile
     // Single-pass matrix-core matvec of the same pipeline, picked per launch by shape: the kernel is
     // mm1_prefix + "nl<N>_" + mm1_tail for N segments per wave (empty prefix: the pipeline has none).
     std::string mm1_prefix, mm1_tail;
@@ -136,11 +133,6 @@ ResolveStatus resolve_pipeline(const std::string& entry, ActDType default_act, s
 // Packed-code layouts the matvec kernels consume.
 enum CodeLayout { kCodesU4 = 0, kCodesBinary1 = 1, kCodesTernary2 = 2, kCodesTrit5 = 3 };
 CodeLayout code_layout(SignedFormat f);
-
-// LDS bytes of the matrix-core matvec kernels (affine u4, 64-column windows).
-size_t mfma_matvec_lds_bytes(CodeLayout layout, uint32_t cols, uint32_t tokens, uint32_t nmat, uint32_t waves, uint32_t kw);
-// waves per row tile the matrix-core matvec uses for a shape; 0 when the shape stays on the vector-ALU kernels
-uint32_t mfma_matvec_kw(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t tokens, uint32_t nmat, size_t lds_limit);
 
 // LDS bytes the matvec kernels need for one packed row stride with `mb` resident activation rows.
 size_t matvec_lds_bytes(CodeLayout layout, uint32_t row_stride_bytes, uint32_t mb);

@@ -43,7 +43,6 @@ struct Pipeline {
     bool ready = false;
     hipFunction_t fn = nullptr;
     hipFunction_t fn_single = nullptr;  // used when the record's batch argument is 1
-    hipFunction_t fn_mm_stream = nullptr, fn_mm_split = nullptr;  // matrix-core variants picked by shape
     hipFunction_t fn_mm1[kMm1MaxSegments + 1] = {};               // single-pass matrix-core matvec, by segments per wave
     hipFunction_t fn_qmt[5][5][3] = {};                           // token-tile qmm, by row tiles and token blocks per wave and waves along K
     hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
@@ -198,7 +197,6 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
         if (L.block[0] != 256) return bad_geom("MFMA qmm kernels run with 256-thread workgroups, got " + std::to_string(L.block[0]));
         return 0;
     };
-    size_t mm_cols = 0, mm_tokens = 1, mm_nmat = 1;  // matrix-core matvec variants: LDS is sized after the switch
     switch (r.family) {
         case kFamAffineMatvec:
         case kFamAffineAdd: {
@@ -210,7 +208,6 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
             need[4] = gy * rows * 2; written[4] = true;
             if (r.family == kFamAffineAdd) need[5] = gy * rows * 2;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
-            mm_cols = cols;
             break;
         }
         case kFamAffineGateUp:
@@ -226,7 +223,6 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
             if (r.family != kFamAffineGateUp) { need[8] = gy * rows * 2; written[8] = true; }
             if (r.family == kFamAffineDualAdd) need[9] = need[10] = gy * rows * 2;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
-            mm_cols = cols; mm_nmat = 2;
             break;
         }
         case kFamNormScaleAffineMatvec: {
@@ -355,7 +351,6 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
             need[yi] = batch * rows * 2; written[yi] = true;
             if (r.family == kFamAffineDualBatched) { need[8] = batch * rows * 2; written[8] = true; }
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), r.lds_variant);
-            mm_cols = cols; mm_tokens = std::min<size_t>(8, std::min(batch, bt)); mm_nmat = r.family == kFamAffineGateUpBatched ? 2 : 1;
             break;
         }
         case kFamSignedMatvec:
@@ -403,7 +398,6 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
             need[3] = batch * cols * 2; align[3] = 16;
             need[4] = batch * (size_t)L.grid[0] * 8; align[4] = 8; written[4] = true;
             L.lds = matvec_lds_bytes(kCodesU4, (uint32_t)(cols / 2), 1);
-            mm_cols = cols;  // one token per pass
             break;
         }
         case kFamLmHeadReduce: {
@@ -867,10 +861,6 @@ int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const 
         default:
             return fail(ctx, SMELT_HIP_ERR_UNKNOWN_PIPELINE, "pipeline '" + p.entry + "' has no launch validator");
     }
-    if (r.mfma_kw > 0) {
-        if (L.block[0] != 256) return bad_geom("matrix-core matvec kernels run with 256-thread workgroups, got " + std::to_string(L.block[0]));
-        L.lds = mfma_matvec_lds_bytes(layout, (uint32_t)mm_cols, (uint32_t)std::max<size_t>(mm_tokens, 1), (uint32_t)mm_nmat, 4, r.mfma_kw);
-    }
     if (L.lds > ctx->lds_limit)
         return bad_geom("needs " + std::to_string(L.lds) + " bytes of LDS, device allows " + std::to_string(ctx->lds_limit));
     for (size_t i = 0; i < L.args.size(); ++i) {
@@ -1161,20 +1151,6 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
                     "pipeline '" + p->entry + "': split-K partials (" + std::to_string(L.ws_partial_need) + " bytes, " +
                         std::to_string(L.ws_counter_need / 4) + " counters) exceed the workspace (" + std::to_string(ws.partial_bytes) +
                         " bytes, " + std::to_string(ws.counter_bytes / 4) + " counters)");
-    if (!routed && p->fn_mm_stream && p->res.rows_arg >= 0 && L.block[0] == 256) {
-        // signed g128 matvec: large matrices run on the matrix cores (same bytes, same arguments + kw)
-        const uint32_t rows = L.args[(size_t)p->res.rows_arg].value, cols = L.args[(size_t)p->res.cols_arg].value;
-        const CodeLayout layout = code_layout(p->res.format);
-        if (const uint32_t kw = mfma_matvec_kw(layout, rows, cols, 128, 1, 1, ctx->lds_limit)) {
-            fn = kw == 1 ? p->fn_mm_stream : p->fn_mm_split;
-            L.lds = mfma_matvec_lds_bytes(layout, cols, 1, 1, 4, kw);
-            Arg a;
-            a.kind = 'U';
-            a.value = kw;
-            L.args.push_back(a);
-        }
-    }
-
     // kernarg block: natural alignment in argument order
     alignas(16) unsigned char kernarg[512];
     size_t pos = 0;
@@ -1401,9 +1377,6 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
         } else {
             p.ready = true;
             if (!p.res.symbol_single.empty() && find(&p.fn_single, p.res.symbol_single) != hipSuccess) p.fn_single = nullptr;
-            if (!p.res.symbol_mm_stream.empty() &&
-                (find(&p.fn_mm_stream, p.res.symbol_mm_stream) != hipSuccess || find(&p.fn_mm_split, p.res.symbol_mm_split) != hipSuccess))
-                p.fn_mm_stream = p.fn_mm_split = nullptr;
             if (!p.res.mm1_prefix.empty())
                 for (uint32_t nl = 1; nl <= kMm1MaxSegments; ++nl)
                     (void)find(&p.fn_mm1[nl], p.res.mm1_prefix + "nl" + std::to_string(nl) + "_" + p.res.mm1_tail);

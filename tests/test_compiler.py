@@ -122,7 +122,6 @@ def test_pipeline_names_resolve_to_kernels_with_the_reference_binding_counts():
     cases = {
         "affine_matvec:1024:64": ("smelt_affine_matvec_f16", 5, 1),
         "affine_matvec_c2048_r151936_g64_rows8": ("smelt_affine_matvec_f16", 5, 0),
-        "affine_matvec_c2048_r151936_g64_rows8_mfma": ("smelt_affine_mm_matvec_stream_f16", 5, 0),   # opt-in matrix-core variant
         "fused_affine_matvec_add_c3584_r1024_g64_rows4": ("smelt_affine_matvec_add_f16", 6, 0),
         "fused_affine_gate_up_swiglu_c1024_r3584_g64_rows4": ("smelt_affine_gate_up_swiglu_f16", 8, 0),
         "fused_dual_affine_matvec:1024:64": ("smelt_affine_dual_matvec_f16", 9, 1),
