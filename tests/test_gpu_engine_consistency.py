@@ -1,8 +1,8 @@
 """What the default (AUTO) engine choice does to the invariants the single-engine tests pin bit for bit.
 
-Under AUTO a step mixes two summation orders: plain, +residual, gate+up and bank matvecs of 1M weights and
-more run the single-pass matrix-core kernel, while the norm-scale, dual, GeGLU and every `_batched*` form
-(the 4-token verify pass included) stay on the vector kernels.  "Fused == staged" and "batched per-token bits
+Under AUTO a step mixes two summation orders: single-token matvecs of 1M weights and more (plain, +residual,
+gate+up, banks, dual, GeGLU, norm-scale forms) run the single-pass matrix-core kernel, while every `_batched*`
+form (the 4-token verify pass included) and the `atomic_norm_*` forms stay on the vector kernels.  "Fused == staged" and "batched per-token bits
 == M = 1 bits" therefore hold bit for bit only on one engine (tests/test_gpu_matvec.py,
 tests/test_gpu_norm_scale.py under VECTOR); across engines they hold to the output tolerance.  This file
 runs the default engine at a shape above the threshold and measures how far apart the two are."""
@@ -66,3 +66,80 @@ def test_auto_engine_decode_against_verify_b4_and_staged(ctx, dtype):
         assert np.array_equal(d1, v4)
     finally:
         ctx.set_matvec_engine(rt.MATVEC_AUTO)
+
+
+def _time_record(ctx, rec):
+    """Median GPU time of one launch of the record (microseconds), whichever kernel the engine routes it to."""
+    return float(np.median(ctx.benchmark_record(rec, warmup=20, iters=120)))
+
+
+def _affine_record(ctx, rows, cols, group, dtype, kind):
+    nmat = 2 if kind == "gate_up" else 1
+    rng = np.random.default_rng(rows * 7 + cols)
+    wf = gh.WeightFile()
+    bufs = []
+    for m in range(nmat):
+        packed = rng.integers(0, 256, size=(rows, cols // 2), dtype=np.uint8)
+        scales = fx.to_bits(np.abs(rng.normal(0, 0.02, (rows, cols // group))).astype(np.float32), dtype)
+        biases = fx.to_bits(rng.normal(0, 0.01, (rows, cols // group)).astype(np.float32), dtype)
+        bufs += [(0, 3 * m + i, wf.add(a)) for i, a in enumerate((packed, scales, biases))]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(gh.X_SLOT, fx.to_bits(rng.normal(0, 1, (1, cols)).astype(np.float32), dtype))
+    ctx.alloc(gh.Y_SLOT, rows * 2)
+    n = 3 * nmat
+    bufs += [(gh.X_SLOT, n, 0), (gh.Y_SLOT, n + 1, 0)]
+    entry = {"matvec": "affine_matvec", "gate_up": "fused_affine_gate_up_swiglu"}[kind] + f":{cols}:{group}"
+    pipe = ctx.pipeline(entry + gh.t_suffix(dtype))
+    return rt.make_record(pipe, bufs, [(n + 2, rows)], (min(1024, (rows + 7) // 8), 1, 1), (256, 1, 1))
+
+
+def _signed_record(ctx, fmt, name, rows, cols, dtype):
+    rng = np.random.default_rng(rows * 5 + cols)
+    stride = {fx.BINARY1: cols // 8, fx.TERNARY2: cols // 4}.get(fmt, (((cols + 4) // 5) + 15) // 16 * 16)
+    packed = rng.integers(0, 243 if fmt == fx.TRIT5 else 256, size=(rows, stride), dtype=np.uint8)
+    # (timing only: a ternary byte may hold the unused code 3 here; nothing is compared)
+    scales = fx.f16_bits(np.abs(rng.normal(0, 0.02, (rows, cols // 128))).astype(np.float32))
+    wf = gh.WeightFile()
+    oc, os_ = wf.add(packed), wf.add(scales)
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(gh.X_SLOT, fx.to_bits(rng.normal(0, 1, (1, cols)).astype(np.float32), dtype))
+    ctx.alloc(gh.Y_SLOT, rows * 2)
+    pipe = ctx.pipeline(f"signed_{name}_matvec_g128_rows8" + gh.t_suffix(dtype))
+    bufs = [(0, 0, oc), (0, 1, os_), (gh.X_SLOT, 2, 0), (gh.Y_SLOT, 3, 0)]
+    return rt.make_record(pipe, bufs, [(4, rows), (5, cols)], (min(1024, (rows + 7) // 8), 1, 1), (256, 1, 1))
+
+
+AFFINE_SWEEP = [(4096, 4096, 64, "matvec"), (11008, 4096, 128, "matvec"), (4096, 11008, 64, "matvec"), (1536, 8960, 64, "matvec"),
+                (32000, 4096, 32, "matvec"), (1024, 1024, 64, "matvec"), (6912, 2304, 64, "gate_up"), (14336, 4096, 128, "gate_up")]
+SIGNED_SWEEP = [(fx.BINARY1, "binary", 8192, 8192), (fx.BINARY1, "binary", 4096, 14336), (fx.BINARY1, "binary", 2048, 2048),
+                (fx.TERNARY2, "ternary", 14336, 4096), (fx.TERNARY2, "ternary", 8192, 2048), (fx.TRIT5, "trit5", 8192, 4096),
+                (fx.TRIT5, "trit5", 2560, 10240)]
+
+
+def test_auto_engine_is_not_the_slower_one(ctx):
+    """AUTO's size thresholds were fitted on the benchmark's shapes.  On a sweep of other shapes (Llama- and
+    Gemma-like projections, a short-and-wide and a tall-and-narrow matrix, one shape at a threshold) the kernel AUTO
+    picks must not lose to the vector kernel by more than run-to-run noise: warm single launches, medians of 120,
+    AUTO <= 1.10 x VECTOR + 0.3 us.  Where AUTO keeps the vector kernel the two times are the same measurement."""
+    dtype = fx.BF16
+    lines, worst = [], 0.0
+
+    def both(rec, what):
+        nonlocal worst
+        t = {}
+        for eng in (rt.MATVEC_AUTO, rt.MATVEC_VECTOR):
+            ctx.set_matvec_engine(eng)
+            t[eng] = _time_record(ctx, rec)
+        ctx.set_matvec_engine(rt.MATVEC_AUTO)
+        lines.append(f"  {what:34s} auto {t[rt.MATVEC_AUTO]:6.2f} us   vector {t[rt.MATVEC_VECTOR]:6.2f} us")
+        worst = max(worst, t[rt.MATVEC_AUTO] / t[rt.MATVEC_VECTOR])
+        assert t[rt.MATVEC_AUTO] <= 1.10 * t[rt.MATVEC_VECTOR] + 0.3, lines[-1]
+
+    try:
+        for rows, cols, group, kind in AFFINE_SWEEP:
+            both(_affine_record(ctx, rows, cols, group, dtype, kind), f"u4 g{group} {kind} {rows}x{cols}")
+        for fmt, name, rows, cols in SIGNED_SWEEP:
+            both(_signed_record(ctx, fmt, name, rows, cols, dtype), f"{name} {rows}x{cols}")
+    finally:
+        ctx.set_matvec_engine(rt.MATVEC_AUTO)
+        print("\n" + "\n".join(lines) + f"\n  worst auto / vector: {worst:.2f}")
