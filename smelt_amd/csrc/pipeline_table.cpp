@@ -468,8 +468,6 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
                 default: break;
             }
             if (a.m1 == kFamAffineGateUp && strstr(a.prefix, "geglu")) out->symbol = "smelt_affine_gate_up_geglu_" + t;
-            const bool prologue = a.m1 == kFamNormScaleAffineMatvec || a.m1 == kFamNormScaleAffineGateUp ||
-                                  a.m1 == kFamNormAddScaleAffineMatvec || a.m1 == kFamNormScaleAffineDual;
             out->appended = {rows, cols, group};
             return kResolveOk;
         }
