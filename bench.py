@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only step|layers|qmm|aux] [--engine auto|matrix|vector]
 
 A step is one pass over the decode-step matvec set of a 24-layer Qwen3.5-0.8B-shaped stack
-(BASELINE configs[1]): the q/k/v projection bank, o, fused gate+up, down (+residual) per layer and
+(the second configuration of the benchmark definition, `configs[1]`): the q/k/v projection bank, o, fused gate+up, down (+residual) per layer and
 the tied lm_head with fused argmax; all affine 4-bit g64 weights, bf16 activations, seeded synthetic
 tensors resident in HBM before the timed region.  The records are emitted by the library's own
 emitters, captured once into a HIP graph and replayed; `value` is weight bytes (packed codes +
