@@ -77,3 +77,34 @@ def test_signed_27b_shapes(ctx, fmt, name, shape):
         staged = so.epilogue_signed_swiglu(y, u, so.BF16)
         steps = np.abs(fused.astype(np.int32) - staged.astype(np.int32))
         assert steps.max() <= 1, int(steps.max())   # the low-precision exp() is not pinned bit-exactly
+
+
+@pytest.mark.parametrize("act", ["swiglu", "geglu"])
+def test_affine_norm_scale_gate_up_27b_shape(ctx, act):
+    """The fused forms a real layer's record list holds in front of the FFN: RMS-norm scale prologue + gate+up with
+    SwiGLU / GeGLU at 2 x 17408 x 5120 (matrix-core kernel under AUTO), against the oracle on the normalised row."""
+    import oracle.oracle as oo
+    from test_gpu_norm_scale import norm_inputs, run_gate_up
+    rows, cols, group, dtype = F, H, 64, fx.BF16
+    rng = fx.rng_for(1, 91)
+
+    def tensor():
+        packed = rng.integers(0, 256, size=(rows, cols // 2), dtype=np.uint8)
+        scales = fx.bf16_bits(np.abs(rng.normal(0, 0.02, size=(rows, cols // 64))).astype(np.float32))
+        biases = fx.bf16_bits(rng.normal(0, 0.01, size=(rows, cols // 64)).astype(np.float32))
+        return packed, scales, biases
+
+    gw, uw = tensor(), tensor()
+    x, w, rs = norm_inputs(1, cols, dtype, seed=5)
+    xn = oo.norm_scale_input(x[0], rs[0], w, dtype).reshape(1, cols)
+    fused = run_gate_up(ctx, gw, uw, dtype, f"norm_scale_affine_gate_up_{act}:{cols}:{group}", [(10, rows)], x, norm=(w, rs))
+    staged = run_gate_up(ctx, gw, uw, dtype, f"fused_affine_gate_up_{act}:{cols}:{group}", [(8, rows)], xn)
+    assert np.array_equal(fused, staged)
+    xf = fx.from_bits(xn, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, group, dtype, threads=True)
+    u = so.affine_matvec(*uw, xf, rows, cols, group, dtype, threads=True)
+    if act == "swiglu":
+        gh.check_outputs(fused, gh.swiglu_unrounded(g, u), dtype, "27B norm-scale gate+up swiglu")
+    else:
+        gh.check_steps(fused, so.epilogue_geglu(g, u, dtype).reshape(np.shape(fused)), dtype, "27B norm-scale gate+up geglu",
+                       max_steps=gh.GEGLU_STEPS)
