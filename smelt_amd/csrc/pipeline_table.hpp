@@ -96,12 +96,12 @@ enum FamilyId {
 enum SignedFormat { kFmtNone = -1, kFmtBinary1 = 0, kFmtTernary2 = 1, kFmtTrit5 = 2 };
 
 struct ResolvedPipeline {
-    FamilyId family;
+    FamilyId family = kFamCount;     // kFamCount: not resolved (a pipeline created with allow_missing keeps it)
     std::string symbol;              // kernel symbol in the code object
     std::string kinds;               // final argument kinds: 'P' pointer, 'U' u32, 'F' f32,
                                      // 'Z' pointer the record does not bind (passed as null)
     std::vector<uint32_t> appended;  // values appended after the record's own bindings
-    ActDType act;
+    ActDType act = kActF16;
     SignedFormat format = kFmtNone;
     uint32_t lds_variant = 0;        // batched matvec: activation rows resident per pass (1, 2, 4);
                                      // qmm: 16-token blocks per workgroup tile (1, 2, 4),
