@@ -139,7 +139,7 @@ size_t cdiv(size_t a, size_t b) { return (a + b - 1) / b; }
 
 // Checks operand extents against what the kernel will touch, and computes its LDS need.
 // Every hand-written kernel is only launched after this passes.
-int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const SplitKWorkspace& ws) {
+int validate_launch(smelt_hip_context* ctx, const Pipeline& p, Launch& L, const SplitKWorkspace& /* checked after routing */) {
     const ResolvedPipeline& r = p.res;
     auto U = [&](size_t i) -> size_t { return L.args[i].value; };
     size_t need[kMaxLaunchArgs] = {};
@@ -1082,17 +1082,17 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         // arguments, its own launch geometry (one workgroup per eight rows)
         uint32_t rows = 0, cols = 0, group = 128;
         size_t ro = 0;   // leading read-only operands (codes, scales[, biases], ..., x)
-        size_t skip = 0; // ... behind this many leading arguments that are not fetched 16 bytes at a time
+        size_t lead = 0; // ... behind this many leading arguments that are not fetched 16 bytes at a time
         auto U = [&](size_t i) { return L.args[i].value; };
         switch (p->res.family) {
             case kFamAffineDual: rows = U(9); cols = U(10); group = U(11); ro = 7; break;
             case kFamAffineDualAdd: rows = U(11); cols = U(12); group = U(13); ro = 7; break;
             // norm-scale prologue: the fp32 scale comes first; x, the norm weight, [the residual,] the
             // normalised row (stored 16 bytes at a time by workgroup 0) and the planes follow
-            case kFamNormScaleAffineMatvec: rows = U(8); cols = U(9); group = U(10); skip = 1; ro = 6; break;
-            case kFamNormAddScaleAffineMatvec: rows = U(9); cols = U(10); group = U(11); skip = 1; ro = 7; break;
-            case kFamNormScaleAffineDual: rows = U(11); cols = U(12); group = U(13); skip = 1; ro = 8; break;
-            case kFamNormScaleAffineGateUp: rows = U(10); cols = U(11); group = U(12); skip = 1; ro = 8; break;
+            case kFamNormScaleAffineMatvec: rows = U(8); cols = U(9); group = U(10); lead = 1; ro = 6; break;
+            case kFamNormAddScaleAffineMatvec: rows = U(9); cols = U(10); group = U(11); lead = 1; ro = 7; break;
+            case kFamNormScaleAffineDual: rows = U(11); cols = U(12); group = U(13); lead = 1; ro = 8; break;
+            case kFamNormScaleAffineGateUp: rows = U(10); cols = U(11); group = U(12); lead = 1; ro = 8; break;
             case kFamAffineMatvec: rows = U(5); cols = U(6); group = U(7); ro = 4; break;
             case kFamAffineAdd: rows = U(6); cols = U(7); group = U(8); ro = 4; break;
             case kFamAffineGateUp: rows = U(8); cols = U(9); group = U(10); ro = 7; break;
@@ -1109,7 +1109,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             default: break;
         }
         Mm1Plan plan;
-        if (rows > 0 && aligned16(skip + ro, skip) && whole_pieces(skip + ro, skip) && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
+        if (rows > 0 && aligned16(lead + ro, lead) && whole_pieces(lead + ro, lead) && mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
                                  ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &plan) &&
             p->fn_mm1[plan.nl]) {
             fn = p->fn_mm1[plan.nl];
