@@ -172,6 +172,21 @@ __host__ __device__ constexpr size_t mm1_lds_bytes(int frags_per_piece, int nl, 
            (size_t)waves * nmat * 32 + (dw == 4 ? 0 : 512);
 }
 
+// v[i] + v[i ^ 16] and v[i] + v[i ^ 32] in every lane, through the lane-swap instructions (no LDS
+// round trip): the swap exchanges the odd rows (the upper half) of its first operand with the even
+// rows (the lower half) of its second, so the two results hold the two addends in the same order in
+// both partner lanes.
+__device__ __forceinline__ float swap_sum16(float v) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+__device__ __forceinline__ float swap_sum32(float v) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+
 __device__ __forceinline__ float quad_sum(float v) {
     v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
     return dpp_add<0x4E>(v);  // quad_perm [2,3,0,1]
@@ -219,20 +234,6 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // Loads return in issue order, so what is needed first is asked for first.  A row or piece
     // past the end re-reads the last valid one and is discarded later (zero scale, no store).
     //
-    // ---- 1. the scale (and bias) rows of the tile: one contiguous block per matrix and plane ----
-    const int plane_pieces = (rows * gpr * 2 + 15) >> 4;
-    uint4_t sp[NMAT][PLANES];
-#pragma unroll
-    for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-        for (int pl = 0; pl < PLANES; ++pl) {
-            const uint4_t* base = reinterpret_cast<const uint4_t*>(pl == 0 ? mats[m].scales : mats[m].biases);
-            int idx = (int)threadIdx.x;
-            if (idx > gpr - 1) idx = gpr - 1;
-            int src = blockIdx.x * gpr + idx;         // row0 * gpr * 2 bytes = blockIdx.x * gpr pieces
-            if (src > plane_pieces - 1) src = plane_pieces - 1;
-            sp[m][pl] = base[src];
-        }
     // ---- 2. this wave's slice of x ---------------------------------------------------------------
     // One item = the columns of one packed dword; item it = 4 * (piece within the run) + dword.
     uint32_t xe[ITEMS][FIELDS / 2];
@@ -276,6 +277,20 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             xe[k][4 * v + 2] = past ? 0u : t.z; xe[k][4 * v + 3] = past ? 0u : t.w;
         }
     }
+    // ---- 1. the scale (and bias) rows of the tile: one contiguous block per matrix and plane ----
+    const int plane_pieces = (rows * gpr * 2 + 15) >> 4;
+    uint4_t sp[NMAT][PLANES];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int pl = 0; pl < PLANES; ++pl) {
+            const uint4_t* base = reinterpret_cast<const uint4_t*>(pl == 0 ? mats[m].scales : mats[m].biases);
+            int idx = (int)threadIdx.x;
+            if (idx > gpr - 1) idx = gpr - 1;
+            int src = blockIdx.x * gpr + idx;         // row0 * gpr * 2 bytes = blockIdx.x * gpr pieces
+            if (src > plane_pieces - 1) src = plane_pieces - 1;
+            sp[m][pl] = base[src];
+        }
     // ---- 3. every weight load of the job -------------------------------------------------------------
     uint4_t codes[NMAT][NL];
     {
@@ -302,16 +317,6 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // ---- 4. scales into LDS ----------------------------------------------------------------------------
     const size_t wave_bytes = mm1_wave_lds_bytes(FPL, NL, DW);
     uint4_t* lds_scales = reinterpret_cast<uint4_t*>(smem + (size_t)kc * wave_bytes);
-#pragma unroll
-    for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-        for (int pl = 0; pl < PLANES; ++pl) {
-            // threads past the end of the block hold its last piece again and store it again
-            int idx = (int)threadIdx.x;
-            if (idx > gpr - 1) idx = gpr - 1;
-            lds_scales[(m * PLANES + pl) * gpr + idx] = sp[m][pl];
-        }
-
     // ---- 5. x as operand fragments, wave-private in LDS --------------------------------------------
     // kFields consecutive activations become the kFPD fragments that dword's MFMAs take (k-slots
     // 2v, 2v+1 of fragment t = columns 4t+v, 4t+v+kPairs).  The four items of a 16-byte piece sit
@@ -354,6 +359,16 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             wsum[it] = __builtin_fmaf(F::kOffset, xs, cb);   // one constant per dword: the job adds them per scale group
         }
     }
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int pl = 0; pl < PLANES; ++pl) {
+            // threads past the end of the block hold its last piece again and store it again
+            int idx = (int)threadIdx.x;
+            if (idx > gpr - 1) idx = gpr - 1;
+            lds_scales[(m * PLANES + pl) * gpr + idx] = sp[m][pl];
+        }
+
     __syncthreads();   // scales of every wave, fragments of this one
 
     // ---- 6. the job --------------------------------------------------------------------------------
@@ -393,6 +408,32 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             }
         }
         const uint4_t* piece_frags = wfrag + (size_t)(i * 8 + a_piece) * PSTRIDE;
+        if constexpr (DW * FPD <= 4 && !F::kDecode) {
+            // few fragments per segment: all of them, and every transpose, are asked for before the first
+            // MFMA, so the LDS round trips overlap each other (and, for the fragments, the weights' flight)
+            uint4_t afr[DW][FPD];
+#pragma unroll
+            for (int d = 0; d < DW; ++d) {
+                const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
+                const uint4_t* pf = a_live ? piece_frags + d * FPD : wzero;
+#pragma unroll
+                for (int f = 0; f < FPD; ++f) afr[d][f] = pf[f];
+            }
+            uint32_t cw[NMAT][DW];
+#pragma unroll
+            for (int d = 0; d < DW; ++d)
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) cw[m][d] = (uint32_t)__builtin_amdgcn_ds_bpermute(xpose, (int)cd[m][d]);
+#pragma unroll
+            for (int d = 0; d < DW; ++d)
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) {
+                    uint4_t ops[FPD];
+                    F::operands(cw[m][d], ops);
+#pragma unroll
+                    for (int f = 0; f < FPD; ++f) acc[m] = E::mfma(afr[d][f], ops[f], acc[m]);
+                }
+        } else {
 #pragma unroll
         for (int d = 0; d < DW; ++d) {
             const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
@@ -408,6 +449,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
 #pragma unroll
                 for (int f = 0; f < FPD; ++f) acc[m] = E::mfma(afr[f], ops[f], acc[m]);
             }
+        }
         }
         const int piece = piece0 + i * 8 + 4 * hh + q;
         const bool piece_ok = piece < pieces;
@@ -452,9 +494,9 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // the eight pieces of a segment: lanes rn + 8 * {0..7}
 #pragma unroll
     for (int m = 0; m < NMAT; ++m) {
-        y[m] += __shfl_xor(y[m], 8);
-        y[m] += __shfl_xor(y[m], 16);
-        y[m] += __shfl_xor(y[m], 32);
+        y[m] = dpp_add<0x128>(y[m]);   // row_ror:8: lane i of a row of sixteen takes lane i ^ 8
+        y[m] = swap_sum16(y[m]);
+        y[m] = swap_sum32(y[m]);
     }
 
     // ---- 7. the kc waves of the workgroup -----------------------------------------------------------
@@ -465,12 +507,18 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             for (int m = 0; m < NMAT; ++m) red[(chunk * NMAT + m) * 8 + lane] = y[m];
         }
         __syncthreads();
-        if (chunk == 0 && lane < 8) {
+        if (chunk == 0) {
+            // lane 8 k + r takes wave k's sum of row r (zero past the last wave; waves 8 .. 15 in a second
+            // value), and the lanes r, r + 8, ... add up as the pieces of a segment did above
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) {
-                float sum = y[m];
-                for (int k = 1; k < kc; ++k) sum += red[(k * NMAT + m) * 8 + lane];
-                y[m] = sum;
+                const int k = lane >> 3, r = lane & 7;
+                const int k0 = k < kc ? k : kc - 1, k1 = k + 8 < kc ? k + 8 : kc - 1;
+                const float v0 = red[(k0 * NMAT + m) * 8 + r], v1 = red[(k1 * NMAT + m) * 8 + r];
+                float sum = (k < kc ? v0 : 0.0f) + (k + 8 < kc ? v1 : 0.0f);
+                sum = dpp_add<0x128>(sum);
+                sum = swap_sum16(sum);
+                y[m] = swap_sum32(sum);
             }
         }
     }
