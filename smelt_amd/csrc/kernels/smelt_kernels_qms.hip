@@ -7,7 +7,6 @@
 #define SMELT_QMS_ALL(T, ACT)                                                                      \
     SMELT_AFFINE_QMS_PLAIN(T, ACT, ACT, 1, 2) SMELT_AFFINE_QMS_PLAIN(T, ACT, ACT, 1, 4)            \
     SMELT_AFFINE_QMS_PLAIN(T, ACT, ACT, 2, 2) SMELT_AFFINE_QMS_PLAIN(T, ACT, ACT, 2, 4)            \
-    SMELT_AFFINE_QMS_PLAIN(T, ACT, ACT, 4, 2) SMELT_AFFINE_QMS_PLAIN(T, ACT, ACT, 4, 4)            \
     SMELT_AFFINE_QMS_GATE_UP(T, ACT, ACT, 2) SMELT_AFFINE_QMS_GATE_UP(T, ACT, ACT, 4)
 
 SMELT_QMS_ALL(f16, smelt::F16)

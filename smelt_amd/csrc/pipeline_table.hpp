@@ -159,7 +159,7 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
 // Launch plan of the streaming skinny qmm: workgroups of `kc` waves over 16 * rt rows each, 16 tokens
 // per grid row; wave c takes the pairs of scale groups c, c + kc, ...  False when the shape has no
 // such kernel.
-constexpr uint32_t kQmsMaxRowTiles = 4;
+constexpr uint32_t kQmsMaxRowTiles = 2;   // what qms_plan returns: one or two
 struct QmsPlan {
     uint32_t rt = 0, kc = 0;
     size_t lds = 0;
