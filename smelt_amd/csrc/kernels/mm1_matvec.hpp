@@ -278,8 +278,27 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         }
     }
     // ---- 1. the scale (and bias) rows of the tile: one contiguous block per matrix and plane ----
+    // Short affine rows (one or two segments per wave: the launches that are a single memory round
+    // trip) skip the block: every lane fetches the two-byte scale and bias of the group it will apply,
+    // no wave waits for another's loads and the workgroup meets only for its final sum.
+    constexpr bool kDirectScales = F::kHasBias && DW == 4 && NL <= 2;
     const int plane_pieces = (rows * gpr * 2 + 15) >> 4;
     uint4_t sp[NMAT][PLANES];
+    uint16_t sdir[NMAT][PLANES][NL];
+    if constexpr (kDirectScales) {
+        int srow = row0 + rn;
+        if (srow > rows - 1) srow = rows - 1;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            int piece = piece0 + i * 8 + 4 * hh + q;
+            if (piece > pieces - 1) piece = pieces - 1;
+            const int g = (piece * F::kPieceCols) >> gshift;
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int pl = 0; pl < PLANES; ++pl) sdir[m][pl][i] = (pl == 0 ? mats[m].scales : mats[m].biases)[(size_t)srow * gpr + g];
+        }
+    } else {
 #pragma unroll
     for (int m = 0; m < NMAT; ++m)
 #pragma unroll
@@ -291,6 +310,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             if (src > plane_pieces - 1) src = plane_pieces - 1;
             sp[m][pl] = base[src];
         }
+    }
     // ---- 3. every weight load of the job -------------------------------------------------------------
     uint4_t codes[NMAT][NL];
     {
@@ -359,6 +379,12 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             wsum[it] = __builtin_fmaf(F::kOffset, xs, cb);   // one constant per dword: the job adds them per scale group
         }
     }
+    if constexpr (kDirectScales) {
+        // the fragments are this wave's own: LDS executes a wave's operations in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
 #pragma unroll
     for (int m = 0; m < NMAT; ++m)
 #pragma unroll
@@ -370,6 +396,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         }
 
     __syncthreads();   // scales of every wave, fragments of this one
+    }
 
     // ---- 6. the job --------------------------------------------------------------------------------
     // A-operand lanes 20q and 20q + 1 (token slots 4q and 4q + 1 in k-block q: the two halves of
@@ -459,11 +486,11 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) {
                 const int sidx = (m * PLANES) * (8 * gpr) + rn * gpr + g;
-                const float sv = F::kSemMul * ScaleT::widen(lds_s16[sidx]);
+                const float sv = F::kSemMul * ScaleT::widen(kDirectScales ? sdir[m][0][i] : lds_s16[sidx]);
                 const float dotp = hh ? acc[m].y : acc[m].x;   // token slot 4q + hh
                 y[m] = __builtin_fmaf(piece_ok ? sv : 0.0f, dotp - cs.x, y[m]);
                 if (F::kHasBias) {
-                    const float bv = ScaleT::widen(lds_s16[sidx + 8 * gpr]);
+                    const float bv = ScaleT::widen(kDirectScales ? sdir[m][PLANES - 1][i] : lds_s16[sidx + 8 * gpr]);
                     y[m] = __builtin_fmaf(piece_ok ? bv : 0.0f, cs.y, y[m]);
                 }
             }
