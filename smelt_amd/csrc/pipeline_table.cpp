@@ -132,10 +132,10 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     }
     if (rows == 0 || cols == 0 || row_stride % 16 != 0 || group < 32 || (group & (group - 1))) return false;
     if (layout != kCodesU4 && group != 128) return false;
-    // small matrices are launch-bound either way and stay where they are tuned
-    // (five-digit bytes: the vector kernel decodes through the same table at twice the cost, so the bar is lower)
-    // (affine: from 1M weights, see the short walk below)
-    if (!force && (uint64_t)rows * cols < (layout == kCodesTrit5 ? (2u << 20) : (layout == kCodesU4 ? (1u << 20) : (8u << 20)))) return false;
+    // Where the vector-ALU kernel stays the default (measured on MI355X, cold, per launch in a graph): affine 4-bit
+    // nowhere (64 x 1024 to 1024 x 1024: 2.1-2.7 us against 2.5-4.0); binary and ternary below 1M weights (not
+    // measured there; from 1M on 2.2-3.1 against 2.8-3.7); five-digit bytes below 2M (equal within a tenth up to 8M).
+    if (!force && (uint64_t)rows * cols < (layout == kCodesTrit5 ? (2u << 20) : (layout == kCodesU4 ? 0u : (1u << 20)))) return false;
     const uint32_t pieces = row_stride / 16, nseg = (pieces + 7) / 8, gpr = (cols + group - 1) / group;
     const uint32_t planes = layout == kCodesU4 ? 2 : 1;
     auto lds_of = [&](uint32_t kc, uint32_t nl) {

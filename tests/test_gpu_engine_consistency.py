@@ -1,11 +1,11 @@
 """What the default (AUTO) engine choice does to the invariants the single-engine tests pin bit for bit.
 
-Under AUTO a step mixes two summation orders: single-token matvecs of 1M weights and more (plain, +residual,
+Under AUTO a step mixes two summation orders: single-token affine matvecs (plain, +residual,
 gate+up, banks, dual, GeGLU, norm-scale forms) run the single-pass matrix-core kernel, while every `_batched*`
 form (the 4-token verify pass included) and the `atomic_norm_*` forms stay on the vector kernels.  "Fused == staged" and "batched per-token bits
 == M = 1 bits" therefore hold bit for bit only on one engine (tests/test_gpu_matvec.py,
 tests/test_gpu_norm_scale.py under VECTOR); across engines they hold to the output tolerance.  This file
-runs the default engine at a shape above the threshold and measures how far apart the two are."""
+runs the default engine and measures how far apart the two are."""
 import numpy as np
 import pytest
 
@@ -34,8 +34,7 @@ def steps_between(a_bits, b_bits, dtype):
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 def test_auto_engine_decode_against_verify_b4_and_staged(ctx, dtype):
-    rows, cols, group = 2048, 1024, 64          # 2M weights: above the 1M threshold of the matrix-core matvec
-    assert rows * cols >= (1 << 20)
+    rows, cols, group = 2048, 1024, 64          # AUTO runs the matrix-core matvec
     packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=31)
     x = fx.synth_activation(4, cols, dtype, config=1, tensor=32)
     xf = fx.from_bits(x, dtype)

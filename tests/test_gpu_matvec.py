@@ -21,8 +21,9 @@ def ctx():
 @pytest.fixture
 def vector_ctx(ctx):
     """The module's context on the vector-ALU kernels: comparisons that are bit for bit between a fused kernel and
-    its staged pair hold there; under AUTO an affine matrix from 1M weights takes the single-pass matrix-core
-    kernel, whose order of accumulation differs (same tolerance against the oracle)."""
+    its staged pair, or a small-batch kernel and the single-token one, hold there; under AUTO a single-token affine
+    matvec takes the single-pass matrix-core kernel, whose order of accumulation differs (same tolerance against
+    the oracle)."""
     ctx.set_matvec_engine(rt.MATVEC_VECTOR)
     yield ctx
     ctx.set_matvec_engine(rt.MATVEC_AUTO)
@@ -246,9 +247,11 @@ def test_affine_gate_up_swiglu_and_dual(vector_ctx):
 
 
 @pytest.mark.parametrize("batch,tile", [(3, 3), (4, 4), (7, 8), (9, 4)])
-def test_affine_small_batch_equals_per_row_matvec(ctx, batch, tile):
+def test_affine_small_batch_equals_per_row_matvec(vector_ctx, batch, tile):
     """Per-token results of the small-batch kernel are the batch-1 kernel's bits
-    (the reference asserts the same of its batched variants)."""
+    (the reference asserts the same of its batched variants).  On the vector-ALU kernels: under AUTO the
+    single-token record runs the matrix-core kernel, which adds up a row in another order."""
+    ctx = vector_ctx
     rows, cols, group = 512, 1024, 64
     dtype = fx.F16
     w = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=2)

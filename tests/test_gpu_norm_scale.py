@@ -427,10 +427,11 @@ def test_norm_fused_into_matvec_and_gate_up(vector_ctx, dtype, threads):
     assert np.array_equal(fused, staged)
 
 
-def test_dual_matvec_per_token_and_small_batch_geglu(ctx):
+def test_dual_matvec_per_token_and_small_batch_geglu(vector_ctx):
     """fused_dual_affine_matvec_*_batched (lut_matvec.metal:7570-7591: grid.y = token) and the
     small-batch GeGLU kernels (:8342-8364, token tiles of 3 and 4): per-token results are the
     single-token kernels' bits."""
+    ctx = vector_ctx
     rows, cols, group, dtype, batch = 512, 1024, 64, fx.F16, 5
     w1 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=10)
     w2 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=11)
@@ -462,12 +463,13 @@ def test_dual_matvec_per_token_and_small_batch_geglu(ctx):
 
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
-def test_generated_small_batch_and_dual_add_names(ctx, dtype):
+def test_generated_small_batch_and_dual_add_names(vector_ctx, dtype):
     """The compiler's generated variants (SmeltGeneratedKernelVariants.swift:17-35, 66-68):
     `_batched_verify_b4` forms of the matvec, gate+up+SwiGLU and dual matvec (token tiles of 4, the token
     count at the binding after the outputs; lut_matvec.metal:3816-3922) and the decode dual matvec with two
     residuals (`fused_dual_affine_matvec_add_*_rows4`, :4660-4733).  Per token they are the single-token
     kernels' bits; the residual form is checked against the oracle's round-then-add."""
+    ctx = vector_ctx
     rows, cols, group, batch = 264, 1024, 64, 6
     w1 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=20)
     w2 = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=21)

@@ -79,16 +79,16 @@ def test_matvec_plans(layout, group):
     # the 27B layer's matrices take the kernel by default in every format
     for rows, cols in [(17408, 5120), (5120, 17408), (5120, 5120)]:
         assert cc.plan_matvec(layout, rows, cols, group) is not None
-    # small matrices stay on the vector kernels unless forced (affine from 1M weights, five-digit bytes from 2M,
-    # binary and ternary from 8M); small affine matrices walk few segments per wave, at most eight waves
+    # small matrices stay on the vector kernels unless forced (binary and ternary below 1M weights, five-digit
+    # bytes below 2M; affine 4-bit never); small affine matrices walk few segments per wave, at most eight waves
     small = cc.plan_matvec(layout, 1024, 2560, group)
-    assert (small is not None) == (layout in (cc.LAYOUT_TRIT5, cc.LAYOUT_U4))
+    assert small is not None
     if layout == cc.LAYOUT_U4:
         assert (small["segments"], small["waves"]) == (2, 5)
         assert cc.plan_matvec(layout, 3584, 1024, group)["segments"] == 1
         assert cc.plan_matvec(layout, 1024, 3584, group)["waves"] <= 8
-        assert cc.plan_matvec(layout, 512, 1024, group) is None
-    assert cc.plan_matvec(layout, 256, 2560, group) is None
+        assert cc.plan_matvec(layout, 512, 1024, group) is not None
+    assert (cc.plan_matvec(layout, 256, 2560, group) is not None) == (layout == cc.LAYOUT_U4)
     assert cc.plan_matvec(layout, 256, 2560, group, force=True) is not None
 
 
