@@ -1086,7 +1086,7 @@ int smelt_hip_plan_qmm(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nm
         return 1;
     }
     smelt_host::QmsPlan q;
-    if (batch > 0 && smelt_host::qms_plan(rows, cols, group, nmat, batch, lds_limit, &q)) {
+    if (batch > 0 && smelt_host::qms_plan(rows, cols, group, nmat, batch, compute_units, lds_limit, &q)) {
         out[0] = 1; out[1] = q.rt; out[2] = q.kc; out[4] = 1;
         out[5] = (rows + 16 * q.rt - 1) / (16 * q.rt); out[6] = (batch + 15) / 16; out[7] = 1;
         out[8] = 64 * q.kc; out[9] = (uint32_t)q.lds;

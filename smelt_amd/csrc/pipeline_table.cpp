@@ -278,7 +278,8 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     return out->lds <= lds_limit;
 }
 
-bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, size_t lds_limit, QmsPlan* out) {
+bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
+              size_t lds_limit, QmsPlan* out) {
     if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;
     const uint32_t gt = cols / 64, npairs = gt / 2;
     // Measured on MI355X at 2560- and 9216-column rows: about four steps per wave hide the memory
@@ -289,12 +290,24 @@ bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     uint32_t kc = (npairs + 3) / 4;
     if (kc < 2) kc = npairs < 2 ? 1 : 2;
     if (kc > 12) kc = 12;
-    const uint32_t steps = (npairs + kc - 1) / kc;
+    uint32_t steps = (npairs + kc - 1) / kc;
     kc = (npairs + steps - 1) / steps;   // same steps per wave, no idle wave
-    if (kc < rt) return false;
     const uint32_t tiles = nmat * rt;
+    auto lds_of = [&](uint32_t waves) {
+        return (size_t)tiles * 16 * (gt + 1) * 8 + (size_t)waves * (16 * 272 + (size_t)tiles * 16 * 72);
+    };
+    // A launch of more workgroups than compute units runs two per unit only if two fit in LDS together, and a
+    // long row's scale table takes a large share: fewer waves with more steps each then beat a second round
+    // (2560 x 9216 at 32 tokens: 14.0 us with nine waves against 16.6 with twelve; 5120 x 17408: 37.6 against 41.4).
+    const uint64_t workgroups = (uint64_t)((rows + 16 * rt - 1) / (16 * rt)) * ((batch + 15) / 16);
+    if (workgroups > compute_units)
+        while (kc > 2 && lds_of(kc) > lds_limit / 2 && lds_of(2) <= lds_limit / 2) {
+            ++steps;
+            kc = (npairs + steps - 1) / steps;
+        }
+    if (kc < rt) return false;
     out->rt = rt; out->kc = kc;
-    out->lds = (size_t)tiles * 16 * (gt + 1) * 8 + (size_t)kc * (16 * 272 + (size_t)tiles * 16 * 72);
+    out->lds = lds_of(kc);
     return out->lds <= lds_limit;
 }
 

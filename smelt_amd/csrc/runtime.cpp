@@ -1137,7 +1137,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             qms_routed = true;
         }
         QmsPlan plan;
-        if (!routed && batch > 0 && qms_plan(rows, cols, group, p->res.qms_nmat, batch, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
+        if (!routed && batch > 0 && qms_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
             fn = p->fn_qms[plan.rt][batch > 8];
             L.grid[0] = (rows + 16 * plan.rt - 1) / (16 * plan.rt); L.grid[1] = (batch + 15) / 16; L.grid[2] = 1;
             L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;

@@ -51,6 +51,25 @@ def test_qmm_k_split_needs_the_workspace():
            {k: with_ws[k] for k in ("kernel", "row_tiles", "k_waves", "grid_x", "grid_y", "lds")}
 
 
+def test_streaming_plan_keeps_two_workgroups_per_unit_when_the_launch_has_them():
+    """A long row's scale table takes a large share of LDS: a launch of more workgroups than compute units takes
+    fewer waves (more steps each) so that two workgroups fit a unit together; a launch that gives every unit at
+    most one workgroup keeps its twelve waves."""
+    one_round = cc.plan_qmm(2560, 9216, 64, 1, 16, CUS, LDS)
+    assert one_round["kernel"] == 1 and one_round["grid_x"] * one_round["grid_y"] <= CUS
+    assert one_round["k_waves"] == 12 and 2 * one_round["lds"] > LDS
+    for rows, cols in [(2560, 9216), (5120, 17408), (4096, 14336)]:
+        p = cc.plan_qmm(rows, cols, 64, 1, 32, CUS, LDS)
+        assert p["kernel"] == 1 and p["grid_x"] * p["grid_y"] > CUS
+        assert 2 * p["lds"] <= LDS and 2 <= p["k_waves"] < 12
+        # every wave has work: no wave past the last pair of scale groups
+        pairs = cols // 128
+        steps = ceil_div(pairs, p["k_waves"])
+        assert (p["k_waves"] - 1) * steps < pairs
+    # short rows never needed it
+    assert cc.plan_qmm(9216, 2560, 64, 1, 32, CUS, LDS)["k_waves"] == 5
+
+
 def test_qmm_plan_rejects_what_no_kernel_takes():
     assert cc.plan_qmm(1024, 1024, 32, 1, 64) is None      # group 32 has no streaming form
     assert cc.plan_qmm(1024, 1024, 64, 1, 0) is None
