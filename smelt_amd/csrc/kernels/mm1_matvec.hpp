@@ -159,9 +159,13 @@ struct M1U4 : M1Codes<4, ActT> {
 //   (five-dword pieces: per dword the folded-out constant, 4 B; and a 512-byte decode table at the end)
 //   Four-dword pieces hold a power-of-two number of fragments, which would put the eight pieces of a
 //   segment (read together, one per A-operand lane) on the same LDS banks: their stride is one
-//   fragment longer.  Five-dword pieces (160 bytes) spread over the banks by themselves.
+//   fragment longer, except for pieces of four fragments (affine 4-bit), where pieces p and p + 4 are the
+//   only ones to meet and the second half of a segment stores fragment d in slot d ^ 1 instead (a long
+//   row's fragments are most of a workgroup's LDS: without the padding three workgroups of a
+//   17408-column matrix fit a compute unit instead of two).  Five-dword pieces (160 bytes) spread over the
+//   banks by themselves.
 __host__ __device__ constexpr int mm1_piece_stride(int frags_per_piece, int dw = 4) {
-    return dw == 4 ? frags_per_piece + 1 : frags_per_piece;
+    return dw == 4 ? (frags_per_piece == 4 ? 4 : frags_per_piece + 1) : frags_per_piece;
 }
 __host__ __device__ constexpr size_t mm1_wave_lds_bytes(int frags_per_piece, int nl, int dw = 4) {
     return (size_t)nl * 8 * mm1_piece_stride(frags_per_piece, dw) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) +
@@ -204,6 +208,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     using E = Elem16<ActT>;
     constexpr int FPD = F::kFPD, FPL = F::kFPL, FIELDS = F::kFields, PAIRS = F::kPairs, DW = F::kDW;
     constexpr int PSTRIDE = mm1_piece_stride(FPL, DW);     // fragments from one piece to the next in LDS
+    constexpr bool kSwizzle = DW == 4 && FPL == 4;         // unpadded pieces: slot d ^ 1 in the second half of a segment
     constexpr int NITEMS = NL * 8 * DW;                    // staging items of a wave: 8 pieces x DW dwords per segment
     constexpr int ITEMS = (NITEMS + kWave - 1) / kWave;    // per lane
     constexpr int PLANES = F::kHasBias ? 2 : 1;
@@ -372,7 +377,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         }
 #pragma unroll
         for (int t = 0; t < FPD; ++t)
-            wfrag[(size_t)pl * PSTRIDE + d * FPD + t] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
+            wfrag[(size_t)pl * PSTRIDE + ((d * FPD + t) ^ (kSwizzle ? (pl >> 2) & 1 : 0))] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
         if constexpr (DW == 4) {
             if (d == 0) *reinterpret_cast<float2*>(wsum + 2 * pl) = float2{__builtin_fmaf(F::kOffset, xs, cb), xs};
         } else {
@@ -442,7 +447,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
 #pragma unroll
             for (int d = 0; d < DW; ++d) {
                 const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
-                const uint4_t* pf = a_live ? piece_frags + d * FPD : wzero;
+                const uint4_t* pf = a_live ? piece_frags + (kSwizzle ? d ^ a_half : d) * FPD : wzero;
 #pragma unroll
                 for (int f = 0; f < FPD; ++f) afr[d][f] = pf[f];
             }
@@ -464,7 +469,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
 #pragma unroll
         for (int d = 0; d < DW; ++d) {
             const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
-            const uint4_t* pf = a_live ? piece_frags + d * FPD : wzero;
+            const uint4_t* pf = a_live ? piece_frags + (kSwizzle ? d ^ a_half : d) * FPD : wzero;
             uint4_t afr[FPD];
 #pragma unroll
             for (int f = 0; f < FPD; ++f) afr[f] = pf[f];

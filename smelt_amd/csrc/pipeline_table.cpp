@@ -139,8 +139,8 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     const uint32_t pieces = row_stride / 16, nseg = (pieces + 7) / 8, gpr = (cols + group - 1) / group;
     const uint32_t planes = layout == kCodesU4 ? 2 : 1;
     auto lds_of = [&](uint32_t kc, uint32_t nl) {
-        // four-dword pieces are stored one fragment apart (LDS banks)
-        const size_t wave = (size_t)nl * 8 * (dw == 4 ? frags + 1 : frags) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) + (size_t)frags * 16;
+        // four-dword pieces are stored one fragment apart (LDS banks), except the four-fragment ones (swizzled instead)
+        const size_t wave = (size_t)nl * 8 * (dw == 4 ? (frags == 4 ? 4 : frags + 1) : frags) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) + (size_t)frags * 16;
         return kc * wave + (size_t)nmat * planes * 8 * gpr * 2 + (size_t)kc * nmat * 32 + (dw == 4 ? 0 : 512);   // + decode table
     };
     Mm1Plan best;
