@@ -236,10 +236,12 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
 
     // Nothing below branches or predicates a load until every load of the job is issued (a load
     // under a branch invites the compiler to move its consumer, and the wait, in there too).
-    // Loads return in issue order, so what is needed first is asked for first.  A row or piece
-    // past the end re-reads the last valid one and is discarded later (zero scale, no store).
+    // Loads return in issue order, so what is needed first is asked for first: the activations (they
+    // come from cache and are turned into fragments while the rest is still in flight), then the
+    // scales, then the weights.  A row or piece past the end re-reads the last valid one and is
+    // discarded later (zero scale, no store).
     //
-    // ---- 2. this wave's slice of x ---------------------------------------------------------------
+    // ---- 1. this wave's slice of x ---------------------------------------------------------------
     // One item = the columns of one packed dword; item it = 4 * (piece within the run) + dword.
     uint32_t xe[ITEMS][FIELDS / 2];
     int item_piece[ITEMS], item_dword[ITEMS];
@@ -282,7 +284,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             xe[k][4 * v + 2] = past ? 0u : t.z; xe[k][4 * v + 3] = past ? 0u : t.w;
         }
     }
-    // ---- 1. the scale (and bias) rows of the tile: one contiguous block per matrix and plane ----
+    // ---- 2. the scale (and bias) rows of the tile: one contiguous block per matrix and plane ----
     // Short affine rows (one or two segments per wave: the launches that are a single memory round
     // trip) skip the block: every lane fetches the two-byte scale and bias of the group it will apply,
     // no wave waits for another's loads and the workgroup meets only for its final sum.
@@ -339,10 +341,9 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         res = epi.prefetch(token, rr < rows ? rr : rows - 1);
     }
 
-    // ---- 4. scales into LDS ----------------------------------------------------------------------------
     const size_t wave_bytes = mm1_wave_lds_bytes(FPL, NL, DW);
     uint4_t* lds_scales = reinterpret_cast<uint4_t*>(smem + (size_t)kc * wave_bytes);
-    // ---- 5. x as operand fragments, wave-private in LDS --------------------------------------------
+    // ---- 4. x as operand fragments, wave-private in LDS --------------------------------------------
     // kFields consecutive activations become the kFPD fragments that dword's MFMAs take (k-slots
     // 2v, 2v+1 of fragment t = columns 4t+v, 4t+v+kPairs).  The four items of a 16-byte piece sit
     // in the four lanes of a quad, which add up their sum(base * x) and sum(x).
@@ -384,8 +385,9 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             wsum[it] = __builtin_fmaf(F::kOffset, xs, cb);   // one constant per dword: the job adds them per scale group
         }
     }
+    // ---- 5. scales into LDS (they were asked for after the activations and arrive after them) ------
     if constexpr (kDirectScales) {
-        // the fragments are this wave's own: LDS executes a wave's operations in order
+        // nothing to share; the fragments are this wave's own: LDS executes a wave's operations in order
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
