@@ -159,11 +159,22 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     static const uint32_t kShortWalk[] = {1, 2, 3, 4, 5, 6};
     const bool small_affine = layout == kCodesU4 && (uint64_t)rows * cols < (8u << 20);
     if (small_affine) order = kShortWalk;
+    // Between 8M and 24M weights (a 4B model's projections: 13 MB, a few workgroups per compute unit) two
+    // segments per wave, as long as twelve waves cover the row and all waves of the launch fit the machine about
+    // at once; measured per launch, cold, against the long walk: 9216 x 2560 5.0 against 5.5 us, 2560 x 9216 (three
+    // segments: twelve waves) 6.4 against 7.0, 4096 x 4096 4.2 against 4.5, 3072 x 3072 3.8 against 4.4.  From 24M
+    // weights on (5120-column rows and longer) the long walk stays: 5120 x 5120 5.7 against 6.0, 17408 x 5120
+    // gate+up 19.5 against 22.4.
+    static const uint32_t kMidWalk[] = {2, 1, 3, 4, 5, 6};
+    const bool mid_affine = layout == kCodesU4 && !small_affine && (uint64_t)rows * cols < (24u << 20);
+    if (mid_affine) order = kMidWalk;
+    const uint64_t tiles = ((uint64_t)rows + 7) / 8;
     for (uint32_t o = 0; o < norder; ++o) {
         const uint32_t nl = order[o];
         if (nl > nl_max || (nl > nseg && nl > 1)) continue;
         const uint32_t kc = (nseg + nl - 1) / nl;
-        if (kc > (small_affine ? 8u : 16u) || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
+        if (kc > (small_affine ? 8u : (mid_affine ? 12u : 16u)) || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
+        if (mid_affine && nl < 6 && tiles * kc > 11264) continue;   // 1.375 x the 8192 wave slots of the machine
         const size_t lds = lds_of(kc, nl);
         if (lds > lds_limit) continue;
         const uint32_t waste = kc * nl - nseg;

@@ -107,6 +107,12 @@ def test_matvec_plans(layout, group):
         assert cc.plan_matvec(layout, 3584, 1024, group)["segments"] == 1
         assert cc.plan_matvec(layout, 1024, 3584, group)["waves"] <= 8
         assert cc.plan_matvec(layout, 512, 1024, group) is not None
+        # 8M to 24M weights: two segments per wave where twelve waves cover the row, else the next that does
+        assert (cc.plan_matvec(layout, 9216, 2560, group)["segments"], cc.plan_matvec(layout, 9216, 2560, group)["waves"]) == (2, 5)
+        assert (cc.plan_matvec(layout, 2560, 9216, group)["segments"], cc.plan_matvec(layout, 2560, 9216, group)["waves"]) == (3, 12)
+        assert cc.plan_matvec(layout, 4096, 4096, group)["segments"] == 2
+        # from 24M weights on the long walk
+        assert cc.plan_matvec(layout, 5120, 5120, group)["segments"] >= 5
     assert (cc.plan_matvec(layout, 256, 2560, group) is not None) == (layout == cc.LAYOUT_U4)
     assert cc.plan_matvec(layout, 256, 2560, group, force=True) is not None
 
