@@ -168,6 +168,11 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     static const uint32_t kMidWalk[] = {2, 1, 3, 4, 5, 6};
     const bool mid_affine = layout == kCodesU4 && !small_affine && (uint64_t)rows * cols < (24u << 20);
     if (mid_affine) order = kMidWalk;
+    // The signed formats below the 27B shapes: one segment per wave (binary 4096 x 4096 3.5 against 3.8 us,
+    // 9216 x 2560 4.25 against 4.5; five-digit bytes 4.55 against 4.9 and 5.3 against 5.7; 2048 x 2048 in all three
+    // 2.6 / 2.6 / 3.35 against 2.8 / 2.8 / 3.8); ternary from 8M weights keeps two (3.5 against 3.7, 4.3 against 4.4).
+    static const uint32_t kSignedShort[] = {1, 2, 3};
+    if (layout != kCodesU4 && (uint64_t)rows * cols < (layout == kCodesTernary2 ? (8u << 20) : (24u << 20))) order = kSignedShort;
     const uint64_t tiles = ((uint64_t)rows + 7) / 8;
     for (uint32_t o = 0; o < norder; ++o) {
         const uint32_t nl = order[o];
