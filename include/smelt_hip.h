@@ -122,11 +122,11 @@ const char *smelt_hip_last_error(const smelt_hip_context *ctx);
  * every quantized matvec (MatvecKernelTable.swift:158-181). */
 int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
 
-/* Which kernel a single-token quantized matvec record runs.  AUTO (the default): affine 4-bit
- * matrices of any size, binary and ternary ones of 1M weights and more, five-digit-byte ones of 2M
- * and more take the single-pass matrix-core kernel of the same pipeline, smaller ones the vector-ALU kernel (the two add up a row in different
- * orders: results agree to the output tolerance, not bit for bit); MATRIX_CORE drops the size threshold (every shape the matrix-core kernel
- * can express takes it); VECTOR keeps every record on the vector-ALU kernels.  The same switch
+/* Which kernel a single-token quantized matvec record runs.  AUTO (the default): every shape the
+ * single-pass matrix-core kernel of the same pipeline can express takes it, the rest the vector-ALU
+ * kernel (the two add up a row in different orders: results agree to the output tolerance, not bit
+ * for bit); MATRIX_CORE asks for the same explicitly (kept from when AUTO had size thresholds);
+ * VECTOR keeps every record on the vector-ALU kernels.  The same switch
  * covers the qmm records: AUTO and MATRIX_CORE run the streaming kernel of the pipeline below 128
  * tokens (K split inside a workgroup, no workspace) and the token-tile kernel from 128 tokens on
  * (matrices with few tiles and long rows split K across workgroups: partial sums in the

@@ -132,10 +132,11 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     }
     if (rows == 0 || cols == 0 || row_stride % 16 != 0 || group < 32 || (group & (group - 1))) return false;
     if (layout != kCodesU4 && group != 128) return false;
-    // Where the vector-ALU kernel stays the default (measured on MI355X, cold, per launch in a graph): affine 4-bit
-    // nowhere (64 x 1024 to 1024 x 1024: 2.1-2.7 us against 2.5-4.0); binary and ternary below 1M weights (not
-    // measured there; from 1M on 2.2-3.1 against 2.8-3.7); five-digit bytes below 2M (equal within a tenth up to 8M).
-    if (!force && (uint64_t)rows * cols < (layout == kCodesTrit5 ? (2u << 20) : (layout == kCodesU4 ? 0u : (1u << 20)))) return false;
+    // No size threshold: measured on MI355X (cold, per launch in a graph) the single-pass kernel is the faster one
+    // at every size once small matrices walk one segment per wave: affine 4-bit 64 x 1024 to 1024 x 1024 2.1-2.7 us
+    // against 2.5-4.0 on the vector-ALU kernel, binary / ternary / five-digit bytes 256 x 1024 to 2048 x 640
+    // 2.1-2.6 / 2.1-2.5 / 2.7-3.0 against 3.2-3.3 / 2.8-3.0 / 3.5-4.0.  (`force` is kept for callers that ask.)
+    (void)force;
     const uint32_t pieces = row_stride / 16, nseg = (pieces + 7) / 8, gpr = (cols + group - 1) / group;
     const uint32_t planes = layout == kCodesU4 ? 2 : 1;
     auto lds_of = [&](uint32_t kc, uint32_t nl) {

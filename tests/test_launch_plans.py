@@ -98,8 +98,7 @@ def test_matvec_plans(layout, group):
     # the 27B layer's matrices take the kernel by default in every format
     for rows, cols in [(17408, 5120), (5120, 17408), (5120, 5120)]:
         assert cc.plan_matvec(layout, rows, cols, group) is not None
-    # small matrices stay on the vector kernels unless forced (binary and ternary below 1M weights, five-digit
-    # bytes below 2M; affine 4-bit never); small affine matrices walk few segments per wave, at most eight waves
+    # no size threshold in any format; small affine matrices walk few segments per wave, at most eight waves
     small = cc.plan_matvec(layout, 1024, 2560, group)
     assert small is not None
     if layout == cc.LAYOUT_U4:
@@ -113,8 +112,12 @@ def test_matvec_plans(layout, group):
         assert cc.plan_matvec(layout, 4096, 4096, group)["segments"] == 2
         # from 24M weights on the long walk
         assert cc.plan_matvec(layout, 5120, 5120, group)["segments"] >= 5
-    assert (cc.plan_matvec(layout, 256, 2560, group) is not None) == (layout == cc.LAYOUT_U4)
-    assert cc.plan_matvec(layout, 256, 2560, group, force=True) is not None
+    assert cc.plan_matvec(layout, 256, 2560, group) == cc.plan_matvec(layout, 256, 2560, group, force=True) is not None
+    if layout != cc.LAYOUT_U4:
+        # the signed formats below the 27B shapes walk one segment per wave (ternary from 8M weights two)
+        assert cc.plan_matvec(layout, 2048, 2048, group)["segments"] == 1
+        assert cc.plan_matvec(layout, 4096, 4096, group)["segments"] == (2 if layout == cc.LAYOUT_TERNARY2 else 1)
+        assert cc.plan_matvec(layout, 17408, 5120, group)["segments"] == 2
 
 
 def test_matvec_plan_rejects_bad_arguments():
