@@ -19,6 +19,13 @@
 SMELT_MM1_EVERY_NL(f16, smelt::F16)
 SMELT_MM1_EVERY_NL(bf16, smelt::BF16)
 
+// affine rows of more than 24576 columns (96 segments: sixteen waves of six) need seven or eight per wave
+#define SMELT_MM1_AFFINE_LONG(T, ACT)                                                             \
+    SMELT_AFFINE_MM1_KERNELS(T, ACT, ACT, 7) SMELT_AFFINE_MM1_BANK(T, ACT, ACT, 7)                 \
+    SMELT_AFFINE_MM1_KERNELS(T, ACT, ACT, 8) SMELT_AFFINE_MM1_BANK(T, ACT, ACT, 8)
+SMELT_MM1_AFFINE_LONG(f16, smelt::F16)
+SMELT_MM1_AFFINE_LONG(bf16, smelt::BF16)
+
 #define SMELT_MM1_TRIT5(T, ACT)                                                                   \
     SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 1) SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 2) \
     SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 3)                                    \

@@ -8,7 +8,8 @@
 #define SMELT_MM1F_EVERY_NL(T, ACT)                                                               \
     SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 1) SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 2)                 \
     SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 3) SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 4)                 \
-    SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 5) SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 6)
+    SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 5) SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 6)                 \
+    SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 7) SMELT_AFFINE_MM1_FUSED(T, ACT, ACT, 8)
 
 SMELT_MM1F_EVERY_NL(f16, smelt::F16)
 SMELT_MM1F_EVERY_NL(bf16, smelt::BF16)

@@ -123,7 +123,7 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
               bool force, Mm1Plan* out) {
     uint32_t row_stride, frags, nl_max, dw = 4;
     switch (layout) {
-        case kCodesU4: row_stride = cols / 2; frags = 4; nl_max = 6; break;
+        case kCodesU4: row_stride = cols / 2; frags = 4; nl_max = 8; break;
         case kCodesTernary2: row_stride = (cols + 127u) / 128u * 32u; frags = 8; nl_max = 3; break;
         case kCodesBinary1: row_stride = (cols + 127u) / 128u * 16u; frags = 16; nl_max = 3; break;
         // five digits per byte: a 16-byte piece is five dwords of sixteen columns, a 128-byte segment five groups
@@ -151,13 +151,14 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     // segments): as many segments per wave as the kernels have.  The signed formats measured best with two
     // (binary 27B layer 33.5 -> 31.5 us, five-digit bytes 50.2 -> 47.6 against three; one or four and more
     // were slower), then three where two would need more than sixteen waves.
-    static const uint32_t kLongRows[] = {6, 5, 4, 3, 2, 1}, kSigned[] = {2, 3, 1};
+    // (seven and eight only where nothing shorter covers the row: rows of more than 24576 columns)
+    static const uint32_t kLongRows[] = {6, 5, 4, 3, 2, 1, 7, 8}, kSigned[] = {2, 3, 1};
     const uint32_t* order = layout == kCodesU4 ? kLongRows : kSigned;
-    const uint32_t norder = layout == kCodesU4 ? 6 : 3;
+    const uint32_t norder = layout == kCodesU4 ? 8 : 3;
     // Affine matrices below 8M weights (a 0.8B model's projections) are a launch and one memory round trip:
     // the more waves share a row the shorter that trip, so the fewest segments per wave that eight waves cover
     // (config-1 step 0.366 -> 0.346 ms against the vector kernels)
-    static const uint32_t kShortWalk[] = {1, 2, 3, 4, 5, 6};
+    static const uint32_t kShortWalk[] = {1, 2, 3, 4, 5, 6, 7, 8};
     const bool small_affine = layout == kCodesU4 && (uint64_t)rows * cols < (8u << 20);
     if (small_affine) order = kShortWalk;
     // Between 8M and 24M weights (a 4B model's projections: 13 MB, a few workgroups per compute unit) two
@@ -166,7 +167,7 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     // segments: twelve waves) 6.4 against 7.0, 4096 x 4096 4.2 against 4.5, 3072 x 3072 3.8 against 4.4.  From 24M
     // weights on (5120-column rows and longer) the long walk stays: 5120 x 5120 5.7 against 6.0, 17408 x 5120
     // gate+up 19.5 against 22.4.
-    static const uint32_t kMidWalk[] = {2, 1, 3, 4, 5, 6};
+    static const uint32_t kMidWalk[] = {2, 1, 3, 4, 5, 6, 7, 8};
     const bool mid_affine = layout == kCodesU4 && !small_affine && (uint64_t)rows * cols < (24u << 20);
     if (mid_affine) order = kMidWalk;
     // The signed formats below the 27B shapes: one segment per wave (binary 4096 x 4096 3.5 against 3.8 us,
@@ -175,12 +176,34 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     static const uint32_t kSignedShort[] = {1, 2, 3};
     if (layout != kCodesU4 && (uint64_t)rows * cols < (layout == kCodesTernary2 ? (8u << 20) : (24u << 20))) order = kSignedShort;
     const uint64_t tiles = ((uint64_t)rows + 7) / 8;
+    // Affine matrices from 24M weights: a wave count that is a multiple of four (every SIMD of the compute unit
+    // carries the same number of the workgroup's waves) with next to no idle segments, eight first, then twelve,
+    // four, sixteen.  Measured per launch, cold, against the long walk below: 8192 x 8192 9.6 against 10.8 us
+    // (four segments on eight waves), 28672 x 8192 27.2 against 31.1, 4096 x 8192 6.25 against 6.9, 14336 x 4096
+    // 8.4 against 8.6 (two on eight), 4096 x 14336 9.7 against 10.5 (five on twelve); 5120- and 17408-column rows
+    // come out as before (five on four, six on twelve).
+    if (layout == kCodesU4 && !small_affine && !mid_affine) {
+        static const uint32_t kWaves[] = {8, 12, 4, 16};
+        for (uint32_t longest : {6u, nl_max})   // seven and eight segments only where six cover no such split
+        for (uint32_t kc : kWaves) {
+            const uint32_t nl = (nseg + kc - 1) / kc;
+            if (nl < 1 || nl > longest || (nseg + nl - 1) / nl != kc || gpr > 64 * kc) continue;
+            const uint32_t waste = kc * nl - nseg;
+            const size_t lds = lds_of(kc, nl);
+            if (waste > tolerated || lds > lds_limit) continue;
+            out->kc = kc; out->nl = nl; out->lds = lds;
+            return true;
+        }
+    }
+    // (a second pass without the size class's own limits: a short matrix of very long rows still has a plan)
+    for (int pass = 0; pass < 2 && best.kc == 0; ++pass)
     for (uint32_t o = 0; o < norder; ++o) {
         const uint32_t nl = order[o];
         if (nl > nl_max || (nl > nseg && nl > 1)) continue;
         const uint32_t kc = (nseg + nl - 1) / nl;
-        if (kc > (small_affine ? 8u : (mid_affine ? 12u : 16u)) || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
-        if (mid_affine && nl < 6 && tiles * kc > 11264) continue;   // 1.375 x the 8192 wave slots of the machine
+        const uint32_t most = pass == 0 ? (small_affine ? 8u : (mid_affine ? 12u : 16u)) : 16u;
+        if (kc > most || gpr > 64 * kc) continue;   // one workgroup; its threads carry one scale piece each
+        if (pass == 0 && mid_affine && nl < 6 && tiles * kc > 11264) continue;   // 1.375 x the 8192 wave slots of the machine
         const size_t lds = lds_of(kc, nl);
         if (lds > lds_limit) continue;
         const uint32_t waste = kc * nl - nseg;

@@ -148,7 +148,7 @@ uint32_t signed_row_stride(SignedFormat f, uint32_t cols);
 // Launch plan of the single-pass matrix-core matvec: one workgroup of `kc` waves per eight rows,
 // `nl` 128-byte row segments per wave.  False when the shape stays on the vector-ALU kernels
 // (`force` drops the size threshold, not the geometry limits).
-constexpr uint32_t kMm1MaxSegments = 6;
+constexpr uint32_t kMm1MaxSegments = 8;
 struct Mm1Plan {
     uint32_t kc = 0, nl = 0;
     size_t lds = 0;

@@ -31,8 +31,9 @@ def vec():
 
 # rows: multiples of 8, ragged tails, fewer than one tile; cols: one 16-byte piece per row, a partial
 # 128-byte segment, several segments per wave, several waves per row
+# (28672 columns: 112 segments, seven per wave on sixteen waves; 8192: four per wave on eight; 30720: eight on fifteen)
 AFFINE_SHAPES = [(8, 32, 32), (5, 64, 64), (50, 1152, 64), (130, 3584, 64), (24, 2560, 128), (264, 5120, 64),
-                 (72, 17408, 64), (33, 9216, 32)]
+                 (72, 17408, 64), (33, 9216, 32), (40, 28672, 64), (8200, 8192, 64), (19, 30720, 128)]
 
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])

@@ -110,8 +110,13 @@ def test_matvec_plans(layout, group):
         assert (cc.plan_matvec(layout, 9216, 2560, group)["segments"], cc.plan_matvec(layout, 9216, 2560, group)["waves"]) == (2, 5)
         assert (cc.plan_matvec(layout, 2560, 9216, group)["segments"], cc.plan_matvec(layout, 2560, 9216, group)["waves"]) == (3, 12)
         assert cc.plan_matvec(layout, 4096, 4096, group)["segments"] == 2
-        # from 24M weights on the long walk
-        assert cc.plan_matvec(layout, 5120, 5120, group)["segments"] >= 5
+        # from 24M weights on: a multiple of four waves with next to no idle segments, else the long walk
+        for rows, cols, want in [(5120, 5120, (5, 4)), (17408, 5120, (5, 4)), (5120, 17408, (6, 12)), (8192, 8192, (4, 8)),
+                                 (14336, 4096, (2, 8)), (4096, 14336, (5, 12)), (8192, 28672, (7, 16))]:
+            p = cc.plan_matvec(layout, rows, cols, group)
+            assert (p["segments"], p["waves"]) == want, (rows, cols, p)
+        assert cc.plan_matvec(layout, 64, 32768, group)["segments"] == 8
+        assert cc.plan_matvec(layout, 64, 32768 + 256, group) is None      # 129 segments: no single workgroup covers the row
     assert cc.plan_matvec(layout, 256, 2560, group) == cc.plan_matvec(layout, 256, 2560, group, force=True) is not None
     if layout != cc.LAYOUT_U4:
         # the signed formats below the 27B shapes walk one segment per wave (ternary from 8M weights two)
