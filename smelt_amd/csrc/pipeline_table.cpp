@@ -124,8 +124,8 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     uint32_t row_stride, frags, nl_max, dw = 4;
     switch (layout) {
         case kCodesU4: row_stride = cols / 2; frags = 4; nl_max = 8; break;
-        case kCodesTernary2: row_stride = (cols + 127u) / 128u * 32u; frags = 8; nl_max = 3; break;
-        case kCodesBinary1: row_stride = (cols + 127u) / 128u * 16u; frags = 16; nl_max = 3; break;
+        case kCodesTernary2: row_stride = (cols + 127u) / 128u * 32u; frags = 8; nl_max = 6; break;
+        case kCodesBinary1: row_stride = (cols + 127u) / 128u * 16u; frags = 16; nl_max = 6; break;
         // five digits per byte: a 16-byte piece is five dwords of sixteen columns, a 128-byte segment five groups
         case kCodesTrit5: if (cols % 16 != 0) return false; row_stride = (((cols + 4u) / 5u) + 15u) & ~15u; frags = 10; nl_max = 3; dw = 5; break;
         default: return false;
@@ -152,9 +152,11 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     // (binary 27B layer 33.5 -> 31.5 us, five-digit bytes 50.2 -> 47.6 against three; one or four and more
     // were slower), then three where two would need more than sixteen waves.
     // (seven and eight only where nothing shorter covers the row: rows of more than 24576 columns)
-    static const uint32_t kLongRows[] = {6, 5, 4, 3, 2, 1, 7, 8}, kSigned[] = {2, 3, 1};
+    // (binary and ternary: four to six only for rows that three per wave on sixteen waves do not cover, ternary
+    // beyond 24576 columns; the five-digit kernels exist for one to three: up to 30720 columns)
+    static const uint32_t kLongRows[] = {6, 5, 4, 3, 2, 1, 7, 8}, kSigned[] = {2, 3, 1, 4, 5, 6, 7, 8};
     const uint32_t* order = layout == kCodesU4 ? kLongRows : kSigned;
-    const uint32_t norder = layout == kCodesU4 ? 8 : 3;
+    const uint32_t norder = 8;
     // Affine matrices below 8M weights (a 0.8B model's projections) are a launch and one memory round trip:
     // the more waves share a row the shorter that trip, so the fewest segments per wave that eight waves cover
     // (config-1 step 0.366 -> 0.346 ms against the vector kernels)
@@ -173,7 +175,7 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     // The signed formats below the 27B shapes: one segment per wave (binary 4096 x 4096 3.5 against 3.8 us,
     // 9216 x 2560 4.25 against 4.5; five-digit bytes 4.55 against 4.9 and 5.3 against 5.7; 2048 x 2048 in all three
     // 2.6 / 2.6 / 3.35 against 2.8 / 2.8 / 3.8); ternary from 8M weights keeps two (3.5 against 3.7, 4.3 against 4.4).
-    static const uint32_t kSignedShort[] = {1, 2, 3};
+    static const uint32_t kSignedShort[] = {1, 2, 3, 4, 5, 6, 7, 8};
     if (layout != kCodesU4 && (uint64_t)rows * cols < (layout == kCodesTernary2 ? (8u << 20) : (24u << 20))) order = kSignedShort;
     const uint64_t tiles = ((uint64_t)rows + 7) / 8;
     // Affine matrices from 24M weights: a wave count that is a multiple of four (every SIMD of the compute unit

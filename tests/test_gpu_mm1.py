@@ -58,7 +58,8 @@ def test_affine_matrix_core_exact_on_dyadic_fixture(ctx):
     assert np.array_equal(y, ref.astype(np.float16).view(np.uint16))
 
 
-SIGNED_SHAPES = [(5, 128), (8, 256), (50, 1152), (1024, 5120), (264, 17408), (77, 9216)]
+# (28672 columns: a ternary row of 56 segments takes four per wave)
+SIGNED_SHAPES = [(5, 128), (8, 256), (50, 1152), (1024, 5120), (264, 17408), (77, 9216), (40, 28672)]
 
 
 def pack_signed(codes, fmt, garbage_padding=False):
