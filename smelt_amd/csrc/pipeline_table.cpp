@@ -183,13 +183,26 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     // four, sixteen.  Measured per launch, cold, against the long walk below: 8192 x 8192 9.6 against 10.8 us
     // (four segments on eight waves), 28672 x 8192 27.2 against 31.1, 4096 x 8192 6.25 against 6.9, 14336 x 4096
     // 8.4 against 8.6 (two on eight), 4096 x 14336 9.7 against 10.5 (five on twelve); 5120- and 17408-column rows
-    // come out as before (five on four, six on twelve).
+    // come out as before (five on four, six on twelve).  Never one segment per wave here: a tall matrix of short
+    // rows (an lm_head read as plain logits) has thousands of tiles and wants few, long waves (151936 x 1024: four
+    // segments on one wave 18.4 us, one on four 27.3, the vector kernel 19-20; 151936 x 2048: 31.8-34.8 against 53).
+    if (layout == kCodesU4 && !small_affine && !mid_affine && tiles >= 16384 && nseg <= 8) {
+        // short rows and more tiles than twice the machine's wave slots: one wave per tile
+        // (151936 x 2048: eight segments on one wave 31.8 us, two on four 34.8-43.3, the vector kernel 38-39)
+        for (uint32_t nl = nl_max < nseg ? nl_max : nseg; nl >= 1; --nl) {
+            const uint32_t kc = (nseg + nl - 1) / nl;
+            const size_t lds = lds_of(kc, nl);
+            if (kc > 16 || gpr > 64 * kc || kc * nl - nseg > tolerated || lds > lds_limit) continue;
+            out->kc = kc; out->nl = nl; out->lds = lds;
+            return true;
+        }
+    }
     if (layout == kCodesU4 && !small_affine && !mid_affine) {
         static const uint32_t kWaves[] = {8, 12, 4, 16};
         for (uint32_t longest : {6u, nl_max})   // seven and eight segments only where six cover no such split
         for (uint32_t kc : kWaves) {
             const uint32_t nl = (nseg + kc - 1) / kc;
-            if (nl < 1 || nl > longest || (nseg + nl - 1) / nl != kc || gpr > 64 * kc) continue;
+            if (nl < 2 || nl > longest || (nseg + nl - 1) / nl != kc || gpr > 64 * kc) continue;
             const uint32_t waste = kc * nl - nseg;
             const size_t lds = lds_of(kc, nl);
             if (waste > tolerated || lds > lds_limit) continue;

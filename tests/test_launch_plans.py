@@ -115,6 +115,10 @@ def test_matvec_plans(layout, group):
                                  (14336, 4096, (2, 8)), (4096, 14336, (5, 12)), (8192, 28672, (7, 16))]:
             p = cc.plan_matvec(layout, rows, cols, group)
             assert (p["segments"], p["waves"]) == want, (rows, cols, p)
+        # never one segment per wave from 24M weights on; a vocabulary-sized matrix of short rows: one wave per tile
+        for rows, cols, want in [(16384, 2048, (2, 4)), (65536, 1024, (4, 1)), (151936, 1024, (4, 1)), (151936, 2048, (8, 1))]:
+            p = cc.plan_matvec(layout, rows, cols, group)
+            assert (p["segments"], p["waves"]) == want, (rows, cols, p)
         assert cc.plan_matvec(layout, 64, 32768, group)["segments"] == 8
         assert cc.plan_matvec(layout, 64, 32768 + 256, group) is None      # 129 segments: no single workgroup covers the row
     assert cc.plan_matvec(layout, 256, 2560, group) == cc.plan_matvec(layout, 256, 2560, group, force=True) is not None
