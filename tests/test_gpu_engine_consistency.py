@@ -108,18 +108,24 @@ def _signed_record(ctx, fmt, name, rows, cols, dtype):
     return rt.make_record(pipe, bufs, [(4, rows), (5, cols)], (min(1024, (rows + 7) // 8), 1, 1), (256, 1, 1))
 
 
+# (the second rows: one shape of each size class of the launch plan: below 1M weights, 8M-24M, from 24M with eight
+# and twelve waves, a row beyond 24576 columns, a tall matrix of short rows)
 AFFINE_SWEEP = [(4096, 4096, 64, "matvec"), (11008, 4096, 128, "matvec"), (4096, 11008, 64, "matvec"), (1536, 8960, 64, "matvec"),
-                (32000, 4096, 32, "matvec"), (1024, 1024, 64, "matvec"), (6912, 2304, 64, "gate_up"), (14336, 4096, 128, "gate_up")]
+                (32000, 4096, 32, "matvec"), (1024, 1024, 64, "matvec"), (6912, 2304, 64, "gate_up"), (14336, 4096, 128, "gate_up"),
+                (512, 1024, 64, "matvec"), (9216, 2560, 64, "matvec"), (8192, 8192, 64, "matvec"), (4096, 14336, 64, "matvec"),
+                (4096, 28672, 64, "matvec"), (32768, 2048, 64, "matvec")]
 SIGNED_SWEEP = [(fx.BINARY1, "binary", 8192, 8192), (fx.BINARY1, "binary", 4096, 14336), (fx.BINARY1, "binary", 2048, 2048),
                 (fx.TERNARY2, "ternary", 14336, 4096), (fx.TERNARY2, "ternary", 8192, 2048), (fx.TRIT5, "trit5", 8192, 4096),
-                (fx.TRIT5, "trit5", 2560, 10240)]
+                (fx.TRIT5, "trit5", 2560, 10240),
+                (fx.BINARY1, "binary", 512, 1024), (fx.TERNARY2, "ternary", 1024, 1024), (fx.TRIT5, "trit5", 1024, 1280)]
 
 
 def test_auto_engine_is_not_the_slower_one(ctx):
-    """AUTO's size thresholds were fitted on the benchmark's shapes.  On a sweep of other shapes (Llama- and
-    Gemma-like projections, a short-and-wide and a tall-and-narrow matrix, one shape at a threshold) the kernel AUTO
-    picks must not lose to the vector kernel by more than run-to-run noise: warm single launches, medians of 120,
-    AUTO <= 1.10 x VECTOR + 0.3 us.  Where AUTO keeps the vector kernel the two times are the same measurement."""
+    """AUTO's launch plans were fitted on a handful of shapes.  On a sweep of other shapes (Llama- and Gemma-like
+    projections, a short-and-wide and a tall-and-narrow matrix, one shape of every size class of the plan) the
+    kernel AUTO picks must not lose to the vector kernel by more than run-to-run noise: warm single launches,
+    medians of 120, AUTO <= 1.10 x VECTOR + 0.3 us.  Where AUTO keeps the vector kernel the two times are the same
+    measurement."""
     dtype = fx.BF16
     lines, worst = [], 0.0
 
