@@ -568,7 +568,7 @@ def qmm_measurements(fx, cc, rt, cus, engine) -> dict:
     layer_bytes = sum(e.size_bytes + e.scales_size_bytes + e.biases_size_bytes for e in ents[0])
     assert layer_bytes == one
     qmm = {}
-    for M in (1, 7, 8, 9, 16, 32, 128, 512):
+    for M in (1, 4, 7, 8, 9, 16, 32, 128, 512):
         em = cc.Emitter(rt.ACT_BF16, cus)
         for layer in ents:
             for e in layer:

@@ -1119,14 +1119,19 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             routed = true;
         }
     }
+    const bool qms_pair = p->res.family == kFamAffineQmmGateUp || p->res.family == kFamAffineGateUpBatched;
+    const bool qms_small_batch = p->res.family == kFamAffineBatched || p->res.family == kFamAffineGateUpBatched;
     if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
-        aligned16(p->res.family == kFamAffineQmmGateUp ? 7 : 4) && whole_pieces(p->res.family == kFamAffineQmmGateUp ? 7 : 4)) {
-        // skinny qmm: the streaming kernel of the same pipeline, same arguments, its own launch
+        aligned16(qms_pair ? 7 : 4) && whole_pieces(qms_pair ? 7 : 4)) {
+        // skinny qmm (and, from two tokens on, the per-token small-batch forms, whose arguments are the
+        // same): the streaming kernel of the same pipeline, same arguments, its own launch
         // geometry (16 * rt rows per workgroup, 16 tokens per grid row); it uses no workspace
-        const size_t o = p->res.family == kFamAffineQmm ? 5 : (p->res.family == kFamAffineQmmAdd ? 7 : 8);
+        const size_t o = qms_pair ? 8 : (p->res.family == kFamAffineQmmAdd ? 7 : 5);
         const uint32_t batch = L.args[o].value, rows = L.args[o + 1].value, cols = L.args[o + 2].value, group = L.args[o + 3].value;
         QmtPlan tplan;
-        if (qmt_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &tplan) && (tplan.per_wave ? p->fn_qmt_per_wave : p->fn_qmt)[tplan.rt][tplan.tb][tplan.kw]) {
+        if (qms_small_batch && batch < 2) {
+            // one token: the kernel the record names
+        } else if (qmt_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &tplan) && (tplan.per_wave ? p->fn_qmt_per_wave : p->fn_qmt)[tplan.rt][tplan.tb][tplan.kw]) {
             fn = (tplan.per_wave ? p->fn_qmt_per_wave : p->fn_qmt)[tplan.rt][tplan.tb][tplan.kw];
             // a split that the workspace of this call cannot hold is not taken
             const uint32_t ksplit = tplan.partial_bytes <= ws.partial_bytes && tplan.counter_bytes <= ws.counter_bytes ? tplan.ksplit : 1;
@@ -1137,7 +1142,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             qms_routed = true;
         }
         QmsPlan plan;
-        if (!routed && batch > 0 && qms_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
+        if (!routed && batch > (qms_small_batch ? 1u : 0u) && qms_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
             fn = p->fn_qms[plan.rt][batch > 8];
             L.grid[0] = (rows + 16 * plan.rt - 1) / (16 * plan.rt); L.grid[1] = (batch + 15) / 16; L.grid[2] = 1;
             L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
