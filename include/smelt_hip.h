@@ -127,13 +127,15 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * kernel (the two add up a row in different orders: results agree to the output tolerance, not bit
  * for bit); MATRIX_CORE asks for the same explicitly (kept from when AUTO had size thresholds);
  * VECTOR keeps every record on the vector-ALU kernels.  The same switch
- * covers the qmm records: AUTO and MATRIX_CORE run the streaming kernel of the pipeline below 128
+ * covers the qmm records and, from two tokens on, the per-token small-batch ("_batched", "_batched_verify_b4")
+ * forms of the group-64 affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's: AUTO and
+ * MATRIX_CORE run the streaming kernel of the pipeline below 128
  * tokens (K split inside a workgroup, no workspace) and the token-tile kernel from 128 tokens on
  * (matrices with few tiles and long rows split K across workgroups: partial sums in the
  * workspace, added in a fixed order), VECTOR the split-K or token-slab kernel the record's geometry
  * describes (split-K: partial sums in the workspace).  Results of the alternatives differ in
  * summation order only.  Consequence under AUTO: the records of one model run on two summation
- * orders, e.g. a matvec at one token (matrix-core kernel) and its batched-verify form (vector
+ * orders, e.g. a matvec at one token (single-pass kernel) and its batched-verify form (streaming
  * kernel) agree to one step of the output type but not bit for bit; a caller that compares such
  * rows bit for bit pins one engine.  On one engine a fused kernel and the staged pair it
  * replaces are bit-identical.  No counterpart in the reference (one kernel per pipeline name there);
