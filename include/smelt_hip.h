@@ -128,7 +128,10 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * for bit); MATRIX_CORE asks for the same explicitly (kept from when AUTO had size thresholds);
  * VECTOR keeps every record on the vector-ALU kernels.  The same switch
  * covers the qmm records and, from two tokens on, the per-token small-batch ("_batched", "_batched_verify_b4")
- * forms of the group-64 affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's: AUTO and
+ * forms of the group-64 affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's, and the
+ * lm_head matvec+argmax over two tokens and more without a logit cap (logits of all tokens through the
+ * streaming kernel into the context workspace, partial keys from a second launch: the record then counts as
+ * two launches): AUTO and
  * MATRIX_CORE run the streaming kernel of the pipeline below 128
  * tokens (K split inside a workgroup, no workspace) and the token-tile kernel from 128 tokens on
  * (matrices with few tiles and long rows split K across workgroups: partial sums in the

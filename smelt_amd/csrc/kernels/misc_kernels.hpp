@@ -190,6 +190,37 @@ SMELT_MISC_KERNEL void smelt_lm_head_argmax_reduce(const smelt::uint2_t* partial
     }
 }
 
+// lm_head over several tokens, second half: the streaming qmm has left the rounded logits of `batch`
+// tokens in `logits` [batch][rows]; this forms the same partial keys the fused matvec+argmax kernel
+// leaves (one per token and grid column, any partition of the rows gives the same final key), so the
+// record's reduce launch reads them unchanged.  Grid (num_partials, batch), one wave per workgroup.
+// The bits are ordered as 16-bit floats of either type (sign and magnitude), so one kernel serves both.
+SMELT_MISC_KERNEL void smelt_logits_argmax_partials(const uint16_t* __restrict__ logits, smelt::uint2_t* partials,
+                                                    uint32_t batch, uint32_t rows, uint32_t num_partials) {
+    using namespace smelt;
+    const uint32_t tok = blockIdx.y;
+    if (tok >= batch || blockIdx.x >= num_partials) return;
+    const uint32_t per = (rows + num_partials - 1) / num_partials;
+    const uint32_t lo = blockIdx.x * per;
+    const uint32_t hi = lo + per < rows ? lo + per : rows;
+    const uint16_t* row = logits + (size_t)tok * rows;
+    uint2_t best = uint2_t{0u, 0u};
+    for (uint32_t r = lo + threadIdx.x; r < hi; r += blockDim.x) {
+        const uint2_t key = argmax_pack_key(row[r], r);
+        if (argmax_key_gt(key, best)) best = key;
+    }
+    best = wave_argmax_key(best);
+    __shared__ uint2_t wave_best[16];
+    const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) wave_best[wave] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t waves = (blockDim.x + kWave - 1) / kWave;
+        for (uint32_t w = 1; w < waves; ++w) best = argmax_key_max(best, wave_best[w]);
+        partials[(size_t)tok * num_partials + blockIdx.x] = best;
+    }
+}
+
 // Plain device copy of n16 16-byte elements (grid-stride).  It moves a known number of bytes
 // each way, which makes it the calibration kernel for memory-traffic counters.
 extern "C" __global__ __launch_bounds__(256) void smelt_copy_u128(const smelt::uint4_t* __restrict__ src,

@@ -284,6 +284,8 @@ void attach_qms(ResolvedPipeline* r) {
     // skinny qmm of their family: from two tokens on they stream too, 9216 x 2560 at four tokens 7.8 against 16.2 us)
     if (r->family == kFamAffineQmm || r->family == kFamAffineBatched) { r->qms_tail = "store_" + t; r->qms_nmat = 1; }
     else if (r->family == kFamAffineQmmAdd) { r->qms_tail = "add_" + t; r->qms_nmat = 1; }
+    // (the lm_head over two tokens and more: logits through the streaming kernel, keys from a second launch)
+    else if (r->family == kFamAffineArgmax) { r->qms_tail = "store_" + t; r->qms_nmat = 1; }
     else if ((r->family == kFamAffineQmmGateUp || r->family == kFamAffineGateUpBatched) && r->symbol.find("swiglu") != std::string::npos) { r->qms_tail = "gate_up_swiglu_" + t; r->qms_nmat = 2; }
 }
 

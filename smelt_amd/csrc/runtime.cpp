@@ -47,6 +47,7 @@ struct Pipeline {
     hipFunction_t fn_qmt[5][5][3] = {};                           // token-tile qmm, by row tiles and token blocks per wave and waves along K
     hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
+    hipFunction_t fn_logits_keys = nullptr;                       // lm_head over several tokens: partial argmax keys from stored logits
     ResolvedPipeline res;
 };
 
@@ -1121,7 +1122,47 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     }
     const bool qms_pair = p->res.family == kFamAffineQmmGateUp || p->res.family == kFamAffineGateUpBatched;
     const bool qms_small_batch = p->res.family == kFamAffineBatched || p->res.family == kFamAffineGateUpBatched;
-    if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
+    if (p->res.family == kFamAffineArgmax) {
+        // lm_head over two tokens and more (W S B X keys batch logit_cap | rows cols group batch_tile): the fused
+        // kernel walks the weights once per token tile; instead the streaming qmm leaves the rounded logits of all
+        // tokens in the workspace and a second launch forms the same partial keys from them (151936 x 1024 at four
+        // tokens: 26 + 3 us against 67).  Not with a logit cap (the fused kernel caps before it rounds), and not
+        // when the workspace is too small for the logits.
+        const uint32_t batch = L.args[5].value, rows = L.args[7].value, cols = L.args[8].value, group = L.args[9].value;
+        QmsPlan plan;
+        if (batch >= 2 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.args[6].value == 0u && p->fn_logits_keys &&
+            aligned16(4) && whole_pieces(4) && (size_t)batch * rows * 2 <= ws.partial_bytes && ws.partial &&
+            qms_plan(rows, cols, group, 1, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) &&
+            p->fn_qms[plan.rt][batch > 8]) {
+            alignas(16) unsigned char ka[128];
+            size_t at = 0;
+            auto put_ptr = [&](const void* v) { at = (at + 7) & ~(size_t)7; memcpy(ka + at, &v, 8); at += 8; };
+            auto put_u32 = [&](uint32_t v) { memcpy(ka + at, &v, 4); at += 4; };
+            for (int i = 0; i < 4; ++i) put_ptr(L.args[(size_t)i].ptr);
+            put_ptr(ws.partial);                       // logits [batch][rows] in the activation type
+            put_u32(batch); put_u32(rows); put_u32(cols); put_u32(group); put_u32(0u);
+            put_ptr(ws.partial); put_ptr(ws.counters);  // the skinny kernels' workspace arguments: unused
+            size_t ka_size = at;
+            void* cfg_a[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size, HIP_LAUNCH_PARAM_END};
+            if (!ctx->batch_open) {
+                HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+                ctx->batch_open = true;
+                ctx->timing_valid = false;
+            }
+            HIP_TRY(ctx, hipModuleLaunchKernel(p->fn_qms[plan.rt][batch > 8], (rows + 16 * plan.rt - 1) / (16 * plan.rt), (batch + 15) / 16, 1,
+                                               64 * plan.kc, 1, 1, (unsigned)plan.lds, ctx->stream, nullptr, cfg_a));
+            alignas(16) unsigned char kb[64];
+            at = 0;
+            auto put_ptr_b = [&](const void* v) { at = (at + 7) & ~(size_t)7; memcpy(kb + at, &v, 8); at += 8; };
+            put_ptr_b(ws.partial); put_ptr_b(L.args[4].ptr);
+            const uint32_t tail[3] = {batch, rows, (uint32_t)L.grid[0]};
+            memcpy(kb + at, tail, sizeof tail); at += sizeof tail;
+            size_t kb_size = at;
+            void* cfg_b[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, kb, HIP_LAUNCH_PARAM_BUFFER_SIZE, &kb_size, HIP_LAUNCH_PARAM_END};
+            HIP_TRY(ctx, hipModuleLaunchKernel(p->fn_logits_keys, L.grid[0], batch, 1, 64, 1, 1, 0, ctx->stream, nullptr, cfg_b));
+            return 2;
+        }
+    } else if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
         aligned16(qms_pair ? 7 : 4) && whole_pieces(qms_pair ? 7 : 4)) {
         // skinny qmm (and, from two tokens on, the per-token small-batch forms, whose arguments are the
         // same): the streaming kernel of the same pipeline, same arguments, its own launch
@@ -1395,6 +1436,7 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
                     else (void)find(&p.fn_qmt[v.rt][v.tb][v.kw], "smelt_affine_qmt_r" + rest);
                 }
             }
+            if (p.res.family == kFamAffineArgmax) (void)find(&p.fn_logits_keys, "smelt_logits_argmax_partials");
             if (!p.res.qms_tail.empty())
                 for (uint32_t rt = 1; rt <= kQmsMaxRowTiles; ++rt)
                     for (uint32_t wide = 0; wide < 2; ++wide)
