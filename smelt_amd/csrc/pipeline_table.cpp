@@ -260,6 +260,13 @@ void attach_mm1(ResolvedPipeline* r) {
         {"smelt_signed_trit5_matvec_add_", "smelt_signed_trit5_mm1_", "matvec_add_", kCodesTrit5, 1},
         {"smelt_signed_trit5_gate_up_swiglu_", "smelt_signed_trit5_mm1_", "gate_up_swiglu_", kCodesTrit5, 2},
         {"smelt_signed_trit5_packed_bank4_matvec_", "smelt_signed_trit5_mm1_", "packed_bank4_matvec_", kCodesTrit5, 1},
+        // the four-token forms: the single-token kernels with one grid row per token
+        {"smelt_signed_binary_matvec_b4_", "smelt_signed_binary_mm1_", "matvec_", kCodesBinary1, 1},
+        {"smelt_signed_binary_gate_up_swiglu_b4_", "smelt_signed_binary_mm1_", "gate_up_swiglu_", kCodesBinary1, 2},
+        {"smelt_signed_ternary_matvec_b4_", "smelt_signed_ternary_mm1_", "matvec_", kCodesTernary2, 1},
+        {"smelt_signed_ternary_gate_up_swiglu_b4_", "smelt_signed_ternary_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},
+        {"smelt_signed_trit5_matvec_b4_", "smelt_signed_trit5_mm1_", "matvec_", kCodesTrit5, 1},
+        {"smelt_signed_trit5_gate_up_swiglu_b4_", "smelt_signed_trit5_mm1_", "gate_up_swiglu_", kCodesTrit5, 2},
         {"smelt_teraff_matvec_", "smelt_teraff_mm1_", "matvec_", kCodesTernary2, 1},
         {"smelt_teraff_matvec_add_", "smelt_teraff_mm1_", "matvec_add_", kCodesTernary2, 1},
         {"smelt_teraff_gate_up_swiglu_", "smelt_teraff_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},

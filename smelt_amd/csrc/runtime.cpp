@@ -1078,10 +1078,13 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             if (L.args[i].kind == 'P' && ((L.args[i].need + 15) & ~(size_t)15) > L.args[i].avail) return false;
         return true;
     };
-    if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.grid[1] == 1) {
+    const bool mm1_b4 = p->res.family == kFamSignedB4 || p->res.family == kFamSignedGateUpB4;
+    // (the signed single-token families take their token from the grid row: a record with several rows keeps them)
+    const bool mm1_per_row = p->res.family == kFamSignedMatvec || p->res.family == kFamSignedAdd || p->res.family == kFamSignedGateUp;
+    if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && (L.grid[1] == 1 || mm1_b4 || mm1_per_row)) {
         // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
         // arguments, its own launch geometry (one workgroup per eight rows)
-        uint32_t rows = 0, cols = 0, group = 128;
+        uint32_t rows = 0, cols = 0, group = 128, tokens = 1;
         size_t ro = 0;   // leading read-only operands (codes, scales[, biases], ..., x)
         size_t lead = 0; // ... behind this many leading arguments that are not fetched 16 bytes at a time
         auto U = [&](size_t i) { return L.args[i].value; };
@@ -1098,9 +1101,13 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             case kFamAffineAdd: rows = U(6); cols = U(7); group = U(8); ro = 4; break;
             case kFamAffineGateUp: rows = U(8); cols = U(9); group = U(10); ro = 7; break;
             case kFamAffineBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); group = U(13); ro = 4; break;
-            case kFamSignedMatvec: rows = U(4); cols = U(5); ro = 3; break;
-            case kFamSignedAdd: rows = U(5); cols = U(6); ro = 3; break;
-            case kFamSignedGateUp: rows = U(6); cols = U(7); ro = 5; break;
+            case kFamSignedMatvec: rows = U(4); cols = U(5); ro = 3; tokens = L.grid[1]; break;
+            case kFamSignedAdd: rows = U(5); cols = U(6); ro = 3; tokens = L.grid[1]; break;
+            case kFamSignedGateUp: rows = U(6); cols = U(7); ro = 5; tokens = L.grid[1]; break;
+            // four tokens per grid row in the record: one grid row per token here (the kernel takes its token from
+            // blockIdx.y; the trailing batch argument is dropped from the argument block)
+            case kFamSignedB4: rows = U(4); cols = U(5); tokens = U(6); ro = 3; break;
+            case kFamSignedGateUpB4: rows = U(6); cols = U(7); tokens = U(8); ro = 5; break;
             case kFamBinaryPackedBank: rows = U(5) + U(6); cols = U(7); ro = 3; break;
             case kFamBinaryPackedBank4: rows = U(7) + U(8) + U(9) + U(10); cols = U(11); ro = 3; break;
             case kFamTerAffMatvec: rows = U(5); cols = U(6); ro = 4; break;
@@ -1114,7 +1121,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
                                  ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &plan) &&
             p->fn_mm1[plan.nl]) {
             fn = p->fn_mm1[plan.nl];
-            L.grid[0] = (rows + 7) / 8; L.grid[1] = 1; L.grid[2] = 1;
+            L.grid[0] = (rows + 7) / 8; L.grid[1] = tokens; L.grid[2] = 1;
+            if (mm1_b4) L.args.count -= 1;
             L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
             L.lds = plan.lds;
             routed = true;

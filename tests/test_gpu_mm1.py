@@ -315,3 +315,32 @@ def test_operands_off_a_16_byte_boundary_keep_the_vector_kernel(ctx, vec):
         out.append(c.read(gh.Y_SLOT, np.uint16, rows).reshape(1, rows))
     gh.check_outputs(out[0], ref, dtype, "misaligned scale plane")
     assert np.array_equal(out[0], out[1])
+
+
+@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary"), (fx.TRIT5, "trit5")])
+@pytest.mark.parametrize("kind", ["matvec", "gate_up"])
+def test_signed_four_token_forms_run_one_grid_row_per_token(fmt, name, kind):
+    """`*_batched_b4` records (four tokens per grid row) and per-token records with several grid rows take the
+    single-pass kernel under the default engine, one grid row per token: each token's row is the single-token
+    kernel's bits and, for the plain matvec, the oracle's values to the usual bar.  Ragged batch (6 = 4 + 2) and
+    ragged rows."""
+    rows, cols, batch, dtype = 1003, 5120, 6, fx.BF16
+    c = rt.Context()
+    try:
+        mats = []
+        for t in range(2 if kind == "gate_up" else 1):
+            codes = fx.synth_signed_codes(fmt, rows, cols, config=2 + fmt, tensor=t)
+            mats.append((pack_signed(codes, fmt), fx.synth_signed_scales(rows, cols, config=2 + fmt, tensor=t)))
+        x = fx.synth_activation(batch, cols, dtype, config=2 + fmt, tensor=77)
+        second = mats[1] if kind == "gate_up" else None
+        y4 = run_signed(c, name, *mats[0], x, dtype, rows, cols, kind=kind, second=second, b4=True)
+        yr = run_signed(c, name, *mats[0], x, dtype, rows, cols, kind=kind, second=second)
+        assert np.array_equal(y4, yr)
+        for b in range(batch):
+            y1 = run_signed(c, name, *mats[0], x[b:b + 1], dtype, rows, cols, kind=kind, second=second)
+            assert np.array_equal(y4[b], y1[0]), b
+        if kind == "matvec":
+            ref = so.signed_matvec(fmt, *mats[0], fx.from_bits(x, dtype), rows, cols, cols, 128)
+            gh.check_outputs(y4, ref, dtype, f"four-token {name}")
+    finally:
+        c.close()
