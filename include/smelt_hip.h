@@ -131,7 +131,9 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * forms of the group-64 affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's, and the
  * lm_head matvec+argmax over two tokens and more without a logit cap (logits of all tokens through the
  * streaming kernel into the context workspace, partial keys from a second launch: the record then counts as
- * two launches): AUTO and
+ * two launches), and the same record at one token where the rows' 16-byte pieces leave the fused kernel's last
+ * pass over a row less than nine tenths full (1536, 2560, 3072, 3584, 5120 columns: the single-pass kernel
+ * with the argmax as its epilogue, tiles that share a partial key meeting in the context workspace): AUTO and
  * MATRIX_CORE run the streaming kernel of the pipeline below 128
  * tokens (K split inside a workgroup, no workspace) and the token-tile kernel from 128 tokens on
  * (matrices with few tiles and long rows split K across workgroups: partial sums in the

@@ -17,6 +17,9 @@ struct EpiBase {
     // An epilogue that reads one 16-bit operand per output row can have it fetched together with
     // the row's last weight item instead of after the reduction (single-token launches only).
     static constexpr bool kPrefetch = false;
+    // An epilogue of the single-pass kernel that works on a whole row tile with a whole wave
+    // (tile(token, row0, rows, lane, sums)) instead of one row per lane.
+    static constexpr bool kTile = false;
     __device__ __forceinline__ void end_chunk(int, int) const {}
 };
 

@@ -556,11 +556,74 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
             }
         }
     }
-    if (chunk == 0 && lane < 8 && row0 + lane < rows) {
+    if constexpr (Epi::kTile) {
+        if (chunk == 0) epi.tile(token, row0, rows, lane, y);
+    } else if (chunk == 0 && lane < 8 && row0 + lane < rows) {
         if constexpr (Epi::kPrefetch) epi.finish(token, row0 + lane, y, res);
         else epi(token, row0 + lane, y);
     }
 }
+
+// lm_head: argmax over the rounded logits, fused (affine_matvec_argmax, one token per grid row).  The
+// pipeline's consumer reads `num_partials` keys per token, any partition of the rows; a tile holds eight
+// rows, so the tiles t, t + num_partials, ... share partial t: each leaves its best key in the workspace
+// and counts itself in, and the last to arrive writes the best of them (keys carry their row, so the
+// result does not depend on the order of arrival).  Keys cross workgroups as agent-scope relaxed atomics
+// (coherent across the compute dies); a tile's store is acknowledged before its arrival is counted, and
+// the last arrival reads only after its count returned.  Counters are left at zero for the next launch.
+template <class ActT>
+struct EpiTileArgmax : EpiBase {
+    static constexpr bool kTile = true;
+    uint2_t* partials;                 // [token][num_partials]
+    unsigned long long* tile_keys;     // workspace: [token][tiles]
+    uint32_t* counters;                // workspace: [token][num_partials]
+    uint32_t num_partials;
+    float logit_cap;
+    __device__ __forceinline__ void tile(int token, int row0, int rows, int lane, const float* y) const {
+        float x = y[0];
+        if (logit_cap > 0.0f) {
+            // cap * tanh(x / cap) as cap * (1 - 2 / (1 + exp(2x / cap))); exp overflow gives +-cap
+            const float e = expf(2.0f * x / logit_cap);
+            x = logit_cap * (1.0f - 2.0f / (1.0f + e));
+        }
+        uint2_t key = {0u, 0u};
+        if (lane < 8 && row0 + lane < rows) key = argmax_pack_key(ActT::narrow(x), (uint32_t)(row0 + lane));
+#pragma unroll
+        for (int off = 4; off > 0; off >>= 1) {
+            uint2_t o;
+            o.x = __shfl_xor(key.x, off);
+            o.y = __shfl_xor(key.y, off);
+            key = argmax_key_max(key, o);
+        }
+        const uint32_t tiles = gridDim.x, parts = num_partials;
+        const uint32_t slot = blockIdx.x % parts;
+        const uint32_t members = tiles / parts + (slot < tiles % parts ? 1u : 0u);
+        uint2_t* out = partials + (size_t)token * parts + slot;
+        if (members == 1u) {
+            if (lane == 0) *out = key;
+            return;
+        }
+        unsigned long long* keys = tile_keys + (size_t)token * tiles;
+        uint32_t* counter = counters + (size_t)token * parts + slot;
+        uint32_t last = 0u;
+        if (lane == 0) {
+            __hip_atomic_store(keys + blockIdx.x, ((unsigned long long)key.x << 32) | key.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): the store is acknowledged
+            last = atomicAdd(counter, 1u) == members - 1u ? 1u : 0u;
+        }
+        if (!__builtin_amdgcn_readfirstlane(last)) return;
+        uint2_t best = {0u, 0u};
+        for (uint32_t j = (uint32_t)lane; j < members; j += kWave) {
+            const unsigned long long v = __hip_atomic_load(keys + slot + (size_t)j * parts, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            best = argmax_key_max(best, uint2_t{(uint32_t)(v >> 32), (uint32_t)v});
+        }
+        best = wave_argmax_key(best);
+        if (lane == 0) {
+            *out = best;
+            *counter = 0u;
+        }
+    }
+};
 
 }  // namespace smelt
 
@@ -709,6 +772,18 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         EpiGeglu<ACT> epi{{}, Y, (int)rows};                                                      \
         mm1_body<M1U4<ACT>, ACT, SC, 2, NLV, EpiGeglu<ACT>, 1>(mats, X, rows, cols, cols / 2, group, epi, \
                                                                NormScale{rs, nw, nullptr});       \
+    }
+
+// lm_head: one launch, one token per grid row; the workspace holds a key per tile and a counter per partial.
+#define SMELT_AFFINE_MM1_ARGMAX(T, ACT, SC, NLV)                                                  \
+    SMELT_MM1_KERNEL void smelt_affine_mm1_nl##NLV##_matvec_argmax_##T(                           \
+        const u8* W, const u16* S, const u16* B, const u16* X, smelt::uint2_t* keys,              \
+        unsigned long long* tile_keys, u32* counters, u32 rows, u32 cols, u32 group,              \
+        u32 num_partials, float logit_cap) {                                                      \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{W, S, B}};                                                      \
+        EpiTileArgmax<ACT> epi{{}, keys, tile_keys, counters, num_partials, logit_cap};           \
+        mm1_body<M1U4<ACT>, ACT, SC, 1, NLV>(mats, X, rows, cols, cols / 2, group, epi);          \
     }
 
 // Ternary "affine" pipelines bind the scale plane a second time where MLX binds a bias plane; it

@@ -5,7 +5,6 @@
 // an in-scope family maps onto a handful of symbols plus appended shape values.
 #include "pipeline_table.hpp"
 
-#include <cstdlib>
 #include <cstring>
 
 namespace smelt_host {
@@ -186,9 +185,11 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     // come out as before (five on four, six on twelve).  Never one segment per wave here: a tall matrix of short
     // rows (an lm_head read as plain logits) has thousands of tiles and wants few, long waves (151936 x 1024: four
     // segments on one wave 18.4 us, one on four 27.3, the vector kernel 19-20; 151936 x 2048: 31.8-34.8 against 53).
-    if (layout == kCodesU4 && !small_affine && !mid_affine && tiles >= 16384 && nseg <= 8) {
-        // short rows and more tiles than twice the machine's wave slots: one wave per tile
-        // (151936 x 2048: eight segments on one wave 31.8 us, two on four 34.8-43.3, the vector kernel 38-39)
+    if (layout == kCodesU4 && !small_affine && !mid_affine && tiles >= 16384 && nseg <= 16) {
+        // more tiles than twice the machine's wave slots: as few waves per tile as cover the row, one up to eight
+        // segments, two up to sixteen (151936 x 2048: eight segments on one wave 31.8 us, two on four 34.8-43.3,
+        // the vector kernel 38-39; cold, 151936 x 3072: six on two 51.0, three on four 58.5, vector 65; 151936 x 3584:
+        // seven on two 61.6, five on three 66.3-68.6, vector 70; 151936 x 4096: two, four and eight waves 74-75)
         for (uint32_t nl = nl_max < nseg ? nl_max : nseg; nl >= 1; --nl) {
             const uint32_t kc = (nseg + nl - 1) / nl;
             const size_t lds = lds_of(kc, nl);
@@ -267,6 +268,8 @@ void attach_mm1(ResolvedPipeline* r) {
         {"smelt_signed_ternary_gate_up_swiglu_b4_", "smelt_signed_ternary_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},
         {"smelt_signed_trit5_matvec_b4_", "smelt_signed_trit5_mm1_", "matvec_", kCodesTrit5, 1},
         {"smelt_signed_trit5_gate_up_swiglu_b4_", "smelt_signed_trit5_mm1_", "gate_up_swiglu_", kCodesTrit5, 2},
+        // the lm_head at one token (its own argument block: a key per tile and a counter per partial in the workspace)
+        {"smelt_affine_matvec_argmax_", "smelt_affine_mm1_", "matvec_argmax_", kCodesU4, 1},
         {"smelt_teraff_matvec_", "smelt_teraff_mm1_", "matvec_", kCodesTernary2, 1},
         {"smelt_teraff_matvec_add_", "smelt_teraff_mm1_", "matvec_add_", kCodesTernary2, 1},
         {"smelt_teraff_gate_up_swiglu_", "smelt_teraff_mm1_", "gate_up_swiglu_", kCodesTernary2, 2},

@@ -1137,6 +1137,44 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         // tokens: 26 + 3 us against 67).  Not with a logit cap (the fused kernel caps before it rounds), and not
         // when the workspace is too small for the logits.
         const uint32_t batch = L.args[5].value, rows = L.args[7].value, cols = L.args[8].value, group = L.args[9].value;
+        // At one token: the single-pass kernel with the argmax as its epilogue, where the fused vector kernel leaves
+        // lanes idle.  That kernel covers a row in whole passes of 64 (32, 16) 16-byte pieces; with the last pass partly
+        // empty it loses (cold, per launch: 151936 x 2560 52 against 43-46 us, x 1536 30 against 27, x 5120 87 against
+        // 80-82, 32000 x 2560 16.0 against 12.9-13.7, x 5120 24.3 against 20.3-20.8), with full passes it wins or ties
+        // (151936 x 1024 19.6 against 21.3, x 2048 33.5 against 34.4, x 4096 64 against 73-75, 32000 x 8192 32.3 against 32).
+        // The record's consumer reads grid-width keys per token, any partition of the rows: the eight-row tiles
+        // t, t + width, ... meet in partial t through the workspace (a key per tile, a counter per partial), so
+        // the route needs at least one tile per partial, at most a wave's worth, and room in the workspace.
+        const uint32_t tiles = (rows + 7) / 8, parts = L.grid[0];
+        const uint32_t units = cols / 32, pass = units > 32 ? 64 : (units > 16 ? 32 : 16);
+        const bool idle_lanes = (uint64_t)units * 10 < (uint64_t)((units + pass - 1) / pass * pass) * 9;
+        Mm1Plan mplan;
+        hipFunction_t fn_argmax = nullptr;
+        if (batch == 1 && idle_lanes && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && p->res.mm1_layout >= 0 && parts > 0 &&
+            aligned16(4) && whole_pieces(4) &&
+            mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, 1, ctx->lds_limit,
+                     ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &mplan) && p->fn_mm1[mplan.nl]) {
+            fn_argmax = p->fn_mm1[mplan.nl];
+        }
+        if (fn_argmax && tiles >= parts && tiles <= 64u * (uint64_t)parts && ws.partial && ws.counters &&
+            (size_t)tiles * 8 <= ws.partial_bytes && (size_t)parts * 4 <= ws.counter_bytes) {
+            alignas(16) unsigned char ka[128];
+            size_t at = 0;
+            auto put_ptr = [&](const void* v) { at = (at + 7) & ~(size_t)7; memcpy(ka + at, &v, 8); at += 8; };
+            auto put_u32 = [&](uint32_t v) { memcpy(ka + at, &v, 4); at += 4; };
+            for (int i = 0; i < 5; ++i) put_ptr(L.args[(size_t)i].ptr);   // W S B X keys
+            put_ptr(ws.partial); put_ptr(ws.counters);
+            put_u32(rows); put_u32(cols); put_u32(group); put_u32(parts); put_u32(L.args[6].value);   // (the cap's float bits)
+            size_t ka_size = at;
+            void* cfg[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size, HIP_LAUNCH_PARAM_END};
+            if (!ctx->batch_open) {
+                HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+                ctx->batch_open = true;
+                ctx->timing_valid = false;
+            }
+            HIP_TRY(ctx, hipModuleLaunchKernel(fn_argmax, tiles, 1, 1, 64 * mplan.kc, 1, 1, (unsigned)mplan.lds, ctx->stream, nullptr, cfg));
+            return 1;
+        }
         QmsPlan plan;
         if (batch >= 2 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.args[6].value == 0u && p->fn_logits_keys &&
             aligned16(4) && whole_pieces(4) && (size_t)batch * rows * 2 <= ws.partial_bytes && ws.partial &&

@@ -109,11 +109,11 @@ def _signed_record(ctx, fmt, name, rows, cols, dtype):
 
 
 # (the second rows: one shape of each size class of the launch plan: below 1M weights, 8M-24M, from 24M with eight
-# and twelve waves, a row beyond 24576 columns, a tall matrix of short rows)
+# and twelve waves, a row beyond 24576 columns, a tall matrix of short rows, a tall matrix with two waves per tile)
 AFFINE_SWEEP = [(4096, 4096, 64, "matvec"), (11008, 4096, 128, "matvec"), (4096, 11008, 64, "matvec"), (1536, 8960, 64, "matvec"),
                 (32000, 4096, 32, "matvec"), (1024, 1024, 64, "matvec"), (6912, 2304, 64, "gate_up"), (14336, 4096, 128, "gate_up"),
                 (512, 1024, 64, "matvec"), (9216, 2560, 64, "matvec"), (8192, 8192, 64, "matvec"), (4096, 14336, 64, "matvec"),
-                (4096, 28672, 64, "matvec"), (32768, 2048, 64, "matvec")]
+                (4096, 28672, 64, "matvec"), (32768, 2048, 64, "matvec"), (131072, 3072, 64, "matvec")]
 SIGNED_SWEEP = [(fx.BINARY1, "binary", 8192, 8192), (fx.BINARY1, "binary", 4096, 14336), (fx.BINARY1, "binary", 2048, 2048),
                 (fx.TERNARY2, "ternary", 14336, 4096), (fx.TERNARY2, "ternary", 8192, 2048), (fx.TRIT5, "trit5", 8192, 4096),
                 (fx.TRIT5, "trit5", 2560, 10240),

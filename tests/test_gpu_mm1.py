@@ -48,6 +48,27 @@ def test_affine_matrix_core_matvec(ctx, dtype, shape):
     print(f"\n  matrix-core affine {shape} dtype={dtype} max rel err {w:.2e}")
 
 
+@pytest.mark.parametrize("cols", [2560, 3584])
+def test_affine_tall_matrix_two_waves_per_tile(ctx, cols):
+    """A vocabulary-sized matrix of rows of ten and fourteen segments: two waves per tile, five and seven segments each.
+    Against the oracle on the first and last rows (ragged last tile), and against the vector kernel everywhere: at most
+    one step of the output type apart."""
+    rows, group, dtype = 131075, 64, fx.BF16
+    packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=cols)
+    x = fx.synth_activation(1, cols, dtype, config=1, tensor=cols + 1)
+    y = run_affine(ctx, packed, scales, biases, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    for sl in (slice(0, 96), slice(rows - 99, rows)):
+        n = sl.stop - sl.start
+        ref = so.affine_matvec(packed[sl], scales[sl], biases[sl], fx.from_bits(x, dtype), n, cols, group, dtype)
+        gh.check_outputs(y[:, sl], ref, dtype, f"tall affine {rows}x{cols} rows {sl.start}..{sl.stop}")
+    ctx.set_matvec_engine(rt.MATVEC_VECTOR)
+    try:
+        y_vec = run_affine(ctx, packed, scales, biases, x, dtype, f"affine_matvec:{cols}:{group}", generic=True)
+    finally:
+        ctx.set_matvec_engine(rt.MATVEC_AUTO)
+    gh.check_steps(y, y_vec, dtype, f"tall affine {rows}x{cols}, single-pass against vector kernel", max_steps=1, min_exact=0.9)
+
+
 def test_affine_matrix_core_exact_on_dyadic_fixture(ctx):
     """KernelLab.swift:2829-2855 buffers: every partial sum is an exact dyadic rational, so the
     matrix cores must give the oracle's bits too."""

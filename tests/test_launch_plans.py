@@ -116,7 +116,10 @@ def test_matvec_plans(layout, group):
             p = cc.plan_matvec(layout, rows, cols, group)
             assert (p["segments"], p["waves"]) == want, (rows, cols, p)
         # never one segment per wave from 24M weights on; a vocabulary-sized matrix of short rows: one wave per tile
-        for rows, cols, want in [(16384, 2048, (2, 4)), (65536, 1024, (4, 1)), (151936, 1024, (4, 1)), (151936, 2048, (8, 1))]:
+        # (... and two waves per tile for rows of nine to sixteen segments)
+        for rows, cols, want in [(16384, 2048, (2, 4)), (65536, 1024, (4, 1)), (151936, 1024, (4, 1)), (151936, 2048, (8, 1)),
+                                 (151936, 2560, (5, 2)), (151936, 3072, (6, 2)), (151936, 3584, (7, 2)), (151936, 4096, (8, 2)),
+                                 (131072, 5120, (5, 4))]:
             p = cc.plan_matvec(layout, rows, cols, group)
             assert (p["segments"], p["waves"]) == want, (rows, cols, p)
         assert cc.plan_matvec(layout, 64, 32768, group)["segments"] == 8
