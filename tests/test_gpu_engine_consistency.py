@@ -87,6 +87,11 @@ def _affine_record(ctx, rows, cols, group, dtype, kind):
     ctx.alloc(gh.Y_SLOT, rows * 2)
     n = 3 * nmat
     bufs += [(gh.X_SLOT, n, 0), (gh.Y_SLOT, n + 1, 0)]
+    if kind == "argmax":
+        # the lm_head record at one token: partial keys (one per grid column) where the other kinds write y
+        ctx.alloc(gh.Y_SLOT, 1024 * 8)
+        pipe = ctx.pipeline(f"affine_matvec_argmax_c{cols}_r{rows}_g{group}_batched" + gh.t_suffix(dtype))
+        return rt.make_record(pipe, bufs, [(5, 1), (6, 0.0)], (1024, 1, 1), (256, 1, 1))
     entry = {"matvec": "affine_matvec", "gate_up": "fused_affine_gate_up_swiglu"}[kind] + f":{cols}:{group}"
     pipe = ctx.pipeline(entry + gh.t_suffix(dtype))
     return rt.make_record(pipe, bufs, [(n + 2, rows)], (min(1024, (rows + 7) // 8), 1, 1), (256, 1, 1))
@@ -109,11 +114,13 @@ def _signed_record(ctx, fmt, name, rows, cols, dtype):
 
 
 # (the second rows: one shape of each size class of the launch plan: below 1M weights, 8M-24M, from 24M with eight
-# and twelve waves, a row beyond 24576 columns, a tall matrix of short rows, a tall matrix with two waves per tile)
+# and twelve waves, a row beyond 24576 columns, a tall matrix of short rows, a tall matrix with two waves per tile;
+# the lm_head record at one token with partly empty and with full vector passes)
 AFFINE_SWEEP = [(4096, 4096, 64, "matvec"), (11008, 4096, 128, "matvec"), (4096, 11008, 64, "matvec"), (1536, 8960, 64, "matvec"),
                 (32000, 4096, 32, "matvec"), (1024, 1024, 64, "matvec"), (6912, 2304, 64, "gate_up"), (14336, 4096, 128, "gate_up"),
                 (512, 1024, 64, "matvec"), (9216, 2560, 64, "matvec"), (8192, 8192, 64, "matvec"), (4096, 14336, 64, "matvec"),
-                (4096, 28672, 64, "matvec"), (32768, 2048, 64, "matvec"), (131072, 3072, 64, "matvec")]
+                (4096, 28672, 64, "matvec"), (32768, 2048, 64, "matvec"), (131072, 3072, 64, "matvec"),
+                (65536, 2560, 64, "argmax"), (32000, 5120, 64, "argmax"), (65536, 1024, 64, "argmax")]
 SIGNED_SWEEP = [(fx.BINARY1, "binary", 8192, 8192), (fx.BINARY1, "binary", 4096, 14336), (fx.BINARY1, "binary", 2048, 2048),
                 (fx.TERNARY2, "ternary", 14336, 4096), (fx.TERNARY2, "ternary", 8192, 2048), (fx.TRIT5, "trit5", 8192, 4096),
                 (fx.TRIT5, "trit5", 2560, 10240),
