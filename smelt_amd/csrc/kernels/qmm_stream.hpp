@@ -1,5 +1,5 @@
 // Streaming small-batch quantized matmul for gfx950:  Y[M, N] = X[M, K] * W[N, K]^T for up to 16
-// tokens per pass, affine u4 weights with one scale group per 64 columns.
+// tokens per pass, affine u4 weights with one scale group per 64 columns, rows of a multiple of 256 columns.
 //
 // At this batch the weights still stream from HBM once and the arithmetic is small; the kernel is
 // the multi-token form of the single-pass matvec.  A wave owns 16 * RT weight rows and, per round,
@@ -79,9 +79,11 @@ constexpr int kQsTokens = 16;          // tokens per pass (blockIdx.y)
 constexpr int kQsXStride = 272;        // bytes per staged token row
 constexpr int kQsWStride = 72;         // bytes per staged weight row
 __host__ __device__ constexpr size_t qms_scale_lds_bytes(int tiles, int groups) { return (size_t)tiles * 16 * (groups + 1) * 8; }
-__host__ __device__ constexpr size_t qms_wave_lds_bytes(int tiles) { return (size_t)16 * kQsXStride + (size_t)tiles * 16 * kQsWStride; }
-__host__ __device__ constexpr size_t qms_lds_bytes(int tiles, int groups, int waves) {
-    return qms_scale_lds_bytes(tiles, groups) + (size_t)waves * qms_wave_lds_bytes(tiles);
+__host__ __device__ constexpr size_t qms_wave_lds_bytes(int tiles, int token_rows = 16) {
+    return (size_t)token_rows * kQsXStride + (size_t)tiles * 16 * kQsWStride;
+}
+__host__ __device__ constexpr size_t qms_lds_bytes(int tiles, int groups, int waves, int token_rows = 16) {
+    return qms_scale_lds_bytes(tiles, groups) + (size_t)waves * qms_wave_lds_bytes(tiles, token_rows);
 }
 
 template <class ActT, class ScaleT, int NMAT, int RT, int XR, class Epi>
@@ -91,7 +93,7 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
     using E = Elem16<ActT>;
     using O = QsOperand<ActT>;
     constexpr int T = NMAT * RT;   // 16-row tiles a wave multiplies by its slice of x
-    static_assert(qms_wave_lds_bytes(T) >= (size_t)T * 1024, "partial sums reuse the staging buffer");
+    static_assert(qms_wave_lds_bytes(T, 4 * XR) >= (size_t)T * 1024, "partial sums reuse the staging buffer");
     static_assert(XR == 2 || XR == 4, "a pass stages eight or sixteen token rows");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1);
@@ -108,7 +110,11 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
     // Nothing below predicates a load; loads return in issue order, so what is needed first is
     // asked for first.
     // ---- scales and biases of the tile: one run of eight groups of one row per thread ------------
-    const int runs = gt >> 3;
+    // (rows of a multiple of 256 but not of 512 columns hold an odd number of four-group halves: runs of four then,
+    // eight bytes per plane and thread; their rows start on 8-byte boundaries only)
+    const bool half_runs = (gt & 7) != 0;
+    const int run_len = half_runs ? 4 : 8;
+    const int runs = half_runs ? gt >> 2 : gt >> 3;
     const int items = T * 16 * runs;
     float2* lds_sb = reinterpret_cast<float2*>(smem);
     const int sstride = gt + 1;
@@ -123,9 +129,16 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
         const uint16_t* bp = B[0];
         if (NMAT > 1 && smat == 1) { sp = S[NMAT - 1]; bp = B[NMAT - 1]; }
         ScaleRun out;
-        out.s = *reinterpret_cast<const uint4_t*>(sp + (size_t)r * gt + 8 * run);
-        out.b = *reinterpret_cast<const uint4_t*>(bp + (size_t)r * gt + 8 * run);
-        out.at = srow * sstride + 8 * run;
+        if (half_runs) {
+            const uint2_t s2 = *reinterpret_cast<const uint2_t*>(sp + (size_t)r * gt + 4 * run);
+            const uint2_t b2 = *reinterpret_cast<const uint2_t*>(bp + (size_t)r * gt + 4 * run);
+            out.s = uint4_t{s2.x, s2.y, 0u, 0u};
+            out.b = uint4_t{b2.x, b2.y, 0u, 0u};
+        } else {
+            out.s = *reinterpret_cast<const uint4_t*>(sp + (size_t)r * gt + 8 * run);
+            out.b = *reinterpret_cast<const uint4_t*>(bp + (size_t)r * gt + 8 * run);
+        }
+        out.at = srow * sstride + run_len * run;
         return out;
     };
     auto store_scales = [&](const ScaleRun& v) {
@@ -134,13 +147,13 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
         for (int e = 0; e < 8; ++e) {
             const float s = ScaleT::widen((uint16_t)(e & 1 ? sd[e >> 1] >> 16 : sd[e >> 1] & 0xFFFFu));
             const float b = ScaleT::widen((uint16_t)(e & 1 ? bd[e >> 1] >> 16 : bd[e >> 1] & 0xFFFFu));
-            lds_sb[v.at + e] = float2{s, __builtin_fmaf(-O::kBase, s, b)};
+            if (e < run_len) lds_sb[v.at + e] = float2{s, __builtin_fmaf(-O::kBase, s, b)};
         }
     };
     const ScaleRun first_run = load_scales((int)threadIdx.x);
 
-    unsigned char* stage = smem + qms_scale_lds_bytes(T, gt) + (size_t)chunk * qms_wave_lds_bytes(T);
-    unsigned char* stage_w = stage + 16 * kQsXStride;
+    unsigned char* stage = smem + qms_scale_lds_bytes(T, gt) + (size_t)chunk * qms_wave_lds_bytes(T, 4 * XR);
+    unsigned char* stage_w = stage + 4 * XR * kQsXStride;
     // load side: sixteen lanes per token row, four lanes per weight row
     const int x_tok = lane >> 4, x_piece = lane & 15;
     const int w_row = lane >> 2, w_piece = lane & 3;
@@ -263,7 +276,7 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
         for (int c = 0; c < kc; ++c)
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) {
-                const float4_t part = reinterpret_cast<const float4_t*>(first + (size_t)c * qms_wave_lds_bytes(T))[(m * RT + t) * kWave + lane];
+                const float4_t part = reinterpret_cast<const float4_t*>(first + (size_t)c * qms_wave_lds_bytes(T, 4 * XR))[(m * RT + t) * kWave + lane];
                 sum[m].x += part.x; sum[m].y += part.y; sum[m].z += part.z; sum[m].w += part.w;
             }
         const int r = row0 + 16 * t + n;

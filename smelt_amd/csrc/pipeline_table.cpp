@@ -349,7 +349,7 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
 
 bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
               size_t lds_limit, QmsPlan* out) {
-    if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;
+    if (group != 64 || cols == 0 || cols % 256 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;
     const uint32_t gt = cols / 64, npairs = gt / 2;
     // Measured on MI355X at 2560- and 9216-column rows: about four steps per wave hide the memory
     // round trips best, up to twelve waves; two row tiles per wave (half the activation traffic per
@@ -361,9 +361,22 @@ bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     if (kc > 12) kc = 12;
     uint32_t steps = (npairs + kc - 1) / kc;
     kc = (npairs + steps - 1) / steps;   // same steps per wave, no idle wave
+    // Matrices of many rows: fewer waves with longer walks, about 3500 waves in the launch's first pass, never
+    // fewer than four, and only a count that leaves no wave idle (cold, 4 / 8 / 16 tokens: 17408 x 5120 four waves
+    // 17.1 / 19.0 / 21.8 us against 19.3 / 20.9 / 24.1 with ten; 14336 x 4096 four 11.8 / 12.3 / 12.6 against 12.3 /
+    // 12.8 / 13.4 with eight; 8192 x 8192 eight 12.5 / 13.0 / 13.6 against 13.2 / 14.0 / 15.0 with eleven; 9216 x 2560
+    // and 4096 x 4096 keep five and eight: fewer were slower).
+    if (nmat == 1) {
+        const uint32_t tiles16 = (rows + 15) / 16;
+        uint32_t want = (3500 + tiles16 / 2) / tiles16;
+        if (want < 4) want = 4;
+        for (uint32_t k = want; k < kc; ++k)
+            if (npairs % k == 0) { kc = k; steps = npairs / k; break; }
+    }
     const uint32_t tiles = nmat * rt;
+    const uint32_t token_rows = batch > 8 ? 16 : 8;   // staged per pass
     auto lds_of = [&](uint32_t waves) {
-        return (size_t)tiles * 16 * (gt + 1) * 8 + (size_t)waves * (16 * 272 + (size_t)tiles * 16 * 72);
+        return (size_t)tiles * 16 * (gt + 1) * 8 + (size_t)waves * (token_rows * 272 + (size_t)tiles * 16 * 72);
     };
     // A launch of more workgroups than compute units runs two per unit only if two fit in LDS together, and a
     // long row's scale table takes a large share: fewer waves with more steps each then beat a second round

@@ -81,6 +81,42 @@ def test_stream_qmm_shapes(ctx, dtype, shape):
     assert np.array_equal(y, again)   # fixed summation order
 
 
+def qmm_full(ctx, w, x_bits, dtype, rows, cols):
+    """A token-slab qmm record (64-row slabs, 16-token grid rows): what the emitter writes where the skinny form
+    does not exist (rows that are not a multiple of 512 columns)."""
+    batch = x_bits.shape[0]
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in w]
+    ctx.upload_weights(0, wf.image())
+    ctx.put(gh.X_SLOT, x_bits)
+    ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+    pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g64_batched_full" + gh.t_suffix(dtype))
+    bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+    rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], ((rows + 63) // 64, 16, 1), (256, 1, 1),
+                         grid_kinds=(0, rt.GRID_SEQ_LEN_CEIL_DIV, 0))
+    assert ctx.encode_prefill(rec, seq_len=batch) == 1
+    ctx.wait()
+    return ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+
+
+# rows of a multiple of 256 but not of 512 columns (11008: a Llama-7B down projection, 86 pairs; 768 = six pairs; 256 =
+# two): scale rows start on 8-byte boundaries only and are staged four groups at a time
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("shape", [(100, 11008, 13), (40, 768, 5), (8200, 2816, 24), (24, 256, 2), (130, 11008, 100)])
+def test_stream_qmm_rows_of_odd_multiples_of_256_columns(ctx, split_k, dtype, shape):
+    rows, cols, batch = shape
+    w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=rows % 7)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=cols % 17, outlier_frac=0.01)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype, threads=True)
+    y = qmm_full(ctx, w, x, dtype, rows, cols)
+    gh.check_outputs(y, ref, dtype, f"stream qmm {shape}")
+    assert np.array_equal(y, qmm_full(ctx, w, x, dtype, rows, cols))   # fixed summation order
+    # the token-slab kernel the record names (vector engine) agrees to the output tolerance
+    slab = qmm_full(split_k, w, x, dtype, rows, cols)
+    gh.check_outputs(slab, ref, dtype, f"slab qmm {shape}")
+    gh.check_steps(y, slab, dtype, f"stream against slab {shape}", max_steps=1)
+
+
 def test_stream_qmm_is_exact_where_the_sums_are(ctx):
     """KernelLab.swift:2829-2855 buffers: every partial sum is an exact dyadic rational, so the
     streaming kernel gives the oracle's bits for every token."""

@@ -42,6 +42,17 @@ def test_qmm_plans_cover_the_output_and_fit_the_machine(nmat):
                 assert p["workspace"] >= tiles * p["ksplit"] * bn * 64 * 4 * nmat // (2 if p["per_wave"] else 1) // 2
 
 
+def test_streaming_plan_rows_of_256_column_multiples_and_tall_matrices():
+    # rows of a multiple of 256 columns stream at every batch (the token-tile kernel takes multiples of 512 only)
+    for batch in (2, 8, 100, 512):
+        p = cc.plan_qmm(4096, 11008, 64, 1, batch, CUS, LDS)
+        assert p is not None and p["kernel"] == 1 and p["grid_y"] == ceil_div(batch, 16)
+    assert cc.plan_qmm(4096, 11008 + 128, 64, 1, 8, CUS, LDS) is None
+    # matrices of many rows: about 3500 waves in the launch, at least four per workgroup, none idle
+    for rows, cols, want in [(17408, 5120, 4), (14336, 4096, 4), (8192, 8192, 8), (9216, 2560, 5), (4096, 4096, 8), (5120, 5120, 10)]:
+        assert cc.plan_qmm(rows, cols, 64, 1, 8, CUS, LDS)["k_waves"] == want, (rows, cols)
+
+
 def test_qmm_k_split_needs_the_workspace():
     with_ws = cc.plan_qmm(2560, 9216, 64, 1, 512, CUS, LDS)
     assert with_ws["ksplit"] > 1
