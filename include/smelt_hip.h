@@ -128,7 +128,9 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * for bit); MATRIX_CORE asks for the same explicitly (kept from when AUTO had size thresholds);
  * VECTOR keeps every record on the vector-ALU kernels.  The same switch
  * covers the qmm records and, from two tokens on, the per-token small-batch ("_batched", "_batched_verify_b4")
- * forms of the group-64 affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's, and the
+ * forms of the group-64 affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's (while
+ * tokens x weights stay below about 20M they run the single-token kernel with a grid row per token, bit for
+ * bit the rows of a one-token record; beyond, the streaming kernel), and the
  * lm_head matvec+argmax over two tokens and more without a logit cap (logits of all tokens through the
  * streaming kernel into the context workspace, partial keys from a second launch: the record then counts as
  * two launches), and the same record at one token where the rows' 16-byte pieces leave the fused kernel's last

@@ -276,6 +276,16 @@ void attach_mm1(ResolvedPipeline* r) {
         {"smelt_teraff_bank4_matvec_", "smelt_teraff_mm1_", "bank4_matvec_", kCodesTernary2, 1},
     };
     const std::string t = act_suffix(r->act);
+    // the per-token small-batch forms of the plain matvec and of gate+up+SwiGLU: the single-token kernels with one
+    // grid row per token (small matrices at a few tokens; the batch argument leaves the argument block)
+    if (r->family == kFamAffineBatched || (r->family == kFamAffineGateUpBatched && r->symbol.find("swiglu") != std::string::npos)) {
+        const bool pair = r->family == kFamAffineGateUpBatched;
+        r->mm1_prefix = "smelt_affine_mm1_";
+        r->mm1_tail = std::string(pair ? "gate_up_swiglu_" : "matvec_") + t;
+        r->mm1_layout = (int)kCodesU4;
+        r->mm1_nmat = pair ? 2 : 1;
+        return;
+    }
     for (const Form& f : kForms) {
         if (r->symbol == std::string(f.stem) + t) {
             r->mm1_prefix = f.prefix;

@@ -1081,7 +1081,23 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     const bool mm1_b4 = p->res.family == kFamSignedB4 || p->res.family == kFamSignedGateUpB4;
     // (the signed single-token families take their token from the grid row: a record with several rows keeps them)
     const bool mm1_per_row = p->res.family == kFamSignedMatvec || p->res.family == kFamSignedAdd || p->res.family == kFamSignedGateUp;
-    if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && (L.grid[1] == 1 || mm1_b4 || mm1_per_row)) {
+    // the per-token small-batch forms of the affine matvec and gate+up (W S B X Y batch | rows cols group tile): a few
+    // tokens of a small matrix are launch-bound, and the single-token kernel with a grid row per token is the shorter
+    // launch while tokens x weights stay below about 20M (cold, streaming kernel against a grid row per token:
+    // 1024 x 1024 at 2 / 4 / 8 / 16 tokens 4.4 / 4.5 / 4.5 / 4.7 us against 2.5 / 2.8 / 3.2 / 4.0; 2048 x 2048 at 2 / 4 / 6
+    // 4.8 / 4.9 / 4.9 against 3.3 / 4.0 / 5.1; 6144 x 1024 at 3 / 4 4.9 / 4.9 against 4.5 / 5.2; 4096 x 4096 at 2 5.5 against 5.7)
+    // (not the skinny and token-slab qmm names: their fused-add sibling writes two outputs, has no such form and
+    // would no longer match the plain record bit for bit)
+    const bool mm1_pair_batch = p->res.family == kFamAffineGateUpBatched;
+    const bool mm1_batch_family = p->res.family == kFamAffineBatched || mm1_pair_batch;
+    bool mm1_small_batch = false;
+    if (mm1_batch_family && p->res.mm1_layout >= 0) {
+        const size_t o = mm1_pair_batch ? 8 : 5;
+        const uint64_t batch = L.args[o].value, weights = (uint64_t)L.args[o + 1].value * L.args[o + 2].value * (mm1_pair_batch ? 2 : 1);
+        mm1_small_batch = batch >= 1 && batch <= 16 && weights * batch <= ((uint64_t)20 << 20);
+    }
+    if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && p->res.family != kFamAffineArgmax &&
+        ((L.grid[1] == 1 && !mm1_batch_family) || mm1_b4 || mm1_per_row || mm1_small_batch)) {
         // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
         // arguments, its own launch geometry (one workgroup per eight rows)
         uint32_t rows = 0, cols = 0, group = 128, tokens = 1;
@@ -1108,6 +1124,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             // blockIdx.y; the trailing batch argument is dropped from the argument block)
             case kFamSignedB4: rows = U(4); cols = U(5); tokens = U(6); ro = 3; break;
             case kFamSignedGateUpB4: rows = U(6); cols = U(7); tokens = U(8); ro = 5; break;
+            case kFamAffineBatched: tokens = U(5); rows = U(6); cols = U(7); group = U(8); ro = 4; break;
+            case kFamAffineGateUpBatched: tokens = U(8); rows = U(9); cols = U(10); group = U(11); ro = 7; break;
             case kFamBinaryPackedBank: rows = U(5) + U(6); cols = U(7); ro = 3; break;
             case kFamBinaryPackedBank4: rows = U(7) + U(8) + U(9) + U(10); cols = U(11); ro = 3; break;
             case kFamTerAffMatvec: rows = U(5); cols = U(6); ro = 4; break;
@@ -1123,6 +1141,12 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             fn = p->fn_mm1[plan.nl];
             L.grid[0] = (rows + 7) / 8; L.grid[1] = tokens; L.grid[2] = 1;
             if (mm1_b4) L.args.count -= 1;
+            if (mm1_small_batch) {
+                // W S B X Y batch rows cols group tile -> W S B X Y rows cols group
+                const size_t o = mm1_pair_batch ? 8 : 5;
+                for (size_t i = o; i + 1 < L.args.count; ++i) L.args[i] = L.args[i + 1];
+                L.args.count -= 2;
+            }
             L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
             L.lds = plan.lds;
             routed = true;
@@ -1208,7 +1232,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             HIP_TRY(ctx, hipModuleLaunchKernel(p->fn_logits_keys, L.grid[0], batch, 1, 64, 1, 1, 0, ctx->stream, nullptr, cfg_b));
             return 2;
         }
-    } else if (!p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
+    } else if (!routed && !p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
         aligned16(qms_pair ? 7 : 4) && whole_pieces(qms_pair ? 7 : 4)) {
         // skinny qmm (and, from two tokens on, the per-token small-batch forms, whose arguments are the
         // same): the streaming kernel of the same pipeline, same arguments, its own launch

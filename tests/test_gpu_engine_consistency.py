@@ -33,8 +33,28 @@ def steps_between(a_bits, b_bits, dtype):
 
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("shape", [(2048, 1024), (1000, 2560), (512, 1024)])
+def test_auto_engine_small_matrices_verify_b4_is_decode_bit_for_bit(ctx, dtype, shape):
+    """While tokens x weights stay below about 20M the per-token small-batch forms run the single-token kernel with a
+    grid row per token: the verify pass then reproduces the decode rows bit for bit under AUTO as well (plain and
+    gate+up+SwiGLU forms, two to four tokens)."""
+    rows, cols = shape
+    group = 64
+    packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=41)
+    x = fx.synth_activation(4, cols, dtype, config=1, tensor=42)
+    decode = np.concatenate([run_affine(ctx, packed, scales, biases, x[t:t + 1], dtype, f"affine_matvec:{cols}:{group}", generic=True)
+                             for t in range(4)])
+    for batch in (2, 3, 4):
+        verify = run_affine(ctx, packed, scales, biases, x[:batch], dtype, f"affine_matvec_c{cols}_r{rows}_g{group}_batched_verify_b4", batched=True, batch_tile=4)
+        assert np.array_equal(verify, decode[:batch]), batch
+    tile4 = run_affine(ctx, packed, scales, biases, x, dtype, f"affine_matvec_c{cols}_r{rows}_g{group}_batched_tile4", batched=True, batch_tile=4)
+    assert np.array_equal(tile4, decode)
+    gh.check_outputs(decode, so.affine_matvec(packed, scales, biases, fx.from_bits(x, dtype), rows, cols, group, dtype), dtype, "decode")
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 def test_auto_engine_decode_against_verify_b4_and_staged(ctx, dtype):
-    rows, cols, group = 2048, 1024, 64          # AUTO runs the matrix-core matvec
+    rows, cols, group = 4096, 2560, 64          # AUTO: single-pass kernel at one token, streaming kernel at four (42M token-weights)
     packed, scales, biases = fx.synth_affine(rows, cols, group, dtype, config=1, tensor=31)
     x = fx.synth_activation(4, cols, dtype, config=1, tensor=32)
     xf = fx.from_bits(x, dtype)
@@ -42,7 +62,7 @@ def test_auto_engine_decode_against_verify_b4_and_staged(ctx, dtype):
     # decode: one token per launch on the engine AUTO picks (matrix core)
     decode = np.concatenate([run_affine(ctx, packed, scales, biases, x[t:t + 1], dtype, f"affine_matvec:{cols}:{group}", generic=True)
                              for t in range(4)])
-    # verify pass: the generated four-token form (vector kernels)
+    # verify pass: the generated four-token form (streaming kernel)
     verify = run_affine(ctx, packed, scales, biases, x, dtype, f"affine_matvec_c{cols}_r{rows}_g{group}_batched_verify_b4", batched=True, batch_tile=4)
     gh.check_outputs(decode, ref, dtype, "AUTO decode")
     gh.check_outputs(verify, ref, dtype, "AUTO verify_b4")
