@@ -137,7 +137,8 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * pass over a row less than nine tenths full (1536, 2560, 3072, 3584, 5120 columns: the single-pass kernel
  * with the argmax as its epilogue, tiles that share a partial key meeting in the context workspace): AUTO and
  * MATRIX_CORE run the streaming kernel of the pipeline below 128
- * tokens (K split inside a workgroup, no workspace) and the token-tile kernel from 128 tokens on
+ * tokens (K split inside a workgroup, no workspace) and the token-tile kernel from 128 tokens on (from 96
+ * for matrices of 20M weights and 2560 rows, from 33 for 40M weights and 3584 rows)
  * (matrices with few tiles and long rows split K across workgroups: partial sums in the
  * workspace, added in a fixed order), VECTOR the split-K or token-slab kernel the record's geometry
  * describes (split-K: partial sums in the workspace).  Results of the alternatives differ in

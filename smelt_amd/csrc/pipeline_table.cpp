@@ -316,10 +316,19 @@ ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType defau
 
 bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
               size_t lds_limit, QmtPlan* out) {
-    // Measured on MI355X at the 4B FFN shapes: below 128 tokens the streaming kernel's 16-token
+    // Measured on MI355X at the 4B FFN shapes: below about 96 tokens the streaming kernel's 16-token
     // passes are as fast or faster (the weights of the later passes come from cache); from there on the
     // shared activation tile wins (128 tokens: 22 against 27 us on 9216 x 2560, 29 against 38 on 2560 x 9216).
-    if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch < 128) return false;
+    if (group != 64 || cols == 0 || cols % 512 != 0 || rows == 0 || nmat == 0 || nmat > 2) return false;
+    // The streaming kernel's time grows with its 16-token passes, this kernel's is flat over a 64-token block, and
+    // the larger the matrix the sooner they cross (cold, streaming against token tiles at 33 / 64 / 96 tokens:
+    // 5120 x 25600 76 / 100 / 140 us against 51 / 53 / 81; 4096 x 12288 29 / 42 / 57 against 26 / 26 / 36; 8192 x 8192
+    // 33 / 41 / 60 against 29 / 28 / 43; 18944 x 3584 33 / 41 / 60 against 28 / 28 / 42; 5120 x 5120 21 / 25 / 33 against
+    // 29 / 30 / 29; 9216 x 2560 14 / 18 / 22 against 17 / 17 / 21; 2560 x 9216 16 / 21 / 27 against 23 / 24 / 24; few rows
+    // leave this kernel short of tiles: 2048 x 16384 22 / 25 / 34 against 28 / 28 / 38).
+    const uint64_t weights = (uint64_t)rows * cols * nmat;
+    const uint32_t min_batch = weights >= (40u << 20) && rows >= 3584 ? 33u : (weights >= (20u << 20) && rows >= 2560 ? 96u : 128u);
+    if (batch < min_batch) return false;
     // buffer loads address the activations and each weight matrix with 32-bit byte offsets
     if ((uint64_t)batch * cols * 2 >= (1ull << 31) || (uint64_t)rows * (cols / 2) >= (1ull << 31)) return false;
     // 96 rows x 64 tokens per workgroup and eight waves (two along K) measured best at 256 to 1024 tokens on

@@ -81,24 +81,6 @@ def test_stream_qmm_shapes(ctx, dtype, shape):
     assert np.array_equal(y, again)   # fixed summation order
 
 
-def qmm_full(ctx, w, x_bits, dtype, rows, cols):
-    """A token-slab qmm record (64-row slabs, 16-token grid rows): what the emitter writes where the skinny form
-    does not exist (rows that are not a multiple of 512 columns)."""
-    batch = x_bits.shape[0]
-    wf = gh.WeightFile()
-    offs = [wf.add(a) for a in w]
-    ctx.upload_weights(0, wf.image())
-    ctx.put(gh.X_SLOT, x_bits)
-    ctx.alloc(gh.Y_SLOT, batch * rows * 2)
-    pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g64_batched_full" + gh.t_suffix(dtype))
-    bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
-    rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], ((rows + 63) // 64, 16, 1), (256, 1, 1),
-                         grid_kinds=(0, rt.GRID_SEQ_LEN_CEIL_DIV, 0))
-    assert ctx.encode_prefill(rec, seq_len=batch) == 1
-    ctx.wait()
-    return ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
-
-
 # rows of a multiple of 256 but not of 512 columns (11008: a Llama-7B down projection, 86 pairs; 768 = six pairs; 256 =
 # two): scale rows start on 8-byte boundaries only and are staged four groups at a time
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
@@ -244,6 +226,20 @@ def test_tile_qmm_4b_shapes(ctx, dtype, batch):
     y = qmm_full(ctx, w, x, dtype, rows, cols)
     worst = gh.check_outputs(y, ref, dtype, f"tile qmm M={batch}")
     print(f"\n  tile qmm M={batch} dtype={dtype} max rel err {worst:.2e}")
+
+
+@pytest.mark.parametrize("batch", [33, 64, 70, 127])
+def test_tile_qmm_takes_large_matrices_from_33_tokens(ctx, split_k, batch):
+    """From 40M weights (and 3584 rows) the token-tile kernel takes the record from 33 tokens on: one ragged 64-token
+    block, one full, two; ragged last row tile.  Against the oracle and against the token-slab kernel."""
+    rows, cols, dtype = 3600, 12288, fx.BF16
+    w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=5)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=batch, outlier_frac=0.01)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype, threads=True)
+    y = qmm_full(ctx, w, x, dtype, rows, cols)
+    gh.check_outputs(y, ref, dtype, f"tile qmm {rows}x{cols} M={batch}")
+    assert np.array_equal(y, qmm_full(ctx, w, x, dtype, rows, cols))
+    gh.check_steps(y, qmm_full(split_k, w, x, dtype, rows, cols), dtype, f"tile against slab M={batch}", max_steps=1)
 
 
 @pytest.mark.parametrize("shape", [(200, 9216, 512), (8200, 1024, 96), (40, 512, 170), (2600, 2560, 520), (2560, 9216, 256),

@@ -16,6 +16,21 @@ def ceil_div(a, b):
     return (a + b - 1) // b
 
 
+def qmt_min_batch(rows, cols, nmat):
+    """From how many tokens the token-tile kernel takes a group-64 record: the larger the matrix, the sooner."""
+    weights = rows * cols * nmat
+    if weights >= 40 << 20 and rows >= 3584:
+        return 33
+    return 96 if weights >= 20 << 20 and rows >= 2560 else 128
+
+
+def test_token_tile_threshold_by_matrix_size():
+    for rows, cols, first in [(5120, 25600, 33), (4096, 12288, 33), (8192, 8192, 33), (18944, 3584, 33), (5120, 5120, 96),
+                              (9216, 2560, 96), (2560, 9216, 96), (2048, 16384, 128), (4096, 4096, 128), (1024, 1024, 128)]:
+        assert cc.plan_qmm(rows, cols, 64, 1, first - 1, CUS, LDS)["kernel"] == 1, (rows, cols)
+        assert cc.plan_qmm(rows, cols, 64, 1, first, CUS, LDS)["kernel"] == 2, (rows, cols)
+
+
 @pytest.mark.parametrize("nmat", [1, 2])
 def test_qmm_plans_cover_the_output_and_fit_the_machine(nmat):
     for (rows, cols), batch in itertools.product(SHAPES, BATCHES):
@@ -23,12 +38,12 @@ def test_qmm_plans_cover_the_output_and_fit_the_machine(nmat):
         assert p is not None, (rows, cols, batch)
         assert p["lds"] <= LDS and p["threads"] <= 1024 and p["threads"] % 64 == 0
         if p["kernel"] == 1:       # streaming: 16 * rt rows, 16 tokens per workgroup, no workspace
-            assert batch < 128 or cols % 512
+            assert batch < qmt_min_batch(rows, cols, nmat) or cols % 512
             assert p["grid_x"] * 16 * p["row_tiles"] >= rows > (p["grid_x"] - 1) * 16 * p["row_tiles"]
             assert p["grid_y"] == ceil_div(batch, 16) and p["grid_z"] == 1 and p["workspace"] == 0
             assert p["threads"] == 64 * p["k_waves"]
         else:                      # token tiles: 64 tokens, 32 * rt rows (16 * rt of each matrix when split by wave)
-            assert p["kernel"] == 2 and batch >= 128 and cols % 512 == 0
+            assert p["kernel"] == 2 and batch >= qmt_min_batch(rows, cols, nmat) and cols % 512 == 0
             bn = (16 if p["per_wave"] else 32) * p["row_tiles"]
             assert p["grid_x"] == ceil_div(rows, bn) and p["grid_y"] == ceil_div(batch, 64)
             assert p["threads"] == 256 * p["k_waves"]
