@@ -327,7 +327,13 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     // 29 / 30 / 29; 9216 x 2560 14 / 18 / 22 against 17 / 17 / 21; 2560 x 9216 16 / 21 / 27 against 23 / 24 / 24; few rows
     // leave this kernel short of tiles: 2048 x 16384 22 / 25 / 34 against 28 / 28 / 38).
     const uint64_t weights = (uint64_t)rows * cols * nmat;
-    const uint32_t min_batch = weights >= (40u << 20) && rows >= 3584 ? 33u : (weights >= (20u << 20) && rows >= 2560 ? 96u : 128u);
+    // Small matrices the other way round: this kernel's walk along K is a latency chain whatever the matrix (9 us at 1024
+    // columns, 19 at 3072) while a streaming pass over a small matrix is short (128 / 256 / 512 / 1024 tokens, streaming
+    // against token tiles: 1024 x 1024 5.0 / 5.7 / 8.0 / 12.7 against 9.1 - 9.2; 1024 x 3072 7.6 / 11.5 / 20.1 / 36 against
+    // 19 - 20; 3072 x 1024 7.3 / 11.0 / 18.0 / 33 against 9.2 / 9.2 / 11.2 / 16; 2048 x 2048 8.8 / 13.0 / 22.4 / 43 against
+    // 14.2 / 14.2 / 14.3 / 26; from 6144 x 1024 on the tiles win at 128: 11.3 against 9.3).
+    const uint32_t min_batch = weights < (2u << 20) ? 1024u : weights < (5u << 20) ? 384u
+                               : weights >= (40u << 20) && rows >= 3584 ? 33u : (weights >= (20u << 20) && rows >= 2560 ? 96u : 128u);
     if (batch < min_batch) return false;
     // buffer loads address the activations and each weight matrix with 32-bit byte offsets
     if ((uint64_t)batch * cols * 2 >= (1ull << 31) || (uint64_t)rows * (cols / 2) >= (1ull << 31)) return false;

@@ -218,8 +218,9 @@ def qmm_full(ctx, w, x_bits, dtype, rows, cols, bt=64):
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 @pytest.mark.parametrize("batch", [49, 64, 100, 127, 128, 129, 300])
 def test_tile_qmm_4b_shapes(ctx, dtype, batch):
-    """Qwen3.5-4B-shaped slab (K=2560, 392 rows: ragged last row tile), ragged last token tile."""
-    rows, cols = 392, 2560
+    """Qwen3.5-4B-shaped slab (K=2560, 2088 rows: ragged last row tile; a matrix of more than 5M weights, which the
+    token-tile kernel takes from 128 tokens; the smaller batches run the streaming kernel), ragged last token tile."""
+    rows, cols = 2088, 2560
     w = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=0)
     x = fx.synth_activation(batch, cols, dtype, config=4, tensor=batch, outlier_frac=0.01)
     ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 64, dtype, threads=True)
@@ -242,11 +243,11 @@ def test_tile_qmm_takes_large_matrices_from_33_tokens(ctx, split_k, batch):
     gh.check_steps(y, qmm_full(split_k, w, x, dtype, rows, cols), dtype, f"tile against slab M={batch}", max_steps=1)
 
 
-@pytest.mark.parametrize("shape", [(200, 9216, 512), (8200, 1024, 96), (40, 512, 170), (2600, 2560, 520), (2560, 9216, 256),
+@pytest.mark.parametrize("shape", [(600, 9216, 512), (8200, 1024, 96), (40, 512, 1100), (2600, 2560, 520), (2560, 9216, 256),
                                    (1000, 6144, 200)])
 def test_tile_qmm_shapes(ctx, split_k, shape):
     """Long rows at a 512-token chunk (three workgroups share each tile along K), many rows in several
-    16-token passes, a matrix smaller than one tile, ragged row and token tiles, the 4B down projection
+    16-token passes, a matrix smaller than one tile (which the token-tile kernel takes from 1024 tokens), ragged row and token tiles, the 4B down projection
     at 256 tokens (64-row tiles, three-way split), a two-way split with uneven halves; against the oracle
     and the token-slab kernel, and twice in a row (the split leaves its counters at zero)."""
     rows, cols, batch = shape
@@ -261,7 +262,7 @@ def test_tile_qmm_shapes(ctx, split_k, shape):
 
 
 def test_tile_qmm_is_exact_where_the_sums_are(ctx):
-    rows, cols, group, batch = 64, 1024, 64, 150
+    rows, cols, group, batch = 5120, 1024, 64, 150      # 5M weights: the token-tile kernel from 128 tokens
     packed, scales, biases, x = fx.kernel_lab_qmm_fixture(rows, cols, group, batch)
     ref = so.affine_matvec(packed, scales, biases, fx.from_bits(x, fx.F16), rows, cols, group)
     y = qmm_full(ctx, (packed, scales, biases), x, fx.F16, rows, cols)
@@ -270,7 +271,7 @@ def test_tile_qmm_is_exact_where_the_sums_are(ctx):
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
 def test_tile_qmm_fused_add_and_gate_up(ctx, dtype):
-    rows, cols, batch = 200, 2560, 140
+    rows, cols, batch = 2100, 2560, 140                 # 5.4M weights: the token-tile kernel from 128 tokens
     gw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=3)
     uw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=4)
     x = fx.synth_activation(batch, cols, dtype, config=4, tensor=8)

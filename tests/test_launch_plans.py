@@ -19,6 +19,8 @@ def ceil_div(a, b):
 def qmt_min_batch(rows, cols, nmat):
     """From how many tokens the token-tile kernel takes a group-64 record: the larger the matrix, the sooner."""
     weights = rows * cols * nmat
+    if weights < 5 << 20:
+        return 1024 if weights < 2 << 20 else 384
     if weights >= 40 << 20 and rows >= 3584:
         return 33
     return 96 if weights >= 20 << 20 and rows >= 2560 else 128
@@ -26,7 +28,8 @@ def qmt_min_batch(rows, cols, nmat):
 
 def test_token_tile_threshold_by_matrix_size():
     for rows, cols, first in [(5120, 25600, 33), (4096, 12288, 33), (8192, 8192, 33), (18944, 3584, 33), (5120, 5120, 96),
-                              (9216, 2560, 96), (2560, 9216, 96), (2048, 16384, 128), (4096, 4096, 128), (1024, 1024, 128)]:
+                              (9216, 2560, 96), (2560, 9216, 96), (2048, 16384, 128), (4096, 4096, 128), (6144, 1024, 128),
+                              (1024, 1024, 1024), (3072, 1024, 384), (2048, 2048, 384)]:
         assert cc.plan_qmm(rows, cols, 64, 1, first - 1, CUS, LDS)["kernel"] == 1, (rows, cols)
         assert cc.plan_qmm(rows, cols, 64, 1, first, CUS, LDS)["kernel"] == 2, (rows, cols)
 
