@@ -1,5 +1,5 @@
 // Streaming small-batch quantized matmul for gfx950:  Y[M, N] = X[M, K] * W[N, K]^T for up to 16
-// tokens per pass, affine u4 weights with one scale group per 64 columns, rows of a multiple of 256 columns.
+// tokens per pass, affine u4 weights with one scale group per 64 (or 128) columns, rows of a multiple of 256 (512) columns.
 //
 // At this batch the weights still stream from HBM once and the arithmetic is small; the kernel is
 // the multi-token form of the single-pass matvec.  A wave owns 16 * RT weight rows and, per round,
@@ -89,7 +89,7 @@ __host__ __device__ constexpr size_t qms_lds_bytes(int tiles, int groups, int wa
 template <class ActT, class ScaleT, int NMAT, int RT, int XR, class Epi>
 __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
                                          const uint16_t* const (&B)[NMAT], const uint16_t* __restrict__ X, int batch,
-                                         int rows, int cols, const Epi& epi) {
+                                         int rows, int cols, int group, const Epi& epi) {
     using E = Elem16<ActT>;
     using O = QsOperand<ActT>;
     constexpr int T = NMAT * RT;   // 16-row tiles a wave multiplies by its slice of x
@@ -100,8 +100,11 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
     const int chunk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int kc = blockDim.x / kWave;
     const int n = lane & 15, q = lane >> 4;
-    const int gt = cols >> 6;          // scale groups per row
-    const int npairs = gt >> 1;
+    // (groups of 128 columns: a step is one group instead of two, everything else is the same)
+    const int g64 = cols >> 6;         // 64-column halves of a step's 128 columns
+    const int gshift = group == 128 ? 1 : 0;
+    const int gt = g64 >> gshift;      // scale groups per row
+    const int npairs = g64 >> 1;
     const int rs = cols >> 1;          // bytes per packed row
     const int row0 = blockIdx.x * (16 * RT);
     const int m0 = blockIdx.y * kQsTokens;
@@ -210,7 +213,7 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         int gi = 2 * pair;
-        if (gi > gt) gi = gt;   // the zero column (gt is even)
+        if (gi > g64) gi = g64;   // past the end: the zero column below
         // with eight staged token rows, MFMA rows 8..15 re-read rows 0..7 (never stored)
         const int xrow = XR == 4 ? n : (n & 7);
 #pragma unroll
@@ -219,7 +222,7 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
             const uint4_t a0 = O::activations(*reinterpret_cast<const uint4_t*>(xr));
             const uint4_t a1 = O::activations(*reinterpret_cast<const uint4_t*>(xr + 16));
             const float4_t xs = E::mfma(a1, ones, E::mfma(a0, ones, zero));
-            const int ge = gi + e < gt ? gi + e : gt;
+            const int ge = gi + e < g64 ? (gi + e) >> gshift : gt;
 #pragma unroll
             for (int m = 0; m < NMAT; ++m)
 #pragma unroll
@@ -330,34 +333,34 @@ struct QsSwiglu {
 #define SMELT_AFFINE_QMS_PLAIN(T, ACT, SC, RTV, XRV)                                                \
     SMELT_QMS_KERNEL void smelt_affine_qms_r##RTV##_x##XRV##_store_##T(                             \
         const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* Y,    \
-        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {     \
+        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t group, uint32_t, float*, uint32_t*) { \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {W};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
         const uint16_t* const b[1] = {B};                                                          \
-        qms_body<ACT, SC, 1, RTV, XRV>(w, s, b, X, batch, rows, cols, QsStore<ACT>{Y});             \
+        qms_body<ACT, SC, 1, RTV, XRV>(w, s, b, X, batch, rows, cols, group, QsStore<ACT>{Y});      \
     }                                                                                              \
     SMELT_QMS_KERNEL void smelt_affine_qms_r##RTV##_x##XRV##_add_##T(                               \
         const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* MV,   \
         const uint16_t* RES, uint16_t* OUT, uint32_t batch, uint32_t rows, uint32_t cols,          \
-        uint32_t, uint32_t, float*, uint32_t*) {                                                   \
+        uint32_t group, uint32_t, float*, uint32_t*) {                                             \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {W};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
         const uint16_t* const b[1] = {B};                                                          \
-        qms_body<ACT, SC, 1, RTV, XRV>(w, s, b, X, batch, rows, cols, QsAdd<ACT>{MV, RES, OUT});    \
+        qms_body<ACT, SC, 1, RTV, XRV>(w, s, b, X, batch, rows, cols, group, QsAdd<ACT>{MV, RES, OUT}); \
     }
 
 #define SMELT_AFFINE_QMS_GATE_UP(T, ACT, SC, XRV)                                                   \
     SMELT_QMS_KERNEL void smelt_affine_qms_r1_x##XRV##_gate_up_swiglu_##T(                          \
         const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
         const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
-        uint32_t rows, uint32_t cols, uint32_t, uint32_t, float*, uint32_t*) {                     \
+        uint32_t rows, uint32_t cols, uint32_t group, uint32_t, float*, uint32_t*) {               \
         using namespace smelt;                                                                     \
         const uint8_t* const w[2] = {gW, uW};                                                      \
         const uint16_t* const s[2] = {gS, uS};                                                     \
         const uint16_t* const b[2] = {gB, uB};                                                     \
-        qms_body<ACT, SC, 2, 1, XRV>(w, s, b, X, batch, rows, cols, QsSwiglu<ACT>{Y});              \
+        qms_body<ACT, SC, 2, 1, XRV>(w, s, b, X, batch, rows, cols, group, QsSwiglu<ACT>{Y});       \
     }
 
 // ---- token-tile form: prefill chunks ------------------------------------------------------------

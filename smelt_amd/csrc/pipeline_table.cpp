@@ -374,8 +374,9 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
 
 bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
               size_t lds_limit, QmsPlan* out) {
-    if (group != 64 || cols == 0 || cols % 256 != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;
-    const uint32_t gt = cols / 64, npairs = gt / 2;
+    // groups of 64 columns (rows of a multiple of 256 columns) or of 128 (512): scale rows are staged four or eight groups at a time
+    if ((group != 64 && group != 128) || cols == 0 || cols % (4 * group) != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;
+    const uint32_t gt = cols / group, npairs = cols / 128;
     // Measured on MI355X at 2560- and 9216-column rows: about four steps per wave hide the memory
     // round trips best, up to twelve waves; two row tiles per wave (half the activation traffic per
     // weight byte) pay once a pass stages sixteen tokens and the matrix still fills the machine

@@ -99,6 +99,34 @@ def test_stream_qmm_rows_of_odd_multiples_of_256_columns(ctx, split_k, dtype, sh
     gh.check_steps(y, slab, dtype, f"stream against slab {shape}", max_steps=1)
 
 
+# groups of 128 columns: one scale per step instead of two; 1536 columns = twelve groups, staged four at a time
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("shape", [(200, 4096, 13), (8200, 1024, 24), (100, 11264, 40), (40, 1536, 3), (130, 5120, 200)])
+def test_stream_qmm_groups_of_128_columns(ctx, split_k, dtype, shape):
+    rows, cols, batch = shape
+    w = fx.synth_affine(rows, cols, 128, dtype, config=4, tensor=rows % 5)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=cols % 19, outlier_frac=0.01)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 128, dtype, threads=True)
+    y = qmm_full(ctx, w, x, dtype, rows, cols, group=128)
+    gh.check_outputs(y, ref, dtype, f"stream qmm g128 {shape}")
+    assert np.array_equal(y, qmm_full(ctx, w, x, dtype, rows, cols, group=128))
+    slab = qmm_full(split_k, w, x, dtype, rows, cols, group=128)
+    gh.check_steps(y, slab, dtype, f"stream against slab, g128 {shape}", max_steps=1)
+    if batch <= 4:
+        # the per-token small-batch form of the same matrix: the streaming kernel, or (small matrices) the single-token
+        # kernel with a grid row per token; either way within the tolerance
+        wf = gh.WeightFile()
+        offs = [wf.add(a) for a in w]
+        ctx.upload_weights(0, wf.image())
+        ctx.put(gh.X_SLOT, x)
+        ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+        pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g128_batched_tile4" + gh.t_suffix(dtype))
+        bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+        assert ctx.encode_decode(rt.make_record(pipe, bufs, [(5, batch)], (min(1024, (rows + 7) // 8), 1, 1), (256, 1, 1))) == 1
+        ctx.wait()
+        gh.check_outputs(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), ref, dtype, "tile4 g128")
+
+
 def test_stream_qmm_is_exact_where_the_sums_are(ctx):
     """KernelLab.swift:2829-2855 buffers: every partial sum is an exact dyadic rational, so the
     streaming kernel gives the oracle's bits for every token."""
@@ -198,7 +226,7 @@ def test_stream_qmm_fused_add_and_gate_up(ctx, dtype):
 
 # ---- token-tile form: 128 tokens and more; below, 16-token passes of the streaming kernel ------
 
-def qmm_full(ctx, w, x_bits, dtype, rows, cols, bt=64):
+def qmm_full(ctx, w, x_bits, dtype, rows, cols, bt=64, group=64):
     """A token-slab qmm record as the emitter writes it for prefill chunks (64-row slabs, bt-token grid rows)."""
     batch = x_bits.shape[0]
     wf = gh.WeightFile()
@@ -206,7 +234,7 @@ def qmm_full(ctx, w, x_bits, dtype, rows, cols, bt=64):
     ctx.upload_weights(0, wf.image())
     ctx.put(gh.X_SLOT, x_bits)
     ctx.alloc(gh.Y_SLOT, batch * rows * 2)
-    pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g64_batched_full_b{bt}" + gh.t_suffix(dtype))
+    pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g{group}_batched_full_b{bt}" + gh.t_suffix(dtype))
     bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
     rec = rt.make_record(pipe, bufs, [(5, 0, rt.CONST_SEQ_LEN)], ((rows + 63) // 64, bt, 1), (256, 1, 1),
                          grid_kinds=(0, rt.GRID_SEQ_LEN_CEIL_DIV, 0))

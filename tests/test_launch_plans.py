@@ -66,6 +66,11 @@ def test_streaming_plan_rows_of_256_column_multiples_and_tall_matrices():
         p = cc.plan_qmm(4096, 11008, 64, 1, batch, CUS, LDS)
         assert p is not None and p["kernel"] == 1 and p["grid_y"] == ceil_div(batch, 16)
     assert cc.plan_qmm(4096, 11008 + 128, 64, 1, 8, CUS, LDS) is None
+    # groups of 128 columns stream too (rows of a multiple of 512 columns), at every batch; other groups do not
+    for batch in (2, 8, 300):
+        p = cc.plan_qmm(4096, 4096, 128, 1, batch, CUS, LDS)
+        assert p is not None and p["kernel"] == 1
+    assert cc.plan_qmm(4096, 11008, 128, 1, 8, CUS, LDS) is None and cc.plan_qmm(4096, 4096, 32, 1, 8, CUS, LDS) is None
     # matrices of many rows: about 3500 waves in the launch, at least four per workgroup, none idle
     for rows, cols, want in [(17408, 5120, 4), (14336, 4096, 4), (8192, 8192, 8), (9216, 2560, 5), (4096, 4096, 8), (5120, 5120, 10)]:
         assert cc.plan_qmm(rows, cols, 64, 1, 8, CUS, LDS)["k_waves"] == want, (rows, cols)
