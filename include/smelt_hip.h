@@ -127,8 +127,9 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * kernel (the two add up a row in different orders: results agree to the output tolerance, not bit
  * for bit); MATRIX_CORE asks for the same explicitly (kept from when AUTO had size thresholds);
  * VECTOR keeps every record on the vector-ALU kernels.  The same switch
- * covers the qmm records and, from two tokens on, the per-token small-batch ("_batched", "_batched_verify_b4")
- * forms of the group-64 affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's (while
+ * covers the qmm records (groups of 64, 128 and 32 columns; rows of a multiple of 256, 512 and 256 columns) and, from
+ * two tokens on, the per-token small-batch ("_batched", "_batched_verify_b4")
+ * forms of the affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's (while
  * tokens x weights stay below about 20M they run the single-token kernel with a grid row per token, bit for
  * bit the rows of a one-token record; beyond, the streaming kernel), and the
  * lm_head matvec+argmax over two tokens and more without a logit cap (logits of all tokens through the

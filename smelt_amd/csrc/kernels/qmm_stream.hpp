@@ -86,7 +86,9 @@ __host__ __device__ constexpr size_t qms_lds_bytes(int tiles, int groups, int wa
     return qms_scale_lds_bytes(tiles, groups) + (size_t)waves * qms_wave_lds_bytes(tiles, token_rows);
 }
 
-template <class ActT, class ScaleT, int NMAT, int RT, int XR, class Epi>
+// G32: groups of 32 columns.  The four k-blocks of an MFMA are the lane quarters q, and q / 2 is the group within a
+// 64-column half, so each half takes its MFMAs twice, once per group with the other group's activations zeroed.
+template <class ActT, class ScaleT, int NMAT, int RT, int XR, class Epi, bool G32 = false>
 __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
                                          const uint16_t* const (&B)[NMAT], const uint16_t* __restrict__ X, int batch,
                                          int rows, int cols, int group, const Epi& epi) {
@@ -103,7 +105,7 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
     // (groups of 128 columns: a step is one group instead of two, everything else is the same)
     const int g64 = cols >> 6;         // 64-column halves of a step's 128 columns
     const int gshift = group == 128 ? 1 : 0;
-    const int gt = g64 >> gshift;      // scale groups per row
+    const int gt = G32 ? g64 << 1 : g64 >> gshift;      // scale groups per row
     const int npairs = g64 >> 1;
     const int rs = cols >> 1;          // bytes per packed row
     const int row0 = blockIdx.x * (16 * RT);
@@ -221,6 +223,36 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
             const unsigned char* xr = stage + xrow * kQsXStride + 128 * e + 32 * q;
             const uint4_t a0 = O::activations(*reinterpret_cast<const uint4_t*>(xr));
             const uint4_t a1 = O::activations(*reinterpret_cast<const uint4_t*>(xr + 16));
+            if constexpr (G32) {
+                uint4_t cx[NMAT][RT], cy[NMAT][RT];
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int t = 0; t < RT; ++t) {
+                        const uint2_t c = *reinterpret_cast<const uint2_t*>(stage_w + ((m * RT + t) * 16 + n) * kQsWStride + 32 * e + 8 * q);
+                        cx[m][t] = O::codes(c.x);
+                        cy[m][t] = O::codes(c.y);
+                    }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const bool mine = (q >> 1) == h;
+                    const uint4_t none = {0u, 0u, 0u, 0u};
+                    const uint4_t a0h = mine ? a0 : none, a1h = mine ? a1 : none;
+                    const float4_t xs = E::mfma(a1h, ones, E::mfma(a0h, ones, zero));
+                    const int ge = gi + e < g64 ? 2 * (gi + e) + h : gt;
+#pragma unroll
+                    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                        for (int t = 0; t < RT; ++t) {
+                            const float4_t d = E::mfma(a1h, cy[m][t], E::mfma(a0h, cx[m][t], zero));
+                            const float2 sb = lds_sb[((m * RT + t) * 16 + n) * sstride + ge];
+                            acc[m][t].x = __builtin_fmaf(sb.x, d.x, __builtin_fmaf(sb.y, xs.x, acc[m][t].x));
+                            acc[m][t].y = __builtin_fmaf(sb.x, d.y, __builtin_fmaf(sb.y, xs.y, acc[m][t].y));
+                            acc[m][t].z = __builtin_fmaf(sb.x, d.z, __builtin_fmaf(sb.y, xs.z, acc[m][t].z));
+                            acc[m][t].w = __builtin_fmaf(sb.x, d.w, __builtin_fmaf(sb.y, xs.w, acc[m][t].w));
+                        }
+                }
+            } else {
             const float4_t xs = E::mfma(a1, ones, E::mfma(a0, ones, zero));
             const int ge = gi + e < g64 ? (gi + e) >> gshift : gt;
 #pragma unroll
@@ -235,6 +267,7 @@ __device__ __forceinline__ void qms_body(const uint8_t* const (&W)[NMAT], const 
                     acc[m][t].z = __builtin_fmaf(sb.x, d.z, __builtin_fmaf(sb.y, xs.z, acc[m][t].z));
                     acc[m][t].w = __builtin_fmaf(sb.x, d.w, __builtin_fmaf(sb.y, xs.w, acc[m][t].w));
                 }
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -361,6 +394,38 @@ struct QsSwiglu {
         const uint16_t* const s[2] = {gS, uS};                                                     \
         const uint16_t* const b[2] = {gB, uB};                                                     \
         qms_body<ACT, SC, 2, 1, XRV>(w, s, b, X, batch, rows, cols, group, QsSwiglu<ACT>{Y});       \
+    }
+
+// Groups of 32 columns: one row tile per wave.
+#define SMELT_AFFINE_QMS_G32(T, ACT, SC, XRV)                                                       \
+    SMELT_QMS_KERNEL void smelt_affine_qms_g32_x##XRV##_store_##T(                                  \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* Y,    \
+        uint32_t batch, uint32_t rows, uint32_t cols, uint32_t group, uint32_t, float*, uint32_t*) { \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        qms_body<ACT, SC, 1, 1, XRV, QsStore<ACT>, true>(w, s, b, X, batch, rows, cols, group, QsStore<ACT>{Y}); \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_affine_qms_g32_x##XRV##_add_##T(                                    \
+        const uint8_t* W, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* MV,   \
+        const uint16_t* RES, uint16_t* OUT, uint32_t batch, uint32_t rows, uint32_t cols,          \
+        uint32_t group, uint32_t, float*, uint32_t*) {                                             \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {W};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        const uint16_t* const b[1] = {B};                                                          \
+        qms_body<ACT, SC, 1, 1, XRV, QsAdd<ACT>, true>(w, s, b, X, batch, rows, cols, group, QsAdd<ACT>{MV, RES, OUT}); \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_affine_qms_g32_x##XRV##_gate_up_swiglu_##T(                         \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t group, uint32_t, float*, uint32_t*) {               \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        qms_body<ACT, SC, 2, 1, XRV, QsSwiglu<ACT>, true>(w, s, b, X, batch, rows, cols, group, QsSwiglu<ACT>{Y}); \
     }
 
 // ---- token-tile form: prefill chunks ------------------------------------------------------------

@@ -374,14 +374,19 @@ bool qmt_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
 
 bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
               size_t lds_limit, QmsPlan* out) {
-    // groups of 64 columns (rows of a multiple of 256 columns) or of 128 (512): scale rows are staged four or eight groups at a time
-    if ((group != 64 && group != 128) || cols == 0 || cols % (4 * group) != 0 || rows == 0 || nmat == 0 || nmat > 2 || batch == 0) return false;
+    // groups of 64 columns (rows of a multiple of 256 columns), of 128 (512) or of 32 (256): scale rows are staged four or
+    // eight groups at a time
+    if ((group != 32 && group != 64 && group != 128) || cols == 0 || cols % (group == 32 ? 256 : 4 * group) != 0 || rows == 0 ||
+        nmat == 0 || nmat > 2 || batch == 0) return false;
+    // (groups of 32 take every 64-column half twice: beyond 256 tokens the token-slab kernel is as fast or faster,
+    // 14336 x 4096 at 512 tokens 283 us against 356)
+    if (group == 32 && batch > 256) return false;
     const uint32_t gt = cols / group, npairs = cols / 128;
     // Measured on MI355X at 2560- and 9216-column rows: about four steps per wave hide the memory
     // round trips best, up to twelve waves; two row tiles per wave (half the activation traffic per
     // weight byte) pay once a pass stages sixteen tokens and the matrix still fills the machine
     // with 32-row workgroups.
-    const uint32_t rt = nmat == 1 && batch > 8 && rows >= 32 * 256 ? 2 : 1;
+    const uint32_t rt = nmat == 1 && batch > 8 && rows >= 32 * 256 && group != 32 ? 2 : 1;   // (the 32-column kernels: one tile)
     uint32_t kc = (npairs + 3) / 4;
     if (kc < 2) kc = npairs < 2 ? 1 : 2;
     if (kc > 12) kc = 12;

@@ -47,6 +47,7 @@ struct Pipeline {
     hipFunction_t fn_qmt[5][5][3] = {};                           // token-tile qmm, by row tiles and token blocks per wave and waves along K
     hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
+    hipFunction_t fn_qms_g32[2] = {};                             // ... for groups of 32 columns
     hipFunction_t fn_logits_keys = nullptr;                       // lm_head over several tokens: partial argmax keys from stored logits
     ResolvedPipeline res;
 };
@@ -1203,7 +1204,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         if (batch >= 2 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && L.args[6].value == 0u && p->fn_logits_keys &&
             aligned16(4) && whole_pieces(4) && (size_t)batch * rows * 2 <= ws.partial_bytes && ws.partial &&
             qms_plan(rows, cols, group, 1, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) &&
-            p->fn_qms[plan.rt][batch > 8]) {
+            (group == 32 ? p->fn_qms_g32[batch > 8] : p->fn_qms[plan.rt][batch > 8])) {
             alignas(16) unsigned char ka[128];
             size_t at = 0;
             auto put_ptr = [&](const void* v) { at = (at + 7) & ~(size_t)7; memcpy(ka + at, &v, 8); at += 8; };
@@ -1219,7 +1220,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
                 ctx->batch_open = true;
                 ctx->timing_valid = false;
             }
-            HIP_TRY(ctx, hipModuleLaunchKernel(p->fn_qms[plan.rt][batch > 8], (rows + 16 * plan.rt - 1) / (16 * plan.rt), (batch + 15) / 16, 1,
+            HIP_TRY(ctx, hipModuleLaunchKernel(group == 32 ? p->fn_qms_g32[batch > 8] : p->fn_qms[plan.rt][batch > 8], (rows + 16 * plan.rt - 1) / (16 * plan.rt), (batch + 15) / 16, 1,
                                                64 * plan.kc, 1, 1, (unsigned)plan.lds, ctx->stream, nullptr, cfg_a));
             alignas(16) unsigned char kb[64];
             at = 0;
@@ -1253,8 +1254,9 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             qms_routed = true;
         }
         QmsPlan plan;
-        if (!routed && batch > (qms_small_batch ? 1u : 0u) && qms_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) && p->fn_qms[plan.rt][batch > 8]) {
-            fn = p->fn_qms[plan.rt][batch > 8];
+        if (!routed && batch > (qms_small_batch ? 1u : 0u) && qms_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) &&
+            (group == 32 ? p->fn_qms_g32[batch > 8] : p->fn_qms[plan.rt][batch > 8])) {
+            fn = group == 32 ? p->fn_qms_g32[batch > 8] : p->fn_qms[plan.rt][batch > 8];
             L.grid[0] = (rows + 16 * plan.rt - 1) / (16 * plan.rt); L.grid[1] = (batch + 15) / 16; L.grid[2] = 1;
             L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
             L.lds = plan.lds;
@@ -1511,6 +1513,9 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
                 for (uint32_t rt = 1; rt <= kQmsMaxRowTiles; ++rt)
                     for (uint32_t wide = 0; wide < 2; ++wide)
                         (void)find(&p.fn_qms[rt][wide], "smelt_affine_qms_r" + std::to_string(rt) + (wide ? "_x4_" : "_x2_") + p.res.qms_tail);
+            if (!p.res.qms_tail.empty())
+                for (uint32_t wide = 0; wide < 2; ++wide)
+                    (void)find(&p.fn_qms_g32[wide], std::string("smelt_affine_qms_g32") + (wide ? "_x4_" : "_x2_") + p.res.qms_tail);
         }
     }
     std::lock_guard<std::mutex> lock(ctx->pipeline_mutex);

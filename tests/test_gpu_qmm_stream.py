@@ -99,19 +99,23 @@ def test_stream_qmm_rows_of_odd_multiples_of_256_columns(ctx, split_k, dtype, sh
     gh.check_steps(y, slab, dtype, f"stream against slab {shape}", max_steps=1)
 
 
-# groups of 128 columns: one scale per step instead of two; 1536 columns = twelve groups, staged four at a time
+# groups of 128 columns: one scale per step instead of two; 1536 columns = twelve groups, staged four at a time.
+# groups of 32: four scales per step, every 64-column half multiplied once per group; 768 and 11008 columns = odd
+# multiples of 256
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
-@pytest.mark.parametrize("shape", [(200, 4096, 13), (8200, 1024, 24), (100, 11264, 40), (40, 1536, 3), (130, 5120, 200)])
-def test_stream_qmm_groups_of_128_columns(ctx, split_k, dtype, shape):
+@pytest.mark.parametrize("group,shape", [(128, (200, 4096, 13)), (128, (8200, 1024, 24)), (128, (100, 11264, 40)), (128, (40, 1536, 3)),
+                                         (128, (130, 5120, 200)), (32, (200, 4096, 13)), (32, (8200, 1024, 24)), (32, (100, 11008, 40)),
+                                         (32, (40, 768, 3)), (32, (130, 5120, 200))])
+def test_stream_qmm_groups_of_128_and_32_columns(ctx, split_k, dtype, group, shape):
     rows, cols, batch = shape
-    w = fx.synth_affine(rows, cols, 128, dtype, config=4, tensor=rows % 5)
+    w = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=rows % 5)
     x = fx.synth_activation(batch, cols, dtype, config=4, tensor=cols % 19, outlier_frac=0.01)
-    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, 128, dtype, threads=True)
-    y = qmm_full(ctx, w, x, dtype, rows, cols, group=128)
-    gh.check_outputs(y, ref, dtype, f"stream qmm g128 {shape}")
-    assert np.array_equal(y, qmm_full(ctx, w, x, dtype, rows, cols, group=128))
-    slab = qmm_full(split_k, w, x, dtype, rows, cols, group=128)
-    gh.check_steps(y, slab, dtype, f"stream against slab, g128 {shape}", max_steps=1)
+    ref = so.affine_matvec(*w, fx.from_bits(x, dtype), rows, cols, group, dtype, threads=True)
+    y = qmm_full(ctx, w, x, dtype, rows, cols, group=group)
+    gh.check_outputs(y, ref, dtype, f"stream qmm g{group} {shape}")
+    assert np.array_equal(y, qmm_full(ctx, w, x, dtype, rows, cols, group=group))
+    slab = qmm_full(split_k, w, x, dtype, rows, cols, group=group)
+    gh.check_steps(y, slab, dtype, f"stream against slab, g{group} {shape}", max_steps=1)
     if batch <= 4:
         # the per-token small-batch form of the same matrix: the streaming kernel, or (small matrices) the single-token
         # kernel with a grid row per token; either way within the tolerance
@@ -120,11 +124,11 @@ def test_stream_qmm_groups_of_128_columns(ctx, split_k, dtype, shape):
         ctx.upload_weights(0, wf.image())
         ctx.put(gh.X_SLOT, x)
         ctx.alloc(gh.Y_SLOT, batch * rows * 2)
-        pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g128_batched_tile4" + gh.t_suffix(dtype))
+        pipe = ctx.pipeline(f"affine_matvec_c{cols}_r{rows}_g{group}_batched_tile4" + gh.t_suffix(dtype))
         bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
         assert ctx.encode_decode(rt.make_record(pipe, bufs, [(5, batch)], (min(1024, (rows + 7) // 8), 1, 1), (256, 1, 1))) == 1
         ctx.wait()
-        gh.check_outputs(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), ref, dtype, "tile4 g128")
+        gh.check_outputs(ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows), ref, dtype, f"tile4 g{group}")
 
 
 def test_stream_qmm_is_exact_where_the_sums_are(ctx):

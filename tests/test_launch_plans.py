@@ -70,7 +70,10 @@ def test_streaming_plan_rows_of_256_column_multiples_and_tall_matrices():
     for batch in (2, 8, 300):
         p = cc.plan_qmm(4096, 4096, 128, 1, batch, CUS, LDS)
         assert p is not None and p["kernel"] == 1
-    assert cc.plan_qmm(4096, 11008, 128, 1, 8, CUS, LDS) is None and cc.plan_qmm(4096, 4096, 32, 1, 8, CUS, LDS) is None
+    p = cc.plan_qmm(16384, 4096, 32, 1, 16, CUS, LDS)       # groups of 32 columns: one row tile per wave
+    assert p is not None and p["kernel"] == 1 and p["row_tiles"] == 1
+    assert cc.plan_qmm(4096, 11008, 128, 1, 8, CUS, LDS) is None and cc.plan_qmm(4096, 4096, 16, 1, 8, CUS, LDS) is None
+    assert cc.plan_qmm(4096, 4096 + 128, 32, 1, 8, CUS, LDS) is None
     # matrices of many rows: about 3500 waves in the launch, at least four per workgroup, none idle
     for rows, cols, want in [(17408, 5120, 4), (14336, 4096, 4), (8192, 8192, 8), (9216, 2560, 5), (4096, 4096, 8), (5120, 5120, 10)]:
         assert cc.plan_qmm(rows, cols, 64, 1, 8, CUS, LDS)["k_waves"] == want, (rows, cols)
@@ -105,7 +108,9 @@ def test_streaming_plan_keeps_two_workgroups_per_unit_when_the_launch_has_them()
 
 
 def test_qmm_plan_rejects_what_no_kernel_takes():
-    assert cc.plan_qmm(1024, 1024, 32, 1, 64) is None      # group 32 has no streaming form
+    assert cc.plan_qmm(1024, 1024, 16, 1, 64) is None      # group 16 has no streaming form
+    assert cc.plan_qmm(1024, 1024, 32, 1, 257) is None     # groups of 32 stream up to 256 tokens
+    assert cc.plan_qmm(1024, 1024, 32, 1, 256) is not None
     assert cc.plan_qmm(1024, 1024, 64, 1, 0) is None
     assert cc.plan_qmm(1024, 1000, 64, 1, 64) is None      # ragged K
     # a small LDS budget: the plan shrinks or gives up, never overshoots
