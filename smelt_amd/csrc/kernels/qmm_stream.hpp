@@ -358,6 +358,20 @@ struct QsSwiglu {
     }
 };
 
+// agent_geglu_product (lut_matvec.metal:2235-2243): gate and up rounded to the 16-bit type, tanh-form GELU of the
+// gate with its argument clamped to +-20, product clamped to the fp16 range
+template <class ActT>
+struct QsGeglu {
+    uint16_t* y;
+    __device__ __forceinline__ void operator()(size_t idx, const float (&v)[2]) const {
+        const float g = ActT::widen(ActT::narrow(v[0])), u = ActT::widen(ActT::narrow(v[1]));
+        float inner = 0.7978845608f * (g + 0.044715f * (g * g * g));
+        inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+        const float gelu = 0.5f * g * (1.0f + tanhf(inner));
+        y[idx] = ActT::narrow(fminf(fmaxf(gelu * u, -65504.0f), 65504.0f));
+    }
+};
+
 }  // namespace smelt
 
 #define SMELT_QMS_KERNEL extern "C" __global__ __launch_bounds__(1024)
@@ -394,6 +408,16 @@ struct QsSwiglu {
         const uint16_t* const s[2] = {gS, uS};                                                     \
         const uint16_t* const b[2] = {gB, uB};                                                     \
         qms_body<ACT, SC, 2, 1, XRV>(w, s, b, X, batch, rows, cols, group, QsSwiglu<ACT>{Y});       \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_affine_qms_r1_x##XRV##_gate_up_geglu_##T(                           \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t group, uint32_t, float*, uint32_t*) {               \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        qms_body<ACT, SC, 2, 1, XRV>(w, s, b, X, batch, rows, cols, group, QsGeglu<ACT>{Y});        \
     }
 
 // Groups of 32 columns: one row tile per wave.
@@ -426,6 +450,16 @@ struct QsSwiglu {
         const uint16_t* const s[2] = {gS, uS};                                                     \
         const uint16_t* const b[2] = {gB, uB};                                                     \
         qms_body<ACT, SC, 2, 1, XRV, QsSwiglu<ACT>, true>(w, s, b, X, batch, rows, cols, group, QsSwiglu<ACT>{Y}); \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_affine_qms_g32_x##XRV##_gate_up_geglu_##T(                          \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t group, uint32_t, float*, uint32_t*) {               \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        qms_body<ACT, SC, 2, 1, XRV, QsGeglu<ACT>, true>(w, s, b, X, batch, rows, cols, group, QsGeglu<ACT>{Y}); \
     }
 
 // ---- token-tile form: prefill chunks ------------------------------------------------------------
@@ -820,4 +854,14 @@ __device__ __forceinline__ void qmt_body(const uint8_t* const (&W)[NMAT], const 
         const uint16_t* const s[2] = {gS, uS};                                                     \
         const uint16_t* const b[2] = {gB, uB};                                                     \
         qmt_body<ACT, SC, 2, RTV, TBV, KWV, PWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsSwiglu<ACT>{Y}); \
+    }                                                                                              \
+    SMELT_QMT_KERNEL(KWV) void smelt_affine_qmt_##TAG##RTV##_t##TBV##_k##KWV##_gate_up_geglu_##T(      \
+        const uint8_t* gW, const uint16_t* gS, const uint16_t* gB, const uint8_t* uW,              \
+        const uint16_t* uS, const uint16_t* uB, const uint16_t* X, uint16_t* Y, uint32_t batch,    \
+        uint32_t rows, uint32_t cols, uint32_t, uint32_t, float* WSP, uint32_t* WSC) {             \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gW, uW};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        const uint16_t* const b[2] = {gB, uB};                                                     \
+        qmt_body<ACT, SC, 2, RTV, TBV, KWV, PWV>(w, s, b, X, batch, rows, cols, WSP, WSC, QsGeglu<ACT>{Y}); \
     }

@@ -276,12 +276,12 @@ void attach_mm1(ResolvedPipeline* r) {
         {"smelt_teraff_bank4_matvec_", "smelt_teraff_mm1_", "bank4_matvec_", kCodesTernary2, 1},
     };
     const std::string t = act_suffix(r->act);
-    // the per-token small-batch forms of the plain matvec and of gate+up+SwiGLU: the single-token kernels with one
+    // the per-token small-batch forms of the plain matvec and of gate+up (SwiGLU, GeGLU): the single-token kernels with one
     // grid row per token (small matrices at a few tokens; the batch argument leaves the argument block)
-    if (r->family == kFamAffineBatched || (r->family == kFamAffineGateUpBatched && r->symbol.find("swiglu") != std::string::npos)) {
+    if (r->family == kFamAffineBatched || r->family == kFamAffineGateUpBatched) {
         const bool pair = r->family == kFamAffineGateUpBatched;
         r->mm1_prefix = "smelt_affine_mm1_";
-        r->mm1_tail = std::string(pair ? "gate_up_swiglu_" : "matvec_") + t;
+        r->mm1_tail = std::string(!pair ? "matvec_" : (r->symbol.find("geglu") != std::string::npos ? "gate_up_geglu_" : "gate_up_swiglu_")) + t;
         r->mm1_layout = (int)kCodesU4;
         r->mm1_nmat = pair ? 2 : 1;
         return;
@@ -307,6 +307,7 @@ void attach_qms(ResolvedPipeline* r) {
     // (the lm_head over two tokens and more: logits through the streaming kernel, keys from a second launch)
     else if (r->family == kFamAffineArgmax) { r->qms_tail = "store_" + t; r->qms_nmat = 1; }
     else if ((r->family == kFamAffineQmmGateUp || r->family == kFamAffineGateUpBatched) && r->symbol.find("swiglu") != std::string::npos) { r->qms_tail = "gate_up_swiglu_" + t; r->qms_nmat = 2; }
+    else if ((r->family == kFamAffineQmmGateUp || r->family == kFamAffineGateUpBatched) && r->symbol.find("geglu") != std::string::npos) { r->qms_tail = "gate_up_geglu_" + t; r->qms_nmat = 2; }
 }
 
 ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType default_act, size_t lds_limit,

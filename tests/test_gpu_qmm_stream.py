@@ -366,3 +366,42 @@ def test_tile_qmm_gate_up_on_a_grid_that_fills_the_machine(ctx):
     u = so.affine_matvec(*uw, xf, rows, cols, 64, dtype, threads=True)
     ref = fx.from_bits(so.epilogue_affine_swiglu(g, u, so.BF16), dtype)
     gh.check_outputs(y, gh.swiglu_unrounded(g, u), dtype, "tile gate_up_swiglu, full grid")
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("shape", [(640, 1024, 21), (2100, 2560, 140), (200, 11008, 9), (512, 1024, 3)])
+def test_geglu_qmm_streams_and_tiles(ctx, split_k, dtype, shape):
+    """The GeGLU gate+up qmm (Gemma-shaped layers) on the streaming kernel (21 and 9 tokens; 11008 columns), on the
+    token-tile kernel (140 tokens of a matrix pair of 10M weights) and, three tokens of a small pair through the per-token
+    small-batch name, on the single-token kernel with a grid row per token: against the oracle's epilogue to the step
+    bound of the GeGLU tests, and against the token-slab kernel the qmm record names."""
+    rows, cols, batch = shape
+    gw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=23)
+    uw = fx.synth_affine(rows, cols, 64, dtype, config=4, tensor=24)
+    x = fx.synth_activation(batch, cols, dtype, config=4, tensor=28)
+    xf = fx.from_bits(x, dtype)
+    g = so.affine_matvec(*gw, xf, rows, cols, 64, dtype, threads=True)
+    u = so.affine_matvec(*uw, xf, rows, cols, 64, dtype, threads=True)
+    ref = so.epilogue_geglu(g, u, dtype)
+
+    def run(c, name, consts, grid):
+        wf = gh.WeightFile()
+        offs = [wf.add(a) for a in (*gw, *uw)]
+        c.upload_weights(0, wf.image())
+        c.put(gh.X_SLOT, x)
+        c.alloc(gh.Y_SLOT, batch * rows * 2)
+        pipe = c.pipeline(name + gh.t_suffix(dtype))
+        bufs = [(0, i, offs[i]) for i in range(6)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)]
+        assert c.encode_prefill(rt.make_record(pipe, bufs, consts, grid, (256, 1, 1)), seq_len=batch) == 1
+        c.wait()
+        return c.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+
+    full = f"fused_affine_gate_up_geglu_c{cols}_r{rows}_g64_batched_full_b64"
+    grid = ((rows + 63) // 64, (batch + 63) // 64, 1)
+    y = run(ctx, full, [(8, batch)], grid)
+    gh.check_steps(y, ref, dtype, f"geglu qmm {shape}", max_steps=gh.GEGLU_STEPS)
+    assert np.array_equal(y, run(ctx, full, [(8, batch)], grid))
+    gh.check_steps(y, run(split_k, full, [(8, batch)], grid), dtype, f"geglu qmm against slab {shape}", max_steps=gh.GEGLU_STEPS)
+    if batch <= 3:
+        small = run(ctx, f"fused_affine_gate_up_geglu_c{cols}_r{rows}_g64_batched", [(8, batch)], (min(1024, (rows + 7) // 8), 1, 1))
+        gh.check_steps(small, ref, dtype, f"geglu small batch {shape}", max_steps=gh.GEGLU_STEPS)
