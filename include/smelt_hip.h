@@ -134,7 +134,8 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * bit the rows of a one-token record; beyond, the streaming kernel), and the
  * lm_head matvec+argmax over two tokens and more without a logit cap (logits of all tokens through the
  * streaming kernel into the context workspace, partial keys from a second launch: the record then counts as
- * two launches), and the same record at one token where the rows' 16-byte pieces leave the fused kernel's last
+ * two launches), the norm-scale prologue qmm records from two tokens on (the normalised rows from a launch of
+ * their own, then the kernel of the plain record: two launches, the bits of the staged pair), and the lm_head record at one token where the rows' 16-byte pieces leave the fused kernel's last
  * pass over a row less than nine tenths full (1536, 2560, 3072, 3584, 5120 columns: the single-pass kernel
  * with the argmax as its epilogue, tiles that share a partial key meeting in the context workspace): AUTO and
  * MATRIX_CORE run the streaming kernel of the pipeline below 128

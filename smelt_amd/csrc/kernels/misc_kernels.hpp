@@ -103,9 +103,32 @@ __device__ __forceinline__ uint16_t trit5_lut_entry(uint32_t b) {
         smelt::signed_gather_body<2, ACT>(C, S, ids, out, hidden, lut);                           \
     }
 
+// The rows a norm-scale qmm multiplies, written out once for all of the matrix's workgroups:
+// out[t][c] = narrow((x[t][c] * rs[t]) * (1 + w[c])), the bits a staged norm stores.  Eight columns per thread
+// (cols is a multiple of eight), grid (columns / 2048 rounded up, tokens).
+#define SMELT_NORM_SCALE_ROWS(T, ACT)                                                             \
+    SMELT_MISC_KERNEL void smelt_norm_scale_rows_##T(                                             \
+        const float* rs, const uint16_t* x, const uint16_t* w, uint16_t* out, uint32_t batch, uint32_t cols) { \
+        using namespace smelt;                                                                    \
+        const uint32_t tok = blockIdx.y, c0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;        \
+        if (tok >= batch || c0 >= cols) return;                                                   \
+        const float r = rs[tok];                                                                  \
+        const uint4_t xv = *reinterpret_cast<const uint4_t*>(x + (size_t)tok * cols + c0);        \
+        const uint4_t wv = *reinterpret_cast<const uint4_t*>(w + c0);                             \
+        uint32_t o[4];                                                                            \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                           \
+            const uint16_t lo = norm_scale_value<ACT>((uint16_t)(xv[j] & 0xFFFFu), r, (uint16_t)(wv[j] & 0xFFFFu)); \
+            const uint16_t hi = norm_scale_value<ACT>((uint16_t)(xv[j] >> 16), r, (uint16_t)(wv[j] >> 16));         \
+            o[j] = (uint32_t)lo | ((uint32_t)hi << 16);                                           \
+        }                                                                                         \
+        *reinterpret_cast<uint4_t*>(out + (size_t)tok * cols + c0) = uint4_t{o[0], o[1], o[2], o[3]}; \
+    }
+
 #ifndef SMELT_NO_INCLUDE_INSTANCES
 SMELT_GATHER_KERNELS(f16, smelt::F16)
 SMELT_GATHER_KERNELS(bf16, smelt::BF16)
+SMELT_NORM_SCALE_ROWS(f16, smelt::F16)
+SMELT_NORM_SCALE_ROWS(bf16, smelt::BF16)
 #endif
 
 #ifndef SMELT_NO_INCLUDE_INSTANCES

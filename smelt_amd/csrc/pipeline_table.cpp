@@ -308,6 +308,9 @@ void attach_qms(ResolvedPipeline* r) {
     else if (r->family == kFamAffineArgmax) { r->qms_tail = "store_" + t; r->qms_nmat = 1; }
     else if ((r->family == kFamAffineQmmGateUp || r->family == kFamAffineGateUpBatched) && r->symbol.find("swiglu") != std::string::npos) { r->qms_tail = "gate_up_swiglu_" + t; r->qms_nmat = 2; }
     else if ((r->family == kFamAffineQmmGateUp || r->family == kFamAffineGateUpBatched) && r->symbol.find("geglu") != std::string::npos) { r->qms_tail = "gate_up_geglu_" + t; r->qms_nmat = 2; }
+    // (the norm-scale prologue forms: the rows are normalised by a launch of their own, then the kernels of the plain forms)
+    else if (r->family == kFamNormScaleAffineQmm || r->family == kFamNormScaleAffineBatched) { r->qms_tail = "store_" + t; r->qms_nmat = 1; }
+    else if (r->family == kFamNormScaleAffineQmmGateUp) { r->qms_tail = std::string(r->symbol.find("geglu") != std::string::npos ? "gate_up_geglu_" : "gate_up_swiglu_") + t; r->qms_nmat = 2; }
 }
 
 ResolveStatus resolve_pipeline_entry(const std::string& entry_in, ActDType default_act, size_t lds_limit,

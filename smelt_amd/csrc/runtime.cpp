@@ -48,6 +48,7 @@ struct Pipeline {
     hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
     hipFunction_t fn_qms_g32[2] = {};                             // ... for groups of 32 columns
+    hipFunction_t fn_norm_rows = nullptr;                         // norm-scale qmm: the normalised rows, written once
     hipFunction_t fn_logits_keys = nullptr;                       // lm_head over several tokens: partial argmax keys from stored logits
     ResolvedPipeline res;
 };
@@ -1233,6 +1234,68 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             HIP_TRY(ctx, hipModuleLaunchKernel(p->fn_logits_keys, L.grid[0], batch, 1, 64, 1, 1, 0, ctx->stream, nullptr, cfg_b));
             return 2;
         }
+    } else if (p->res.family == kFamNormScaleAffineQmm || p->res.family == kFamNormScaleAffineQmmGateUp || p->res.family == kFamNormScaleAffineBatched) {
+        // Norm-scale prologue in front of a qmm (rs X nw XN W S B Y batch | rows cols group tile; gate+up: rs X nw gW gS gB
+        // uW uS uB Y batch | ...): the fused kernels are the token-slab and vector ones; instead one launch writes the
+        // normalised rows (into the record's XN, or into the end of the workspace where the record has none) and the
+        // streaming or token-tile kernel of the plain form multiplies them: the bits of the staged pair.  From two tokens on.
+        const bool pair = p->res.family == kFamNormScaleAffineQmmGateUp;
+        const size_t o = pair ? 10 : 8;
+        const uint32_t batch = L.args[o].value, rows = L.args[o + 1].value, cols = L.args[o + 2].value, group = L.args[o + 3].value;
+        const size_t xn_bytes = ((size_t)batch * cols * 2 + 255) & ~(size_t)255;
+        char* xn = !pair && L.args[3].ptr ? L.args[3].ptr : nullptr;
+        const bool scratch = xn == nullptr;
+        if (scratch && ws.partial && xn_bytes <= ws.partial_bytes) xn = (char*)ws.partial + (ws.partial_bytes - xn_bytes);
+        const size_t ws_left = scratch ? ws.partial_bytes - (xn ? xn_bytes : 0) : ws.partial_bytes;
+        const size_t wfirst = pair ? 3 : 4, wcount = pair ? 6 : 3;
+        hipFunction_t fn2 = nullptr;
+        uint32_t g2[3] = {0, 0, 0}, block2 = 0;
+        size_t lds2 = 0;
+        QmtPlan tplan;
+        QmsPlan plan;
+        if (batch >= 2 && xn && (reinterpret_cast<uintptr_t>(xn) & 15u) == 0 && p->fn_norm_rows && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && cols % 8 == 0 &&
+            aligned16(wfirst + wcount, wfirst) && whole_pieces(wfirst + wcount, wfirst) && aligned16(3, 1)) {
+            if (qmt_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &tplan) &&
+                (tplan.per_wave ? p->fn_qmt_per_wave : p->fn_qmt)[tplan.rt][tplan.tb][tplan.kw]) {
+                fn2 = (tplan.per_wave ? p->fn_qmt_per_wave : p->fn_qmt)[tplan.rt][tplan.tb][tplan.kw];
+                const uint32_t ksplit = tplan.partial_bytes <= ws_left && tplan.counter_bytes <= ws.counter_bytes ? tplan.ksplit : 1;
+                g2[0] = (rows + tplan.bn - 1) / tplan.bn; g2[1] = (batch + tplan.bm - 1) / tplan.bm; g2[2] = ksplit;
+                block2 = 256 * tplan.kw; lds2 = tplan.lds;
+            } else if (qms_plan(rows, cols, group, p->res.qms_nmat, batch, (uint32_t)ctx->props.multiProcessorCount, ctx->lds_limit, &plan) &&
+                       (group == 32 ? p->fn_qms_g32[batch > 8] : p->fn_qms[plan.rt][batch > 8])) {
+                fn2 = group == 32 ? p->fn_qms_g32[batch > 8] : p->fn_qms[plan.rt][batch > 8];
+                g2[0] = (rows + 16 * plan.rt - 1) / (16 * plan.rt); g2[1] = (batch + 15) / 16; g2[2] = 1;
+                block2 = 64 * plan.kc; lds2 = plan.lds;
+            }
+        }
+        if (fn2) {
+            alignas(16) unsigned char ka[64], kb[160];
+            size_t at = 0;
+            auto put = [&](unsigned char* buf, const void* v, size_t n, size_t align) { at = (at + align - 1) & ~(align - 1); memcpy(buf + at, v, n); at += n; };
+            const void* rs = L.args[0].ptr; const void* xin = L.args[1].ptr; const void* nw = L.args[2].ptr;
+            put(ka, &rs, 8, 8); put(ka, &xin, 8, 8); put(ka, &nw, 8, 8); put(ka, &xn, 8, 8); put(ka, &batch, 4, 4); put(ka, &cols, 4, 4);
+            size_t ka_size = at;
+            void* cfg_a[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size, HIP_LAUNCH_PARAM_END};
+            if (!ctx->batch_open) {
+                HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+                ctx->batch_open = true;
+                ctx->timing_valid = false;
+            }
+            HIP_TRY(ctx, hipModuleLaunchKernel(p->fn_norm_rows, (cols / 8 + 255) / 256, batch, 1, 256, 1, 1, 0, ctx->stream, nullptr, cfg_a));
+            at = 0;
+            for (size_t i = 0; i < wcount; ++i) { const void* w = L.args[wfirst + i].ptr; put(kb, &w, 8, 8); }
+            put(kb, &xn, 8, 8);
+            const void* y = L.args[pair ? 9 : 7].ptr;
+            put(kb, &y, 8, 8);
+            const uint32_t tail[5] = {batch, rows, cols, group, L.args[o + 4].value};
+            put(kb, tail, sizeof tail, 4);
+            const void* wsp = ws.partial; const void* wsc = ws.counters;
+            put(kb, &wsp, 8, 8); put(kb, &wsc, 8, 8);
+            size_t kb_size = at;
+            void* cfg_b[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, kb, HIP_LAUNCH_PARAM_BUFFER_SIZE, &kb_size, HIP_LAUNCH_PARAM_END};
+            HIP_TRY(ctx, hipModuleLaunchKernel(fn2, g2[0], g2[1], g2[2], block2, 1, 1, (unsigned)lds2, ctx->stream, nullptr, cfg_b));
+            return 2;
+        }
     } else if (!routed && !p->res.qms_tail.empty() && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR &&
         aligned16(qms_pair ? 7 : 4) && whole_pieces(qms_pair ? 7 : 4)) {
         // skinny qmm (and, from two tokens on, the per-token small-batch forms, whose arguments are the
@@ -1509,6 +1572,8 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
                 }
             }
             if (p.res.family == kFamAffineArgmax) (void)find(&p.fn_logits_keys, "smelt_logits_argmax_partials");
+            if (p.res.family == kFamNormScaleAffineQmm || p.res.family == kFamNormScaleAffineQmmGateUp || p.res.family == kFamNormScaleAffineBatched)
+                (void)find(&p.fn_norm_rows, std::string("smelt_norm_scale_rows_") + (p.res.act == kActBF16 ? "bf16" : "f16"));
             if (!p.res.qms_tail.empty())
                 for (uint32_t rt = 1; rt <= kQmsMaxRowTiles; ++rt)
                     for (uint32_t wide = 0; wide < 2; ++wide)

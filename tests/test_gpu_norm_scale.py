@@ -255,11 +255,11 @@ def test_emitted_scale_only_plus_norm_scale_pair_equals_norm_then_matvec(dtype):
         ctx.close()
 
 
-def run_qmm(ctx, entry, dtype, batch, bufs_fn, rows, grid_w, bt, batch_index):
+def run_qmm(ctx, entry, dtype, batch, bufs_fn, rows, grid_w, bt, batch_index, launches=1):
     pipe = ctx.pipeline(entry + gh.t_suffix(dtype))
     ctx.alloc(gh.Y_SLOT, batch * rows * 2)
     rec = rt.make_record(pipe, bufs_fn(), [(batch_index, batch)], (grid_w, (batch + bt - 1) // bt, 1), (256, 1, 1))
-    assert ctx.encode_decode(rec) == 1
+    assert ctx.encode_decode(rec) == launches
     ctx.wait()
     return ctx.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
 
@@ -296,6 +296,40 @@ def test_norm_scale_qmm_equals_plain_qmm_on_the_stored_rows(ctx, dtype, batch, s
     gh.check_outputs(fused, ref, dtype, "norm_scale qmm")
 
 
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("batch,suffix,bt,rows,cols", [(14, "_batched_full", 16, 1000, 1024), (140, "_batched_full_b64", 64, 2100, 2560),
+                                                       (3, "_batched", 8, 1000, 1024), (37, "_batched_full", 16, 200, 11008)])
+def test_norm_scale_qmm_under_the_default_engine_is_the_staged_pair(ctx, dtype, batch, suffix, bt, rows, cols):
+    """Under AUTO the norm-scale qmm records (token-slab and per-token small-batch names) run as two launches: the
+    normalised rows (stored to the record's output, the bits of a staged norm), then the streaming or token-tile
+    kernel of the plain record (140 tokens of a 5.4M-weight matrix: token tiles).  Equal bit for bit to the plain
+    record run on the stored rows, which takes the same kernel."""
+    group = 64
+    weights = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=2)
+    x, w, rs = norm_inputs(batch, cols, dtype, seed=batch)
+    wf = gh.WeightFile()
+    ow, os_, ob = (wf.add(a) for a in weights)
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
+    ctx.alloc(XN_SLOT, batch * cols * 2)
+    shape = f"_c{cols}_r{rows}_g{group}"
+    grid_w = (rows + 63) // 64 if "full" in suffix else min(1024, (rows + 7) // 8)
+    fused = run_qmm(ctx, "norm_scale_affine_matvec" + shape + suffix, dtype, batch,
+                    lambda: [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0), (XN_SLOT, 3, 0), (0, 4, ow), (0, 5, os_),
+                             (0, 6, ob), (gh.Y_SLOT, 7, 0)], rows, grid_w, bt, 8, launches=2)
+    xn = ctx.read(XN_SLOT, np.uint16, batch * cols).reshape(batch, cols)
+    for b in range(batch):
+        assert np.array_equal(xn[b], so.norm_scale_input(x[b], rs[b], w, dtype)), b
+    ctx.put(gh.X_SLOT, xn)
+    plain = "_batched_full" if suffix == "_batched" else suffix     # (three tokens of a 1M-weight matrix stream either way)
+    staged = run_qmm(ctx, "affine_matvec" + shape + plain, dtype, batch,
+                     lambda: [(0, 0, ow), (0, 1, os_), (0, 2, ob), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)],
+                     rows, (rows + 63) // 64, 16 if plain == "_batched_full" else bt, 5)
+    assert np.array_equal(fused, staged)
+    ref = so.affine_matvec(*weights, fx.from_bits(xn, dtype), rows, cols, group, dtype, threads=True)
+    gh.check_outputs(fused, ref, dtype, "norm_scale qmm, default engine")
+
+
 @pytest.mark.parametrize("act", ["swiglu", "geglu"])
 def test_norm_scale_gate_up_qmm_and_geglu_qmm(ctx, act):
     rows, cols, group, dtype, batch, bt = 640, 1024, 64, fx.F16, 21, 16
@@ -308,16 +342,22 @@ def test_norm_scale_gate_up_qmm_and_geglu_qmm(ctx, act):
     ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
     ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
     shape = f"_c{cols}_r{rows}_g{group}_batched_full"
-    fused = run_qmm(ctx, f"norm_scale_affine_gate_up_{act}" + shape, dtype, batch,
-                    lambda: [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0)] + [(0, 3 + i, o) for i, o in enumerate(offs)] +
-                            [(gh.Y_SLOT, 9, 0)], rows, (rows + 63) // 64, bt, 10)
-    ctx.put(gh.X_SLOT, xn)
-    ctx.set_matvec_engine(rt.MATVEC_VECTOR)   # the staged record on the token-slab kernel the fused form shares its tile code with
-    staged = run_qmm(ctx, f"fused_affine_gate_up_{act}" + shape, dtype, batch,
-                     lambda: [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)],
-                     rows, (rows + 63) // 64, bt, 8)
-    ctx.set_matvec_engine(rt.MATVEC_AUTO)
-    assert np.array_equal(fused, staged)
+    # on either engine the fused record equals the staged pair bit for bit: under AUTO two launches (the normalised rows
+    # into the workspace, then the streaming kernel of the plain gate+up), under VECTOR the token-slab kernel both share
+    for engine, launches in ((rt.MATVEC_AUTO, 2), (rt.MATVEC_VECTOR, 1)):
+        ctx.set_matvec_engine(engine)
+        try:
+            ctx.put(gh.X_SLOT, x)
+            fused = run_qmm(ctx, f"norm_scale_affine_gate_up_{act}" + shape, dtype, batch,
+                            lambda: [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0)] + [(0, 3 + i, o) for i, o in enumerate(offs)] +
+                                    [(gh.Y_SLOT, 9, 0)], rows, (rows + 63) // 64, bt, 10, launches=launches)
+            ctx.put(gh.X_SLOT, xn)
+            staged = run_qmm(ctx, f"fused_affine_gate_up_{act}" + shape, dtype, batch,
+                             lambda: [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 6, 0), (gh.Y_SLOT, 7, 0)],
+                             rows, (rows + 63) // 64, bt, 8)
+        finally:
+            ctx.set_matvec_engine(rt.MATVEC_AUTO)
+        assert np.array_equal(fused, staged), engine
     xf = fx.from_bits(xn, dtype)
     g = so.affine_matvec(*gw, xf, rows, cols, group, dtype)
     u = so.affine_matvec(*uw, xf, rows, cols, group, dtype)
