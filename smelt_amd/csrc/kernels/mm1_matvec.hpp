@@ -167,13 +167,13 @@ struct M1U4 : M1Codes<4, ActT> {
 __host__ __device__ constexpr int mm1_piece_stride(int frags_per_piece, int dw = 4) {
     return dw == 4 ? (frags_per_piece == 4 ? 4 : frags_per_piece + 1) : frags_per_piece;
 }
-__host__ __device__ constexpr size_t mm1_wave_lds_bytes(int frags_per_piece, int nl, int dw = 4) {
-    return (size_t)nl * 8 * mm1_piece_stride(frags_per_piece, dw) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) +
+__host__ __device__ constexpr size_t mm1_wave_lds_bytes(int frags_per_piece, int nl, int dw = 4, int tok = 1) {
+    return (size_t)tok * ((size_t)nl * 8 * mm1_piece_stride(frags_per_piece, dw) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4)) +
            (size_t)frags_per_piece * 16;
 }
-__host__ __device__ constexpr size_t mm1_lds_bytes(int frags_per_piece, int nl, int waves, int nmat, int gpr, bool has_bias, int dw = 4) {
-    return (size_t)waves * mm1_wave_lds_bytes(frags_per_piece, nl, dw) + (size_t)nmat * (has_bias ? 2 : 1) * 8 * gpr * 2 +
-           (size_t)waves * nmat * 32 + (dw == 4 ? 0 : 512);
+__host__ __device__ constexpr size_t mm1_lds_bytes(int frags_per_piece, int nl, int waves, int nmat, int gpr, bool has_bias, int dw = 4, int tok = 1) {
+    return (size_t)waves * mm1_wave_lds_bytes(frags_per_piece, nl, dw, tok) + (size_t)nmat * (has_bias ? 2 : 1) * 8 * gpr * 2 +
+           (size_t)waves * nmat * tok * 32 + (dw == 4 ? 0 : 512);
 }
 
 // v[i] + v[i ^ 16] and v[i] + v[i ^ 32] in every lane, through the lane-swap instructions (no LDS
@@ -201,10 +201,13 @@ __device__ __forceinline__ float quad_sum(float v) {
 // NORM: 0 = x is multiplied as it is; 1 = the norm-scale prologue (what is multiplied is
 // narrow((x * rs[token]) * (1 + weight)), the bits a staged norm would have stored; workgroup 0 also
 // stores that row to ns.out); 2 = the same followed by the residual add of the norm_add_scale form.
-template <class F, class ActT, class ScaleT, int NMAT, int NL, class Epi, int NORM = 0>
+// TOK = 2: two tokens per pass (grid row r takes tokens 2r and 2r + 1 of `tokens`).  With four-dword pieces the
+// token slots 4q + 2 and 4q + 3 of an MFMA are free: they carry the second token's fragments, so the weights are
+// unpacked and multiplied once for both tokens.
+template <class F, class ActT, class ScaleT, int NMAT, int NL, class Epi, int NORM = 0, int TOK = 1>
 __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint16_t* __restrict__ x_all, int rows,
                                          int cols, int row_stride, int group, const Epi& epi,
-                                         const NormScale& ns = NormScale{}) {
+                                         const NormScale& ns = NormScale{}, int tokens = 0) {
     using E = Elem16<ActT>;
     constexpr int FPD = F::kFPD, FPL = F::kFPL, FIELDS = F::kFields, PAIRS = F::kPairs, DW = F::kDW;
     constexpr int PSTRIDE = mm1_piece_stride(FPL, DW);     // fragments from one piece to the next in LDS
@@ -212,6 +215,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     constexpr int NITEMS = NL * 8 * DW;                    // staging items of a wave: 8 pieces x DW dwords per segment
     constexpr int ITEMS = (NITEMS + kWave - 1) / kWave;    // per lane
     constexpr int PLANES = F::kHasBias ? 2 : 1;
+    static_assert(TOK == 1 || (TOK == 2 && DW == 4 && NORM == 0 && !Epi::kTile), "two tokens per pass: four-dword pieces, no prologue");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
     // five-digit bytes: the 512-byte decode table sits at the start of LDS (a lookup address is the byte
     // value times two), everything else behind it
@@ -220,8 +224,11 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     const int chunk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int kc = blockDim.x / kWave;
     const int n = lane & 15, q = lane >> 4;
-    const int token = blockIdx.y;
+    const int token = blockIdx.y * TOK;
+    // (a second token past the batch re-reads the last one and is never stored)
+    const int token_b = TOK == 2 && token + 1 < tokens ? token + 1 : token;
     const uint16_t* __restrict__ x = x_all + (size_t)token * cols;
+    const uint16_t* __restrict__ x_b = x_all + (size_t)token_b * cols;
     const int pieces = row_stride >> 4;               // 16-byte pieces per packed row
     const int gshift = ilog2((uint32_t)group);
     const int gpr = (cols + group - 1) >> gshift;     // 16-byte pieces of one plane's scale block, too
@@ -243,7 +250,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     //
     // ---- 1. this wave's slice of x ---------------------------------------------------------------
     // One item = the columns of one packed dword; item it = 4 * (piece within the run) + dword.
-    uint32_t xe[ITEMS][FIELDS / 2];
+    uint32_t xe[TOK][ITEMS][FIELDS / 2];
     int item_piece[ITEMS], item_dword[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
@@ -256,8 +263,10 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         const bool past = DW != 4 && col0 > cols - FIELDS;
         if (col0 > cols - FIELDS) col0 = cols - FIELDS;   // cols is a multiple of kFields
 #pragma unroll
+        for (int tk = 0; tk < TOK; ++tk)
+#pragma unroll
         for (int v = 0; v < FIELDS / 8; ++v) {
-            uint4_t t = *reinterpret_cast<const uint4_t*>(x + col0 + 8 * v);
+            uint4_t t = *reinterpret_cast<const uint4_t*>((tk == 0 ? x : x_b) + col0 + 8 * v);
             if constexpr (NORM != 0) {
                 // eight activations through the prologue, each rounded as the staged norm rounds it
                 const float rs = ns.rs[token];
@@ -280,8 +289,8 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
                 // (lanes past the last item hold the last item again and store the same bits again)
                 if (blockIdx.x == 0 && ns.out != nullptr) *reinterpret_cast<uint4_t*>(ns.out + (size_t)token * cols + col0 + 8 * v) = t;
             }
-            xe[k][4 * v] = past ? 0u : t.x; xe[k][4 * v + 1] = past ? 0u : t.y;
-            xe[k][4 * v + 2] = past ? 0u : t.z; xe[k][4 * v + 3] = past ? 0u : t.w;
+            xe[tk][k][4 * v] = past ? 0u : t.x; xe[tk][k][4 * v + 1] = past ? 0u : t.y;
+            xe[tk][k][4 * v + 2] = past ? 0u : t.z; xe[tk][k][4 * v + 3] = past ? 0u : t.w;
         }
     }
     // ---- 2. the scale (and bias) rows of the tile: one contiguous block per matrix and plane ----
@@ -335,13 +344,15 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // the epilogue's operand, by every lane of every wave (clamped to the tile's rows): under a branch
     // the load brings its own wait on everything issued before it, and wave 0 would stage x only
     // after all its weights have arrived
-    uint16_t res = 0;
+    uint16_t res[TOK] = {};
     if constexpr (Epi::kPrefetch) {
         const int rr = row0 + (lane & 7);
-        res = epi.prefetch(token, rr < rows ? rr : rows - 1);
+        res[0] = epi.prefetch(token, rr < rows ? rr : rows - 1);
+        if constexpr (TOK == 2) res[1] = epi.prefetch(token_b, rr < rows ? rr : rows - 1);
     }
 
-    const size_t wave_bytes = mm1_wave_lds_bytes(FPL, NL, DW);
+    const size_t wave_bytes = mm1_wave_lds_bytes(FPL, NL, DW, TOK);
+    constexpr int kTokStride = NL * 8 * PSTRIDE + (DW == 4 ? NL * 4 : 0);   // fragments and sums of one token, in 16-byte units
     uint4_t* lds_scales = reinterpret_cast<uint4_t*>(smem + (size_t)kc * wave_bytes);
     // ---- 4. x as operand fragments, wave-private in LDS --------------------------------------------
     // kFields consecutive activations become the kFPD fragments that dword's MFMAs take (k-slots
@@ -349,7 +360,9 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // in the four lanes of a quad, which add up their sum(base * x) and sum(x).
     uint4_t* wfrag = reinterpret_cast<uint4_t*>(smem + (size_t)chunk * wave_bytes);
     float* wsum = reinterpret_cast<float*>(wfrag + (size_t)NL * 8 * PSTRIDE);   // [piece][2]: constant, sum x ([piece][DW]: constants)
-    uint4_t* wzero = reinterpret_cast<uint4_t*>(wsum + (DW == 4 ? NL * 16 : NL * 8 * DW));   // FPL zero fragments
+    // (a second token's fragments and sums follow the first's; the zero fragments come last)
+    uint4_t* wzero = TOK == 2 ? wfrag + (size_t)TOK * kTokStride
+                              : reinterpret_cast<uint4_t*>(wsum + (DW == 4 ? NL * 16 : NL * 8 * DW));   // FPL zero fragments
     // decode table of the five-digit bytes, copied from constant memory; visible after the barrier below
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem_all);
     if constexpr (F::kDecode) {
@@ -358,16 +371,20 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     }
     if (lane < FPL) wzero[lane] = uint4_t{0u, 0u, 0u, 0u};
 #pragma unroll
+    for (int tk = 0; tk < TOK; ++tk)
+#pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         // lanes past the last item hold the last item again (whole quads of them: d == 3) and store
         // the same fragments again
         const int pl = item_piece[k], d = item_dword[k], it = pl * DW + d;
+        uint4_t* const wfrag_t = wfrag + (size_t)tk * kTokStride;
+        float* const wsum_t = wsum + (size_t)tk * kTokStride * 4;
         float cb = 0.0f, xs = 0.0f;
         constexpr uint32_t kOnes = F::both((uint32_t)E::kExpBias << E::kMant);   // (1.0, 1.0)
         uint32_t fr[PAIRS];
 #pragma unroll
         for (int j = 0; j < PAIRS; ++j) {
-            const uint32_t lo = xe[k][j >> 1], hi = xe[k][(PAIRS >> 1) + (j >> 1)];
+            const uint32_t lo = xe[tk][k][j >> 1], hi = xe[tk][k][(PAIRS >> 1) + (j >> 1)];
             fr[j] = __builtin_amdgcn_perm(hi, lo, (j & 1) ? 0x07060302u : 0x05040100u);   // (x[j], x[j + kPairs])
             cb = E::dot2k(fr[j], F::base_pair(j), cb);
             xs = E::dot2k(fr[j], kOnes, xs);
@@ -378,11 +395,11 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         }
 #pragma unroll
         for (int t = 0; t < FPD; ++t)
-            wfrag[(size_t)pl * PSTRIDE + ((d * FPD + t) ^ (kSwizzle ? (pl >> 2) & 1 : 0))] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
+            wfrag_t[(size_t)pl * PSTRIDE + ((d * FPD + t) ^ (kSwizzle ? (pl >> 2) & 1 : 0))] = uint4_t{fr[4 * t], fr[4 * t + 1], fr[4 * t + 2], fr[4 * t + 3]};
         if constexpr (DW == 4) {
-            if (d == 0) *reinterpret_cast<float2*>(wsum + 2 * pl) = float2{__builtin_fmaf(F::kOffset, xs, cb), xs};
+            if (d == 0) *reinterpret_cast<float2*>(wsum_t + 2 * pl) = float2{__builtin_fmaf(F::kOffset, xs, cb), xs};
         } else {
-            wsum[it] = __builtin_fmaf(F::kOffset, xs, cb);   // one constant per dword: the job adds them per scale group
+            wsum_t[it] = __builtin_fmaf(F::kOffset, xs, cb);   // one constant per dword: the job adds them per scale group
         }
     }
     // ---- 5. scales into LDS (they were asked for after the activations and arrive after them) ------
@@ -413,7 +430,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     // second group go to token slots 4q + 2 and 4q + 3 instead, i.e. for those dwords A lanes 20q + 2
     // and 20q + 3 are the ones that read fragments.
     const int a_slot = n - 4 * q;                       // 0..3 for the lanes that ever read fragments
-    const bool a_valid = DW == 4 ? (a_slot == 0 || a_slot == 1) : (a_slot >= 0 && a_slot < 4);
+    const bool a_valid = DW == 4 && TOK == 1 ? (a_slot == 0 || a_slot == 1) : (a_slot >= 0 && a_slot < 4);
     const int a_half = a_slot & 1, a_second = a_slot >> 1;
     const int a_piece = 4 * a_half + q;                 // piece of the segment this lane feeds
     auto first_group_dwords = [](int piece_in_segment) {
@@ -423,9 +440,11 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
     };
     const int a_split = first_group_dwords(a_piece);
     const uint16_t* lds_s16 = reinterpret_cast<const uint16_t*>(lds_scales);
-    float y[NMAT];
+    float y[TOK][NMAT];
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m) y[m] = 0.0f;
+    for (int tk = 0; tk < TOK; ++tk)
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) y[tk][m] = 0.0f;
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         float4_t acc[NMAT];
@@ -441,14 +460,15 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
                 cd[m][0] = codes[m][i].x; cd[m][1] = codes[m][i].y; cd[m][2] = codes[m][i].z; cd[m][3] = codes[m][i].w;
             }
         }
-        const uint4_t* piece_frags = wfrag + (size_t)(i * 8 + a_piece) * PSTRIDE;
+        // (two tokens: slots 4q + 2 and 4q + 3 read the second token's fragments of the same pieces)
+        const uint4_t* piece_frags = wfrag + (TOK == 2 ? (size_t)a_second * kTokStride : (size_t)0) + (size_t)(i * 8 + a_piece) * PSTRIDE;
         if constexpr (DW * FPD <= 4 && !F::kDecode) {
             // few fragments per segment: all of them, and every transpose, are asked for before the first
             // MFMA, so the LDS round trips overlap each other (and, for the fragments, the weights' flight)
             uint4_t afr[DW][FPD];
 #pragma unroll
             for (int d = 0; d < DW; ++d) {
-                const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
+                const bool a_live = a_valid && (TOK == 2 || (d >= a_split) == (a_second == 1));
                 const uint4_t* pf = a_live ? piece_frags + (kSwizzle ? d ^ a_half : d) * FPD : wzero;
 #pragma unroll
                 for (int f = 0; f < FPD; ++f) afr[d][f] = pf[f];
@@ -470,7 +490,7 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         } else {
 #pragma unroll
         for (int d = 0; d < DW; ++d) {
-            const bool a_live = a_valid && ((d >= a_split) == (a_second == 1));
+            const bool a_live = a_valid && (TOK == 2 || (d >= a_split) == (a_second == 1));
             const uint4_t* pf = a_live ? piece_frags + (kSwizzle ? d ^ a_half : d) * FPD : wzero;
             uint4_t afr[FPD];
 #pragma unroll
@@ -489,17 +509,21 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         const bool piece_ok = piece < pieces;
         const int g = ((piece_ok ? piece : pieces - 1) * F::kPieceCols) >> gshift;
         if constexpr (DW == 4) {
-            const float2 cs = *reinterpret_cast<const float2*>(wsum + 2 * (i * 8 + 4 * hh + q));
+#pragma unroll
+            for (int tk = 0; tk < TOK; ++tk) {
+            const float2 cs = *reinterpret_cast<const float2*>(wsum + (size_t)tk * kTokStride * 4 + 2 * (i * 8 + 4 * hh + q));
 #pragma unroll
             for (int m = 0; m < NMAT; ++m) {
                 const int sidx = (m * PLANES) * (8 * gpr) + rn * gpr + g;
                 const float sv = F::kSemMul * ScaleT::widen(kDirectScales ? sdir[m][0][i] : lds_s16[sidx]);
-                const float dotp = hh ? acc[m].y : acc[m].x;   // token slot 4q + hh
-                y[m] = __builtin_fmaf(piece_ok ? sv : 0.0f, dotp - cs.x, y[m]);
+                // token slot 4q + hh (the second token: 4q + 2 + hh)
+                const float dotp = tk == 0 ? (hh ? acc[m].y : acc[m].x) : (hh ? acc[m].w : acc[m].z);
+                y[tk][m] = __builtin_fmaf(piece_ok ? sv : 0.0f, dotp - cs.x, y[tk][m]);
                 if (F::kHasBias) {
                     const float bv = ScaleT::widen(kDirectScales ? sdir[m][PLANES - 1][i] : lds_s16[sidx + 8 * gpr]);
-                    y[m] = __builtin_fmaf(piece_ok ? bv : 0.0f, cs.y, y[m]);
+                    y[tk][m] = __builtin_fmaf(piece_ok ? bv : 0.0f, cs.y, y[tk][m]);
                 }
+            }
             }
         } else {
             // the folded-out constants of the piece's dwords, per scale group
@@ -520,17 +544,19 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
                 const float s2 = F::kSemMul * ScaleT::widen(lds_s16[srow + g2]);
                 const float d1 = hh ? acc[m].y : acc[m].x;   // token slot 4q + hh: first group
                 const float d2 = hh ? acc[m].w : acc[m].z;   // token slot 4q + 2 + hh: second group
-                y[m] = __builtin_fmaf(piece_ok ? s1 : 0.0f, d1 - c_first, y[m]);
-                y[m] = __builtin_fmaf(piece_ok ? s2 : 0.0f, d2 - c_second, y[m]);
+                y[0][m] = __builtin_fmaf(piece_ok ? s1 : 0.0f, d1 - c_first, y[0][m]);
+                y[0][m] = __builtin_fmaf(piece_ok ? s2 : 0.0f, d2 - c_second, y[0][m]);
             }
         }
     }
     // the eight pieces of a segment: lanes rn + 8 * {0..7}
 #pragma unroll
+    for (int tk = 0; tk < TOK; ++tk)
+#pragma unroll
     for (int m = 0; m < NMAT; ++m) {
-        y[m] = dpp_add<0x128>(y[m]);   // row_ror:8: lane i of a row of sixteen takes lane i ^ 8
-        y[m] = swap_sum16(y[m]);
-        y[m] = swap_sum32(y[m]);
+        y[tk][m] = dpp_add<0x128>(y[tk][m]);   // row_ror:8: lane i of a row of sixteen takes lane i ^ 8
+        y[tk][m] = swap_sum16(y[tk][m]);
+        y[tk][m] = swap_sum32(y[tk][m]);
     }
 
     // ---- 7. the kc waves of the workgroup -----------------------------------------------------------
@@ -538,29 +564,39 @@ __device__ __forceinline__ void mm1_body(const MatPtrs (&mats)[NMAT], const uint
         float* red = reinterpret_cast<float*>(smem + (size_t)kc * wave_bytes + (size_t)NMAT * PLANES * 8 * gpr * 2);
         if (lane < 8) {
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m) red[(chunk * NMAT + m) * 8 + lane] = y[m];
+            for (int tk = 0; tk < TOK; ++tk)
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) red[((chunk * TOK + tk) * NMAT + m) * 8 + lane] = y[tk][m];
         }
         __syncthreads();
         if (chunk == 0) {
             // lane 8 k + r takes wave k's sum of row r (zero past the last wave; waves 8 .. 15 in a second
             // value), and the lanes r, r + 8, ... add up as the pieces of a segment did above
 #pragma unroll
+            for (int tk = 0; tk < TOK; ++tk)
+#pragma unroll
             for (int m = 0; m < NMAT; ++m) {
                 const int k = lane >> 3, r = lane & 7;
                 const int k0 = k < kc ? k : kc - 1, k1 = k + 8 < kc ? k + 8 : kc - 1;
-                const float v0 = red[(k0 * NMAT + m) * 8 + r], v1 = red[(k1 * NMAT + m) * 8 + r];
+                const float v0 = red[((k0 * TOK + tk) * NMAT + m) * 8 + r], v1 = red[((k1 * TOK + tk) * NMAT + m) * 8 + r];
                 float sum = (k < kc ? v0 : 0.0f) + (k + 8 < kc ? v1 : 0.0f);
                 sum = dpp_add<0x128>(sum);
                 sum = swap_sum16(sum);
-                y[m] = swap_sum32(sum);
+                y[tk][m] = swap_sum32(sum);
             }
         }
     }
     if constexpr (Epi::kTile) {
-        if (chunk == 0) epi.tile(token, row0, rows, lane, y);
+        if (chunk == 0) epi.tile(token, row0, rows, lane, y[0]);
     } else if (chunk == 0 && lane < 8 && row0 + lane < rows) {
-        if constexpr (Epi::kPrefetch) epi.finish(token, row0 + lane, y, res);
-        else epi(token, row0 + lane, y);
+        if constexpr (Epi::kPrefetch) epi.finish(token, row0 + lane, y[0], res[0]);
+        else epi(token, row0 + lane, y[0]);
+        if constexpr (TOK == 2) {
+            if (token + 1 < tokens) {
+                if constexpr (Epi::kPrefetch) epi.finish(token + 1, row0 + lane, y[1], res[1]);
+                else epi(token + 1, row0 + lane, y[1]);
+            }
+        }
     }
 }
 
@@ -659,6 +695,68 @@ struct EpiTileArgmax : EpiBase {
         EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
         mm1_body<F, ACT, F16, 2, NLV>(mats, X, rows, cols,                                   \
                                            F::row_stride((int)cols), 128, epi);  \
+    }
+
+// Two tokens per pass (binary and ternary codes): the argument lists above plus the number of tokens; grid row r
+// takes tokens 2r and 2r + 1.
+#define SMELT_SIGNED_MM1_KERNELS_T2(FN, FMT, T, ACT, NLV)                                         \
+    SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_t2_matvec_##T(                        \
+        const u8* C, const u16* S, const u16* X, u16* Y, u32 rows, u32 cols, u32 tokens) {        \
+        using namespace smelt;                                                                    \
+        using F = FMT<ACT>;                                                                       \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<F, ACT, F16, 1, NLV, EpiStore<ACT>, 0, 2>(mats, X, rows, cols, F::row_stride((int)cols), 128, epi, \
+                                                           NormScale{}, (int)tokens);             \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_t2_matvec_add_##T(                    \
+        const u8* C, const u16* S, const u16* X, u16* Y, const u16* res, u32 rows, u32 cols,      \
+        u32 tokens) {                                                                             \
+        using namespace smelt;                                                                    \
+        using F = FMT<ACT>;                                                                       \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        mm1_body<F, ACT, F16, 1, NLV, EpiAdd<ACT>, 0, 2>(mats, X, rows, cols, F::row_stride((int)cols), 128, epi, \
+                                                         NormScale{}, (int)tokens);               \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_signed_##FN##_mm1_nl##NLV##_t2_gate_up_swiglu_##T(                \
+        const u8* gC, const u16* gS, const u8* uC, const u16* uS, const u16* X, u16* Y, u32 rows, \
+        u32 cols, u32 tokens) {                                                                   \
+        using namespace smelt;                                                                    \
+        using F = FMT<ACT>;                                                                       \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        mm1_body<F, ACT, F16, 2, NLV, EpiSignedSwiglu<ACT>, 0, 2>(mats, X, rows, cols, F::row_stride((int)cols), 128, \
+                                                                  epi, NormScale{}, (int)tokens); \
+    }
+
+#define SMELT_TERAFF_MM1_KERNELS_T2(T, ACT, NLV)                                                  \
+    SMELT_MM1_KERNEL void smelt_teraff_mm1_nl##NLV##_t2_matvec_##T(                               \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* Y, u32 rows, u32 cols,          \
+        u32 tokens) {                                                                             \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiStore<ACT> epi{{}, Y, (int)rows};                                                      \
+        mm1_body<M1Ter2<ACT>, ACT, F16, 1, NLV, EpiStore<ACT>, 0, 2>(mats, X, rows, cols, cols / 4, 128, epi, \
+                                                                     NormScale{}, (int)tokens);   \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_teraff_mm1_nl##NLV##_t2_matvec_add_##T(                           \
+        const u8* C, const u16* S, const u16*, const u16* X, u16* Y, const u16* res, u32 rows,    \
+        u32 cols, u32 tokens) {                                                                   \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[1] = {{C, S, nullptr}};                                                \
+        EpiAdd<ACT> epi{{}, Y, res, (int)rows};                                                   \
+        mm1_body<M1Ter2<ACT>, ACT, F16, 1, NLV, EpiAdd<ACT>, 0, 2>(mats, X, rows, cols, cols / 4, 128, epi, \
+                                                                   NormScale{}, (int)tokens);     \
+    }                                                                                             \
+    SMELT_MM1_KERNEL void smelt_teraff_mm1_nl##NLV##_t2_gate_up_swiglu_##T(                       \
+        const u8* gC, const u16* gS, const u16*, const u8* uC, const u16* uS, const u16*,         \
+        const u16* X, u16* Y, u32 rows, u32 cols, u32 tokens) {                                   \
+        using namespace smelt;                                                                    \
+        const MatPtrs mats[2] = {{gC, gS, nullptr}, {uC, uS, nullptr}};                           \
+        EpiSignedSwiglu<ACT> epi{{}, Y, (int)rows};                                               \
+        mm1_body<M1Ter2<ACT>, ACT, F16, 2, NLV, EpiSignedSwiglu<ACT>, 0, 2>(mats, X, rows, cols, cols / 4, 128, \
+                                                                            epi, NormScale{}, (int)tokens); \
     }
 
 // Affine 4-bit: argument lists of the vector-ALU kernels of the same pipelines.

@@ -26,6 +26,17 @@ SMELT_MM1_EVERY_NL(bf16, smelt::BF16)
 SMELT_MM1_AFFINE_LONG(f16, smelt::F16)
 SMELT_MM1_AFFINE_LONG(bf16, smelt::BF16)
 
+// two tokens per pass: binary and ternary codes (the per-row and four-token forms from two tokens on)
+#define SMELT_MM1_T2(T, ACT, NLV)                                                                 \
+    SMELT_SIGNED_MM1_KERNELS_T2(binary, smelt::M1Bin, T, ACT, NLV)                                \
+    SMELT_SIGNED_MM1_KERNELS_T2(ternary, smelt::M1Ter2, T, ACT, NLV)                              \
+    SMELT_TERAFF_MM1_KERNELS_T2(T, ACT, NLV)
+#define SMELT_MM1_T2_EVERY_NL(T, ACT)                                                             \
+    SMELT_MM1_T2(T, ACT, 1) SMELT_MM1_T2(T, ACT, 2) SMELT_MM1_T2(T, ACT, 3)                       \
+    SMELT_MM1_T2(T, ACT, 4) SMELT_MM1_T2(T, ACT, 5) SMELT_MM1_T2(T, ACT, 6)
+SMELT_MM1_T2_EVERY_NL(f16, smelt::F16)
+SMELT_MM1_T2_EVERY_NL(bf16, smelt::BF16)
+
 #define SMELT_MM1_TRIT5(T, ACT)                                                                   \
     SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 1) SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 2) \
     SMELT_SIGNED_MM1_KERNELS(trit5, smelt::M1Trit5, T, ACT, 3)                                    \

@@ -119,7 +119,7 @@ uint32_t signed_row_stride(SignedFormat f, uint32_t cols) {
 }
 
 bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
-              bool force, Mm1Plan* out) {
+              bool force, Mm1Plan* out, uint32_t tokens_per_pass) {
     uint32_t row_stride, frags, nl_max, dw = 4;
     switch (layout) {
         case kCodesU4: row_stride = cols / 2; frags = 4; nl_max = 8; break;
@@ -130,6 +130,7 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
         default: return false;
     }
     if (rows == 0 || cols == 0 || row_stride % 16 != 0 || group < 32 || (group & (group - 1))) return false;
+    if (tokens_per_pass != 1 && (tokens_per_pass != 2 || dw != 4)) return false;
     if (layout != kCodesU4 && group != 128) return false;
     // No size threshold: measured on MI355X (cold, per launch in a graph) the single-pass kernel is the faster one
     // at every size once small matrices walk one segment per wave: affine 4-bit 64 x 1024 to 1024 x 1024 2.1-2.7 us
@@ -140,8 +141,9 @@ bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, u
     const uint32_t planes = layout == kCodesU4 ? 2 : 1;
     auto lds_of = [&](uint32_t kc, uint32_t nl) {
         // four-dword pieces are stored one fragment apart (LDS banks), except the four-fragment ones (swizzled instead)
-        const size_t wave = (size_t)nl * 8 * (dw == 4 ? (frags == 4 ? 4 : frags + 1) : frags) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4) + (size_t)frags * 16;
-        return kc * wave + (size_t)nmat * planes * 8 * gpr * 2 + (size_t)kc * nmat * 32 + (dw == 4 ? 0 : 512);   // + decode table
+        const size_t tok = tokens_per_pass;
+        const size_t wave = tok * ((size_t)nl * 8 * (dw == 4 ? (frags == 4 ? 4 : frags + 1) : frags) * 16 + (dw == 4 ? (size_t)nl * 8 * 8 : (size_t)nl * 8 * dw * 4)) + (size_t)frags * 16;
+        return kc * wave + (size_t)nmat * planes * 8 * gpr * 2 + (size_t)kc * nmat * tok * 32 + (dw == 4 ? 0 : 512);   // + decode table
     };
     Mm1Plan best;
     uint32_t best_waste = ~0u;

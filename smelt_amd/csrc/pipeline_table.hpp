@@ -153,8 +153,9 @@ struct Mm1Plan {
     uint32_t kc = 0, nl = 0;
     size_t lds = 0;
 };
+// (`tokens_per_pass` 2: the kernels that multiply two tokens per pass stage two sets of activation fragments)
 bool mm1_plan(CodeLayout layout, uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, size_t lds_limit,
-              bool force, Mm1Plan* out);
+              bool force, Mm1Plan* out, uint32_t tokens_per_pass = 1);
 
 // Launch plan of the streaming skinny qmm: workgroups of `kc` waves over 16 * rt rows each, 16 tokens
 // per grid row; wave c takes the pairs of scale groups c, c + kc, ...  False when the shape has no

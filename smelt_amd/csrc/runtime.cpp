@@ -44,6 +44,7 @@ struct Pipeline {
     hipFunction_t fn = nullptr;
     hipFunction_t fn_single = nullptr;  // used when the record's batch argument is 1
     hipFunction_t fn_mm1[kMm1MaxSegments + 1] = {};               // single-pass matrix-core matvec, by segments per wave
+    hipFunction_t fn_mm1_t2[kMm1MaxSegments + 1] = {};            // ... two tokens per pass (binary and ternary codes)
     hipFunction_t fn_qmt[5][5][3] = {};                           // token-tile qmm, by row tiles and token blocks per wave and waves along K
     hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
@@ -1082,7 +1083,8 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     };
     const bool mm1_b4 = p->res.family == kFamSignedB4 || p->res.family == kFamSignedGateUpB4;
     // (the signed single-token families take their token from the grid row: a record with several rows keeps them)
-    const bool mm1_per_row = p->res.family == kFamSignedMatvec || p->res.family == kFamSignedAdd || p->res.family == kFamSignedGateUp;
+    const bool mm1_per_row = p->res.family == kFamSignedMatvec || p->res.family == kFamSignedAdd || p->res.family == kFamSignedGateUp ||
+                             p->res.family == kFamTerAffMatvec || p->res.family == kFamTerAffAdd || p->res.family == kFamTerAffGateUp;
     // the per-token small-batch forms of the affine matvec and gate+up (W S B X Y batch | rows cols group tile): a few
     // tokens of a small matrix are launch-bound, and the single-token kernel with a grid row per token is the shorter
     // launch while tokens x weights stay below about 20M (cold, streaming kernel against a grid row per token:
@@ -1130,9 +1132,9 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             case kFamAffineGateUpBatched: tokens = U(8); rows = U(9); cols = U(10); group = U(11); ro = 7; break;
             case kFamBinaryPackedBank: rows = U(5) + U(6); cols = U(7); ro = 3; break;
             case kFamBinaryPackedBank4: rows = U(7) + U(8) + U(9) + U(10); cols = U(11); ro = 3; break;
-            case kFamTerAffMatvec: rows = U(5); cols = U(6); ro = 4; break;
-            case kFamTerAffAdd: rows = U(6); cols = U(7); ro = 4; break;
-            case kFamTerAffGateUp: rows = U(8); cols = U(9); ro = 7; break;
+            case kFamTerAffMatvec: rows = U(5); cols = U(6); ro = 4; tokens = L.grid[1]; break;
+            case kFamTerAffAdd: rows = U(6); cols = U(7); ro = 4; tokens = L.grid[1]; break;
+            case kFamTerAffGateUp: rows = U(8); cols = U(9); ro = 7; tokens = L.grid[1]; break;
             case kFamTerAffBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); ro = 4; break;
             default: break;
         }
@@ -1142,7 +1144,18 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             p->fn_mm1[plan.nl]) {
             fn = p->fn_mm1[plan.nl];
             L.grid[0] = (rows + 7) / 8; L.grid[1] = tokens; L.grid[2] = 1;
-            if (mm1_b4) L.args.count -= 1;
+            // binary and ternary codes from two tokens on: two tokens per pass (the weights are unpacked and multiplied
+            // once for both; the token count is the kernels' last argument: the four-token forms bring it along)
+            Mm1Plan plan2;
+            const bool two = tokens >= 2 && (mm1_b4 || mm1_per_row) &&
+                             mm1_plan((CodeLayout)p->res.mm1_layout, rows, cols, group, p->res.mm1_nmat, ctx->lds_limit,
+                                      ctx->matvec_engine == SMELT_HIP_MATVEC_MATRIX_CORE, &plan2, 2) && p->fn_mm1_t2[plan2.nl];
+            if (two) {
+                plan = plan2;
+                fn = p->fn_mm1_t2[plan.nl];
+                L.grid[1] = (tokens + 1) / 2;
+                if (!mm1_b4) { Arg a; a.kind = 'U'; a.value = tokens; L.args.push_back(a); }
+            } else if (mm1_b4) L.args.count -= 1;
             if (mm1_small_batch) {
                 // W S B X Y batch rows cols group tile -> W S B X Y rows cols group
                 const size_t o = mm1_pair_batch ? 8 : 5;
@@ -1561,6 +1574,9 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
             if (!p.res.mm1_prefix.empty())
                 for (uint32_t nl = 1; nl <= kMm1MaxSegments; ++nl)
                     (void)find(&p.fn_mm1[nl], p.res.mm1_prefix + "nl" + std::to_string(nl) + "_" + p.res.mm1_tail);
+            if (!p.res.mm1_prefix.empty() && (p.res.mm1_layout == (int)kCodesBinary1 || p.res.mm1_layout == (int)kCodesTernary2))
+                for (uint32_t nl = 1; nl <= kMm1MaxSegments; ++nl)
+                    (void)find(&p.fn_mm1_t2[nl], p.res.mm1_prefix + "nl" + std::to_string(nl) + "_t2_" + p.res.mm1_tail);
             if (!p.res.qms_tail.empty()) {
                 // the variants qmt_plan can return: (row tiles, token blocks, waves along K), one matrix per wave or not
                 static const struct { uint32_t rt, tb, kw; bool per_wave; } kQmtVariants[] = {

@@ -340,12 +340,14 @@ def test_operands_off_a_16_byte_boundary_keep_the_vector_kernel(ctx, vec):
 
 @pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary"), (fx.TRIT5, "trit5")])
 @pytest.mark.parametrize("kind", ["matvec", "gate_up"])
-def test_signed_four_token_forms_run_one_grid_row_per_token(fmt, name, kind):
+@pytest.mark.parametrize("batch", [6, 5, 2])
+def test_signed_four_token_forms_run_one_grid_row_per_token(fmt, name, kind, batch):
     """`*_batched_b4` records (four tokens per grid row) and per-token records with several grid rows take the
-    single-pass kernel under the default engine, one grid row per token: each token's row is the single-token
-    kernel's bits and, for the plain matvec, the oracle's values to the usual bar.  Ragged batch (6 = 4 + 2) and
-    ragged rows."""
-    rows, cols, batch, dtype = 1003, 5120, 6, fx.BF16
+    single-pass kernel under the default engine: two tokens per pass for binary and ternary codes (the second token
+    in the MFMA's free token slots), one grid row per token for five-digit bytes.  Each token's row is the
+    single-token kernel's bits and, for the plain matvec, the oracle's values to the usual bar.  Ragged batches
+    (6 = 4 + 2; 5: the last pass holds one token) and ragged rows."""
+    rows, cols, dtype = 1003, 5120, fx.BF16
     c = rt.Context()
     try:
         mats = []
@@ -363,5 +365,39 @@ def test_signed_four_token_forms_run_one_grid_row_per_token(fmt, name, kind):
         if kind == "matvec":
             ref = so.signed_matvec(fmt, *mats[0], fx.from_bits(x, dtype), rows, cols, cols, 128)
             gh.check_outputs(y4, ref, dtype, f"four-token {name}")
+    finally:
+        c.close()
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_ternary_affine_rows_over_several_tokens(dtype):
+    """`signed_ternary_affine_matvec_g128_rows8` with one grid row per token (what the reference launches below six
+    tokens): two tokens per pass on the single-pass kernel; every row is the one-token launch's bits."""
+    rows, cols, batch = 777, 2560, 5
+    c = rt.Context()
+    try:
+        codes = fx.synth_signed_codes(fx.TERNARY2, rows, cols, config=3, tensor=5)
+        scales = fx.synth_signed_scales(rows, cols, config=3, tensor=5)
+        packed = fx.pack_signed_np(codes, fx.TERNARY2)
+        x = fx.synth_activation(batch, cols, dtype, config=3, tensor=15)
+        wf = gh.WeightFile()
+        oc, os_ = wf.add(packed), wf.add(scales)
+        c.upload_weights(0, wf.image())
+        pipe = c.pipeline("signed_ternary_affine_matvec_g128_rows8" + gh.t_suffix(dtype))
+
+        def run(xb):
+            n = xb.shape[0]
+            c.put(gh.X_SLOT, xb)
+            c.alloc(gh.Y_SLOT, n * rows * 2)
+            bufs = [(0, 0, oc), (0, 1, os_), (0, 2, os_), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+            assert c.encode_decode(rt.make_record(pipe, bufs, [(5, rows), (6, cols)], ((rows + 7) // 8, n, 1), (256, 1, 1))) == 1
+            c.wait()
+            return c.read(gh.Y_SLOT, np.uint16, n * rows).reshape(n, rows)
+
+        y = run(x)
+        for b in range(batch):
+            assert np.array_equal(y[b], run(x[b:b + 1])[0]), b
+        ref = so.signed_matvec(so.TERNARY2, packed, scales, fx.from_bits(x, dtype), rows, cols, cols, 128)
+        gh.check_outputs(y, ref, dtype, "ternary affine rows, five tokens")
     finally:
         c.close()
