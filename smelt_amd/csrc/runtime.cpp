@@ -1082,7 +1082,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         return true;
     };
     const bool mm1_b4 = p->res.family == kFamSignedB4 || p->res.family == kFamSignedGateUpB4;
-    // (the signed single-token families take their token from the grid row: a record with several rows keeps them)
+    // (the single-token families of the binary and ternary codes: with several grid rows, two tokens per pass)
     const bool mm1_per_row = p->res.family == kFamSignedMatvec || p->res.family == kFamSignedAdd || p->res.family == kFamSignedGateUp ||
                              p->res.family == kFamTerAffMatvec || p->res.family == kFamTerAffAdd || p->res.family == kFamTerAffGateUp;
     // the per-token small-batch forms of the affine matvec and gate+up (W S B X Y batch | rows cols group tile): a few
@@ -1101,10 +1101,12 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
         mm1_small_batch = batch >= 1 && batch <= 16 && weights * batch <= ((uint64_t)20 << 20);
     }
     if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && p->res.family != kFamAffineArgmax &&
-        ((L.grid[1] == 1 && !mm1_batch_family) || mm1_b4 || mm1_per_row || mm1_small_batch)) {
+        (!mm1_batch_family || mm1_small_batch)) {
         // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
         // arguments, its own launch geometry (one workgroup per eight rows)
-        uint32_t rows = 0, cols = 0, group = 128, tokens = 1;
+        // (every single-token kernel takes its token from the grid row: a record with several rows is one launch per token
+        // of the same kernel, each row the one-token launch's bits)
+        uint32_t rows = 0, cols = 0, group = 128, tokens = L.grid[1];
         size_t ro = 0;   // leading read-only operands (codes, scales[, biases], ..., x)
         size_t lead = 0; // ... behind this many leading arguments that are not fetched 16 bytes at a time
         auto U = [&](size_t i) { return L.args[i].value; };
@@ -1121,9 +1123,9 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             case kFamAffineAdd: rows = U(6); cols = U(7); group = U(8); ro = 4; break;
             case kFamAffineGateUp: rows = U(8); cols = U(9); group = U(10); ro = 7; break;
             case kFamAffineBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); group = U(13); ro = 4; break;
-            case kFamSignedMatvec: rows = U(4); cols = U(5); ro = 3; tokens = L.grid[1]; break;
-            case kFamSignedAdd: rows = U(5); cols = U(6); ro = 3; tokens = L.grid[1]; break;
-            case kFamSignedGateUp: rows = U(6); cols = U(7); ro = 5; tokens = L.grid[1]; break;
+            case kFamSignedMatvec: rows = U(4); cols = U(5); ro = 3; break;
+            case kFamSignedAdd: rows = U(5); cols = U(6); ro = 3; break;
+            case kFamSignedGateUp: rows = U(6); cols = U(7); ro = 5; break;
             // four tokens per grid row in the record: one grid row per token here (the kernel takes its token from
             // blockIdx.y; the trailing batch argument is dropped from the argument block)
             case kFamSignedB4: rows = U(4); cols = U(5); tokens = U(6); ro = 3; break;
@@ -1132,9 +1134,9 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             case kFamAffineGateUpBatched: tokens = U(8); rows = U(9); cols = U(10); group = U(11); ro = 7; break;
             case kFamBinaryPackedBank: rows = U(5) + U(6); cols = U(7); ro = 3; break;
             case kFamBinaryPackedBank4: rows = U(7) + U(8) + U(9) + U(10); cols = U(11); ro = 3; break;
-            case kFamTerAffMatvec: rows = U(5); cols = U(6); ro = 4; tokens = L.grid[1]; break;
-            case kFamTerAffAdd: rows = U(6); cols = U(7); ro = 4; tokens = L.grid[1]; break;
-            case kFamTerAffGateUp: rows = U(8); cols = U(9); ro = 7; tokens = L.grid[1]; break;
+            case kFamTerAffMatvec: rows = U(5); cols = U(6); ro = 4; break;
+            case kFamTerAffAdd: rows = U(6); cols = U(7); ro = 4; break;
+            case kFamTerAffGateUp: rows = U(8); cols = U(9); ro = 7; break;
             case kFamTerAffBank4: rows = U(8) + U(9) + U(10) + U(11); cols = U(12); ro = 4; break;
             default: break;
         }
