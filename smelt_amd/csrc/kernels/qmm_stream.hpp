@@ -462,6 +462,200 @@ struct QsGeglu {
         qms_body<ACT, SC, 2, 1, XRV, QsGeglu<ACT>, true>(w, s, b, X, batch, rows, cols, group, QsGeglu<ACT>{Y}); \
     }
 
+// ---- ternary codes (two bits, groups of 128 columns): the streaming form of the ternary qmm ------------
+// The skeleton of qms_body with a dequantised fp16 weight operand in place of exact codes and scale FMAs: the
+// value of an element is the token-slab kernel's (signed_quant_precise.metal:407-439), rounded to fp16 once:
+// the two-bit field keeps its place inside its byte, byte lane k multiplies it by its own subscale
+// fp16(scale / 4^k), and -bias (a plane of its own) is added.  Activations are multiplied as fp16 (bf16 rows are
+// converted at staging, as that kernel does).  A wave owns sixteen rows and walks 128-column steps (one scale
+// group each); the waves of a workgroup split K; tokens are the A operand in memory order, so lane (n, q) takes
+// the four bytes of row n that hold columns 16 q .. 16 q + 15 of a 64-column half: byte j is registers 2 j
+// (codes in byte lanes 0 and 1) and 2 j + 1 (lanes 2 and 3) of the two MFMAs' B operands.
+namespace smelt {
+
+typedef _Float16 half2v_t __attribute__((ext_vector_type(2)));
+constexpr int kQtsWStride = 40;        // bytes per staged weight row of a step (32 + 8 of padding)
+__host__ __device__ constexpr size_t qts_scale_lds_bytes(int groups) { return (size_t)16 * (groups + 1) * 4; }
+__host__ __device__ constexpr size_t qts_wave_lds_bytes(int token_rows) {
+    return (size_t)token_rows * kQsXStride + 16 * kQtsWStride < 1024 ? (size_t)1024 : (size_t)token_rows * kQsXStride + 16 * kQtsWStride;
+}
+
+template <class ActT, int XR>
+__device__ __forceinline__ void qts_body(const uint8_t* __restrict__ W, const uint16_t* __restrict__ S,
+                                         const uint16_t* __restrict__ B, const uint16_t* __restrict__ X,
+                                         uint16_t* __restrict__ Y, int batch, int rows, int cols) {
+    using E = Elem16<F16>;
+    static_assert(XR == 2 || XR == 4, "a pass stages eight or sixteen token rows");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int chunk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int kc = blockDim.x / kWave;
+    const int n = lane & 15, q = lane >> 4;
+    const int gt = cols >> 7;          // scale groups per row = steps
+    const int rs = cols >> 2;          // bytes per packed row
+    const int row0 = blockIdx.x * 16;
+    const int m0 = blockIdx.y * kQsTokens;
+    const int last_tok = (batch < m0 + kQsTokens ? batch : m0 + kQsTokens) - 1;
+
+    // ---- (scale, -bias) of the sixteen rows and every group, plus one zero column: four or eight groups per thread
+    const bool half_runs = (gt & 7) != 0;
+    const int run_len = half_runs ? 4 : 8;
+    const int runs = half_runs ? gt >> 2 : gt >> 3;
+    const int items = 16 * runs;
+    uint32_t* lds_sb = reinterpret_cast<uint32_t*>(smem);
+    const int sstride = gt + 1;
+    struct ScaleRun { uint4_t s, b; int at; };
+    auto load_scales = [&](int item) {
+        if (item > items - 1) item = items - 1;
+        const int srow = item / runs, run = item - srow * runs;
+        int r = row0 + srow;
+        if (r > rows - 1) r = rows - 1;
+        ScaleRun out;
+        if (half_runs) {
+            const uint2_t s2 = *reinterpret_cast<const uint2_t*>(S + (size_t)r * gt + 4 * run);
+            const uint2_t b2 = *reinterpret_cast<const uint2_t*>(B + (size_t)r * gt + 4 * run);
+            out.s = uint4_t{s2.x, s2.y, 0u, 0u};
+            out.b = uint4_t{b2.x, b2.y, 0u, 0u};
+        } else {
+            out.s = *reinterpret_cast<const uint4_t*>(S + (size_t)r * gt + 8 * run);
+            out.b = *reinterpret_cast<const uint4_t*>(B + (size_t)r * gt + 8 * run);
+        }
+        out.at = srow * sstride + run_len * run;
+        return out;
+    };
+    auto store_scales = [&](const ScaleRun& v) {
+        const uint32_t sd[4] = {v.s.x, v.s.y, v.s.z, v.s.w}, bd[4] = {v.b.x, v.b.y, v.b.z, v.b.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t sc = e & 1 ? sd[e >> 1] >> 16 : sd[e >> 1] & 0xFFFFu;
+            const uint32_t bi = e & 1 ? bd[e >> 1] >> 16 : bd[e >> 1] & 0xFFFFu;
+            if (e < run_len) lds_sb[v.at + e] = sc | ((bi ^ 0x8000u) << 16);   // (scale, -bias) as fp16
+        }
+    };
+    const ScaleRun first_run = load_scales((int)threadIdx.x);
+
+    unsigned char* stage = smem + qts_scale_lds_bytes(gt) + (size_t)chunk * qts_wave_lds_bytes(4 * XR);
+    unsigned char* stage_w = stage + 4 * XR * kQsXStride;
+    const int x_tok = lane >> 4, x_piece = lane & 15;
+    const int w_row = lane >> 2, w_piece = lane & 3;
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    struct Step { uint4_t x[XR]; uint2_t w; };
+    const uint16_t* x_base[XR];
+#pragma unroll
+    for (int r = 0; r < XR; ++r) {
+        int tok = m0 + 4 * r + x_tok;
+        if (tok > last_tok) tok = last_tok;
+        x_base[r] = X + (size_t)tok * cols + 8 * x_piece;
+    }
+    const uint8_t* w_base;
+    {
+        int r = row0 + w_row;
+        if (r > rows - 1) r = rows - 1;
+        w_base = W + (size_t)r * rs + 8 * w_piece;
+    }
+    auto issue = [&](Step& st, int step) {
+        if (step > gt - 1) step = gt - 1;   // past the end: the last step again, under a zero scale and bias
+#pragma unroll
+        for (int r = 0; r < XR; ++r) st.x[r] = *reinterpret_cast<const uint4_t*>(x_base[r] + 128 * step);
+        st.w = *reinterpret_cast<const uint2_t*>(w_base + 32 * step);
+    };
+    auto consume = [&](const Step& st, int step) {
+#pragma unroll
+        for (int r = 0; r < XR; ++r) {
+            uint4_t v = st.x[r];
+            if (!ActT::kIsF16) {
+                uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    p[i] = (uint32_t)ActT::to_f16_bits((uint16_t)(p[i] & 0xFFFFu)) | ((uint32_t)ActT::to_f16_bits((uint16_t)(p[i] >> 16)) << 16);
+                v = uint4_t{p[0], p[1], p[2], p[3]};
+            }
+            *reinterpret_cast<uint4_t*>(stage + (4 * r + x_tok) * kQsXStride + 16 * x_piece) = v;
+        }
+        *reinterpret_cast<uint2_t*>(stage_w + w_row * kQtsWStride + 8 * w_piece) = st.w;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int gi = step < gt ? step : gt;   // the zero column
+        const uint32_t sb = lds_sb[n * sstride + gi];
+        const _Float16 sc = __builtin_bit_cast(_Float16, (uint16_t)(sb & 0xFFFFu));
+        const _Float16 nb = __builtin_bit_cast(_Float16, (uint16_t)(sb >> 16));
+        const half2v_t s01 = half2v_t{sc, sc} * half2v_t{(_Float16)1.0f, (_Float16)0.25f};
+        const half2v_t s23 = half2v_t{sc, sc} * half2v_t{(_Float16)0.0625f, (_Float16)0.015625f};
+        const half2v_t nb2 = {nb, nb};
+        const half2v_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+        const int xrow = XR == 4 ? n : (n & 7);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const unsigned char* xr = stage + xrow * kQsXStride + 128 * e + 32 * q;
+            const uint4_t a0 = *reinterpret_cast<const uint4_t*>(xr);
+            const uint4_t a1 = *reinterpret_cast<const uint4_t*>(xr + 16);
+            const uint32_t c = *reinterpret_cast<const uint32_t*>(stage_w + n * kQtsWStride + 16 * e + 4 * q);
+            uint32_t bw[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // byte j in both half-words, then its lanes 0|1 and 2|3 as (1024 + field) pairs
+                const uint32_t rep = __builtin_amdgcn_perm(c, c, 0x0c000c00u | (uint32_t)j | ((uint32_t)j << 16));
+                const half2v_t f01 = __builtin_bit_cast(half2v_t, and_or(rep, 0x000C0003u, 0x64006400u)) - k1024;
+                const half2v_t f23 = __builtin_bit_cast(half2v_t, and_or(rep, 0x00C00030u, 0x64006400u)) - k1024;
+                bw[2 * j] = __builtin_bit_cast(uint32_t, s01 * f01 + nb2);
+                bw[2 * j + 1] = __builtin_bit_cast(uint32_t, s23 * f23 + nb2);
+            }
+            acc = E::mfma(a0, uint4_t{bw[0], bw[1], bw[2], bw[3]}, acc);
+            acc = E::mfma(a1, uint4_t{bw[4], bw[5], bw[6], bw[7]}, acc);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    Step s0, s1;
+    int step = chunk;
+    issue(s0, step);
+    issue(s1, step + kc);
+    store_scales(first_run);
+    for (int base = (int)blockDim.x; base < items; base += (int)blockDim.x) store_scales(load_scales(base + (int)threadIdx.x));
+    if (threadIdx.x < 16) lds_sb[threadIdx.x * sstride + gt] = 0u;
+    __syncthreads();
+    for (; step < gt; step += 2 * kc) {
+        consume(s0, step);
+        issue(s0, step + 2 * kc);
+        consume(s1, step + kc);
+        issue(s1, step + 3 * kc);
+    }
+
+    // ---- the kc waves of the workgroup, in wave order ------------------------------------------------
+    reinterpret_cast<float4_t*>(stage)[lane] = acc;
+    __syncthreads();
+    if (chunk == 0) {
+        const unsigned char* first = smem + qts_scale_lds_bytes(gt);
+        float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int c = 0; c < kc; ++c) {
+            const float4_t part = reinterpret_cast<const float4_t*>(first + (size_t)c * qts_wave_lds_bytes(4 * XR))[lane];
+            sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+        }
+        const int r = row0 + n;
+        if (r < rows) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int tok = m0 + 4 * q + v;
+                if (tok <= last_tok) Y[(size_t)tok * rows + r] = ActT::narrow(v == 0 ? sum.x : (v == 1 ? sum.y : (v == 2 ? sum.z : sum.w)));
+            }
+        }
+    }
+}
+
+}  // namespace smelt
+
+// Argument list of the ternary token-slab qmm (the bias plane is the scale plane bound a second time).
+#define SMELT_TERNARY_QMS(T, ACT, XRV)                                                              \
+    SMELT_QMS_KERNEL void smelt_ternary_qms_x##XRV##_##T(                                           \
+        const uint8_t* C, const uint16_t* S, const uint16_t* B, const uint16_t* X, uint16_t* Y,    \
+        uint32_t rows, uint32_t cols, uint32_t batch) {                                            \
+        smelt::qts_body<ACT, XRV>(C, S, B, X, Y, (int)batch, (int)rows, (int)cols);                \
+    }
+
 // ---- token-tile form: prefill chunks ------------------------------------------------------------
 // The same arithmetic for many tokens.  A workgroup of four waves (two along the rows, two along the
 // tokens) owns 32 * RT weight rows times 32 * TB tokens and walks K one pair of scale groups at a time.

@@ -430,6 +430,28 @@ bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
     return out->lds <= lds_limit;
 }
 
+bool qts_plan(uint32_t rows, uint32_t cols, uint32_t batch, size_t lds_limit, QmsPlan* out) {
+    // scale rows are staged four or eight groups at a time: rows of a multiple of 512 columns
+    if (rows == 0 || cols == 0 || cols % 512 != 0 || batch == 0) return false;
+    const uint32_t gt = cols / 128;
+    uint32_t kc = (gt + 3) / 4;          // about four steps per wave, at most twelve waves, none idle
+    if (kc < 1) kc = 1;
+    if (kc > 12) kc = 12;
+    uint32_t steps = (gt + kc - 1) / kc;
+    kc = (gt + steps - 1) / steps;
+    const uint32_t tiles16 = (rows + 15) / 16;
+    uint32_t want = (3500 + tiles16 / 2) / tiles16;   // matrices of many rows: fewer waves, longer walks (as qms_plan)
+    if (want < 4) want = 4;
+    for (uint32_t k = want; k < kc; ++k)
+        if (gt % k == 0) { kc = k; break; }
+    const size_t token_rows = batch > 8 ? 16 : 8;
+    size_t wave = token_rows * 272 + 16 * 40;
+    if (wave < 1024) wave = 1024;
+    out->rt = 1; out->kc = kc;
+    out->lds = (size_t)16 * (gt + 1) * 4 + kc * wave;
+    return out->lds <= lds_limit;
+}
+
 ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act,
                                size_t lds_limit, ResolvedPipeline* out, std::string* why) {
     const ResolveStatus st = resolve_pipeline_entry(entry_in, default_act, lds_limit, out, why);

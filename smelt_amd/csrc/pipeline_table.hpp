@@ -167,6 +167,10 @@ struct QmsPlan {
 };
 bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint32_t batch, uint32_t compute_units,
               size_t lds_limit, QmsPlan* out);
+// Launch plan of the streaming ternary qmm (two-bit codes, groups of 128 columns): workgroups of `kc` waves over
+// sixteen rows, sixteen tokens per grid row, wave c takes the 128-column steps c, c + kc, ...
+bool qts_plan(uint32_t rows, uint32_t cols, uint32_t batch, size_t lds_limit, QmsPlan* out);
+
 
 // Launch plan of the token-tile qmm: workgroups of 4 * kw waves over 32 * rt rows (per matrix) and
 // 32 * tb tokens.  False when the shape has no such kernel or too few tokens to pay for the tiles.

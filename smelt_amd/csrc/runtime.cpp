@@ -49,6 +49,7 @@ struct Pipeline {
     hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
     hipFunction_t fn_qms_g32[2] = {};                             // ... for groups of 32 columns
+    hipFunction_t fn_tqs[2] = {};                                 // streaming ternary qmm, eight / sixteen staged token rows
     hipFunction_t fn_norm_rows = nullptr;                         // norm-scale qmm: the normalised rows, written once
     hipFunction_t fn_logits_keys = nullptr;                       // lm_head over several tokens: partial argmax keys from stored logits
     ResolvedPipeline res;
@@ -1342,6 +1343,22 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             qms_routed = true;
         }
     }
+    if (p->res.family == kFamTerAffQmm && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && aligned16(4) && whole_pieces(4)) {
+        // ternary qmm (C S S2 X Y rows cols batch): the streaming kernel, same arguments, its own geometry, up to 128
+        // tokens (256 for matrices of fewer than 8192 rows, which leave the token-slab kernel short of slabs).  Cold,
+        // streaming against token slabs at 8 / 32 / 128 / 256 / 512 tokens: 17408 x 5120 15 / 33 / 101 / 183 / 341 us against
+        // 57 / 62 / 104 / 168 / 291; 5120 x 17408 20 / 35 / 107 / 194 / 367 against 156 / 203 / 208 / 253 / 328; 4096 x 4096
+        // 5.2 / 9.0 / 23 / 40 / 76 against 37 / 41 / 41 / 48 / 73.
+        const uint32_t rows = L.args[5].value, cols = L.args[6].value, batch = L.args[7].value;
+        QmsPlan plan;
+        if (batch <= (rows < 8192 ? 256u : 128u) && qts_plan(rows, cols, batch, ctx->lds_limit, &plan) && p->fn_tqs[batch > 8]) {
+            fn = p->fn_tqs[batch > 8];
+            L.grid[0] = (rows + 15) / 16; L.grid[1] = (batch + 15) / 16; L.grid[2] = 1;
+            L.block[0] = 64 * plan.kc; L.block[1] = 1; L.block[2] = 1;
+            L.lds = plan.lds;
+            routed = true;
+        }
+    }
     if (!qms_routed && (L.ws_partial_need > ws.partial_bytes || L.ws_counter_need > ws.counter_bytes))
         return fail(ctx, SMELT_HIP_ERR_UNSUPPORTED_GEOMETRY,
                     "pipeline '" + p->entry + "': split-K partials (" + std::to_string(L.ws_partial_need) + " bytes, " +
@@ -1590,6 +1607,9 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
                 }
             }
             if (p.res.family == kFamAffineArgmax) (void)find(&p.fn_logits_keys, "smelt_logits_argmax_partials");
+            if (p.res.family == kFamTerAffQmm)
+                for (uint32_t wide = 0; wide < 2; ++wide)
+                    (void)find(&p.fn_tqs[wide], std::string("smelt_ternary_qms_") + (wide ? "x4_" : "x2_") + (p.res.act == kActBF16 ? "bf16" : "f16"));
             if (p.res.family == kFamNormScaleAffineQmm || p.res.family == kFamNormScaleAffineQmmGateUp || p.res.family == kFamNormScaleAffineBatched)
                 (void)find(&p.fn_norm_rows, std::string("smelt_norm_scale_rows_") + (p.res.act == kActBF16 ? "bf16" : "f16"));
             if (!p.res.qms_tail.empty())

@@ -461,3 +461,75 @@ def test_fused_argmax_at_the_largest_vocabulary(ctx):
         bufs = [(0, i, o) for i, o in enumerate(offs)] + [(gh.X_SLOT, 3, 0), (gh.AUX_SLOT, 4, 0)]
         ctx.encode_decode(rt.make_record(ctx.pipeline(f"affine_matvec_argmax_c{cols}_r{rows + 8}_g{group}_batched"), bufs,
                                          [(5, 1), (6, 0.0)], (grid_w, 1, 1), (256, 1, 1)))
+
+
+@pytest.fixture(scope="module")
+def auto_ctx():
+    c = rt.Context()            # default engine: the ternary qmm record takes the streaming kernel up to 64 tokens
+    yield c
+    c.close()
+
+
+def test_ternary_qmm_streaming_kernel_reproduces_the_golden_bits_too(auto_ctx):
+    test_ternary_qmm_reproduces_mlx_golden_bits_and_byte_lane_subscales(auto_ctx)
+    test_ternary_qmm_matches_per_row_matvec_and_oracle(auto_ctx)
+
+
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+@pytest.mark.parametrize("shape", [(1003, 5120, 14), (40, 512, 6), (200, 17408, 33), (2050, 1536, 64), (96, 1024, 9)])
+def test_ternary_qmm_streaming_kernel_shapes(ctx, auto_ctx, dtype, shape):
+    """The streaming ternary qmm against the oracle's per-element fp16 dequantisation and against the token-slab
+    kernel (one output step apart at most: the two add up a row in different orders): ragged rows, one to four
+    16-token passes, eight and sixteen staged token rows, rows of four, twelve, forty and 136 groups, separate
+    bias plane, bf16 rows (converted to fp16 as in the token-slab kernel)."""
+    rows, cols, batch = shape
+    codes = fx.synth_signed_codes(fx.TERNARY2, rows, cols, config=3, tensor=rows % 7)
+    scales = fx.synth_signed_scales(rows, cols, config=3, tensor=rows % 7)
+    bias_scales = np.roll(scales, 3, axis=0)
+    packed = fx.pack_signed_np(codes, fx.TERNARY2)
+    x = fx.synth_activation(batch, cols, dtype, config=3, tensor=batch)
+    out = {}
+    for name, c in (("stream", auto_ctx), ("slab", ctx)):
+        wf = gh.WeightFile()
+        oc, os_, ob = wf.add(packed), wf.add(scales), wf.add(bias_scales)
+        c.upload_weights(0, wf.image())
+        c.put(gh.X_SLOT, x)
+        c.alloc(gh.Y_SLOT, batch * rows * 2)
+        rec = rt.make_record(c.pipeline("signed_ternary_affine_qmm_g128_bm32_bn32_bk32" + gh.t_suffix(dtype)),
+                             [(0, 0, oc), (0, 1, os_), (0, 2, ob), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)],
+                             [(5, rows), (6, cols), (7, batch)], ((rows + 63) // 64, (batch + 31) // 32, 1), (256, 1, 1))
+        assert c.encode_decode(rec) == 1
+        c.wait()
+        out[name] = c.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+        assert np.array_equal(out[name], (c.encode_decode(rec), c.wait(), c.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows))[2])
+    gh.check_steps(out["stream"], out["slab"], dtype, f"ternary qmm, streaming against token-slab {shape}", max_steps=1, min_exact=0.9)
+    if dtype == fx.F16:
+        ref = so.ternary_affine_qmm(packed, scales, x, rows, cols, bias_scales=bias_scales)
+        gh.check_outputs(out["stream"], ref, dtype, f"ternary qmm streaming {shape}")
+
+
+def test_ternary_qmm_streaming_kernel_is_bit_exact_where_the_sums_are(auto_ctx):
+    """The MLX fixture of the golden test at 512 and 1024 columns (the streaming kernel takes multiples of 512; the
+    golden shape itself has 256 and keeps the token-slab kernel): every partial sum is exact, so the bits must be the
+    oracle's, with ordinary scales, with scales whose quarter, sixteenth and sixty-fourth round in the fp16
+    subnormal range, and with a separate bias plane."""
+    case = fx.golden_vectors()["ternary_qmm_mlx_m14"]
+    small = ["1b95", "1797", "1b93", "17ff", "1a01"]
+    for cols, rows, batch in ((512, 24, 14), (1024, 40, 37)):
+        for scale_bits, separate_bias in ((case["scale_bits"], False), (small, False), (small, True)):
+            codes, scales, x = fx.mlx_ternary_qmm_fixture(rows, cols, batch, scale_bits)
+            bias_scales = np.roll(scales, 1, axis=0) if separate_bias else scales
+            packed = fx.pack_signed_np(codes, fx.TERNARY2)
+            ref = so.ternary_affine_qmm(packed, scales, x, rows, cols, bias_scales=bias_scales)
+            want = ref.astype(np.float16).view(np.uint16).ravel()
+            wf = gh.WeightFile()
+            oc, os_, ob = wf.add(packed), wf.add(scales), wf.add(bias_scales)
+            auto_ctx.upload_weights(0, wf.image())
+            auto_ctx.put(gh.X_SLOT, x)
+            auto_ctx.alloc(gh.Y_SLOT, batch * rows * 2)
+            auto_ctx.encode_decode(rt.make_record(
+                auto_ctx.pipeline("signed_ternary_affine_qmm_g128_bm32_bn32_bk32"),
+                [(0, 0, oc), (0, 1, os_), (0, 2, ob), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)],
+                [(5, rows), (6, cols), (7, batch)], (1, (batch + 31) // 32, 1), (256, 1, 1)))
+            auto_ctx.wait()
+            assert np.array_equal(auto_ctx.read(gh.Y_SLOT, np.uint16, want.size), want), (cols, scale_bits, separate_bias)
