@@ -127,7 +127,7 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * kernel (the two add up a row in different orders: results agree to the output tolerance, not bit
  * for bit); MATRIX_CORE asks for the same explicitly (kept from when AUTO had size thresholds);
  * VECTOR keeps every record on the vector-ALU kernels.  The ternary qmm record takes a streaming kernel up to
- * 128 tokens (same dequantised fp16 weights, rows of a multiple of 512 columns).  Binary and ternary records over several tokens
+ * 128 tokens (same dequantised fp16 weights, rows of a multiple of 256 columns).  Binary and ternary records over several tokens
  * (the "_batched_b4" forms, per-token records with several grid rows) take the same kernel two tokens per
  * pass, each token's row bit for bit the one-token launch's.  The same switch
  * covers the qmm records (groups of 64, 128 and 32 columns; rows of a multiple of 256, 512 and 256 columns) and, from

@@ -497,10 +497,12 @@ __device__ __forceinline__ void qts_body(const uint8_t* __restrict__ W, const ui
     const int m0 = blockIdx.y * kQsTokens;
     const int last_tok = (batch < m0 + kQsTokens ? batch : m0 + kQsTokens) - 1;
 
-    // ---- (scale, -bias) of the sixteen rows and every group, plus one zero column: four or eight groups per thread
+    // ---- (scale, -bias) of the sixteen rows and every group, plus one zero column: eight, four or two groups per
+    // thread (rows of a multiple of 1024, 512 or 256 columns; the scale rows start on 16-, 8- or 4-byte boundaries)
     const bool half_runs = (gt & 7) != 0;
-    const int run_len = half_runs ? 4 : 8;
-    const int runs = half_runs ? gt >> 2 : gt >> 3;
+    const bool quarter_runs = (gt & 3) != 0;
+    const int run_len = quarter_runs ? 2 : (half_runs ? 4 : 8);
+    const int runs = gt / run_len;
     const int items = 16 * runs;
     uint32_t* lds_sb = reinterpret_cast<uint32_t*>(smem);
     const int sstride = gt + 1;
@@ -511,7 +513,10 @@ __device__ __forceinline__ void qts_body(const uint8_t* __restrict__ W, const ui
         int r = row0 + srow;
         if (r > rows - 1) r = rows - 1;
         ScaleRun out;
-        if (half_runs) {
+        if (quarter_runs) {
+            out.s = uint4_t{*reinterpret_cast<const uint32_t*>(S + (size_t)r * gt + 2 * run), 0u, 0u, 0u};
+            out.b = uint4_t{*reinterpret_cast<const uint32_t*>(B + (size_t)r * gt + 2 * run), 0u, 0u, 0u};
+        } else if (half_runs) {
             const uint2_t s2 = *reinterpret_cast<const uint2_t*>(S + (size_t)r * gt + 4 * run);
             const uint2_t b2 = *reinterpret_cast<const uint2_t*>(B + (size_t)r * gt + 4 * run);
             out.s = uint4_t{s2.x, s2.y, 0u, 0u};

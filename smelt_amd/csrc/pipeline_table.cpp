@@ -431,8 +431,8 @@ bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
 }
 
 bool qts_plan(uint32_t rows, uint32_t cols, uint32_t batch, size_t lds_limit, QmsPlan* out) {
-    // scale rows are staged four or eight groups at a time: rows of a multiple of 512 columns
-    if (rows == 0 || cols == 0 || cols % 512 != 0 || batch == 0) return false;
+    // scale rows are staged two, four or eight groups at a time: rows of a multiple of 256 columns
+    if (rows == 0 || cols == 0 || cols % 256 != 0 || batch == 0) return false;
     const uint32_t gt = cols / 128;
     uint32_t kc = (gt + 3) / 4;          // about four steps per wave, at most twelve waves, none idle
     if (kc < 1) kc = 1;

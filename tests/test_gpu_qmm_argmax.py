@@ -476,7 +476,7 @@ def test_ternary_qmm_streaming_kernel_reproduces_the_golden_bits_too(auto_ctx):
 
 
 @pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
-@pytest.mark.parametrize("shape", [(1003, 5120, 14), (40, 512, 6), (200, 17408, 33), (2050, 1536, 64), (96, 1024, 9)])
+@pytest.mark.parametrize("shape", [(1003, 5120, 14), (40, 512, 6), (200, 17408, 33), (2050, 1536, 64), (96, 1024, 9), (77, 2816, 20)])
 def test_ternary_qmm_streaming_kernel_shapes(ctx, auto_ctx, dtype, shape):
     """The streaming ternary qmm against the oracle's per-element fp16 dequantisation and against the token-slab
     kernel (one output step apart at most: the two add up a row in different orders): ragged rows, one to four
@@ -509,13 +509,13 @@ def test_ternary_qmm_streaming_kernel_shapes(ctx, auto_ctx, dtype, shape):
 
 
 def test_ternary_qmm_streaming_kernel_is_bit_exact_where_the_sums_are(auto_ctx):
-    """The MLX fixture of the golden test at 512 and 1024 columns (the streaming kernel takes multiples of 512; the
-    golden shape itself has 256 and keeps the token-slab kernel): every partial sum is exact, so the bits must be the
-    oracle's, with ordinary scales, with scales whose quarter, sixteenth and sixty-fourth round in the fp16
-    subnormal range, and with a separate bias plane."""
+    """The MLX fixture of the golden test at 512, 768 and 1024 columns (the golden shape itself, 256 columns, runs on the
+    streaming kernel in `test_ternary_qmm_streaming_kernel_reproduces_the_golden_bits_too`): every partial sum is exact,
+    so the bits must be the oracle's, with ordinary scales, with scales whose quarter, sixteenth and sixty-fourth round
+    in the fp16 subnormal range, and with a separate bias plane."""
     case = fx.golden_vectors()["ternary_qmm_mlx_m14"]
     small = ["1b95", "1797", "1b93", "17ff", "1a01"]
-    for cols, rows, batch in ((512, 24, 14), (1024, 40, 37)):
+    for cols, rows, batch in ((512, 24, 14), (1024, 40, 37), (768, 19, 9)):
         for scale_bits, separate_bias in ((case["scale_bits"], False), (small, False), (small, True)):
             codes, scales, x = fx.mlx_ternary_qmm_fixture(rows, cols, batch, scale_bits)
             bias_scales = np.roll(scales, 1, axis=0) if separate_bias else scales
