@@ -661,6 +661,273 @@ __device__ __forceinline__ void qts_body(const uint8_t* __restrict__ W, const ui
         smelt::qts_body<ACT, XRV>(C, S, B, X, Y, (int)batch, (int)rows, (int)cols);                \
     }
 
+// ---- binary and ternary codes (groups of 128 columns) over many tokens ------------------------------
+// The per-token records of the signed formats (one grid row per token) from eight tokens on, fp16 activations:
+// the skeleton of qts_body with exact operands (2 code - 1 for one-bit codes, code - 1 for two-bit codes, as fp16)
+// and the group's scale applied in fp32 to each step's sums, i.e. the arithmetic of the single-token kernels in
+// another summation order.  NMAT = 2: gate and up of one tile (the fused SwiGLU form).  Epilogues are the
+// single-token kernels' ((token, row, sums)).
+namespace smelt {
+
+template <int BITS, int NMAT, int XR, class Epi>
+__device__ __forceinline__ void qss_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
+                                         const uint16_t* __restrict__ X, int batch, int rows, int cols, const Epi& epi) {
+    using E = Elem16<F16>;
+    static_assert(BITS == 1 || BITS == 2, "one- or two-bit codes");
+    constexpr int kWB = 16 * BITS;            // bytes of a row per 128-column step
+    constexpr int kWStride = kWB + 8;         // staged, with padding
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int chunk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int kc = blockDim.x / kWave;
+    const int n = lane & 15, q = lane >> 4;
+    const int gt = cols >> 7;
+    const int rs = gt * kWB;
+    const int row0 = blockIdx.x * 16;
+    const int m0 = blockIdx.y * kQsTokens;
+    const int last_tok = (batch < m0 + kQsTokens ? batch : m0 + kQsTokens) - 1;
+
+    // ---- scales of the tile (fp32), plus one zero column: eight, four or two groups per thread
+    const bool half_runs = (gt & 7) != 0, quarter_runs = (gt & 3) != 0;
+    const int run_len = quarter_runs ? 2 : (half_runs ? 4 : 8);
+    const int runs = gt / run_len;
+    const int items = NMAT * 16 * runs;
+    float* lds_s = reinterpret_cast<float*>(smem);
+    const int sstride = gt + 1;
+    struct ScaleRun { uint4_t s; int at; };
+    auto load_scales = [&](int item) {
+        if (item > items - 1) item = items - 1;
+        const int srow = item / runs, run = item - srow * runs;   // srow = matrix * 16 + row in tile
+        const int m = srow >> 4;
+        int r = row0 + (srow & 15);
+        if (r > rows - 1) r = rows - 1;
+        const uint16_t* sp = NMAT > 1 && m == 1 ? S[NMAT - 1] : S[0];
+        ScaleRun out;
+        if (quarter_runs) out.s = uint4_t{*reinterpret_cast<const uint32_t*>(sp + (size_t)r * gt + 2 * run), 0u, 0u, 0u};
+        else if (half_runs) {
+            const uint2_t s2 = *reinterpret_cast<const uint2_t*>(sp + (size_t)r * gt + 4 * run);
+            out.s = uint4_t{s2.x, s2.y, 0u, 0u};
+        } else out.s = *reinterpret_cast<const uint4_t*>(sp + (size_t)r * gt + 8 * run);
+        out.at = srow * sstride + run_len * run;
+        return out;
+    };
+    auto store_scales = [&](const ScaleRun& v) {
+        const uint32_t sd[4] = {v.s.x, v.s.y, v.s.z, v.s.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (e < run_len) lds_s[v.at + e] = F16::widen((uint16_t)(e & 1 ? sd[e >> 1] >> 16 : sd[e >> 1] & 0xFFFFu));
+    };
+    const ScaleRun first_run = load_scales((int)threadIdx.x);
+
+    constexpr size_t kWaveBytes = (size_t)4 * XR * kQsXStride + (size_t)NMAT * 16 * kWStride < (size_t)NMAT * 1024
+                                      ? (size_t)NMAT * 1024 : (size_t)4 * XR * kQsXStride + (size_t)NMAT * 16 * kWStride;
+    unsigned char* stage = smem + (size_t)NMAT * 16 * sstride * 4 + (size_t)chunk * kWaveBytes;
+    unsigned char* stage_w = stage + 4 * XR * kQsXStride;
+    const int x_tok = lane >> 4, x_piece = lane & 15;
+    const int w_row = lane >> 2, w_piece = lane & 3;
+    const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    float4_t acc[NMAT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) acc[m] = zero;
+
+    struct Step { uint4_t x[XR]; uint32_t w[NMAT][BITS]; };
+    const uint16_t* x_base[XR];
+#pragma unroll
+    for (int r = 0; r < XR; ++r) {
+        int tok = m0 + 4 * r + x_tok;
+        if (tok > last_tok) tok = last_tok;
+        x_base[r] = X + (size_t)tok * cols + 8 * x_piece;
+    }
+    const uint8_t* w_base[NMAT];
+    {
+        int r = row0 + w_row;
+        if (r > rows - 1) r = rows - 1;
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) w_base[m] = W[m] + (size_t)r * rs + 4 * BITS * w_piece;
+    }
+    auto issue = [&](Step& st, int step) {
+        if (step > gt - 1) step = gt - 1;   // past the end: the last step again, under a zero scale
+#pragma unroll
+        for (int r = 0; r < XR; ++r) st.x[r] = *reinterpret_cast<const uint4_t*>(x_base[r] + 128 * step);
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int d = 0; d < BITS; ++d) st.w[m][d] = *reinterpret_cast<const uint32_t*>(w_base[m] + kWB * step + 4 * d);
+    };
+    auto consume = [&](const Step& st, int step) {
+#pragma unroll
+        for (int r = 0; r < XR; ++r)
+            *reinterpret_cast<uint4_t*>(stage + (4 * r + x_tok) * kQsXStride + 16 * x_piece) = st.x[r];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int d = 0; d < BITS; ++d)
+                *reinterpret_cast<uint32_t*>(stage_w + (m * 16 + w_row) * kWStride + 4 * BITS * w_piece + 4 * d) = st.w[m][d];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int gi = step < gt ? step : gt;   // the zero column
+        const half2v_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+        const half2v_t minus1 = {(_Float16)-1.0f, (_Float16)-1.0f};
+        const int xrow = XR == 4 ? n : (n & 7);
+        float4_t d[NMAT];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) d[m] = zero;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const unsigned char* xr = stage + xrow * kQsXStride + 128 * e + 32 * q;
+            const uint4_t a0 = *reinterpret_cast<const uint4_t*>(xr);
+            const uint4_t a1 = *reinterpret_cast<const uint4_t*>(xr + 16);
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                uint32_t bw[8];
+                if constexpr (BITS == 2) {
+                    const uint32_t c = *reinterpret_cast<const uint32_t*>(stage_w + (m * 16 + n) * kWStride + 16 * e + 4 * q);
+                    const half2v_t r01 = {(_Float16)1.0f, (_Float16)0.25f}, r23 = {(_Float16)0.0625f, (_Float16)0.015625f};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t rep = __builtin_amdgcn_perm(c, c, 0x0c000c00u | (uint32_t)j | ((uint32_t)j << 16));
+                        const half2v_t f01 = __builtin_bit_cast(half2v_t, and_or(rep, 0x000C0003u, 0x64006400u)) - k1024;
+                        const half2v_t f23 = __builtin_bit_cast(half2v_t, and_or(rep, 0x00C00030u, 0x64006400u)) - k1024;
+                        bw[2 * j] = __builtin_bit_cast(uint32_t, f01 * r01 + minus1);        // code - 1, exact
+                        bw[2 * j + 1] = __builtin_bit_cast(uint32_t, f23 * r23 + minus1);
+                    }
+                } else {
+                    const uint32_t c = *reinterpret_cast<const uint16_t*>(stage_w + (m * 16 + n) * kWStride + 8 * e + 2 * q);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const uint32_t rep = __builtin_amdgcn_perm(c, c, 0x0c000c00u | (uint32_t)j | ((uint32_t)j << 16));
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const uint32_t mask = (1u << (2 * r)) | (1u << (2 * r + 1 + 16));
+                            const half2v_t f = __builtin_bit_cast(half2v_t, and_or(rep, mask, 0x64006400u)) - k1024;
+                            const half2v_t rc = {(_Float16)(2.0f / (float)(1 << (2 * r))), (_Float16)(2.0f / (float)(1 << (2 * r + 1)))};
+                            bw[4 * j + r] = __builtin_bit_cast(uint32_t, f * rc + minus1);   // 2 bit - 1, exact
+                        }
+                    }
+                }
+                d[m] = E::mfma(a0, uint4_t{bw[0], bw[1], bw[2], bw[3]}, d[m]);
+                d[m] = E::mfma(a1, uint4_t{bw[4], bw[5], bw[6], bw[7]}, d[m]);
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            const float sc = lds_s[(m * 16 + n) * sstride + gi];
+            acc[m].x = __builtin_fmaf(sc, d[m].x, acc[m].x);
+            acc[m].y = __builtin_fmaf(sc, d[m].y, acc[m].y);
+            acc[m].z = __builtin_fmaf(sc, d[m].z, acc[m].z);
+            acc[m].w = __builtin_fmaf(sc, d[m].w, acc[m].w);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    Step s0, s1;
+    int step = chunk;
+    issue(s0, step);
+    issue(s1, step + kc);
+    store_scales(first_run);
+    for (int base = (int)blockDim.x; base < items; base += (int)blockDim.x) store_scales(load_scales(base + (int)threadIdx.x));
+    if (threadIdx.x < NMAT * 16) lds_s[threadIdx.x * sstride + gt] = 0.0f;
+    __syncthreads();
+    for (; step < gt; step += 2 * kc) {
+        consume(s0, step);
+        issue(s0, step + 2 * kc);
+        consume(s1, step + kc);
+        issue(s1, step + 3 * kc);
+    }
+
+    {
+        float4_t* mine = reinterpret_cast<float4_t*>(stage);
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) mine[m * kWave + lane] = acc[m];
+    }
+    __syncthreads();
+    if (chunk == 0) {
+        const unsigned char* first = smem + (size_t)NMAT * 16 * sstride * 4;
+        float4_t sum[NMAT];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) sum[m] = zero;
+        for (int c = 0; c < kc; ++c)
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                const float4_t part = reinterpret_cast<const float4_t*>(first + (size_t)c * kWaveBytes)[m * kWave + lane];
+                sum[m].x += part.x; sum[m].y += part.y; sum[m].z += part.z; sum[m].w += part.w;
+            }
+        const int r = row0 + n;
+        if (r < rows) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int tok = m0 + 4 * q + v;
+                if (tok <= last_tok) {
+                    float val[NMAT];
+#pragma unroll
+                    for (int m = 0; m < NMAT; ++m) val[m] = v == 0 ? sum[m].x : (v == 1 ? sum[m].y : (v == 2 ? sum[m].z : sum[m].w));
+                    epi(tok, r, val);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace smelt
+
+// Argument lists of the single-token kernels of the same pipelines plus the number of tokens.
+#define SMELT_SIGNED_QSS(FN, BITSV, XRV)                                                            \
+    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_matvec_f16(                              \
+        const uint8_t* C, const uint16_t* S, const uint16_t* X, uint16_t* Y, uint32_t rows,        \
+        uint32_t cols, uint32_t tokens) {                                                          \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {C};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        qss_body<BITSV, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiStore<F16>{{}, Y, (int)rows}); \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_matvec_add_f16(                          \
+        const uint8_t* C, const uint16_t* S, const uint16_t* X, uint16_t* Y, const uint16_t* res,  \
+        uint32_t rows, uint32_t cols, uint32_t tokens) {                                           \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {C};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        qss_body<BITSV, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiAdd<F16>{{}, Y, res, (int)rows}); \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_gate_up_swiglu_f16(                      \
+        const uint8_t* gC, const uint16_t* gS, const uint8_t* uC, const uint16_t* uS,              \
+        const uint16_t* X, uint16_t* Y, uint32_t rows, uint32_t cols, uint32_t tokens) {           \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gC, uC};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        qss_body<BITSV, 2, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiSignedSwiglu<F16>{{}, Y, (int)rows}); \
+    }
+
+// the ternary-affine names: the scale plane bound a second time is ignored, as in the single-token kernels
+#define SMELT_TERAFF_QSS(XRV)                                                                       \
+    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_matvec_f16(                                     \
+        const uint8_t* C, const uint16_t* S, const uint16_t*, const uint16_t* X, uint16_t* Y,      \
+        uint32_t rows, uint32_t cols, uint32_t tokens) {                                           \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {C};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        qss_body<2, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiStore<F16>{{}, Y, (int)rows}); \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_matvec_add_f16(                                 \
+        const uint8_t* C, const uint16_t* S, const uint16_t*, const uint16_t* X, uint16_t* Y,      \
+        const uint16_t* res, uint32_t rows, uint32_t cols, uint32_t tokens) {                      \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[1] = {C};                                                           \
+        const uint16_t* const s[1] = {S};                                                          \
+        qss_body<2, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiAdd<F16>{{}, Y, res, (int)rows}); \
+    }                                                                                              \
+    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_gate_up_swiglu_f16(                             \
+        const uint8_t* gC, const uint16_t* gS, const uint16_t*, const uint8_t* uC,                 \
+        const uint16_t* uS, const uint16_t*, const uint16_t* X, uint16_t* Y, uint32_t rows,        \
+        uint32_t cols, uint32_t tokens) {                                                          \
+        using namespace smelt;                                                                     \
+        const uint8_t* const w[2] = {gC, uC};                                                      \
+        const uint16_t* const s[2] = {gS, uS};                                                     \
+        qss_body<2, 2, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiSignedSwiglu<F16>{{}, Y, (int)rows}); \
+    }
+
 // ---- token-tile form: prefill chunks ------------------------------------------------------------
 // The same arithmetic for many tokens.  A workgroup of four waves (two along the rows, two along the
 // tokens) owns 32 * RT weight rows times 32 * TB tokens and walks K one pair of scale groups at a time.

@@ -452,6 +452,16 @@ bool qts_plan(uint32_t rows, uint32_t cols, uint32_t batch, size_t lds_limit, Qm
     return out->lds <= lds_limit;
 }
 
+bool qss_plan(uint32_t bits, uint32_t nmat, uint32_t rows, uint32_t cols, uint32_t batch, size_t lds_limit, QmsPlan* out) {
+    if ((bits != 1 && bits != 2) || nmat < 1 || nmat > 2 || !qts_plan(rows, cols, batch, lds_limit, out)) return false;
+    const uint32_t gt = cols / 128;
+    const size_t token_rows = batch > 8 ? 16 : 8;
+    size_t wave = token_rows * 272 + (size_t)nmat * 16 * (16 * bits + 8);
+    if (wave < (size_t)nmat * 1024) wave = (size_t)nmat * 1024;
+    out->lds = (size_t)nmat * 16 * (gt + 1) * 4 + out->kc * wave;
+    return out->lds <= lds_limit;
+}
+
 ResolveStatus resolve_pipeline(const std::string& entry_in, ActDType default_act,
                                size_t lds_limit, ResolvedPipeline* out, std::string* why) {
     const ResolveStatus st = resolve_pipeline_entry(entry_in, default_act, lds_limit, out, why);

@@ -170,6 +170,8 @@ bool qms_plan(uint32_t rows, uint32_t cols, uint32_t group, uint32_t nmat, uint3
 // Launch plan of the streaming ternary qmm (two-bit codes, groups of 128 columns): workgroups of `kc` waves over
 // sixteen rows, sixteen tokens per grid row, wave c takes the 128-column steps c, c + kc, ...
 bool qts_plan(uint32_t rows, uint32_t cols, uint32_t batch, size_t lds_limit, QmsPlan* out);
+// ... and of the streaming kernels of the binary (bits = 1) and ternary (2) per-token records over many tokens.
+bool qss_plan(uint32_t bits, uint32_t nmat, uint32_t rows, uint32_t cols, uint32_t batch, size_t lds_limit, QmsPlan* out);
 
 
 // Launch plan of the token-tile qmm: workgroups of 4 * kw waves over 32 * rt rows (per matrix) and

@@ -401,3 +401,68 @@ def test_ternary_affine_rows_over_several_tokens(dtype):
         gh.check_outputs(y, ref, dtype, "ternary affine rows, five tokens")
     finally:
         c.close()
+
+
+@pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")])
+@pytest.mark.parametrize("kind", ["matvec", "add", "gate_up"])
+@pytest.mark.parametrize("shape", [(1003, 5120, 13), (40, 768, 8), (264, 2560, 33)])
+def test_signed_rows_over_many_tokens_stream(fmt, name, kind, shape):
+    """Per-token binary and ternary records (one grid row per token) from eight tokens on, fp16 activations: the
+    streaming kernel of the format (the weights pass once per sixteen tokens).  Against the single-token kernel's
+    rows (the same exact operands and fp32 scales in another summation order: one output step at most for the
+    plain and +residual forms, the SwiGLU step bound for gate+up) and, for the plain matvec, the oracle."""
+    rows, cols, batch = shape
+    dtype = fx.F16
+    c = rt.Context()
+    try:
+        mats = []
+        for t in range(2 if kind == "gate_up" else 1):
+            codes = fx.synth_signed_codes(fmt, rows, cols, config=2 + fmt, tensor=10 + t)
+            mats.append((pack_signed(codes, fmt), fx.synth_signed_scales(rows, cols, config=2 + fmt, tensor=10 + t)))
+        x = fx.synth_activation(batch, cols, dtype, config=2 + fmt, tensor=78)
+        res = fx.to_bits(fx.rng_for(2, 79).normal(0, 1, (batch, rows)).astype(np.float32), dtype) if kind == "add" else None
+        second = mats[1] if kind == "gate_up" else None
+        y = run_signed(c, name, *mats[0], x, dtype, rows, cols, kind=kind, second=second, residual=res)
+        assert np.array_equal(y, run_signed(c, name, *mats[0], x, dtype, rows, cols, kind=kind, second=second, residual=res))
+        if kind == "add":
+            # the residual form is the plain form's rounded sums plus the residual, bit for bit (a comparison with the
+            # single-token rows would measure the projection's last place against a sum that may cancel)
+            plain = run_signed(c, name, *mats[0], x, dtype, rows, cols, kind="matvec")
+            assert np.array_equal(y, so.narrow(fx.from_bits(plain, dtype) + fx.from_bits(res, dtype), dtype))
+        else:
+            rows1 = np.concatenate([run_signed(c, name, *mats[0], x[b:b + 1], dtype, rows, cols, kind=kind, second=second)
+                                    for b in range(batch)])
+            gh.check_steps(y, rows1, dtype, f"{name} {kind} over {batch} tokens against single-token rows",
+                           max_steps=4 if kind == "gate_up" else 1, min_exact=0.8 if kind == "gate_up" else 0.9)
+        if kind == "matvec":
+            ref = so.signed_matvec(fmt, *mats[0], fx.from_bits(x, dtype), rows, cols, cols, 128)
+            gh.check_outputs(y, ref, dtype, f"{name} over {batch} tokens")
+    finally:
+        c.close()
+
+
+def test_ternary_affine_rows_over_many_tokens_stream():
+    """`signed_ternary_affine_matvec_g128_rows8` with one grid row per token at thirteen tokens (fp16): the streaming
+    kernel, the second binding of the scale plane ignored as in the single-token kernel."""
+    rows, cols, batch, dtype = 777, 2560, 13, fx.F16
+    c = rt.Context()
+    try:
+        codes = fx.synth_signed_codes(fx.TERNARY2, rows, cols, config=3, tensor=6)
+        scales = fx.synth_signed_scales(rows, cols, config=3, tensor=6)
+        other = np.roll(scales, 2, axis=0)
+        packed = fx.pack_signed_np(codes, fx.TERNARY2)
+        x = fx.synth_activation(batch, cols, dtype, config=3, tensor=16)
+        wf = gh.WeightFile()
+        oc, os_, oo = wf.add(packed), wf.add(scales), wf.add(other)
+        c.upload_weights(0, wf.image())
+        c.put(gh.X_SLOT, x)
+        c.alloc(gh.Y_SLOT, batch * rows * 2)
+        pipe = c.pipeline("signed_ternary_affine_matvec_g128_rows8")
+        bufs = [(0, 0, oc), (0, 1, os_), (0, 2, oo), (gh.X_SLOT, 3, 0), (gh.Y_SLOT, 4, 0)]
+        assert c.encode_decode(rt.make_record(pipe, bufs, [(5, rows), (6, cols)], ((rows + 7) // 8, batch, 1), (256, 1, 1))) == 1
+        c.wait()
+        y = c.read(gh.Y_SLOT, np.uint16, batch * rows).reshape(batch, rows)
+        ref = so.signed_matvec(so.TERNARY2, packed, scales, fx.from_bits(x, dtype), rows, cols, cols, 128)
+        gh.check_outputs(y, ref, dtype, "ternary affine rows, thirteen tokens")
+    finally:
+        c.close()
