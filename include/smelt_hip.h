@@ -129,8 +129,8 @@ int smelt_hip_set_activation_dtype(smelt_hip_context *ctx, int act_dtype);
  * VECTOR keeps every record on the vector-ALU kernels.  The ternary qmm record takes a streaming kernel up to
  * 128 tokens (same dequantised fp16 weights, rows of a multiple of 256 columns).  Binary and ternary records over several tokens
  * (the "_batched_b4" forms, per-token records with several grid rows) take the same kernel two tokens per
- * pass, each token's row bit for bit the one-token launch's; from eight tokens on, with fp16 activations, a
- * streaming kernel (the weights pass once per sixteen tokens; one output step from those rows at most).  The same switch
+ * pass, each token's row bit for bit the one-token launch's; from eight tokens on a streaming kernel (the
+ * weights pass once per sixteen tokens; bf16 rows converted to fp16; one output step from those rows at most).  The same switch
  * covers the qmm records (groups of 64, 128 and 32 columns; rows of a multiple of 256, 512 and 256 columns) and, from
  * two tokens on, the per-token small-batch ("_batched", "_batched_verify_b4")
  * forms of the affine matvec and gate+up+SwiGLU, whose arguments are the skinny qmm's (while

@@ -662,14 +662,14 @@ __device__ __forceinline__ void qts_body(const uint8_t* __restrict__ W, const ui
     }
 
 // ---- binary and ternary codes (groups of 128 columns) over many tokens ------------------------------
-// The per-token records of the signed formats (one grid row per token) from eight tokens on, fp16 activations:
+// The per-token records of the signed formats (one grid row per token) from eight tokens on (bf16 rows converted to fp16):
 // the skeleton of qts_body with exact operands (2 code - 1 for one-bit codes, code - 1 for two-bit codes, as fp16)
 // and the group's scale applied in fp32 to each step's sums, i.e. the arithmetic of the single-token kernels in
 // another summation order.  NMAT = 2: gate and up of one tile (the fused SwiGLU form).  Epilogues are the
 // single-token kernels' ((token, row, sums)).
 namespace smelt {
 
-template <int BITS, int NMAT, int XR, class Epi>
+template <class ActT, int BITS, int NMAT, int XR, class Epi>
 __device__ __forceinline__ void qss_body(const uint8_t* const (&W)[NMAT], const uint16_t* const (&S)[NMAT],
                                          const uint16_t* __restrict__ X, int batch, int rows, int cols, const Epi& epi) {
     using E = Elem16<F16>;
@@ -756,8 +756,17 @@ __device__ __forceinline__ void qss_body(const uint8_t* const (&W)[NMAT], const 
     };
     auto consume = [&](const Step& st, int step) {
 #pragma unroll
-        for (int r = 0; r < XR; ++r)
-            *reinterpret_cast<uint4_t*>(stage + (4 * r + x_tok) * kQsXStride + 16 * x_piece) = st.x[r];
+        for (int r = 0; r < XR; ++r) {
+            uint4_t v = st.x[r];
+            if (!ActT::kIsF16) {   // bf16 rows are multiplied as fp16, as in the vector kernels of these formats
+                uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    p[i] = (uint32_t)ActT::to_f16_bits((uint16_t)(p[i] & 0xFFFFu)) | ((uint32_t)ActT::to_f16_bits((uint16_t)(p[i] >> 16)) << 16);
+                v = uint4_t{p[0], p[1], p[2], p[3]};
+            }
+            *reinterpret_cast<uint4_t*>(stage + (4 * r + x_tok) * kQsXStride + 16 * x_piece) = v;
+        }
 #pragma unroll
         for (int m = 0; m < NMAT; ++m)
 #pragma unroll
@@ -874,58 +883,58 @@ __device__ __forceinline__ void qss_body(const uint8_t* const (&W)[NMAT], const 
 }  // namespace smelt
 
 // Argument lists of the single-token kernels of the same pipelines plus the number of tokens.
-#define SMELT_SIGNED_QSS(FN, BITSV, XRV)                                                            \
-    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_matvec_f16(                              \
+#define SMELT_SIGNED_QSS(FN, BITSV, XRV, T, ACT)                                                            \
+    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_matvec_##T(                              \
         const uint8_t* C, const uint16_t* S, const uint16_t* X, uint16_t* Y, uint32_t rows,        \
         uint32_t cols, uint32_t tokens) {                                                          \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {C};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
-        qss_body<BITSV, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiStore<F16>{{}, Y, (int)rows}); \
+        qss_body<ACT, BITSV, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiStore<ACT>{{}, Y, (int)rows}); \
     }                                                                                              \
-    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_matvec_add_f16(                          \
+    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_matvec_add_##T(                          \
         const uint8_t* C, const uint16_t* S, const uint16_t* X, uint16_t* Y, const uint16_t* res,  \
         uint32_t rows, uint32_t cols, uint32_t tokens) {                                           \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {C};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
-        qss_body<BITSV, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiAdd<F16>{{}, Y, res, (int)rows}); \
+        qss_body<ACT, BITSV, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiAdd<ACT>{{}, Y, res, (int)rows}); \
     }                                                                                              \
-    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_gate_up_swiglu_f16(                      \
+    SMELT_QMS_KERNEL void smelt_signed_##FN##_qss_x##XRV##_gate_up_swiglu_##T(                      \
         const uint8_t* gC, const uint16_t* gS, const uint8_t* uC, const uint16_t* uS,              \
         const uint16_t* X, uint16_t* Y, uint32_t rows, uint32_t cols, uint32_t tokens) {           \
         using namespace smelt;                                                                     \
         const uint8_t* const w[2] = {gC, uC};                                                      \
         const uint16_t* const s[2] = {gS, uS};                                                     \
-        qss_body<BITSV, 2, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiSignedSwiglu<F16>{{}, Y, (int)rows}); \
+        qss_body<ACT, BITSV, 2, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiSignedSwiglu<ACT>{{}, Y, (int)rows}); \
     }
 
 // the ternary-affine names: the scale plane bound a second time is ignored, as in the single-token kernels
-#define SMELT_TERAFF_QSS(XRV)                                                                       \
-    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_matvec_f16(                                     \
+#define SMELT_TERAFF_QSS(XRV, T, ACT)                                                                       \
+    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_matvec_##T(                                     \
         const uint8_t* C, const uint16_t* S, const uint16_t*, const uint16_t* X, uint16_t* Y,      \
         uint32_t rows, uint32_t cols, uint32_t tokens) {                                           \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {C};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
-        qss_body<2, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiStore<F16>{{}, Y, (int)rows}); \
+        qss_body<ACT, 2, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiStore<ACT>{{}, Y, (int)rows}); \
     }                                                                                              \
-    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_matvec_add_f16(                                 \
+    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_matvec_add_##T(                                 \
         const uint8_t* C, const uint16_t* S, const uint16_t*, const uint16_t* X, uint16_t* Y,      \
         const uint16_t* res, uint32_t rows, uint32_t cols, uint32_t tokens) {                      \
         using namespace smelt;                                                                     \
         const uint8_t* const w[1] = {C};                                                           \
         const uint16_t* const s[1] = {S};                                                          \
-        qss_body<2, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiAdd<F16>{{}, Y, res, (int)rows}); \
+        qss_body<ACT, 2, 1, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiAdd<ACT>{{}, Y, res, (int)rows}); \
     }                                                                                              \
-    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_gate_up_swiglu_f16(                             \
+    SMELT_QMS_KERNEL void smelt_teraff_qss_x##XRV##_gate_up_swiglu_##T(                             \
         const uint8_t* gC, const uint16_t* gS, const uint16_t*, const uint8_t* uC,                 \
         const uint16_t* uS, const uint16_t*, const uint16_t* X, uint16_t* Y, uint32_t rows,        \
         uint32_t cols, uint32_t tokens) {                                                          \
         using namespace smelt;                                                                     \
         const uint8_t* const w[2] = {gC, uC};                                                      \
         const uint16_t* const s[2] = {gS, uS};                                                     \
-        qss_body<2, 2, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiSignedSwiglu<F16>{{}, Y, (int)rows}); \
+        qss_body<ACT, 2, 2, XRV>(w, s, X, (int)tokens, (int)rows, (int)cols, EpiSignedSwiglu<ACT>{{}, Y, (int)rows}); \
     }
 
 // ---- token-tile form: prefill chunks ------------------------------------------------------------

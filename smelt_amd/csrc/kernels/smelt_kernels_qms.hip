@@ -15,7 +15,10 @@
 SMELT_QMS_ALL(f16, smelt::F16)
 SMELT_QMS_ALL(bf16, smelt::BF16)
 
-// binary and ternary per-token records over many tokens (fp16 activations)
-SMELT_SIGNED_QSS(binary, 1, 2) SMELT_SIGNED_QSS(binary, 1, 4)
-SMELT_SIGNED_QSS(ternary, 2, 2) SMELT_SIGNED_QSS(ternary, 2, 4)
-SMELT_TERAFF_QSS(2) SMELT_TERAFF_QSS(4)
+// binary and ternary per-token records over many tokens
+#define SMELT_QSS_ALL(T, ACT)                                                                      \
+    SMELT_SIGNED_QSS(binary, 1, 2, T, ACT) SMELT_SIGNED_QSS(binary, 1, 4, T, ACT)                  \
+    SMELT_SIGNED_QSS(ternary, 2, 2, T, ACT) SMELT_SIGNED_QSS(ternary, 2, 4, T, ACT)                \
+    SMELT_TERAFF_QSS(2, T, ACT) SMELT_TERAFF_QSS(4, T, ACT)
+SMELT_QSS_ALL(f16, smelt::F16)
+SMELT_QSS_ALL(bf16, smelt::BF16)

@@ -49,7 +49,7 @@ struct Pipeline {
     hipFunction_t fn_qmt_per_wave[5][5][3] = {};                  // ... with one matrix per wave along the rows (gate and up)
     hipFunction_t fn_qms[kQmsMaxRowTiles + 1][2] = {};            // streaming skinny qmm, by row tiles per wave and 8 / 16 staged token rows
     hipFunction_t fn_qms_g32[2] = {};                             // ... for groups of 32 columns
-    hipFunction_t fn_qss[2] = {};                                 // binary / ternary per-token records over many tokens (fp16)
+    hipFunction_t fn_qss[2] = {};                                 // binary / ternary per-token records over many tokens
     hipFunction_t fn_tqs[2] = {};                                 // streaming ternary qmm, eight / sixteen staged token rows
     hipFunction_t fn_norm_rows = nullptr;                         // norm-scale qmm: the normalised rows, written once
     hipFunction_t fn_logits_keys = nullptr;                       // lm_head over several tokens: partial argmax keys from stored logits
@@ -1150,7 +1150,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             L.grid[0] = (rows + 7) / 8; L.grid[1] = tokens; L.grid[2] = 1;
             // binary and ternary codes from two tokens on: two tokens per pass (the weights are unpacked and multiplied
             // once for both; the token count is the kernels' last argument: the four-token forms bring it along)
-            // ... and from eight tokens on (fp16 activations, rows of a multiple of 256 columns) the streaming kernel
+            // ... and from eight tokens on (rows of a multiple of 256 columns; bf16 rows converted to fp16) the streaming kernel
             // of the format: the weights pass once per sixteen tokens
             // (cold, binary gate+up 2 x 17408 x 5120 at 8 / 16 / 32 / 64 tokens: 20 / 23 / 36 / 67 us against 47 / 89 / 173 / 325
             // two tokens per pass; binary 5120 x 5120 7.5 / 9.6 / 12 / 20 against 11 / 19 / 33 / 62; 2048 x 2048 at eight 4.3 against 4.0)
@@ -1625,7 +1625,7 @@ int smelt_hip_pipeline_create(smelt_hip_context* ctx, const char* entry, int all
                 }
             }
             if (p.res.family == kFamAffineArgmax) (void)find(&p.fn_logits_keys, "smelt_logits_argmax_partials");
-            if (p.res.act == kActF16 && !p.res.mm1_prefix.empty() && p.res.mm1_prefix.size() > 4 &&
+            if (!p.res.mm1_prefix.empty() && p.res.mm1_prefix.size() > 4 &&
                 (p.res.mm1_layout == (int)kCodesBinary1 || p.res.mm1_layout == (int)kCodesTernary2))
                 for (uint32_t wide = 0; wide < 2; ++wide)
                     (void)find(&p.fn_qss[wide], p.res.mm1_prefix.substr(0, p.res.mm1_prefix.size() - 4) + (wide ? "qss_x4_" : "qss_x2_") + p.res.mm1_tail);

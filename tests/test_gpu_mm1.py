@@ -406,13 +406,13 @@ def test_ternary_affine_rows_over_several_tokens(dtype):
 @pytest.mark.parametrize("fmt,name", [(fx.BINARY1, "binary"), (fx.TERNARY2, "ternary")])
 @pytest.mark.parametrize("kind", ["matvec", "add", "gate_up"])
 @pytest.mark.parametrize("shape", [(1003, 5120, 13), (40, 768, 8), (264, 2560, 33)])
-def test_signed_rows_over_many_tokens_stream(fmt, name, kind, shape):
-    """Per-token binary and ternary records (one grid row per token) from eight tokens on, fp16 activations: the
+@pytest.mark.parametrize("dtype", [fx.F16, fx.BF16])
+def test_signed_rows_over_many_tokens_stream(fmt, name, kind, shape, dtype):
+    """Per-token binary and ternary records (one grid row per token) from eight tokens on (bf16 rows converted to fp16): the
     streaming kernel of the format (the weights pass once per sixteen tokens).  Against the single-token kernel's
     rows (the same exact operands and fp32 scales in another summation order: one output step at most for the
     plain and +residual forms, the SwiGLU step bound for gate+up) and, for the plain matvec, the oracle."""
     rows, cols, batch = shape
-    dtype = fx.F16
     c = rt.Context()
     try:
         mats = []
