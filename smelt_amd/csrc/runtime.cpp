@@ -1155,13 +1155,13 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
             // (cold, binary gate+up 2 x 17408 x 5120 at 8 / 16 / 32 / 64 tokens: 20 / 23 / 36 / 67 us against 47 / 89 / 173 / 325
             // two tokens per pass; binary 5120 x 5120 7.5 / 9.6 / 12 / 20 against 11 / 19 / 33 / 62; 2048 x 2048 at eight 4.3 against 4.0)
             QmsPlan splan;
-            if (mm1_per_row && tokens >= 8u && p->fn_qss[tokens > 8] &&
+            if ((mm1_per_row || mm1_b4) && tokens >= 8u && p->fn_qss[tokens > 8] &&
                 qss_plan(p->res.mm1_layout == (int)kCodesBinary1 ? 1 : 2, p->res.mm1_nmat, rows, cols, tokens, ctx->lds_limit, &splan)) {
                 fn = p->fn_qss[tokens > 8];
                 L.grid[0] = (rows + 15) / 16; L.grid[1] = (tokens + 15) / 16; L.grid[2] = 1;
                 L.block[0] = 64 * splan.kc; L.block[1] = 1; L.block[2] = 1;
                 L.lds = splan.lds;
-                Arg a; a.kind = 'U'; a.value = tokens; L.args.push_back(a);
+                if (!mm1_b4) { Arg a; a.kind = 'U'; a.value = tokens; L.args.push_back(a); }   // (the four-token forms bring the count along)
                 routed = true;
             }
             const bool streamed = routed;
@@ -1174,7 +1174,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
                 fn = p->fn_mm1_t2[plan.nl];
                 L.grid[1] = (tokens + 1) / 2;
                 if (!mm1_b4) { Arg a; a.kind = 'U'; a.value = tokens; L.args.push_back(a); }
-            } else if (mm1_b4) L.args.count -= 1;
+            } else if (mm1_b4 && !streamed) L.args.count -= 1;
             if (mm1_small_batch) {
                 // W S B X Y batch rows cols group tile -> W S B X Y rows cols group
                 const size_t o = mm1_pair_batch ? 8 : 5;

@@ -424,6 +424,9 @@ def test_signed_rows_over_many_tokens_stream(fmt, name, kind, shape, dtype):
         second = mats[1] if kind == "gate_up" else None
         y = run_signed(c, name, *mats[0], x, dtype, rows, cols, kind=kind, second=second, residual=res)
         assert np.array_equal(y, run_signed(c, name, *mats[0], x, dtype, rows, cols, kind=kind, second=second, residual=res))
+        if kind != "add":
+            # the four-token form of the same record takes the same kernel
+            assert np.array_equal(y, run_signed(c, name, *mats[0], x, dtype, rows, cols, kind=kind, second=second, b4=True))
         if kind == "add":
             # the residual form is the plain form's rounded sums plus the residual, bit for bit (a comparison with the
             # single-token rows would measure the projection's last place against a sum that may cancel)
