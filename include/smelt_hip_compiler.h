@@ -228,8 +228,11 @@ int smelt_hip_resolve_pipeline_name(const char *entry, int default_act, char *sy
  * what a record will run).  Each writes its answer as unsigned 32-bit fields and returns 1 when
  * the shape takes the kernel, 0 when it keeps the kernel its pipeline names, negative on error.
  *
- * smelt_hip_plan_qmm: an affine g64 qmm record (plain, +add: nmat 1; gate+up: nmat 2) of `batch`
- * tokens.  out[0] = 1 streaming kernel, 2 token-tile kernel; out[1] row tiles per wave;
+ * smelt_hip_plan_qmm: an affine qmm record (groups of 64, 128 or 32 columns; plain, +add: nmat 1;
+ * gate+up: nmat 2) of `batch` tokens.  (The plans of the other re-routed forms are not exposed here: the per-token
+ * small-batch names of small matrices, which take the single-token kernel with a grid row per token, the norm-scale
+ * qmm names, which run as normalised rows plus this plan, the ternary qmm and the binary / ternary records over
+ * several tokens.)  out[0] = 1 streaming kernel, 2 token-tile kernel; out[1] row tiles per wave;
  * out[2] waves along K (streaming: waves of the workgroup); out[3] = 1 when the two matrices go to
  * separate waves; out[4] workgroups that share a tile along K; out[5..7] grid; out[8] threads;
  * out[9] LDS bytes; out[10] workspace bytes of the K split (low 32 bits).
