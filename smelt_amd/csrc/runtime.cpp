@@ -1104,7 +1104,7 @@ int encode_record(smelt_hip_context* ctx, const SmeltDispatchRecord* rec, int cu
     }
     if (p->res.mm1_layout >= 0 && ctx->matvec_engine != SMELT_HIP_MATVEC_VECTOR && p->res.family != kFamAffineArgmax &&
         (!mm1_batch_family || mm1_small_batch)) {
-        // large single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
+        // single-token matvecs: the single-pass matrix-core kernel of the same pipeline, same
         // arguments, its own launch geometry (one workgroup per eight rows)
         // (every single-token kernel takes its token from the grid row: a record with several rows is one launch per token
         // of the same kernel, each row the one-token launch's bits)
