@@ -569,3 +569,45 @@ def test_generated_small_batch_and_dual_add_names(vector_ctx, dtype):
     gh.check_outputs(s2[:1], a2, dtype, "dual, second projection")
     assert np.array_equal(y1, so.epilogue_residual_add(fx.from_bits(s1[:1], dtype), r1, odt))
     assert np.array_equal(y2, so.epilogue_residual_add(fx.from_bits(s2[:1], dtype), r2, odt))
+
+
+def test_two_launch_routes_replay_in_a_graph(ctx):
+    """A captured table of records that the default engine runs as several launches (a norm-scale qmm: normalised rows
+    plus the streaming kernel; a norm-scale gate+up, whose rows live in the context workspace) replayed three times
+    with new inputs in between: every replay equals the eager result."""
+    rows, cols, group, dtype, batch = 640, 1024, 64, fx.BF16, 11
+    weights = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=2)
+    gw = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=3)
+    uw = fx.synth_affine(rows, cols, group, dtype, config=4, tensor=4)
+    wf = gh.WeightFile()
+    offs = [wf.add(a) for a in (*weights, *gw, *uw)]
+    ctx.upload_weights(gh.WEIGHTS_SLOT, wf.image())
+    F2 = 12
+    ctx.alloc(XN_SLOT, batch * cols * 2); ctx.alloc(gh.Y_SLOT, batch * rows * 2); ctx.alloc(F2, batch * rows * 2)
+    shape = f"_c{cols}_r{rows}_g{group}_batched_full"
+    t = gh.t_suffix(dtype)
+    r1 = rt.make_record(ctx.pipeline("norm_scale_affine_matvec" + shape + t),
+                        [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0), (XN_SLOT, 3, 0)] + [(0, 4 + i, offs[i]) for i in range(3)] +
+                        [(gh.Y_SLOT, 7, 0)], [(8, batch)], ((rows + 63) // 64, 1, 1), (256, 1, 1))
+    r2 = rt.make_record(ctx.pipeline("norm_scale_affine_gate_up_swiglu" + shape + t),
+                        [(RS_SLOT, 0, 0), (gh.X_SLOT, 1, 0), (NW_SLOT, 2, 0)] + [(0, 3 + i, offs[3 + i]) for i in range(6)] + [(F2, 9, 0)],
+                        [(10, batch)], ((rows + 63) // 64, 1, 1), (256, 1, 1))
+    table = ctx.table([r1, r2])
+    x0, w0, rs0 = norm_inputs(batch, cols, dtype, seed=5)
+    ctx.put(RS_SLOT, rs0); ctx.put(gh.X_SLOT, x0); ctx.put(NW_SLOT, w0)
+    graph, n = ctx.capture_decode(table)
+    assert n == 4
+    try:
+        for seed in (6, 7, 8):
+            x, w, rs = norm_inputs(batch, cols, dtype, seed=seed)
+            ctx.put(RS_SLOT, rs); ctx.put(gh.X_SLOT, x); ctx.put(NW_SLOT, w)
+            assert ctx.interpret_decode(table) == 4
+            ctx.wait()
+            eager = (ctx.read(gh.Y_SLOT, np.uint16, batch * rows).copy(), ctx.read(F2, np.uint16, batch * rows).copy())
+            ctx.put(gh.Y_SLOT, np.zeros(batch * rows, np.uint16)); ctx.put(F2, np.zeros(batch * rows, np.uint16))
+            ctx.graph_launch(graph); ctx.wait()
+            assert np.array_equal(ctx.read(gh.Y_SLOT, np.uint16, batch * rows), eager[0]), seed
+            assert np.array_equal(ctx.read(F2, np.uint16, batch * rows), eager[1]), seed
+            assert np.abs(fx.from_bits(eager[0], dtype)).max() > 0
+    finally:
+        ctx.graph_destroy(graph)
